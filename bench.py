@@ -1,0 +1,199 @@
+#!/usr/bin/env python3
+"""Benchmark of the paged KV-cache attention path on one MI355X.
+
+A step is one decode layer-step over one batch of synthetic input resident in HBM:
+KV append (one token per sequence) -> split-KV grouped-query decode map -> log-sum-exp combine.
+Default workload: batch 32, contexts uniform in [1024, 8192], 24 Q / 4 KV heads, head_dim 256,
+bf16 K/V in 16-token pages from a shuffled pool, 512-token partitions.
+
+Prints ONE JSON line.  `value` is the achieved HBM bandwidth of the whole layer-step (algorithmic
+bytes / wall time); `us_per_layer_step` is the time itself.  `roofline` prices the dominant kernel
+(the split-KV map) against the 8 TB/s HBM3E peak from its own HIP-event timings; `cpu_baseline`
+times the scalar CPU oracle on a bounded sample of the same workload on this box's host cores.
+"""
+import argparse
+import importlib
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBPS = 8000.0
+
+
+def parse_args():
+    p = argparse.ArgumentParser()
+    p.add_argument("--gpus", type=int, default=1)
+    p.add_argument("--steps", type=int, default=200)
+    p.add_argument("--warmup", type=int, default=20)
+    p.add_argument("--batch", type=int, default=32)
+    p.add_argument("--ctx-lo", type=int, default=1024)
+    p.add_argument("--ctx-hi", type=int, default=8192)
+    p.add_argument("--partition", type=int, default=512, help="split-KV partition length in tokens")
+    p.add_argument("--arenas", type=int, default=2, help="independent page arenas rotated between steps")
+    p.add_argument("--seed", type=int, default=2)
+    p.add_argument("--cpu-seconds", type=float, default=12.0, help="budget of the CPU baseline sample")
+    p.add_argument("--no-cpu-baseline", action="store_true")
+    p.add_argument("--kernel-only", action="store_true", help="time only the map kernel (for profiling runs)")
+    return p.parse_args()
+
+
+def read_profile_traffic(workload_key):
+    """HBM bytes per map launch measured with rocprofv3 --pmc (FETCH_SIZE + WRITE_SIZE), if the
+    committed summary covers this workload."""
+    path = os.path.join(ROOT, "profiles", "split_kv_decode_map_c2_pmc.txt")
+    try:
+        with open(path) as f:
+            text = f.read()
+    except OSError:
+        return None
+    if f"workload={workload_key}" not in text:
+        return None
+    for line in text.splitlines():
+        if line.startswith("traffic_bytes_per_launch="):
+            return float(line.split("=", 1)[1])
+    return None
+
+
+def cpu_baseline(psi, wl, w, dw, budget_s):
+    """Scalar oracle (a C restatement of the reference's sequential f32 oracle) on the first
+    requests of the batch, one thread, on this box's host cores."""
+    import numpy as np
+
+    from oracle import binding as oracle
+
+    dt = {0: oracle.F32, 1: oracle.BF16, 2: oracle.F16}[int(w.dtype)]
+    pages = dw.pages_host()
+    layout = (w.layout.num_req_slots, w.layout.num_gqa_layers, w.layout.num_blocks, w.layout.num_page_ids_per_block)
+    es = w.dtype.item_size()
+
+    def run(n_reqs, threads):
+        cu = w.cu_tokens[: n_reqs + 1]
+        t0 = time.perf_counter()
+        oracle.paged_gqa(w.num_q_heads, w.num_kv_heads, w.head_dim, w.scale, w.page_bytes, dt, layout, w.layer,
+                         w.req_slots[:n_reqs], w.token_indices[:n_reqs], cu, w.q[: int(cu[-1])], pages, w.page_ids,
+                         num_threads=threads)
+        dt_s = time.perf_counter() - t0
+        ctx = int(w.context_lens[:n_reqs].astype(np.int64).sum())
+        nbytes = ctx * 2 * w.num_kv_heads * w.head_dim * es + 2 * int(cu[-1]) * w.num_q_heads * w.head_dim * es
+        return dt_s, nbytes
+
+    t1, b1 = run(1, 1)
+    n = int(max(1, min(len(w.req_slots), budget_s / max(t1, 1e-3))))
+    t, b = (t1, b1) if n == 1 else run(n, 1)
+    cores = os.cpu_count() or 1
+    threads = min(cores, 16)
+    tp, bp = run(n, threads)
+    return {
+        "value": b / t / 1e9,
+        "unit": "GB/s",
+        "cores": 1,
+        "kind": "port",
+        "sample": f"attention of the first {n} of {len(w.req_slots)} requests of the same batch "
+                  f"({b / 1e6:.1f} MB algorithmic), scalar f32 oracle, {t:.2f} s",
+        "us_per_layer_step_extrapolated": t * 1e6 * (w.algorithmic_bytes() / b),
+        "openmp": {"value": bp / tp / 1e9, "unit": "GB/s", "cores": threads, "seconds": tp},
+    }
+
+
+def main():
+    args = parse_args()
+    if args.gpus != 1:
+        print(f"bench.py measures one GPU only (got --gpus {args.gpus}); the path does not shard in this build",
+              file=sys.stderr)
+        sys.exit(2)
+    import numpy as np
+    import torch
+
+    psi = importlib.import_module("psi-dec_amd")
+    wl = importlib.import_module("psi-dec_amd.workloads")
+    if not torch.cuda.is_available():
+        print("bench.py needs a GPU", file=sys.stderr)
+        sys.exit(1)
+    device = psi.Device(0)
+
+    arenas = []
+    for i in range(max(1, args.arenas)):
+        w = wl.config_c2(seed=args.seed, batch=args.batch, host_pages=False, lo=args.ctx_lo, hi=args.ctx_hi)
+        w.seed = args.seed + 1000 * i  # same geometry, different page contents
+        arenas.append(wl.DeviceWorkload(device, w, partition_tokens=args.partition))
+    w = arenas[0].w
+    shape = arenas[0].shape
+    step_bytes = w.algorithmic_bytes()
+    map_bytes = w.map_algorithmic_bytes()
+
+    def run_steps(n):
+        for i in range(n):
+            arenas[i % len(arenas)].step()
+
+    def run_maps(n):
+        for i in range(n):
+            arenas[i % len(arenas)].map()
+
+    body = run_maps if args.kernel_only else run_steps
+    body(args.warmup)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    body(args.steps)
+    torch.cuda.synchronize()
+    elapsed = time.perf_counter() - t0
+    ms_per_step = elapsed * 1e3 / args.steps
+
+    # Dominant kernel, timed by HIP events on the launch stream around every map launch.
+    device.set_timing(True)
+    device.reset_timing()
+    run_maps(min(args.steps, 100))
+    map_ms, map_launches = device.kernel_time_ms("split_kv_map")
+    device.set_timing(False)
+    map_avg_s = map_ms / max(map_launches, 1) / 1e3
+    achieved = map_bytes / map_avg_s / 1e9
+
+    workload_key = (f"decode_b{args.batch}_ctx{args.ctx_lo}-{args.ctx_hi}_24q4kv_d256_bf16_p16_part{args.partition}"
+                    f"_seed{args.seed}")
+    result = {
+        "metric": "decode attn achieved HBM GB/s per layer-step (B=32, ctx 1k-8k); us/layer-step alongside",
+        "value": (map_bytes if args.kernel_only else step_bytes) / (ms_per_step / 1e3) / 1e9,
+        "unit": "GB/s",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": ms_per_step,
+        "us_per_layer_step": ms_per_step * 1e3,
+        "hbm_frac_of_peak": (map_bytes if args.kernel_only else step_bytes) / (ms_per_step / 1e3) / 1e9 / HBM_PEAK_GBPS,
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "bf16",
+        "data": "synthetic",
+        "config": {
+            "workload": workload_key,
+            "step": "map kernel only" if args.kernel_only else "kv append -> split-KV map -> LSE combine",
+            "batch": args.batch,
+            "context_tokens_total": int(w.context_lens.astype(np.int64).sum()),
+            "kv_splits": shape.num_sdpa_map_task_templates,
+            "algorithmic_bytes_per_step": step_bytes,
+            "arenas_rotated": len(arenas),
+        },
+        "roofline": {
+            "bound": "hbm",
+            "kernel": "split_kv_decode_map",
+            "achieved": achieved,
+            "peak": HBM_PEAK_GBPS,
+            "unit": "GB/s",
+            "frac": achieved / HBM_PEAK_GBPS,
+            "traffic": read_profile_traffic(workload_key),
+            "algorithmic_bytes_per_launch": map_bytes,
+            "avg_launch_us": map_avg_s * 1e6,
+            "launches_timed": int(map_launches),
+        },
+    }
+    if not args.no_cpu_baseline:
+        result["cpu_baseline"] = cpu_baseline(psi, wl, w, arenas[0], args.cpu_seconds)
+    print(json.dumps(result))
+
+
+if __name__ == "__main__":
+    main()

@@ -1,0 +1,268 @@
+/*
+ * psi_hip.h -- C ABI of the MI355X (gfx950) paged KV-cache attention path.
+ *
+ * This is the layer an `inference-backend-hip` crate (a sibling of the reference's
+ * `inference-backend-metal`) binds: every entry point takes plain pointers and sizes, returns an
+ * `int` status, never throws and never aborts.  Device pointers are ordinary HIP device
+ * addresses owned by the caller; the library allocates no device memory in any entry point below.
+ *
+ * Status codes: 0 = ok; negative = error, text available from psi_hip_last_error() (per thread).
+ * Contract violations that make the reference `panic!`/`assert!` come back as
+ * PSI_HIP_ERR_INVALID_ARGUMENT with the reference's message.
+ *
+ * Each declaration cites the reference interface it replaces (paths relative to the reference
+ * repository root).
+ */
+#ifndef PSI_HIP_H
+#define PSI_HIP_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define PSI_HIP_OK 0
+#define PSI_HIP_ERR_INVALID_ARGUMENT (-1)
+#define PSI_HIP_ERR_RESOURCE_EXHAUSTED (-2)
+#define PSI_HIP_ERR_RUNTIME (-3)
+#define PSI_HIP_ERR_UNSUPPORTED (-4)
+
+/* Element type of q / K / V / pages / output.  The reference's `Dtype::{Float32, Bfloat16}`
+ * (crates/inference-backend-metal/src/components/gqa_split_kv.rs:33); F16 is added for the
+ * fp16-page configuration and is byte-compatible with the u16 page write. */
+#define PSI_HIP_F32 0u
+#define PSI_HIP_BF16 1u
+#define PSI_HIP_F16 2u
+
+#define PSI_HIP_SENTINEL 0xffffffffu /* padding value of kv_splits rows (u32::MAX) */
+
+/* SplitKV variant tags, `GQASplitKVVariant` (gqa_split_kv.rs:8-19). */
+#define PSI_HIP_VARIANT_SINGLE_Q 0u
+#define PSI_HIP_VARIANT_TILED_Q 1u
+
+typedef struct psi_hip_ctx psi_hip_ctx;
+
+/* Fixed workload facts: `GQASplitKVConfig` / `GQAKVPageWriteConfig` / `GQASplitKVSingleQConfig`
+ * (gqa_split_kv.rs:23-29, gqa_kv_page_write.rs:42-48, gqa_split_kv_single_q.rs:47-58).  `scale`
+ * is the model's attention scale; kernels never substitute 1/sqrt(head_dim). */
+typedef struct psi_hip_gqa_config {
+    uint32_t num_q_heads;
+    uint32_t num_kv_heads;
+    uint32_t head_dim;
+    float scale;
+    uint32_t page_bytes;
+    uint32_t dtype;
+} psi_hip_gqa_config;
+
+/* `GQAPageTableLayout`: u32 page_ids[num_req_slots][num_gqa_layers][num_blocks][num_page_ids_per_block]
+ * (crates/inference-executor-core/src/attn/gqa/core.rs:146-183). */
+typedef struct psi_hip_page_table_layout {
+    uint32_t num_req_slots;
+    uint32_t num_gqa_layers;
+    uint32_t num_blocks;
+    uint32_t num_page_ids_per_block;
+} psi_hip_page_table_layout;
+
+/* `GQASplitKVVariant` with its geometry (gqa_split_kv.rs:8-19).  SingleQ uses kv_token_tile_size,
+ * num_threads_per_threadblock, q_head_tile_size; TiledQ uses q_token_tile_size,
+ * kv_token_tile_size, q_head_tile_size.  The tile fields drive the metadata planner (split
+ * boundaries fall on kv_token_tile_size multiples); the HIP kernels choose their own launch shape. */
+typedef struct psi_hip_split_kv_variant {
+    uint32_t kind;
+    uint32_t q_token_tile_size;
+    uint32_t kv_token_tile_size;
+    uint32_t num_threads_per_threadblock;
+    uint32_t q_head_tile_size;
+} psi_hip_split_kv_variant;
+
+/* `GQAReplayShape` (core.rs:94-143). */
+typedef struct psi_hip_gqa_replay_shape {
+    uint32_t num_tokens;
+    uint32_t num_total_tokens;
+    uint32_t num_q_token_tiles;
+    uint32_t num_total_q_token_tiles;
+    uint32_t num_kv_splits;       /* num_sdpa_map_task_templates */
+    uint32_t num_total_kv_splits; /* num_total_sdpa_map_task_templates */
+    uint32_t reduce_sdpa_partial_outputs;
+} psi_hip_gqa_replay_shape;
+
+/* ------------------------------------------------------------------ library / context */
+
+const char* psi_hip_last_error(void);
+const char* psi_hip_version(void);
+
+/* Replaces `Device::system_default()` + `Stream::new` (crates/inference-backend-metal/src/metal/mod.rs:12-40).
+ * `stream` is a hipStream_t (NULL = the default stream); every launch of this context goes to
+ * it.  A context is confined to one thread, like the reference's executor. */
+int psi_hip_ctx_create(int device, void* stream, psi_hip_ctx** out_ctx);
+int psi_hip_ctx_destroy(psi_hip_ctx* ctx);
+int psi_hip_ctx_set_stream(psi_hip_ctx* ctx, void* stream);
+/* `ReplaySubmission::wait` (stream synchronisation). */
+int psi_hip_sync(psi_hip_ctx* ctx);
+/* Per-kernel timing for measurement harnesses: when enabled, every launch is bracketed by HIP
+ * events on the context's stream; psi_hip_ctx_kernel_time_ms drains them (synchronises) and
+ * returns the accumulated milliseconds and launch count of the kernel with that name
+ * ("kv_page_write", "split_kv_map", "split_kv_reduce", "tiled_q_map", "tiled_q_reduce"). */
+int psi_hip_ctx_set_timing(psi_hip_ctx* ctx, int enabled);
+int psi_hip_ctx_kernel_time_ms(psi_hip_ctx* ctx, const char* kernel, double* out_total_ms, uint64_t* out_launches);
+int psi_hip_ctx_reset_timing(psi_hip_ctx* ctx);
+/* Behaviour switches.  FORCE_GENERIC routes every attention launch to the shape-generic kernels
+ * (the cross-check variant, like the reference's `--validate` runs that compare two variants). */
+#define PSI_HIP_FLAG_FORCE_GENERIC 1u
+/* F32_OUTPUT makes the combine kernels store the attention output as f32 [tokens, Hq, D] instead of
+ * the io dtype, so a harness can check the f32-accumulated result before output rounding. */
+#define PSI_HIP_FLAG_F32_OUTPUT 2u
+int psi_hip_ctx_set_flag(psi_hip_ctx* ctx, uint32_t flag, uint32_t value);
+
+/* ------------------------------------------------------------------ geometry (host only) */
+
+/* `GQAKVPageWriteConfig::num_tokens_per_page` (gqa_kv_page_write.rs:57-70). */
+int psi_hip_gqa_tokens_per_page(const psi_hip_gqa_config* cfg, uint32_t* out_tokens_per_page);
+
+/* `GQASplitKV::new(config).select(num_tokens, num_q_token_tiles)` (gqa_split_kv.rs:86-156);
+ * dspark_history != 0 selects `new_dspark_history` (SingleQ partial layout only). */
+int psi_hip_split_kv_select(const psi_hip_gqa_config* cfg, int dspark_history, uint32_t num_tokens,
+                            uint32_t num_q_token_tiles, psi_hip_split_kv_variant* out_variant);
+/* `GQASplitKV::max_q_tokens_per_partial_output` (gqa_split_kv.rs:127-133). */
+int psi_hip_split_kv_max_q_tokens_per_partial_output(const psi_hip_gqa_config* cfg, int dspark_history,
+                                                     uint32_t* out);
+/* `select_split_kv_variant` (crates/inference-executor-metal/src/attn/gqa/mod.rs:64-94), including
+ * the (head_dim 256, 8 tokens/page) work model of mod.rs:96-316.  bucket_max_tokens = 0 means no
+ * replay bucket policy (exact power-of-two padding). */
+int psi_hip_split_kv_select_batch(const psi_hip_gqa_config* cfg, uint32_t max_tokens, uint32_t bucket_max_tokens,
+                                  const uint32_t* token_indices, const uint32_t* cu_tokens, uint32_t num_reqs,
+                                  psi_hip_split_kv_variant* out_variant);
+
+/* `ReplayBucketPolicy::with_topology_boundaries(max, boundaries).buckets()` and `.capacity(active)`
+ * (crates/inference-executor-core/src/replay.rs:4-87).  out_buckets may be NULL to query the count. */
+int psi_hip_replay_buckets(uint32_t max_capacity, const uint32_t* topology_boundaries, uint32_t num_boundaries,
+                           uint32_t* out_buckets, uint32_t buckets_capacity, uint32_t* out_num_buckets);
+int psi_hip_replay_bucket_capacity(uint32_t max_capacity, const uint32_t* topology_boundaries,
+                                   uint32_t num_boundaries, uint32_t active, uint32_t* out_capacity);
+
+/* ------------------------------------------------------------------ batch metadata (host only) */
+
+#define PSI_HIP_CAPACITY_EXACT 0u             /* `GQAMetadataBuffers::update` */
+#define PSI_HIP_CAPACITY_BUCKETED 1u          /* `update_bucketed` */
+#define PSI_HIP_CAPACITY_CALLER_TOKENS 2u     /* `update_bucketed_with_token_capacity` */
+#define PSI_HIP_CAPACITY_FIXED_PARTITION 3u   /* fixed-length partitions; not in the reference */
+
+/* `GQAMetadataBuffers::update*` (crates/inference-executor-metal/src/attn/gqa/batch_metadata.rs:128-317)
+ * with `build_single_q_kv_splits` (:352-424) and `build_tiled_q_kv_splits` (:433-523).
+ * Host arrays, each with capacity for max_tokens entries as in `GQAMetadataBuffers::new` (:92-126):
+ *   req_slots_by_token[max_tokens], flat_token_indices[max_tokens], q_token_tiles[max_tokens][2],
+ *   kv_splits[max_tokens][3], cu_kv_splits[max_tokens + 1].
+ * Only the ranges the reference writes are written (tails keep the caller's bytes); kv_splits is
+ * padded with PSI_HIP_SENTINEL up to shape->num_total_kv_splits rows.
+ * capacity_mode FIXED_PARTITION ignores the greedy budget: token t gets ceil(ctx_t / partition_tokens)
+ * splits of partition_tokens (a multiple of variant->kv_token_tile_size); kv_splits must then hold
+ * `kv_splits_capacity` rows (>= the plan) and is padded to the bucketed/exact capacity within it. */
+int psi_hip_gqa_metadata_update(uint32_t max_tokens, const uint32_t* req_slots, const uint32_t* token_indices,
+                                const uint32_t* cu_tokens, uint32_t num_reqs,
+                                const psi_hip_split_kv_variant* variant, uint32_t capacity_mode,
+                                uint32_t caller_num_total_tokens, const uint32_t* topology_boundaries,
+                                uint32_t num_boundaries, uint32_t partition_tokens, uint32_t kv_splits_capacity,
+                                uint32_t* req_slots_by_token, uint32_t* flat_token_indices,
+                                uint32_t* q_token_tiles, uint32_t* kv_splits, uint32_t* cu_kv_splits,
+                                psi_hip_gqa_replay_shape* out_shape);
+
+/* ------------------------------------------------------------------ KV append */
+
+/* `GQAKVPageWrite::invoke_bucketed(...)` recorded and submitted
+ * (crates/inference-backend-metal/src/components/gqa_kv_page_write.rs:130-234; kernel
+ * metal/gqa_kv_page_write.metal:5-53).  Argument order follows the Metal binding indices 0..10.
+ * pages: device, the page arena (written); pages_bytes bounds it (0 = unchecked).
+ * flat_k, flat_v: device [num_total_token_writes, num_kv_heads, head_dim].
+ * req_slots, flat_token_indices: device u32[num_total_token_writes].
+ * page_ids: device u32 table laid out per `layout`.
+ * Writes with index >= num_active_token_writes touch nothing. */
+int psi_hip_kv_page_write(psi_hip_ctx* ctx, const psi_hip_gqa_config* cfg, const psi_hip_page_table_layout* layout,
+                          void* pages, uint64_t pages_bytes, const void* flat_k, const void* flat_v,
+                          const uint32_t* req_slots, const uint32_t* flat_token_indices, const uint32_t* page_ids,
+                          uint32_t num_total_token_writes, uint32_t num_active_token_writes,
+                          uint32_t gqa_layer_index);
+
+/* ------------------------------------------------------------------ split-KV decode (SingleQ) */
+
+/* Scratch for the partial states of `num_total_kv_splits` splits: replaces `GQASplitKVSingleQScratch::new`
+ * (gqa_split_kv_single_q.rs:236-246).  The layout is private to the library. */
+int psi_hip_split_kv_single_q_scratch_bytes(const psi_hip_gqa_config* cfg, uint32_t num_total_kv_splits,
+                                            uint64_t* out_bytes);
+
+/* `GQASplitKVSingleQKernels::invoke_map_bucketed` (gqa_split_kv_single_q.rs:320-351; kernel
+ * metal/gqa_split_kv_single_q_map.metal:31-253).  q: device [num_total_tokens, Hq, D];
+ * kv_splits: device u32[num_total_kv_splits][3] = {q_token, kv_begin, kv_end}; rows whose
+ * q_token >= num_active_tokens (sentinel padding) and rows >= num_active_kv_splits write nothing. */
+int psi_hip_split_kv_single_q_map(psi_hip_ctx* ctx, const psi_hip_gqa_config* cfg,
+                                  const psi_hip_page_table_layout* layout, const void* q, const void* kv_pages,
+                                  uint64_t kv_pages_bytes, const uint32_t* req_slots, const uint32_t* page_ids,
+                                  const uint32_t* kv_splits, void* scratch, uint64_t scratch_bytes,
+                                  uint32_t gqa_layer_index, uint32_t num_total_tokens,
+                                  uint32_t num_total_kv_splits, uint32_t num_active_tokens,
+                                  uint32_t num_active_kv_splits);
+
+/* `GQASplitKVSingleQKernels::invoke_reduce_bucketed` (gqa_split_kv_single_q.rs:353-383; kernel
+ * metal/gqa_split_kv_single_q_reduce.metal:10-49).  cu_kv_splits: device u32[num_total_tokens + 1];
+ * output: device [num_total_tokens, Hq, D]; rows >= num_active_tokens keep their bytes. */
+int psi_hip_split_kv_single_q_reduce(psi_hip_ctx* ctx, const psi_hip_gqa_config* cfg, const void* scratch,
+                                     uint64_t scratch_bytes, const uint32_t* cu_kv_splits, void* output,
+                                     uint32_t num_total_tokens, uint32_t num_total_kv_splits,
+                                     uint32_t num_active_tokens);
+
+/* ------------------------------------------------------------------ split-KV verify / prefill (TiledQ) */
+
+/* `GQASplitKVTiledQConfig::partial_output_bytes + 2 * partial_output_stats_bytes`
+ * (gqa_split_kv_tiled_q.rs:131-157). */
+int psi_hip_split_kv_tiled_q_scratch_bytes(const psi_hip_gqa_config* cfg, uint32_t q_token_tile_size,
+                                           uint32_t num_total_kv_splits, uint64_t* out_bytes);
+
+/* `GQASplitKVTiledQKernels::invoke_map_bucketed` (gqa_split_kv_tiled_q.rs:279-300; kernel
+ * metal/gqa_split_kv_tiled_q.metal:49-319).  q_token_tiles: device u32[num_total_q_token_tiles][2];
+ * kv_splits rows index q-token tiles.  Causal mask: key position > flat_token_indices[q] is hidden. */
+int psi_hip_split_kv_tiled_q_map(psi_hip_ctx* ctx, const psi_hip_gqa_config* cfg,
+                                 const psi_hip_page_table_layout* layout, uint32_t q_token_tile_size,
+                                 const void* q, const void* kv_pages, uint64_t kv_pages_bytes,
+                                 const uint32_t* req_slots, const uint32_t* page_ids,
+                                 const uint32_t* flat_token_indices, const uint32_t* q_token_tiles,
+                                 const uint32_t* kv_splits, void* scratch, uint64_t scratch_bytes,
+                                 uint32_t gqa_layer_index, uint32_t num_total_tokens,
+                                 uint32_t num_total_q_token_tiles, uint32_t num_total_kv_splits,
+                                 uint32_t num_active_tokens, uint32_t num_active_q_token_tiles,
+                                 uint32_t num_active_kv_splits);
+
+/* `GQASplitKVTiledQKernels::invoke_reduce_bucketed` (gqa_split_kv_tiled_q.rs:314-327; kernel
+ * metal/gqa_split_kv_tiled_q.metal:324-378). */
+int psi_hip_split_kv_tiled_q_reduce(psi_hip_ctx* ctx, const psi_hip_gqa_config* cfg, uint32_t q_token_tile_size,
+                                    const void* scratch, uint64_t scratch_bytes, const uint32_t* q_token_tiles,
+                                    const uint32_t* cu_kv_splits, void* output, uint32_t num_total_tokens,
+                                    uint32_t num_total_q_token_tiles, uint32_t num_total_kv_splits,
+                                    uint32_t num_active_q_token_tiles);
+
+/* ------------------------------------------------------------------ request page table */
+
+/* `GQARequestPageTable::write_page_ids` (crates/inference-executor-metal/src/attn/gqa/request_page_table.rs:58-69):
+ * copies `count` (= num_page_ids_per_block) host IDs into the device table row
+ * (req_slot, layer_index, block_index) on the context's stream.  IDs >= num_cache_pages are
+ * rejected (crates/inference-executor-metal/src/model/qwen/v3_x/state/gqa.rs:97-102); 0 = unchecked. */
+int psi_hip_page_table_write_page_ids(psi_hip_ctx* ctx, const psi_hip_page_table_layout* layout,
+                                      uint32_t* page_ids_device, uint32_t req_slot, uint32_t layer_index,
+                                      uint32_t block_index, const uint32_t* ids, uint32_t count,
+                                      uint32_t num_cache_pages);
+/* `GQARequestPageTable::reset_req_slot` (request_page_table.rs:71-77): zeroes one slot's rows. */
+int psi_hip_page_table_reset_req_slot(psi_hip_ctx* ctx, const psi_hip_page_table_layout* layout,
+                                      uint32_t* page_ids_device, uint32_t req_slot);
+/* Flat index of (req_slot, layer, block, 0), `page_ids_start_index` (request_page_table.rs:112-117). */
+int psi_hip_page_table_start_index(const psi_hip_page_table_layout* layout, uint32_t req_slot,
+                                   uint32_t layer_index, uint32_t block_index, uint64_t* out_index);
+/* `page_ids_by_layer_for_lane` (crates/inference-executor-core/src/model/replayable_model.rs:182-212):
+ * splits one synced block's flat list [layer][id] into per-layer rows; block_ids has
+ * num_gqa_layers * num_page_ids_per_block entries, out_by_layer the same count (layer-major). */
+int psi_hip_page_ids_by_layer(const uint32_t* block_ids, uint32_t block_ids_len, uint32_t num_gqa_layers,
+                              uint32_t num_page_ids_per_block, uint32_t* out_by_layer);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* PSI_HIP_H */

@@ -1,0 +1,166 @@
+"""ctypes binding of libpsi_hip.so (the C ABI declared in include/psi_hip.h).
+
+The library is loaded from psi-dec_amd/lib/; there is no CPU fallback: if the shared object is
+missing, `load()` raises with the build command.
+"""
+import ctypes
+import os
+from ctypes import POINTER, c_char_p, c_double, c_float, c_int, c_uint32, c_uint64, c_void_p
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(_HERE, "lib", "libpsi_hip.so")
+
+OK = 0
+ERR_INVALID_ARGUMENT = -1
+ERR_RESOURCE_EXHAUSTED = -2
+ERR_RUNTIME = -3
+ERR_UNSUPPORTED = -4
+
+F32, BF16, F16 = 0, 1, 2
+SENTINEL = 0xFFFFFFFF
+VARIANT_SINGLE_Q, VARIANT_TILED_Q = 0, 1
+CAPACITY_EXACT, CAPACITY_BUCKETED, CAPACITY_CALLER_TOKENS, CAPACITY_FIXED_PARTITION = 0, 1, 2, 3
+FLAG_FORCE_GENERIC = 1
+FLAG_F32_OUTPUT = 2
+
+
+class PsiHipError(RuntimeError):
+    """A non-zero status from the C ABI; `.code` is the status, the text is psi_hip_last_error()."""
+
+    def __init__(self, code, message):
+        super().__init__(f"psi_hip error {code}: {message}")
+        self.code = code
+        self.message = message
+
+
+class GQAConfigStruct(ctypes.Structure):
+    _fields_ = [
+        ("num_q_heads", c_uint32),
+        ("num_kv_heads", c_uint32),
+        ("head_dim", c_uint32),
+        ("scale", c_float),
+        ("page_bytes", c_uint32),
+        ("dtype", c_uint32),
+    ]
+
+
+class PageTableLayoutStruct(ctypes.Structure):
+    _fields_ = [
+        ("num_req_slots", c_uint32),
+        ("num_gqa_layers", c_uint32),
+        ("num_blocks", c_uint32),
+        ("num_page_ids_per_block", c_uint32),
+    ]
+
+
+class VariantStruct(ctypes.Structure):
+    _fields_ = [
+        ("kind", c_uint32),
+        ("q_token_tile_size", c_uint32),
+        ("kv_token_tile_size", c_uint32),
+        ("num_threads_per_threadblock", c_uint32),
+        ("q_head_tile_size", c_uint32),
+    ]
+
+
+class ReplayShapeStruct(ctypes.Structure):
+    _fields_ = [
+        ("num_tokens", c_uint32),
+        ("num_total_tokens", c_uint32),
+        ("num_q_token_tiles", c_uint32),
+        ("num_total_q_token_tiles", c_uint32),
+        ("num_kv_splits", c_uint32),
+        ("num_total_kv_splits", c_uint32),
+        ("reduce_sdpa_partial_outputs", c_uint32),
+    ]
+
+
+_U32P = POINTER(c_uint32)
+_CFG = POINTER(GQAConfigStruct)
+_LAYOUT = POINTER(PageTableLayoutStruct)
+_VARIANT = POINTER(VariantStruct)
+
+# name -> (restype, argtypes); every symbol include/psi_hip.h declares.
+PROTOTYPES = {
+    "psi_hip_last_error": (c_char_p, []),
+    "psi_hip_version": (c_char_p, []),
+    "psi_hip_ctx_create": (c_int, [c_int, c_void_p, POINTER(c_void_p)]),
+    "psi_hip_ctx_destroy": (c_int, [c_void_p]),
+    "psi_hip_ctx_set_stream": (c_int, [c_void_p, c_void_p]),
+    "psi_hip_sync": (c_int, [c_void_p]),
+    "psi_hip_ctx_set_timing": (c_int, [c_void_p, c_int]),
+    "psi_hip_ctx_kernel_time_ms": (c_int, [c_void_p, c_char_p, POINTER(c_double), POINTER(c_uint64)]),
+    "psi_hip_ctx_reset_timing": (c_int, [c_void_p]),
+    "psi_hip_ctx_set_flag": (c_int, [c_void_p, c_uint32, c_uint32]),
+    "psi_hip_gqa_tokens_per_page": (c_int, [_CFG, _U32P]),
+    "psi_hip_split_kv_select": (c_int, [_CFG, c_int, c_uint32, c_uint32, _VARIANT]),
+    "psi_hip_split_kv_max_q_tokens_per_partial_output": (c_int, [_CFG, c_int, _U32P]),
+    "psi_hip_split_kv_select_batch": (c_int, [_CFG, c_uint32, c_uint32, _U32P, _U32P, c_uint32, _VARIANT]),
+    "psi_hip_replay_buckets": (c_int, [c_uint32, _U32P, c_uint32, _U32P, c_uint32, _U32P]),
+    "psi_hip_replay_bucket_capacity": (c_int, [c_uint32, _U32P, c_uint32, c_uint32, _U32P]),
+    "psi_hip_gqa_metadata_update": (
+        c_int,
+        [c_uint32, _U32P, _U32P, _U32P, c_uint32, _VARIANT, c_uint32, c_uint32, _U32P, c_uint32, c_uint32, c_uint32,
+         _U32P, _U32P, _U32P, _U32P, _U32P, POINTER(ReplayShapeStruct)],
+    ),
+    "psi_hip_kv_page_write": (
+        c_int,
+        [c_void_p, _CFG, _LAYOUT, c_void_p, c_uint64, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_uint32,
+         c_uint32, c_uint32],
+    ),
+    "psi_hip_split_kv_single_q_scratch_bytes": (c_int, [_CFG, c_uint32, POINTER(c_uint64)]),
+    "psi_hip_split_kv_single_q_map": (
+        c_int,
+        [c_void_p, _CFG, _LAYOUT, c_void_p, c_void_p, c_uint64, c_void_p, c_void_p, c_void_p, c_void_p, c_uint64,
+         c_uint32, c_uint32, c_uint32, c_uint32, c_uint32],
+    ),
+    "psi_hip_split_kv_single_q_reduce": (
+        c_int, [c_void_p, _CFG, c_void_p, c_uint64, c_void_p, c_void_p, c_uint32, c_uint32, c_uint32]),
+    "psi_hip_split_kv_tiled_q_scratch_bytes": (c_int, [_CFG, c_uint32, c_uint32, POINTER(c_uint64)]),
+    "psi_hip_split_kv_tiled_q_map": (
+        c_int,
+        [c_void_p, _CFG, _LAYOUT, c_uint32, c_void_p, c_void_p, c_uint64, c_void_p, c_void_p, c_void_p, c_void_p,
+         c_void_p, c_void_p, c_uint64, c_uint32, c_uint32, c_uint32, c_uint32, c_uint32, c_uint32, c_uint32],
+    ),
+    "psi_hip_split_kv_tiled_q_reduce": (
+        c_int,
+        [c_void_p, _CFG, c_uint32, c_void_p, c_uint64, c_void_p, c_void_p, c_void_p, c_uint32, c_uint32, c_uint32,
+         c_uint32],
+    ),
+    "psi_hip_page_table_write_page_ids": (
+        c_int, [c_void_p, _LAYOUT, c_void_p, c_uint32, c_uint32, c_uint32, _U32P, c_uint32, c_uint32]),
+    "psi_hip_page_table_reset_req_slot": (c_int, [c_void_p, _LAYOUT, c_void_p, c_uint32]),
+    "psi_hip_page_table_start_index": (c_int, [_LAYOUT, c_uint32, c_uint32, c_uint32, POINTER(c_uint64)]),
+    "psi_hip_page_ids_by_layer": (c_int, [_U32P, c_uint32, c_uint32, c_uint32, _U32P]),
+}
+
+_lib = None
+
+
+def load():
+    """Loads libpsi_hip.so once and installs the prototypes.  Raises if it has not been built."""
+    global _lib
+    if _lib is not None:
+        return _lib
+    if not os.path.exists(LIB_PATH):
+        raise RuntimeError(
+            f"{LIB_PATH} is missing: build it with `make -C {_HERE}` (or __graft_entry__.build()); "
+            "there is no CPU fallback for the attention path"
+        )
+    lib = ctypes.CDLL(LIB_PATH)
+    for name, (restype, argtypes) in PROTOTYPES.items():
+        fn = getattr(lib, name)
+        fn.restype = restype
+        fn.argtypes = argtypes
+    _lib = lib
+    return lib
+
+
+def check(status):
+    if status != OK:
+        raise PsiHipError(status, load().psi_hip_last_error().decode("utf-8", "replace"))
+
+
+def u32_array(values):
+    values = [int(v) for v in values]
+    return (c_uint32 * max(len(values), 1))(*values)

@@ -1,0 +1,504 @@
+// Host-side planning of a GQA batch: replay capacity buckets, SplitKV variant selection and the
+// per-batch metadata (per-token slots/positions, Q-token tiles, KV splits).  Pure integer logic,
+// no device work.  Follows
+//   crates/inference-executor-core/src/replay.rs:4-87                      (buckets)
+//   crates/inference-backend-metal/src/components/gqa_split_kv.rs:86-156   (variant geometry)
+//   crates/inference-executor-metal/src/attn/gqa/mod.rs:64-316             (batch selector)
+//   crates/inference-executor-metal/src/attn/gqa/batch_metadata.rs:192-523 (metadata + split plans)
+#include <algorithm>
+#include <queue>
+
+#include "common.h"
+
+namespace psi {
+
+// ---------------------------------------------------------------- replay buckets (replay.rs)
+
+static const uint32_t kBaseBuckets[] = {1, 2, 4, 6, 8, 12, 16, 20, 24, 32, 40, 48, 56, 64};
+
+struct BucketPolicy {
+    uint32_t max_capacity = 0;
+    std::vector<uint32_t> buckets;
+
+    // First bucket that holds `active` (replay.rs:56-61).
+    int capacity(uint32_t active, uint32_t* out) const {
+        PSI_REQUIRE(active > 0, "replay bucket requires active work");
+        PSI_REQUIRE(active <= max_capacity, "replay active work exceeds capacity");
+        *out = *std::lower_bound(buckets.begin(), buckets.end(), active);
+        return PSI_HIP_OK;
+    }
+};
+
+static int make_bucket_policy(uint32_t max_capacity, const uint32_t* boundaries, uint32_t num_boundaries,
+                              BucketPolicy* policy) {
+    PSI_REQUIRE(max_capacity > 0, "replay bucket capacity must be positive");
+    std::vector<uint32_t>& b = policy->buckets;
+    b.clear();
+    for (uint32_t base : kBaseBuckets)
+        if (base <= max_capacity) b.push_back(base);
+    // Above 64: quarters of each power-of-two interval, stopping before max_capacity (replay.rs:69-87).
+    bool done = false;
+    for (uint64_t lower = 64; !done && lower < max_capacity; lower *= 2) {
+        const uint64_t step = lower / 4;
+        for (uint64_t part = 1; part <= 4; ++part) {
+            const uint64_t candidate = std::min<uint64_t>(lower + step * part, UINT32_MAX);
+            if (candidate >= max_capacity) {
+                done = true;
+                break;
+            }
+            b.push_back((uint32_t)candidate);
+        }
+    }
+    for (uint32_t i = 0; i < num_boundaries; ++i) {
+        PSI_REQUIRE(boundaries[i] > 0, "replay topology boundary must be positive");
+        if (boundaries[i] > 1 && boundaries[i] <= max_capacity) b.push_back(boundaries[i] - 1);
+    }
+    b.push_back(max_capacity);
+    std::sort(b.begin(), b.end());
+    b.erase(std::unique(b.begin(), b.end()), b.end());
+    policy->max_capacity = max_capacity;
+    return PSI_HIP_OK;
+}
+
+// ---------------------------------------------------------------- variant geometry (gqa_split_kv.rs)
+
+struct SplitKVSelector {
+    uint32_t group;
+    bool supports_tiled_q;
+    bool full_group_for_tiled_q;
+    uint32_t single_q_tile;  // = threads per threadblock
+    uint32_t tiled_q_token_tile = 8;
+    uint32_t tiled_kv_token_tile = 16;
+    uint32_t max_q_head_tile;
+
+    psi_hip_split_kv_variant single_q() const {
+        psi_hip_split_kv_variant v{};
+        v.kind = PSI_HIP_VARIANT_SINGLE_Q;
+        v.q_token_tile_size = 1;
+        v.kv_token_tile_size = single_q_tile;
+        v.num_threads_per_threadblock = single_q_tile;
+        v.q_head_tile_size = std::min(group, max_q_head_tile);
+        return v;
+    }
+
+    int select(uint32_t num_tokens, uint32_t num_q_token_tiles, psi_hip_split_kv_variant* out) const {
+        PSI_REQUIRE(num_tokens > 0, "GQA SplitKV selection requires tokens");
+        PSI_REQUIRE(num_q_token_tiles > 0 && num_q_token_tiles <= num_tokens,
+                    "GQA SplitKV selection requires 0 < q_token_tiles <= tokens");
+        if (!supports_tiled_q || (uint64_t)num_tokens < 2ull * num_q_token_tiles) {
+            *out = single_q();
+            return PSI_HIP_OK;
+        }
+        const uint32_t desired = (!full_group_for_tiled_q && (uint64_t)num_tokens < 4ull * num_q_token_tiles)
+                                     ? (group + 1) / 2
+                                     : group;
+        psi_hip_split_kv_variant v{};
+        v.kind = PSI_HIP_VARIANT_TILED_Q;
+        v.q_token_tile_size = tiled_q_token_tile;
+        v.kv_token_tile_size = tiled_kv_token_tile;
+        v.num_threads_per_threadblock = 0;
+        v.q_head_tile_size = std::min(desired, max_q_head_tile);
+        *out = v;
+        return PSI_HIP_OK;
+    }
+};
+
+static uint32_t next_pow2_u32(uint32_t v) {
+    uint32_t p = 1;
+    while (p < v) p <<= 1;
+    return p;
+}
+
+static int make_selector(const psi_hip_gqa_config* cfg, bool dspark_history, SplitKVSelector* sel,
+                         Geometry* geometry_out = nullptr) {
+    Geometry g;
+    int rc = make_geometry(cfg, &g);
+    if (rc != PSI_HIP_OK) return rc;
+    // The reference's attention kernels accept f32 and bf16 only; f16 shares the bf16 geometry here.
+    const bool two_byte = g.dtype != PSI_HIP_F32;
+    const bool profile = (g.d == 128 && g.tokens_per_page == 8) ||
+                         (g.d == 256 && (g.tokens_per_page == 8 || g.tokens_per_page == 16));
+    sel->group = g.group;
+    sel->supports_tiled_q = !dspark_history && two_byte && profile && g.group <= 8;
+    sel->full_group_for_tiled_q = !dspark_history && g.d == 128 && g.tokens_per_page == 8;
+    sel->single_q_tile = next_pow2_u32(std::max(std::min(g.d, 256u), 32u));
+    sel->max_q_head_tile = 256 / (sel->tiled_q_token_tile / 8 * 32);
+    if (geometry_out) *geometry_out = g;
+    return PSI_HIP_OK;
+}
+
+// ---------------------------------------------------------------- split plans (batch_metadata.rs)
+
+struct QTile {
+    uint32_t flat_begin, flat_end, context_len;
+    uint64_t num_splits;
+};
+
+static inline uint64_t div_ceil_u64(uint64_t a, uint64_t b) { return (a + b - 1) / b; }
+
+// Greedy budgeted split count assignment shared by both variants (batch_metadata.rs:364-386 and
+// :466-488): repeatedly give one more split to the tile whose splits currently span the most KV
+// tiles; ties go to the lowest tile index; a tile is skipped when its partial-state cost no longer
+// fits.  `cost(tile)` is 1 for SingleQ and the tile's token count for TiledQ.
+static void assign_greedy_splits(std::vector<QTile>& tiles, uint32_t kv_tile, uint64_t budget, bool cost_is_tokens) {
+    uint64_t used = 0;
+    for (auto& t : tiles) used += cost_is_tokens ? (t.flat_end - t.flat_begin) : 1;
+    // Max-heap on (kv tiles per split, lowest index first).  Popping the best candidate, bumping it
+    // and pushing it back reproduces the reference's full rescan: priorities of other tiles do not
+    // change between steps, and a tile rejected for cost can never fit later (the budget only shrinks).
+    struct Entry {
+        uint64_t per_split;
+        uint32_t index;
+        bool operator<(const Entry& o) const {
+            return per_split != o.per_split ? per_split < o.per_split : index > o.index;
+        }
+    };
+    std::priority_queue<Entry> heap;
+    auto kv_tiles = [&](const QTile& t) { return div_ceil_u64(t.context_len, kv_tile); };
+    for (uint32_t i = 0; i < tiles.size(); ++i)
+        if (tiles[i].num_splits < kv_tiles(tiles[i])) heap.push({div_ceil_u64(kv_tiles(tiles[i]), tiles[i].num_splits), i});
+    while (used < budget && !heap.empty()) {
+        const Entry e = heap.top();
+        heap.pop();
+        QTile& t = tiles[e.index];
+        const uint64_t cost = cost_is_tokens ? (t.flat_end - t.flat_begin) : 1;
+        if (used + cost > budget) continue;  // cannot fit now or later
+        t.num_splits += 1;
+        used += cost;
+        if (t.num_splits < kv_tiles(t)) heap.push({div_ceil_u64(kv_tiles(t), t.num_splits), e.index});
+    }
+}
+
+static int emit_splits(const std::vector<QTile>& tiles, uint32_t kv_tile, std::vector<uint32_t>* kv_splits,
+                       std::vector<uint32_t>* cu) {
+    kv_splits->clear();
+    cu->assign(1, 0u);
+    for (uint32_t i = 0; i < tiles.size(); ++i) {
+        const QTile& t = tiles[i];
+        const uint64_t n_tiles = div_ceil_u64(t.context_len, kv_tile);
+        for (uint64_t s = 0; s < t.num_splits; ++s) {
+            const uint64_t tb = n_tiles * s / t.num_splits, te = n_tiles * (s + 1) / t.num_splits;
+            const uint64_t begin = tb * kv_tile, end = te * kv_tile;
+            PSI_REQUIRE(begin <= UINT32_MAX, "GQA map KV split KV-token begin must fit u32");
+            PSI_REQUIRE(end <= UINT32_MAX, "GQA map KV split KV-token end must fit u32");
+            kv_splits->push_back(i);
+            kv_splits->push_back((uint32_t)begin);
+            kv_splits->push_back(std::min(t.context_len, (uint32_t)end));
+        }
+        PSI_REQUIRE(kv_splits->size() / 3 <= UINT32_MAX, "GQA map KV split count must fit u32");
+        cu->push_back((uint32_t)(kv_splits->size() / 3));
+    }
+    return PSI_HIP_OK;
+}
+
+static std::vector<QTile> single_q_tiles(const std::vector<uint32_t>& flat_token_indices) {
+    std::vector<QTile> tiles;
+    tiles.reserve(flat_token_indices.size());
+    for (uint32_t i = 0; i < flat_token_indices.size(); ++i)
+        tiles.push_back({i, i + 1, flat_token_indices[i] + 1, 1});
+    return tiles;
+}
+
+// Request-local chunks of at most q_tile tokens (batch_metadata.rs:443-461).
+static std::vector<QTile> tiled_q_tiles(const uint32_t* token_indices, const uint32_t* cu_tokens, uint32_t num_reqs,
+                                        uint32_t q_tile) {
+    std::vector<QTile> tiles;
+    for (uint32_t r = 0; r < num_reqs; ++r) {
+        uint32_t begin = cu_tokens[r];
+        const uint32_t req_end = cu_tokens[r + 1];
+        while (begin < req_end) {
+            const uint32_t end = begin + std::min(req_end - begin, q_tile);
+            tiles.push_back({begin, end, token_indices[r] + (end - cu_tokens[r]), 1});
+            begin = end;
+        }
+    }
+    return tiles;
+}
+
+// ---------------------------------------------------------------- batch selector (attn/gqa/mod.rs)
+
+struct SelectionWork {
+    uint64_t num_kv_splits, scheduled_map_work, active_map_work, map_blocks_per_kv_head, map_waves_per_kv_head,
+        active_partial_states, padded_replay_work;
+    uint64_t bookkeeping() const {
+        return map_blocks_per_kv_head + map_waves_per_kv_head + active_partial_states + padded_replay_work;
+    }
+};
+
+static int padded_kv_splits(uint64_t num_kv_splits, uint32_t max_tokens, const BucketPolicy* policy, uint64_t* out) {
+    if (policy) {
+        uint32_t cap;
+        PSI_REQUIRE(num_kv_splits <= UINT32_MAX, "GQA active KV-split count must fit u32");
+        int rc = policy->capacity((uint32_t)num_kv_splits, &cap);
+        if (rc != PSI_HIP_OK) return rc;
+        *out = cap;
+        return PSI_HIP_OK;
+    }
+    uint64_t p = 1;
+    while (p < num_kv_splits) p <<= 1;
+    *out = std::min<uint64_t>(p, max_tokens);
+    return PSI_HIP_OK;
+}
+
+// mod.rs:221-274: the same greedy loop as the metadata builder, priced in partial-state tokens.
+static int selection_work(std::vector<QTile> tiles, uint32_t kv_tile, uint32_t scheduled_q_tokens,
+                          uint32_t map_blocks_per_split, uint32_t waves_per_map_block, uint32_t max_tokens,
+                          const BucketPolicy* policy, SelectionWork* out) {
+    PSI_REQUIRE(!tiles.empty(), "GQA SplitKV selection requires tiles");
+    uint64_t active = 0;
+    for (auto& t : tiles) active += t.flat_end - t.flat_begin;
+    PSI_REQUIRE(active <= max_tokens, "GQA SplitKV selection tokens exceed max_tokens");
+    assign_greedy_splits(tiles, kv_tile, max_tokens, true);
+    SelectionWork w{};
+    for (auto& t : tiles) {
+        const uint64_t n_tiles = div_ceil_u64(t.context_len, kv_tile);
+        w.num_kv_splits += t.num_splits;
+        w.scheduled_map_work += n_tiles * ((uint64_t)kv_tile * scheduled_q_tokens);
+        w.active_map_work += n_tiles * ((uint64_t)kv_tile * (t.flat_end - t.flat_begin));
+        w.active_partial_states += (uint64_t)(t.flat_end - t.flat_begin) * t.num_splits;
+    }
+    w.map_blocks_per_kv_head = w.num_kv_splits * map_blocks_per_split;
+    w.map_waves_per_kv_head = w.map_blocks_per_kv_head * waves_per_map_block;
+    uint64_t padded;
+    int rc = padded_kv_splits(w.num_kv_splits, max_tokens, policy, &padded);
+    if (rc != PSI_HIP_OK) return rc;
+    w.padded_replay_work = padded * scheduled_q_tokens;
+    *out = w;
+    return PSI_HIP_OK;
+}
+
+static int check_batch(const uint32_t* token_indices, const uint32_t* cu_tokens, uint32_t num_reqs) {
+    PSI_REQUIRE(token_indices && cu_tokens, "GQA batch arrays must not be null");
+    PSI_REQUIRE(cu_tokens[0] == 0, "GQA batch cu_tokens must start at zero");
+    for (uint32_t r = 0; r < num_reqs; ++r) {
+        PSI_REQUIRE(cu_tokens[r] <= cu_tokens[r + 1], "GQA batch cu_tokens must be nondecreasing");
+        PSI_REQUIRE((uint64_t)token_indices[r] + (cu_tokens[r + 1] - cu_tokens[r]) <= UINT32_MAX,
+                    "GQA request context length must fit u32");
+    }
+    return PSI_HIP_OK;
+}
+
+}  // namespace psi
+
+using namespace psi;
+
+extern "C" int psi_hip_replay_buckets(uint32_t max_capacity, const uint32_t* topology_boundaries,
+                                      uint32_t num_boundaries, uint32_t* out_buckets, uint32_t buckets_capacity,
+                                      uint32_t* out_num_buckets) {
+    BucketPolicy policy;
+    int rc = make_bucket_policy(max_capacity, topology_boundaries, num_boundaries, &policy);
+    if (rc != PSI_HIP_OK) return rc;
+    PSI_REQUIRE(out_num_buckets != nullptr, "out_num_buckets must not be null");
+    *out_num_buckets = (uint32_t)policy.buckets.size();
+    if (out_buckets) {
+        PSI_REQUIRE(buckets_capacity >= policy.buckets.size(), "bucket output array too small");
+        std::copy(policy.buckets.begin(), policy.buckets.end(), out_buckets);
+    }
+    return PSI_HIP_OK;
+}
+
+extern "C" int psi_hip_replay_bucket_capacity(uint32_t max_capacity, const uint32_t* topology_boundaries,
+                                              uint32_t num_boundaries, uint32_t active, uint32_t* out_capacity) {
+    BucketPolicy policy;
+    int rc = make_bucket_policy(max_capacity, topology_boundaries, num_boundaries, &policy);
+    if (rc != PSI_HIP_OK) return rc;
+    PSI_REQUIRE(out_capacity != nullptr, "out_capacity must not be null");
+    return policy.capacity(active, out_capacity);
+}
+
+extern "C" int psi_hip_split_kv_select(const psi_hip_gqa_config* cfg, int dspark_history, uint32_t num_tokens,
+                                       uint32_t num_q_token_tiles, psi_hip_split_kv_variant* out_variant) {
+    SplitKVSelector sel;
+    int rc = make_selector(cfg, dspark_history != 0, &sel);
+    if (rc != PSI_HIP_OK) return rc;
+    PSI_REQUIRE(out_variant != nullptr, "out_variant must not be null");
+    return sel.select(num_tokens, num_q_token_tiles, out_variant);
+}
+
+extern "C" int psi_hip_split_kv_max_q_tokens_per_partial_output(const psi_hip_gqa_config* cfg, int dspark_history,
+                                                                uint32_t* out) {
+    SplitKVSelector sel;
+    int rc = make_selector(cfg, dspark_history != 0, &sel);
+    if (rc != PSI_HIP_OK) return rc;
+    PSI_REQUIRE(out != nullptr, "out pointer must not be null");
+    *out = sel.supports_tiled_q ? sel.tiled_q_token_tile : 1;
+    return PSI_HIP_OK;
+}
+
+extern "C" int psi_hip_split_kv_select_batch(const psi_hip_gqa_config* cfg, uint32_t max_tokens,
+                                             uint32_t bucket_max_tokens, const uint32_t* token_indices,
+                                             const uint32_t* cu_tokens, uint32_t num_reqs,
+                                             psi_hip_split_kv_variant* out_variant) {
+    SplitKVSelector sel;
+    Geometry g;
+    int rc = make_selector(cfg, false, &sel, &g);
+    if (rc != PSI_HIP_OK) return rc;
+    PSI_REQUIRE(out_variant != nullptr, "out_variant must not be null");
+    rc = check_batch(token_indices, cu_tokens, num_reqs);
+    if (rc != PSI_HIP_OK) return rc;
+    const uint32_t num_tokens = cu_tokens[num_reqs];
+    PSI_REQUIRE(num_tokens > 0, "GQA batch metadata requires tokens");
+    uint64_t num_q_token_tiles = 0;
+    for (uint32_t r = 0; r < num_reqs; ++r)
+        num_q_token_tiles += div_ceil_u64(cu_tokens[r + 1] - cu_tokens[r], sel.tiled_q_token_tile);
+    psi_hip_split_kv_variant candidate;
+    rc = sel.select(num_tokens, (uint32_t)num_q_token_tiles, &candidate);
+    if (rc != PSI_HIP_OK) return rc;
+    const bool d256_page8 = g.d == 256 && g.tokens_per_page == 8;
+    if (!d256_page8 || candidate.kind != PSI_HIP_VARIANT_TILED_Q) {
+        *out_variant = candidate;
+        return PSI_HIP_OK;
+    }
+    // mod.rs:96-127: compare both plans' bookkeeping and require enough useful map work.
+    BucketPolicy policy;
+    const BucketPolicy* policy_ptr = nullptr;
+    if (bucket_max_tokens > 0) {
+        rc = make_bucket_policy(bucket_max_tokens, nullptr, 0, &policy);
+        if (rc != PSI_HIP_OK) return rc;
+        policy_ptr = &policy;
+    }
+    const psi_hip_split_kv_variant single = sel.single_q();
+    std::vector<uint32_t> flat;
+    uint64_t logical_pairs = 0;
+    for (uint32_t r = 0; r < num_reqs; ++r)
+        for (uint32_t i = 0; i < cu_tokens[r + 1] - cu_tokens[r]; ++i) {
+            flat.push_back(token_indices[r] + i);
+            logical_pairs += (uint64_t)token_indices[r] + i + 1;
+        }
+    SelectionWork single_work, tiled_work;
+    rc = selection_work(single_q_tiles(flat), single.kv_token_tile_size, 1, 1, single.num_threads_per_threadblock / 32,
+                        max_tokens, policy_ptr, &single_work);
+    if (rc != PSI_HIP_OK) return rc;
+    rc = selection_work(tiled_q_tiles(token_indices, cu_tokens, num_reqs, candidate.q_token_tile_size),
+                        candidate.kv_token_tile_size, candidate.q_token_tile_size,
+                        (uint32_t)div_ceil_u64(single.q_head_tile_size, candidate.q_head_tile_size),
+                        candidate.q_token_tile_size / 8 * candidate.q_head_tile_size, max_tokens, policy_ptr,
+                        &tiled_work);
+    if (rc != PSI_HIP_OK) return rc;
+    const uint64_t complete_plan_work = logical_pairs + std::min(single_work.bookkeeping(), tiled_work.bookkeeping());
+    const bool enough_utilization = tiled_work.active_map_work * 2 >= tiled_work.scheduled_map_work;
+    *out_variant = (enough_utilization && complete_plan_work >= 2048) ? candidate : single;
+    return PSI_HIP_OK;
+}
+
+extern "C" int psi_hip_gqa_metadata_update(uint32_t max_tokens, const uint32_t* req_slots,
+                                           const uint32_t* token_indices, const uint32_t* cu_tokens,
+                                           uint32_t num_reqs, const psi_hip_split_kv_variant* variant,
+                                           uint32_t capacity_mode, uint32_t caller_num_total_tokens,
+                                           const uint32_t* topology_boundaries, uint32_t num_boundaries,
+                                           uint32_t partition_tokens, uint32_t kv_splits_capacity,
+                                           uint32_t* req_slots_by_token, uint32_t* flat_token_indices,
+                                           uint32_t* q_token_tiles, uint32_t* kv_splits, uint32_t* cu_kv_splits,
+                                           psi_hip_gqa_replay_shape* out_shape) {
+    PSI_REQUIRE(max_tokens > 0, "GQA batch metadata requires tokens");
+    PSI_REQUIRE(req_slots && variant && req_slots_by_token && flat_token_indices && kv_splits && cu_kv_splits &&
+                    out_shape,
+                "GQA batch metadata arrays must not be null");
+    int rc = check_batch(token_indices, cu_tokens, num_reqs);
+    if (rc != PSI_HIP_OK) return rc;
+    const bool tiled = variant->kind == PSI_HIP_VARIANT_TILED_Q;
+    PSI_REQUIRE(variant->kind == PSI_HIP_VARIANT_SINGLE_Q || tiled, "unknown SplitKV variant kind %u", variant->kind);
+    PSI_REQUIRE(variant->kv_token_tile_size > 0, "GQA KV-token tile size must be positive");
+    PSI_REQUIRE(!tiled || variant->q_token_tile_size > 0, "GQA Q-token tile size must be positive");
+    PSI_REQUIRE(!tiled || q_token_tiles != nullptr, "GQA Q-token tile array must not be null");
+    const uint32_t num_tokens = cu_tokens[num_reqs];
+    PSI_REQUIRE(num_tokens > 0, "GQA batch metadata requires tokens");
+    PSI_REQUIRE(num_tokens <= max_tokens, "GQA batch tokens exceed the metadata capacity");
+    const bool fixed = capacity_mode == PSI_HIP_CAPACITY_FIXED_PARTITION;
+    const uint32_t max_kv_splits = fixed ? kv_splits_capacity : max_tokens;
+    if (capacity_mode == PSI_HIP_CAPACITY_CALLER_TOKENS) {
+        PSI_REQUIRE(num_tokens <= caller_num_total_tokens,
+                    "GQA active token count must not exceed the caller-owned token capacity");
+        PSI_REQUIRE(caller_num_total_tokens <= max_tokens,
+                    "GQA caller-owned token capacity must not exceed the metadata capacity");
+    }
+    PSI_REQUIRE(capacity_mode <= PSI_HIP_CAPACITY_FIXED_PARTITION, "unknown capacity mode %u", capacity_mode);
+
+    // Per-token expansion (batch_metadata.rs:234-246).
+    std::vector<uint32_t> flat;
+    flat.reserve(num_tokens);
+    for (uint32_t r = 0; r < num_reqs; ++r)
+        for (uint32_t i = 0; i < cu_tokens[r + 1] - cu_tokens[r]; ++i) {
+            req_slots_by_token[flat.size()] = req_slots[r];
+            flat_token_indices[flat.size()] = token_indices[r] + i;
+            flat.push_back(token_indices[r] + i);
+        }
+
+    std::vector<QTile> tiles = tiled ? tiled_q_tiles(token_indices, cu_tokens, num_reqs, variant->q_token_tile_size)
+                                     : single_q_tiles(flat);
+    if (fixed) {
+        PSI_REQUIRE(partition_tokens > 0 && partition_tokens % variant->kv_token_tile_size == 0,
+                    "partition_tokens must be a positive multiple of the KV-token tile size");
+        for (auto& t : tiles) t.num_splits = div_ceil_u64(t.context_len, partition_tokens);
+    } else if (tiled) {
+        uint64_t partial_tokens = 0;
+        for (auto& t : tiles) partial_tokens += t.flat_end - t.flat_begin;
+        PSI_REQUIRE(partial_tokens <= max_tokens, "GQA tiled partial-output tokens exceed the metadata capacity");
+        assign_greedy_splits(tiles, variant->kv_token_tile_size, max_tokens, true);
+    } else {
+        PSI_REQUIRE(max_kv_splits >= flat.size(), "GQA KV-split capacity is smaller than the token count");
+        assign_greedy_splits(tiles, variant->kv_token_tile_size, max_kv_splits, false);
+    }
+    std::vector<uint32_t> splits, cu;
+    if (fixed) {
+        // Fixed partitions cut on partition boundaries rather than on even tile shares.
+        cu.assign(1, 0u);
+        for (uint32_t i = 0; i < tiles.size(); ++i) {
+            for (uint64_t s = 0; s < tiles[i].num_splits; ++s) {
+                splits.push_back(i);
+                splits.push_back((uint32_t)(s * partition_tokens));
+                splits.push_back((uint32_t)std::min<uint64_t>(tiles[i].context_len, (s + 1) * partition_tokens));
+            }
+            cu.push_back((uint32_t)(splits.size() / 3));
+        }
+    } else {
+        rc = emit_splits(tiles, variant->kv_token_tile_size, &splits, &cu);
+        if (rc != PSI_HIP_OK) return rc;
+    }
+    const uint32_t num_kv_splits = (uint32_t)(splits.size() / 3);
+    const uint32_t num_q_token_tiles = tiled ? (uint32_t)tiles.size() : num_tokens;
+    PSI_REQUIRE(num_kv_splits <= max_kv_splits, "GQA KV-split plan exceeds the KV-split capacity: %u > %u",
+                num_kv_splits, max_kv_splits);
+
+    // Recorded capacities (batch_metadata.rs:277-294).
+    uint32_t total_tokens = num_tokens, total_tiles = num_q_token_tiles, total_splits = num_kv_splits;
+    if (capacity_mode == PSI_HIP_CAPACITY_EXACT || fixed) {
+        total_splits = (uint32_t)std::min<uint64_t>(next_pow2_u32(num_kv_splits), max_kv_splits);
+        if (fixed) total_splits = num_kv_splits;  // fixed partitions launch exactly the planned splits
+    } else {
+        BucketPolicy tokens_policy, plain_policy;
+        rc = make_bucket_policy(max_tokens, topology_boundaries, num_boundaries, &tokens_policy);
+        if (rc != PSI_HIP_OK) return rc;
+        rc = make_bucket_policy(max_tokens, nullptr, 0, &plain_policy);
+        if (rc != PSI_HIP_OK) return rc;
+        if (capacity_mode == PSI_HIP_CAPACITY_BUCKETED) {
+            rc = tokens_policy.capacity(num_tokens, &total_tokens);
+            if (rc != PSI_HIP_OK) return rc;
+        } else {
+            total_tokens = caller_num_total_tokens;
+        }
+        rc = plain_policy.capacity(num_q_token_tiles, &total_tiles);
+        if (rc != PSI_HIP_OK) return rc;
+        rc = plain_policy.capacity(num_kv_splits, &total_splits);
+        if (rc != PSI_HIP_OK) return rc;
+    }
+    PSI_REQUIRE(total_splits >= num_kv_splits, "GQA recorded KV-split capacity is below the plan");
+
+    if (tiled)
+        for (uint32_t i = 0; i < tiles.size(); ++i) {
+            q_token_tiles[2 * i] = tiles[i].flat_begin;
+            q_token_tiles[2 * i + 1] = tiles[i].flat_end;
+        }
+    std::copy(splits.begin(), splits.end(), kv_splits);
+    std::fill(kv_splits + splits.size(), kv_splits + (size_t)total_splits * 3, PSI_HIP_SENTINEL);
+    std::copy(cu.begin(), cu.end(), cu_kv_splits);
+
+    out_shape->num_tokens = num_tokens;
+    out_shape->num_total_tokens = total_tokens;
+    out_shape->num_q_token_tiles = num_q_token_tiles;
+    out_shape->num_total_q_token_tiles = total_tiles;
+    out_shape->num_kv_splits = num_kv_splits;
+    out_shape->num_total_kv_splits = total_splits;
+    out_shape->reduce_sdpa_partial_outputs = (tiled || num_kv_splits > num_tokens) ? 1u : 0u;
+    return PSI_HIP_OK;
+}

@@ -1,0 +1,78 @@
+// Shared declarations of the split-KV attention kernels: scratch layout and kernel arguments.
+#pragma once
+#include "common.h"
+#include "device_types.h"
+
+namespace psi {
+
+// Partial state of one (kv_split, q_head [, q_token_in_tile]) row, private to this library:
+//   max2 : running maximum of the logits in the log2 domain (logit * scale * log2(e)), -inf if empty
+//   sum  : sum of exp2(logit2 - max2) over the split's keys
+//   acc  : un-normalised sum of exp2(logit2 - max2) * V, f32 [head_dim]
+// Arrays are laid out [row][...] with row = (split * num_q_heads + q_head) * rows_per_split_head + r.
+struct PartialLayout {
+    uint64_t rows;
+    uint64_t max_offset, sum_offset, acc_offset, total_bytes;
+};
+
+inline PartialLayout partial_layout(uint64_t num_total_kv_splits, uint32_t hq, uint32_t d,
+                                    uint32_t rows_per_split_head) {
+    PartialLayout l;
+    l.rows = num_total_kv_splits * hq * rows_per_split_head;
+    auto align = [](uint64_t v) { return (v + 255) & ~uint64_t(255); };
+    l.max_offset = 0;
+    l.sum_offset = align(l.rows * 4);
+    l.acc_offset = l.sum_offset + align(l.rows * 4);
+    l.total_bytes = l.acc_offset + align(l.rows * d * 4);
+    return l;
+}
+
+struct MapArgs {
+    const void* q;
+    const void* kv_pages;
+    const uint32_t* req_slots;
+    const uint32_t* kv_splits;
+    float* part_max;
+    float* part_sum;
+    float* part_acc;
+    PageWalk walk;
+    uint32_t layer;
+    uint32_t hq, group;
+    uint32_t num_total_kv_splits;
+    uint32_t num_active_tokens, num_active_kv_splits;
+    float scale_log2;  // scale * log2(e)
+    // TiledQ only (null / 1 / 0 for SingleQ): kv_splits rows then name Q-token tiles.
+    const uint32_t* q_token_tiles = nullptr;       // [tiles][2] = flat token begin, end
+    const uint32_t* flat_token_indices = nullptr;  // request-absolute position of each flat token
+    uint32_t rows_per_split_head = 1;              // q_token_tile_size
+    uint32_t num_active_q_token_tiles = 0;
+};
+
+struct ReduceArgs {
+    const float* part_max;
+    const float* part_sum;
+    const float* part_acc;
+    const uint32_t* cu_kv_splits;
+    void* output;
+    uint32_t hq, d;
+    uint32_t num_active_tokens;
+    uint32_t out_dtype = PSI_HIP_F32;  // element type of `output`
+    // TiledQ only: cu_kv_splits is indexed by Q-token tile.
+    const uint32_t* q_token_tiles = nullptr;
+    uint32_t rows_per_split_head = 1;
+    uint32_t num_active_q_token_tiles = 0;
+};
+
+// Shape-generic kernels (any head_dim / page size / element type), SingleQ and TiledQ layouts.
+void launch_map_generic(psi_hip_ctx* ctx, const Geometry& g, const MapArgs& a);
+void launch_reduce_generic(psi_hip_ctx* ctx, const Geometry& g, const ReduceArgs& a, uint32_t num_total_tokens);
+void fill_walk(PageWalk* walk, const Geometry& g, const psi_hip_page_table_layout* layout, const uint32_t* page_ids);
+
+// Fast decode map for head_dim 256 / 128, 2-byte elements, power-of-two pages; returns
+// PSI_HIP_ERR_UNSUPPORTED when the shape is outside its domain (caller falls back).
+int launch_decode_map_fast(psi_hip_ctx* ctx, const Geometry& g, const MapArgs& a);
+int launch_reduce_fast(psi_hip_ctx* ctx, const Geometry& g, const ReduceArgs& a);
+// MFMA TiledQ map for bf16 / f16, head_dim 256 / 128; PSI_HIP_ERR_UNSUPPORTED outside its domain.
+int launch_tiled_map_fast(psi_hip_ctx* ctx, const Geometry& g, const MapArgs& a);
+
+}  // namespace psi

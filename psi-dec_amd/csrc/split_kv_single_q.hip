@@ -1,0 +1,141 @@
+// Split-KV decode attention (SingleQ): C-ABI entry points and dispatch between the gfx950 fast
+// kernels and the shape-generic ones.  Semantics follow
+// crates/inference-backend-metal/src/components/metal/gqa_split_kv_single_q_map.metal:31-253 and
+// gqa_split_kv_single_q_reduce.metal:10-49: one partial state per (kv_split, q_head), online
+// softmax over the split's keys, log-sum-exp combine over the splits of each token.
+#include <cmath>
+
+#include "split_kv.h"
+
+namespace psi {
+
+constexpr float kLog2e = 1.4426950408889634f;
+
+// Reference shape checks: gqa_split_kv_single_q.rs:197-209.
+static int check_single_q_shape(const Geometry& g, uint32_t num_total_tokens, uint32_t num_total_kv_splits) {
+    PSI_REQUIRE(g.scale > 0.0f, "GQA attention scale must be positive");
+    PSI_REQUIRE(num_total_tokens > 0, "GQA SDPA requires tokens");
+    PSI_REQUIRE(num_total_kv_splits > 0, "GQA SDPA requires KV splits");
+    const uint64_t out_values = (uint64_t)num_total_tokens * g.hq * g.d;
+    PSI_REQUIRE(out_values <= UINT32_MAX, "GQA SDPA query/output exceeds the shader u32 count domain: count=%llu",
+                (unsigned long long)out_values);
+    const uint64_t stats = (uint64_t)num_total_kv_splits * g.hq;
+    PSI_REQUIRE(stats - 1 <= UINT32_MAX, "GQA SDPA partial-output stats exceeds the shader u32 element-index domain");
+    PSI_REQUIRE(stats * g.d - 1 <= UINT32_MAX,
+                "GQA SDPA partial output exceeds the shader u32 element-index domain");
+    return PSI_HIP_OK;
+}
+
+}  // namespace psi
+
+using namespace psi;
+
+extern "C" int psi_hip_split_kv_single_q_scratch_bytes(const psi_hip_gqa_config* cfg, uint32_t num_total_kv_splits,
+                                                       uint64_t* out_bytes) {
+    Geometry g;
+    int rc = make_geometry(cfg, &g);
+    if (rc != PSI_HIP_OK) return rc;
+    PSI_REQUIRE(out_bytes != nullptr, "out pointer must not be null");
+    PSI_REQUIRE(num_total_kv_splits > 0, "GQA SDPA requires KV splits");
+    *out_bytes = partial_layout(num_total_kv_splits, g.hq, g.d, 1).total_bytes;
+    return PSI_HIP_OK;
+}
+
+extern "C" int psi_hip_split_kv_single_q_map(psi_hip_ctx* ctx, const psi_hip_gqa_config* cfg,
+                                             const psi_hip_page_table_layout* layout, const void* q,
+                                             const void* kv_pages, uint64_t kv_pages_bytes,
+                                             const uint32_t* req_slots, const uint32_t* page_ids,
+                                             const uint32_t* kv_splits, void* scratch, uint64_t scratch_bytes,
+                                             uint32_t gqa_layer_index, uint32_t num_total_tokens,
+                                             uint32_t num_total_kv_splits, uint32_t num_active_tokens,
+                                             uint32_t num_active_kv_splits) {
+    PSI_REQUIRE(ctx != nullptr, "ctx must not be null");
+    Geometry g;
+    int rc = make_geometry(cfg, &g);
+    if (rc != PSI_HIP_OK) return rc;
+    rc = check_layout(layout);
+    if (rc != PSI_HIP_OK) return rc;
+    rc = check_single_q_shape(g, num_total_tokens, num_total_kv_splits);
+    if (rc != PSI_HIP_OK) return rc;
+    PSI_REQUIRE(q && kv_pages && req_slots && page_ids && kv_splits && scratch,
+                "GQA SplitKV SingleQ map buffers must not be null");
+    PSI_REQUIRE(gqa_layer_index < layout->num_gqa_layers, "GQA page-table index exceeds layer count");
+    PSI_REQUIRE(num_active_tokens > 0, "GQA SplitKV SingleQ active token count must be positive");
+    PSI_REQUIRE(num_active_tokens <= num_total_tokens,
+                "GQA SplitKV SingleQ active token count exceeds recorded capacity");
+    PSI_REQUIRE(num_active_kv_splits > 0, "GQA SplitKV SingleQ active KV split count must be positive");
+    PSI_REQUIRE(num_active_kv_splits <= num_total_kv_splits,
+                "GQA SplitKV SingleQ active KV split count exceeds recorded capacity");
+    PSI_REQUIRE(kv_pages_bytes == 0 || kv_pages_bytes >= cfg->page_bytes, "GQA page arena is smaller than one page");
+    const PartialLayout pl = partial_layout(num_total_kv_splits, g.hq, g.d, 1);
+    PSI_REQUIRE(scratch_bytes >= pl.total_bytes, "GQA SplitKV SingleQ scratch too small: %llu < %llu",
+                (unsigned long long)scratch_bytes, (unsigned long long)pl.total_bytes);
+
+    MapArgs a;
+    a.q = q;
+    a.kv_pages = kv_pages;
+    a.req_slots = req_slots;
+    a.kv_splits = kv_splits;
+    a.part_max = reinterpret_cast<float*>(static_cast<char*>(scratch) + pl.max_offset);
+    a.part_sum = reinterpret_cast<float*>(static_cast<char*>(scratch) + pl.sum_offset);
+    a.part_acc = reinterpret_cast<float*>(static_cast<char*>(scratch) + pl.acc_offset);
+    fill_walk(&a.walk, g, layout, page_ids);
+    a.layer = gqa_layer_index;
+    a.hq = g.hq;
+    a.group = g.group;
+    a.num_total_kv_splits = num_total_kv_splits;
+    a.num_active_tokens = num_active_tokens;
+    a.num_active_kv_splits = num_active_kv_splits;
+    a.scale_log2 = g.scale * kLog2e;
+
+    LaunchScope scope(ctx, "split_kv_map");
+    rc = launch_decode_map_fast(ctx, g, a);
+    if (rc == PSI_HIP_ERR_UNSUPPORTED) {
+        const uint64_t grid = (uint64_t)num_total_kv_splits * g.hq * ((g.d + 63) / 64);
+        PSI_REQUIRE(grid <= 0x7fffffffull, "GQA SDPA map threads exceeds the shader u32 count domain");
+        launch_map_generic(ctx, g, a);
+        rc = PSI_HIP_OK;
+    }
+    if (rc != PSI_HIP_OK) return rc;
+    PSI_HIP_CHECK(hipGetLastError());
+    return PSI_HIP_OK;
+}
+
+extern "C" int psi_hip_split_kv_single_q_reduce(psi_hip_ctx* ctx, const psi_hip_gqa_config* cfg, const void* scratch,
+                                                uint64_t scratch_bytes, const uint32_t* cu_kv_splits, void* output,
+                                                uint32_t num_total_tokens, uint32_t num_total_kv_splits,
+                                                uint32_t num_active_tokens) {
+    PSI_REQUIRE(ctx != nullptr, "ctx must not be null");
+    Geometry g;
+    int rc = make_geometry(cfg, &g);
+    if (rc != PSI_HIP_OK) return rc;
+    rc = check_single_q_shape(g, num_total_tokens, num_total_kv_splits);
+    if (rc != PSI_HIP_OK) return rc;
+    PSI_REQUIRE(scratch && cu_kv_splits && output, "GQA SplitKV SingleQ reduce buffers must not be null");
+    PSI_REQUIRE(num_active_tokens > 0, "GQA SplitKV SingleQ active token count must be positive");
+    PSI_REQUIRE(num_active_tokens <= num_total_tokens,
+                "GQA SplitKV SingleQ active token count exceeds recorded capacity");
+    const PartialLayout pl = partial_layout(num_total_kv_splits, g.hq, g.d, 1);
+    PSI_REQUIRE(scratch_bytes >= pl.total_bytes, "GQA SplitKV SingleQ scratch too small: %llu < %llu",
+                (unsigned long long)scratch_bytes, (unsigned long long)pl.total_bytes);
+    ReduceArgs a;
+    a.part_max = reinterpret_cast<const float*>(static_cast<const char*>(scratch) + pl.max_offset);
+    a.part_sum = reinterpret_cast<const float*>(static_cast<const char*>(scratch) + pl.sum_offset);
+    a.part_acc = reinterpret_cast<const float*>(static_cast<const char*>(scratch) + pl.acc_offset);
+    a.cu_kv_splits = cu_kv_splits;
+    a.output = output;
+    a.hq = g.hq;
+    a.d = g.d;
+    a.out_dtype = ctx->f32_output ? PSI_HIP_F32 : g.dtype;
+    a.num_active_tokens = num_active_tokens;
+
+    LaunchScope scope(ctx, "split_kv_reduce");
+    rc = launch_reduce_fast(ctx, g, a);
+    if (rc == PSI_HIP_ERR_UNSUPPORTED) {
+        launch_reduce_generic(ctx, g, a, 0);
+        rc = PSI_HIP_OK;
+    }
+    if (rc != PSI_HIP_OK) return rc;
+    PSI_HIP_CHECK(hipGetLastError());
+    return PSI_HIP_OK;
+}

@@ -1,0 +1,284 @@
+"""Seeded synthetic workloads for the paged-attention path: page pools, block tables, K/V history,
+new-token K/V and queries in the shapes the benchmark configurations name.  Host arrays are numpy;
+`DeviceWorkload` uploads them and drives one layer-step (append -> split-KV map -> combine)
+through the library.  Nothing here computes attention.
+"""
+from dataclasses import dataclass
+from typing import List, Optional, Sequence
+
+import numpy as np
+
+from . import gqa as G
+
+
+def f32_to_bf16_bits(x: np.ndarray) -> np.ndarray:
+    bits = np.ascontiguousarray(x, dtype=np.float32).view(np.uint32)
+    rounded = bits + np.uint32(0x7FFF) + ((bits >> np.uint32(16)) & np.uint32(1))
+    return (rounded >> np.uint32(16)).astype(np.uint16)
+
+
+def to_storage(x: np.ndarray, dtype: G.Dtype) -> np.ndarray:
+    """f32 values -> the element storage of `dtype` (f32, or uint16 bit patterns)."""
+    if dtype == G.Dtype.Float32:
+        return np.ascontiguousarray(x, dtype=np.float32)
+    if dtype == G.Dtype.Bfloat16:
+        return f32_to_bf16_bits(x)
+    return np.ascontiguousarray(x, dtype=np.float32).astype(np.float16).view(np.uint16)
+
+
+@dataclass
+class Workload:
+    """One layer-step of a batch: `q_lens[r]` new tokens per request on top of `token_indices[r]`
+    cached ones.  The page arena holds random history everywhere; the new tokens' K/V arrive in
+    flat_k / flat_v and are appended by the step itself."""
+
+    num_q_heads: int
+    num_kv_heads: int
+    head_dim: int
+    dtype: G.Dtype
+    scale: float
+    tokens_per_page: int
+    layout: G.GQAPageTableLayout
+    layer: int
+    num_pages: int
+    req_slots: np.ndarray        # [requests]
+    token_indices: np.ndarray    # [requests] position of the first new token
+    cu_tokens: np.ndarray        # [requests + 1]
+    page_ids: np.ndarray         # the table, flat u32
+    pages: Optional[np.ndarray]  # arena storage [num_pages, 2, Hkv, P, D] (None when filled on device)
+    q: np.ndarray                # storage [tokens, Hq, D]
+    flat_k: np.ndarray           # storage [tokens, Hkv, D]
+    flat_v: np.ndarray
+    seed: int
+
+    @property
+    def page_bytes(self) -> int:
+        return 2 * self.num_kv_heads * self.tokens_per_page * self.head_dim * self.dtype.item_size()
+
+    @property
+    def num_tokens(self) -> int:
+        return int(self.cu_tokens[-1])
+
+    @property
+    def context_lens(self) -> np.ndarray:
+        """Context length of each request after the append."""
+        return self.token_indices + np.diff(self.cu_tokens)
+
+    def algorithmic_bytes(self) -> int:
+        """Bytes one layer-step must move: every visible K and V element once, Q read, O write,
+        append read + write."""
+        es = self.dtype.item_size()
+        kv = int(self.context_lens.astype(np.int64).sum()) * 2 * self.num_kv_heads * self.head_dim * es
+        t = self.num_tokens
+        qo = 2 * t * self.num_q_heads * self.head_dim * es
+        append = t * 2 * self.num_kv_heads * self.head_dim * es * 2
+        return kv + qo + append
+
+    def map_algorithmic_bytes(self) -> int:
+        """Bytes of the split-KV map kernel alone: visible K and V once plus the Q read."""
+        es = self.dtype.item_size()
+        q_lens = np.diff(self.cu_tokens).astype(np.int64)
+        # with more than one new token per request the tokens share one pass over the context
+        kv = int(self.context_lens.astype(np.int64).sum()) * 2 * self.num_kv_heads * self.head_dim * es
+        return kv + int(q_lens.sum()) * self.num_q_heads * self.head_dim * es
+
+
+def make_workload(seed: int, context_lens: Sequence[int], num_q_heads: int, num_kv_heads: int, head_dim: int,
+                  dtype: G.Dtype, tokens_per_page: int = 16, q_lens=1, scale: Optional[float] = None,
+                  input_scale: float = 1.0, num_gqa_layers: int = 1, layer: int = 0, num_page_ids_per_block: int = 1,
+                  spare_pages: int = 3, host_pages: bool = True, outlier_rate: float = 0.0,
+                  outlier_sigma: float = 8.0, shuffle_slots: bool = True) -> Workload:
+    """`context_lens[r]` counts the tokens of request r after this step's append."""
+    rng = np.random.default_rng(seed)
+    context_lens = np.asarray(context_lens, dtype=np.int64)
+    batch = len(context_lens)
+    q_lens = np.full(batch, q_lens, dtype=np.int64) if np.isscalar(q_lens) else np.asarray(q_lens, dtype=np.int64)
+    assert (context_lens >= q_lens).all() and (q_lens >= 1).all()
+    token_indices = (context_lens - q_lens).astype(np.uint32)
+    cu_tokens = np.concatenate([[0], np.cumsum(q_lens)]).astype(np.uint32)
+    pages_per_req = -(-context_lens // tokens_per_page)
+    blocks_per_req = -(-pages_per_req // num_page_ids_per_block)
+    num_blocks = int(blocks_per_req.max())
+    num_req_slots = batch + 1
+    layout = G.GQAPageTableLayout(num_req_slots, num_gqa_layers, num_blocks, num_page_ids_per_block)
+    req_slots = (rng.permutation(num_req_slots)[:batch] if shuffle_slots else np.arange(batch)).astype(np.uint32)
+    num_pages = int(pages_per_req.sum()) + spare_pages
+    pool = rng.permutation(num_pages).astype(np.uint32)
+    table = np.zeros(layout.num_page_ids(), dtype=np.uint32)
+    # rows of other layers stay zero on purpose: a kernel that walks the wrong layer reads page 0
+    cursor = 0
+    per_slot = num_gqa_layers * num_blocks * num_page_ids_per_block
+    for r in range(batch):
+        n = int(pages_per_req[r])
+        start = int(req_slots[r]) * per_slot + layer * num_blocks * num_page_ids_per_block
+        table[start:start + n] = pool[cursor:cursor + n]
+        cursor += n
+    total_tokens = int(cu_tokens[-1])
+    elems_per_page = 2 * num_kv_heads * tokens_per_page * head_dim
+
+    def normal(shape):
+        return rng.standard_normal(shape, dtype=np.float32) * np.float32(input_scale)
+
+    pages = None
+    if host_pages:
+        values = normal((num_pages, elems_per_page))
+        if outlier_rate > 0:
+            # large-magnitude K outliers: the K half of each page is [0, elems/2)
+            k_part = values[:, :elems_per_page // 2]
+            mask = rng.random(k_part.shape) < outlier_rate
+            signs = np.where(rng.random(k_part.shape) < 0.5, -1.0, 1.0).astype(np.float32)
+            k_part[mask] = (outlier_sigma * input_scale) * signs[mask]
+        pages = to_storage(values, dtype).reshape(num_pages, 2, num_kv_heads, tokens_per_page, head_dim)
+    q = to_storage(normal((total_tokens, num_q_heads, head_dim)), dtype)
+    flat_k = to_storage(normal((total_tokens, num_kv_heads, head_dim)), dtype)
+    flat_v = to_storage(normal((total_tokens, num_kv_heads, head_dim)), dtype)
+    if scale is None:
+        scale = 1.0 / float(np.sqrt(head_dim))
+    return Workload(num_q_heads, num_kv_heads, head_dim, dtype, float(scale), tokens_per_page, layout, layer,
+                    num_pages, req_slots, token_indices, cu_tokens, table, pages, q, flat_k, flat_v, seed)
+
+
+class DeviceWorkload:
+    """A workload resident in HBM plus the metadata and scratch one layer-step needs."""
+
+    def __init__(self, device: G.Device, w: Workload, partition_tokens: Optional[int] = None,
+                 max_tokens: Optional[int] = None, variant: Optional[G.GQASplitKVVariant] = None,
+                 f32_output: bool = False):
+        import torch
+
+        self.device, self.w = device, w
+        self.torch_dtype = w.dtype.torch()
+        dev = device.torch_device
+        if w.pages is not None:
+            self.pages = device.from_numpy(w.pages.reshape(-1))
+        else:
+            n = w.num_pages * 2 * w.num_kv_heads * w.tokens_per_page * w.head_dim
+            gen = torch.Generator(device=dev)
+            gen.manual_seed(w.seed)
+            self.pages = torch.empty(n, dtype=self.torch_dtype, device=dev)
+            chunk = 1 << 26
+            for start in range(0, n, chunk):
+                end = min(n, start + chunk)
+                self.pages[start:end] = torch.randn(end - start, generator=gen, device=dev,
+                                                    dtype=torch.float32).to(self.torch_dtype)
+        self.q = device.from_numpy(w.q.reshape(-1))
+        self.flat_k = device.from_numpy(w.flat_k.reshape(-1))
+        self.flat_v = device.from_numpy(w.flat_v.reshape(-1))
+        self.page_ids = device.from_numpy(w.page_ids)
+        split_kv = G.GQASplitKV.new(G.GQASplitKVConfig(w.dtype, w.page_bytes, w.num_q_heads, w.num_kv_heads,
+                                                       w.head_dim))
+        q_lens = np.diff(w.cu_tokens)
+        if variant is None:
+            variant = split_kv.select(w.num_tokens, int(sum(-(-int(n) // 8) for n in q_lens)))
+        self.variant = variant
+        rows = variant.q_token_tile_size if variant.is_tiled() else 1
+        if partition_tokens is not None:
+            if variant.is_tiled():
+                tile = variant.q_token_tile_size
+                splits_cap = int(sum(-(-int(c) // partition_tokens) * -(-int(n) // tile)
+                                     for c, n in zip(w.context_lens, q_lens)))
+            else:
+                splits_cap = int(sum(-(-(int(t) + i + 1) // partition_tokens)
+                                     for t, n in zip(w.token_indices, q_lens) for i in range(int(n))))
+            self.meta = G.GQAMetadataBuffers(device, max(w.num_tokens, 1), max_kv_splits=splits_cap)
+            self.shape = self.meta.update_fixed_partition(w.req_slots, w.token_indices, w.cu_tokens, variant,
+                                                          partition_tokens)
+        else:
+            self.meta = G.GQAMetadataBuffers(device, max_tokens or max(w.num_tokens, 1))
+            self.shape = self.meta.update(w.req_slots, w.token_indices, w.cu_tokens, variant)
+        s = self.shape
+        self.write = G.GQAKVPageWrite(device, G.GQAKVPageWriteConfig(w.num_kv_heads, w.head_dim, w.page_bytes,
+                                                                     w.dtype))
+        self.write_shape = G.GQAKVPageWriteShape(s.num_total_tokens, w.layout)
+        self.f32_output = f32_output
+        out_dtype = torch.float32 if f32_output else self.torch_dtype
+        self.output = torch.zeros(s.num_total_tokens * w.num_q_heads * w.head_dim, dtype=out_dtype, device=dev)
+        if variant.is_tiled():
+            self.cfg = G.GQASplitKVTiledQConfig(w.num_q_heads, w.num_kv_heads, w.head_dim, variant.q_head_tile_size,
+                                                variant.q_token_tile_size, variant.kv_token_tile_size, w.scale,
+                                                w.page_bytes, w.dtype, w.layout)
+            self.kshape = G.GQASplitKVTiledQShape(s.num_total_tokens, s.num_total_q_token_tiles,
+                                                  s.num_total_sdpa_map_task_templates)
+            self.kernels = G.GQASplitKVTiledQKernels(device, self.cfg, self.kshape)
+            self.scratch = G.GQASplitKVTiledQScratch(device, self.cfg, self.kshape)
+        else:
+            self.cfg = G.GQASplitKVSingleQConfig(w.num_q_heads, w.num_kv_heads, w.head_dim, w.scale, w.page_bytes,
+                                                 w.layout, variant.kv_token_tile_size,
+                                                 variant.num_threads_per_threadblock, variant.q_head_tile_size,
+                                                 w.dtype)
+            self.kshape = G.GQASplitKVSingleQShape(s.num_total_tokens, s.num_total_sdpa_map_task_templates)
+            self.kernels = G.GQASplitKVSingleQKernels(device, self.cfg, self.kshape)
+            self.scratch = G.GQASplitKVSingleQScratch(device, self.cfg, self.kshape)
+        self._rows = rows
+
+    def append(self):
+        m = self.meta
+        self.write.invoke_bucketed(
+            self.write_shape,
+            G.GQAKVPageWriteBuffers(self.pages, self.flat_k, self.flat_v, m.d_req_slots, m.d_flat_token_indices,
+                                    self.page_ids),
+            self.shape.num_tokens, self.w.layer)
+
+    def map(self):
+        m, s = self.meta, self.shape
+        if self.variant.is_tiled():
+            self.kernels.invoke_map_bucketed(self.q, self.pages, m.d_req_slots, self.page_ids,
+                                             m.d_flat_token_indices, m.d_q_token_tiles, m.d_kv_splits, self.scratch,
+                                             self.w.layer, s.num_tokens, s.num_q_token_tiles,
+                                             s.num_sdpa_map_task_templates)
+        else:
+            self.kernels.invoke_map_bucketed(self.q, self.pages, m.d_req_slots, self.page_ids, m.d_kv_splits,
+                                             self.scratch, self.w.layer, s.num_tokens,
+                                             s.num_sdpa_map_task_templates)
+
+    def reduce(self):
+        m, s = self.meta, self.shape
+        self.device.f32_output(self.f32_output)
+        if self.variant.is_tiled():
+            self.kernels.invoke_reduce_bucketed(self.scratch, m.d_q_token_tiles, m.d_cu_kv_splits, self.output,
+                                                s.num_q_token_tiles)
+        else:
+            self.kernels.invoke_reduce_bucketed(self.scratch, m.d_cu_kv_splits, self.output, s.num_tokens)
+        self.device.f32_output(False)
+
+    def step(self):
+        """One layer-step: append the new tokens, then attend (the new tokens see themselves)."""
+        self.append()
+        self.map()
+        self.reduce()
+
+    def output_f32(self) -> np.ndarray:
+        import torch
+
+        self.device.sync()
+        n = self.w.num_tokens * self.w.num_q_heads * self.w.head_dim
+        return self.output[:n].to(torch.float32).cpu().numpy()
+
+    def pages_host(self) -> np.ndarray:
+        """The arena's bytes as the storage dtype (uint16 bit patterns for 2-byte types)."""
+        import torch
+
+        self.device.sync()
+        t = self.pages
+        if t.dtype in (torch.bfloat16, torch.float16, torch.int16):
+            return t.view(torch.int16).cpu().numpy().view(np.uint16)
+        return t.cpu().numpy()
+
+
+def config_c1(seed: int = 1) -> Workload:
+    """Single-sequence decode: batch 1, context 512 after the append, 16 Q / 2 KV heads, D=256, fp16,
+    16-token pages; inputs N(0,1)/sqrt(256).  Appending position 511 keeps the pool at 32 pages."""
+    return make_workload(seed, [512], 16, 2, 256, G.Dtype.Float16, 16, input_scale=1.0 / 16.0, spare_pages=0,
+                         shuffle_slots=False)
+
+
+def config_c2_context_lens(seed: int = 2, batch: int = 32, lo: int = 1024, hi: int = 8192) -> np.ndarray:
+    rng = np.random.default_rng(seed)
+    return rng.integers(lo, hi + 1, size=batch)
+
+
+def config_c2(seed: int = 2, batch: int = 32, host_pages: bool = False, lo: int = 1024, hi: int = 8192) -> Workload:
+    """Batched ragged decode: contexts uniform in [lo, hi] (before the append), 24 Q / 4 KV heads,
+    D=256, bf16, 16-token pages from a shuffled pool; each step appends one token per sequence."""
+    ctx = config_c2_context_lens(seed, batch, lo, hi) + 1
+    return make_workload(seed, ctx, 24, 4, 256, G.Dtype.Bfloat16, 16, host_pages=host_pages)
