@@ -114,6 +114,9 @@ int psi_hip_ctx_reset_timing(psi_hip_ctx* ctx);
 /* F32_OUTPUT makes the combine kernels store the attention output as f32 [tokens, Hq, D] instead of
  * the io dtype, so a harness can check the f32-accumulated result before output rounding. */
 #define PSI_HIP_FLAG_F32_OUTPUT 2u
+/* DECODE_VALU_QK selects the decode map variant that computes QK^T with packed dot products on the
+ * vector ALU instead of MFMA tiles (kept for counter comparisons; same results within tolerance). */
+#define PSI_HIP_FLAG_DECODE_VALU_QK 3u
 int psi_hip_ctx_set_flag(psi_hip_ctx* ctx, uint32_t flag, uint32_t value);
 
 /* ------------------------------------------------------------------ geometry (host only) */

@@ -22,6 +22,7 @@ VARIANT_SINGLE_Q, VARIANT_TILED_Q = 0, 1
 CAPACITY_EXACT, CAPACITY_BUCKETED, CAPACITY_CALLER_TOKENS, CAPACITY_FIXED_PARTITION = 0, 1, 2, 3
 FLAG_FORCE_GENERIC = 1
 FLAG_F32_OUTPUT = 2
+FLAG_DECODE_VALU_QK = 3
 
 
 class PsiHipError(RuntimeError):

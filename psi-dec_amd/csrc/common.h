@@ -57,6 +57,7 @@ struct psi_hip_ctx {
     bool timing = false;
     bool force_generic = false;  // route every launch to the shape-generic kernels
     bool f32_output = false;     // combine kernels store f32 instead of the io dtype
+    bool decode_valu_qk = false; // decode map computes QK^T on the vector ALU instead of MFMA
     std::map<std::string, psi::KernelTimer> timers;
     std::vector<hipEvent_t> event_pool;
 };

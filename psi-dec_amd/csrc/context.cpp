@@ -131,9 +131,12 @@ int psi_hip_sync(psi_hip_ctx* ctx) {
 
 int psi_hip_ctx_set_flag(psi_hip_ctx* ctx, uint32_t flag, uint32_t value) {
     PSI_REQUIRE(ctx != nullptr, "ctx must not be null");
-    PSI_REQUIRE(flag == PSI_HIP_FLAG_FORCE_GENERIC || flag == PSI_HIP_FLAG_F32_OUTPUT, "unknown context flag %u", flag);
+    PSI_REQUIRE(flag == PSI_HIP_FLAG_FORCE_GENERIC || flag == PSI_HIP_FLAG_F32_OUTPUT ||
+                    flag == PSI_HIP_FLAG_DECODE_VALU_QK,
+                "unknown context flag %u", flag);
     if (flag == PSI_HIP_FLAG_FORCE_GENERIC) ctx->force_generic = value != 0;
-    else ctx->f32_output = value != 0;
+    else if (flag == PSI_HIP_FLAG_F32_OUTPUT) ctx->f32_output = value != 0;
+    else ctx->decode_valu_qk = value != 0;
     return PSI_HIP_OK;
 }
 

@@ -90,6 +90,10 @@ class Device:
     def force_generic(self, on: bool):
         L.check(self.lib.psi_hip_ctx_set_flag(self.ctx, L.FLAG_FORCE_GENERIC, int(on)))
 
+    def decode_valu_qk(self, on: bool):
+        """Decode map variant with QK^T on the vector ALU instead of MFMA (for comparisons)."""
+        L.check(self.lib.psi_hip_ctx_set_flag(self.ctx, L.FLAG_DECODE_VALU_QK, int(on)))
+
     def f32_output(self, on: bool):
         """Combine kernels then store f32 outputs (for checking the result before output rounding)."""
         L.check(self.lib.psi_hip_ctx_set_flag(self.ctx, L.FLAG_F32_OUTPUT, int(on)))
