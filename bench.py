@@ -37,6 +37,9 @@ def parse_args():
     p.add_argument("--seed", type=int, default=2)
     p.add_argument("--cpu-seconds", type=float, default=12.0, help="budget of the CPU baseline sample")
     p.add_argument("--no-cpu-baseline", action="store_true")
+    p.add_argument("--identity-pages", action="store_true", help="unshuffled page pool (diagnostic)")
+    p.add_argument("--decode-waves", type=int, default=0, help="waves per decode workgroup (0 = automatic)")
+    p.add_argument("--balance", action="store_true", help="equal-tile worker plan instead of one workgroup per partition")
     p.add_argument("--kernel-only", action="store_true", help="time only the map kernel (for profiling runs)")
     return p.parse_args()
 
@@ -114,12 +117,14 @@ def main():
         print("bench.py needs a GPU", file=sys.stderr)
         sys.exit(1)
     device = psi.Device(0)
+    device.decode_waves(args.decode_waves)
 
     arenas = []
     for i in range(max(1, args.arenas)):
-        w = wl.config_c2(seed=args.seed, batch=args.batch, host_pages=False, lo=args.ctx_lo, hi=args.ctx_hi)
+        w = wl.config_c2(seed=args.seed, batch=args.batch, host_pages=False, lo=args.ctx_lo, hi=args.ctx_hi,
+                         shuffle_pages=not args.identity_pages)
         w.seed = args.seed + 1000 * i  # same geometry, different page contents
-        arenas.append(wl.DeviceWorkload(device, w, partition_tokens=args.partition))
+        arenas.append(wl.DeviceWorkload(device, w, partition_tokens=args.partition, balanced=args.balance))
     w = arenas[0].w
     shape = arenas[0].shape
     step_bytes = w.algorithmic_bytes()

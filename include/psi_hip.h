@@ -117,6 +117,9 @@ int psi_hip_ctx_reset_timing(psi_hip_ctx* ctx);
 /* DECODE_VALU_QK selects the decode map variant that computes QK^T with packed dot products on the
  * vector ALU instead of MFMA tiles (kept for counter comparisons; same results within tolerance). */
 #define PSI_HIP_FLAG_DECODE_VALU_QK 3u
+/* DECODE_WAVES fixes the number of waves per decode-map workgroup (1, 2 or 4); 0 restores the
+ * automatic choice from the grid size. */
+#define PSI_HIP_FLAG_DECODE_WAVES 4u
 int psi_hip_ctx_set_flag(psi_hip_ctx* ctx, uint32_t flag, uint32_t value);
 
 /* ------------------------------------------------------------------ geometry (host only) */
@@ -171,6 +174,20 @@ int psi_hip_gqa_metadata_update(uint32_t max_tokens, const uint32_t* req_slots, 
                                 uint32_t* q_token_tiles, uint32_t* kv_splits, uint32_t* cu_kv_splits,
                                 psi_hip_gqa_replay_shape* out_shape);
 
+/* Balanced decode plan (no counterpart in the reference, whose planner budgets partial states, not
+ * device occupancy).  Cuts the rows of an existing SingleQ plan at tile boundaries so that
+ * `num_workers` consecutive groups of rows hold equal numbers of 16-token tiles; a decode-map
+ * workgroup then serves one group per KV head and all workgroups finish together.
+ * kv_splits_in[num_rows_in][3] / cu_in[num_tokens + 1] -> kv_splits_out (capacity rows_capacity
+ * rows, at most num_rows_in + num_workers are produced), cu_out[num_tokens + 1],
+ * worker_cu_out[num_workers + 1].  Every output row lies inside one input row. */
+int psi_hip_split_kv_balance_plan(const uint32_t* kv_splits_in, uint32_t num_rows_in, const uint32_t* cu_in,
+                                  uint32_t num_tokens, uint32_t num_workers, uint32_t* kv_splits_out,
+                                  uint32_t rows_capacity, uint32_t* cu_out, uint32_t* worker_cu_out,
+                                  uint32_t* out_num_rows);
+/* Workers per KV head that fill the device exactly once with decode-map workgroups. */
+int psi_hip_split_kv_balanced_workers(const psi_hip_gqa_config* cfg, uint32_t* out_num_workers);
+
 /* ------------------------------------------------------------------ KV append */
 
 /* `GQAKVPageWrite::invoke_bucketed(...)` recorded and submitted
@@ -205,6 +222,19 @@ int psi_hip_split_kv_single_q_map(psi_hip_ctx* ctx, const psi_hip_gqa_config* cf
                                   uint32_t gqa_layer_index, uint32_t num_total_tokens,
                                   uint32_t num_total_kv_splits, uint32_t num_active_tokens,
                                   uint32_t num_active_kv_splits);
+
+/* The same map launched over a balanced plan: workgroup w of each KV head serves kv_splits rows
+ * [worker_cu[w], worker_cu[w + 1]) (device u32[num_workers + 1], from psi_hip_split_kv_balance_plan).
+ * Falls back to the row-per-workgroup launch for shapes outside the gfx950 kernels' domain. */
+int psi_hip_split_kv_single_q_map_balanced(psi_hip_ctx* ctx, const psi_hip_gqa_config* cfg,
+                                           const psi_hip_page_table_layout* layout, const void* q,
+                                           const void* kv_pages, uint64_t kv_pages_bytes,
+                                           const uint32_t* req_slots, const uint32_t* page_ids,
+                                           const uint32_t* kv_splits, const uint32_t* worker_cu,
+                                           uint32_t num_workers, void* scratch, uint64_t scratch_bytes,
+                                           uint32_t gqa_layer_index, uint32_t num_total_tokens,
+                                           uint32_t num_total_kv_splits, uint32_t num_active_tokens,
+                                           uint32_t num_active_kv_splits);
 
 /* `GQASplitKVSingleQKernels::invoke_reduce_bucketed` (gqa_split_kv_single_q.rs:353-383; kernel
  * metal/gqa_split_kv_single_q_reduce.metal:10-49).  cu_kv_splits: device u32[num_total_tokens + 1];

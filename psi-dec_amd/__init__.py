@@ -37,5 +37,6 @@ from .gqa import (  # noqa: F401
     GQASplitKVTiledQShape,
     GQASplitKVVariant,
     ReplayBucketPolicy,
+    balanced_workers,
     select_split_kv_variant,
 )

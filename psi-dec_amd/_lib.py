@@ -23,6 +23,7 @@ CAPACITY_EXACT, CAPACITY_BUCKETED, CAPACITY_CALLER_TOKENS, CAPACITY_FIXED_PARTIT
 FLAG_FORCE_GENERIC = 1
 FLAG_F32_OUTPUT = 2
 FLAG_DECODE_VALU_QK = 3
+FLAG_DECODE_WAVES = 4
 
 
 class PsiHipError(RuntimeError):
@@ -103,6 +104,14 @@ PROTOTYPES = {
         c_int,
         [c_uint32, _U32P, _U32P, _U32P, c_uint32, _VARIANT, c_uint32, c_uint32, _U32P, c_uint32, c_uint32, c_uint32,
          _U32P, _U32P, _U32P, _U32P, _U32P, POINTER(ReplayShapeStruct)],
+    ),
+    "psi_hip_split_kv_balance_plan": (
+        c_int, [_U32P, c_uint32, _U32P, c_uint32, c_uint32, _U32P, c_uint32, _U32P, _U32P, _U32P]),
+    "psi_hip_split_kv_balanced_workers": (c_int, [_CFG, _U32P]),
+    "psi_hip_split_kv_single_q_map_balanced": (
+        c_int,
+        [c_void_p, _CFG, _LAYOUT, c_void_p, c_void_p, c_uint64, c_void_p, c_void_p, c_void_p, c_void_p, c_uint32,
+         c_void_p, c_uint64, c_uint32, c_uint32, c_uint32, c_uint32, c_uint32],
     ),
     "psi_hip_kv_page_write": (
         c_int,

@@ -58,6 +58,7 @@ struct psi_hip_ctx {
     bool force_generic = false;  // route every launch to the shape-generic kernels
     bool f32_output = false;     // combine kernels store f32 instead of the io dtype
     bool decode_valu_qk = false; // decode map computes QK^T on the vector ALU instead of MFMA
+    int decode_waves_override = 0;  // 0 = choose waves per decode workgroup from the grid size
     std::map<std::string, psi::KernelTimer> timers;
     std::vector<hipEvent_t> event_pool;
 };

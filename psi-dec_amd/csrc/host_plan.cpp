@@ -502,3 +502,70 @@ extern "C" int psi_hip_gqa_metadata_update(uint32_t max_tokens, const uint32_t* 
     out_shape->reduce_sdpa_partial_outputs = (tiled || num_kv_splits > num_tokens) ? 1u : 0u;
     return PSI_HIP_OK;
 }
+
+extern "C" int psi_hip_split_kv_balanced_workers(const psi_hip_gqa_config* cfg, uint32_t* out_num_workers) {
+    Geometry g;
+    int rc = make_geometry(cfg, &g);
+    if (rc != PSI_HIP_OK) return rc;
+    PSI_REQUIRE(out_num_workers != nullptr, "out pointer must not be null");
+    // 256 compute units, three 4-wave workgroups resident on each
+    *out_num_workers = std::max(1u, (256u * 3u) / g.hkv);
+    return PSI_HIP_OK;
+}
+
+extern "C" int psi_hip_split_kv_balance_plan(const uint32_t* kv_splits_in, uint32_t num_rows_in,
+                                             const uint32_t* cu_in, uint32_t num_tokens, uint32_t num_workers,
+                                             uint32_t* kv_splits_out, uint32_t rows_capacity, uint32_t* cu_out,
+                                             uint32_t* worker_cu_out, uint32_t* out_num_rows) {
+    PSI_REQUIRE(kv_splits_in && cu_in && kv_splits_out && cu_out && worker_cu_out && out_num_rows,
+                "balanced plan arrays must not be null");
+    PSI_REQUIRE(num_workers > 0 && num_tokens > 0, "balanced plan needs workers and tokens");
+    PSI_REQUIRE(cu_in[0] == 0 && cu_in[num_tokens] == num_rows_in, "cu_kv_splits must cover every input row");
+    constexpr uint32_t kTile = 16;
+    auto tiles_of = [&](uint32_t r) -> uint64_t {
+        const uint32_t b = kv_splits_in[3 * r + 1], e = kv_splits_in[3 * r + 2];
+        return e > b ? (uint64_t)(e + kTile - 1) / kTile - b / kTile : 0;
+    };
+    uint64_t total = 0;
+    for (uint32_t r = 0; r < num_rows_in; ++r) {
+        PSI_REQUIRE(kv_splits_in[3 * r] < num_tokens, "balanced plan input must not hold padding rows");
+        total += tiles_of(r);
+    }
+    uint32_t out_rows = 0, worker = 0;
+    uint64_t linear = 0;  // tiles emitted so far
+    auto worker_end = [&](uint32_t w) { return total * (w + 1) / num_workers; };
+    worker_cu_out[0] = 0;
+    uint32_t token = 0;
+    cu_out[0] = 0;
+    for (uint32_t r = 0; r < num_rows_in; ++r) {
+        while (token < num_tokens && r >= cu_in[token + 1]) cu_out[++token] = out_rows;
+        const uint32_t b = kv_splits_in[3 * r + 1], e = kv_splits_in[3 * r + 2];
+        uint64_t remaining = tiles_of(r);
+        uint32_t tile_cursor = b / kTile;
+        if (remaining == 0) {  // degenerate row: keep it so that row counts per token stay positive
+            PSI_REQUIRE(out_rows < rows_capacity, "balanced plan exceeds the row capacity");
+            kv_splits_out[3 * out_rows] = kv_splits_in[3 * r];
+            kv_splits_out[3 * out_rows + 1] = b;
+            kv_splits_out[3 * out_rows + 2] = e;
+            ++out_rows;
+            continue;
+        }
+        while (remaining > 0) {
+            while (worker + 1 < num_workers && linear >= worker_end(worker)) worker_cu_out[++worker] = out_rows;
+            const uint64_t room = worker + 1 < num_workers ? worker_end(worker) - linear : remaining;
+            const uint64_t take = std::min<uint64_t>(remaining, std::max<uint64_t>(room, 1));
+            PSI_REQUIRE(out_rows < rows_capacity, "balanced plan exceeds the row capacity");
+            kv_splits_out[3 * out_rows] = kv_splits_in[3 * r];
+            kv_splits_out[3 * out_rows + 1] = std::max<uint32_t>(b, tile_cursor * kTile);
+            kv_splits_out[3 * out_rows + 2] = (uint32_t)std::min<uint64_t>(e, (uint64_t)(tile_cursor + take) * kTile);
+            ++out_rows;
+            tile_cursor += (uint32_t)take;
+            remaining -= take;
+            linear += take;
+        }
+    }
+    while (token < num_tokens) cu_out[++token] = out_rows;
+    while (worker < num_workers) worker_cu_out[++worker] = out_rows;
+    *out_num_rows = out_rows;
+    return PSI_HIP_OK;
+}

@@ -46,6 +46,10 @@ struct MapArgs {
     const uint32_t* flat_token_indices = nullptr;  // request-absolute position of each flat token
     uint32_t rows_per_split_head = 1;              // q_token_tile_size
     uint32_t num_active_q_token_tiles = 0;
+    // Balanced decode launch only: workgroup w of a KV head serves kv_splits rows
+    // [worker_cu[w], worker_cu[w + 1]).
+    const uint32_t* worker_cu = nullptr;
+    uint32_t num_workers = 0;
 };
 
 struct ReduceArgs {

@@ -1,0 +1,8 @@
+// Instantiates the gfx950 decode map for f16 K/V, head_dim 256 (all group sizes and workgroup widths).
+#include "split_kv_decode_kernel.h"
+
+namespace psi {
+int launch_decode_map_f16_d256(psi_hip_ctx* ctx, const Geometry& g, const MapArgs& a) {
+    return launch_decode_map_group<F16Tag, 256>(ctx, g, a);
+}
+}  // namespace psi

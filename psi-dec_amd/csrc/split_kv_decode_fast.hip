@@ -1,336 +1,13 @@
-// gfx950 split-KV grouped-query decode map and log-sum-exp combine for 2-byte K/V (bf16 / f16),
-// head_dim 128 or 256, pages of 16*k tokens.
-//
-// Work decomposition
-//   one workgroup (4 waves) = one (kv_split, kv_head); it serves all G query heads of that KV head
-//   one wave = every 4th 16-token tile of the split, with its own online-softmax state; the four
-//   wave states are merged through LDS once, at the end.
-//
-// Per 16-token tile and wave
-//   QK^T  one 16x16 MFMA tile: A = the K tile (16 tokens x head_dim, read straight from the page
-//         with 128-bit loads, lane = (token lane%16, 8-dim chunk lane/16)), B = the query group
-//         (G rows, zero-padded to 16) held in registers for the whole split.  The contraction runs
-//         over head_dim, which is the contiguous axis of a K line, so no transpose is needed.
-//   softmax  the MFMA result leaves each lane with 4 tokens of one query row; tile maximum by two
-//         cross-row exchanges; probabilities go to LDS as P[token][head].
-//   PV    vector ALU: lane = (token parity, 8 dims); each 128-bit load instruction covers 1 KiB of
-//         contiguous V lines; acc[G][8] stays in registers for the whole split.  (PV contracts
-//         over tokens, the strided axis of V, so it stays on the vector ALU with P broadcast
-//         from LDS.)
-//   Loads are software-pipelined one tile ahead: every K / V register is re-requested for the
-//   next tile right after its last use in the current one.
-//
-// Algorithmic bytes per (kv token, kv head): 2 * head_dim * 2 (one K and one V line), read once.
-#include <type_traits>
-
+// Dispatch of the gfx950 split-KV decode map (instantiated per element type and head_dim in the
+// split_kv_decode_*.hip files) and the gfx950 log-sum-exp combine kernel.
 #include "split_kv.h"
 
 namespace psi {
 
-typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8_t;
-typedef __attribute__((ext_vector_type(8))) _Float16 f16x8_t;
-typedef __attribute__((ext_vector_type(4))) float f32x4_t;
-typedef __attribute__((ext_vector_type(2))) _Float16 f16x2_t;
-
-// D(16x16, f32) += A(16x32) * B(32x16).  Lane l holds A[row l%16][k 8*(l/16)..+8],
-// B[k 8*(l/16)..+8][col l%16] and D[row 4*(l/16)+r][col l%16], r = 0..3.
-template <typename Tag>
-__device__ __forceinline__ f32x4_t mfma_16x16x32(uint4 a, uint4 b, f32x4_t c);
-template <>
-__device__ __forceinline__ f32x4_t mfma_16x16x32<BF16Tag>(uint4 a, uint4 b, f32x4_t c) {
-    return __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8_t, a), __builtin_bit_cast(bf16x8_t, b), c,
-                                                   0, 0, 0);
-}
-template <>
-__device__ __forceinline__ f32x4_t mfma_16x16x32<F16Tag>(uint4 a, uint4 b, f32x4_t c) {
-    return __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(f16x8_t, a), __builtin_bit_cast(f16x8_t, b), c,
-                                                  0, 0, 0);
-}
-
-template <typename Tag>
-__device__ __forceinline__ void unpack2(uint32_t packed, float& lo, float& hi);
-template <>
-__device__ __forceinline__ void unpack2<BF16Tag>(uint32_t packed, float& lo, float& hi) {
-    lo = __uint_as_float(packed << 16);
-    hi = __uint_as_float(packed & 0xffff0000u);
-}
-template <>
-__device__ __forceinline__ void unpack2<F16Tag>(uint32_t packed, float& lo, float& hi) {
-    const f16x2_t h = __builtin_bit_cast(f16x2_t, packed);
-    lo = (float)h.x;
-    hi = (float)h.y;
-}
-
-// Orders this wave's LDS traffic: earlier LDS operations have completed and the compiler keeps
-// later ones after this point.  A wave's LDS operations execute in issue order.
-__device__ __forceinline__ void wave_lds_fence() { asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory"); }
-
-constexpr int kTileTokens = 16;
-constexpr int kWaves = 4;
-
-template <typename Tag, int D, int G>
-__global__ __launch_bounds__(256, 2) void split_kv_decode_map(
-    MapArgs a, const uint32_t* __restrict__ page_ids, const uint32_t* __restrict__ kv_splits,
-    const uint32_t* __restrict__ req_slots, const uint16_t* __restrict__ q, const uint16_t* __restrict__ pages) {
-    constexpr int kVLanesPerToken = D / 8;                  // 32 (D=256) or 16 (D=128)
-    constexpr int kVTokensPerLoad = 64 / kVLanesPerToken;   // 2 or 4
-    constexpr int kVLoads = kTileTokens / kVTokensPerLoad;  // 8 or 4
-    constexpr int kKSteps = D / 32;                         // 8 or 4 MFMA k-steps
-    constexpr int kPStride = 8;                             // floats per token row of P in LDS
-
-    const uint32_t kv_head = blockIdx.x % a.walk.hkv;
-    const uint32_t split = blockIdx.x / a.walk.hkv;
-    if (split >= a.num_active_kv_splits) return;
-    const uint32_t q_token = kv_splits[split * 3];
-    if (q_token >= a.num_active_tokens) return;  // sentinel padding or a slot owned by another producer
-    const uint32_t kv_begin = kv_splits[split * 3 + 1];
-    const uint32_t kv_end = kv_splits[split * 3 + 2];
-    const uint32_t req_slot = req_slots[q_token];
-
-    const uint32_t tid = threadIdx.x;
-    const uint32_t lane = tid & 63;
-    const uint32_t wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-
-    __shared__ __attribute__((aligned(16))) float p_lds[kWaves][kTileTokens * kPStride];
-    __shared__ __attribute__((aligned(16))) float alpha_lds[kWaves][8];
-    __shared__ __attribute__((aligned(16))) float merge_acc[kWaves][G * D];
-    __shared__ float merge_max[kWaves][G];
-    __shared__ float merge_sum[kWaves][G];
-
-    // MFMA lane coordinates: row of A (token) and column of B / D (query row); 8-dim chunk of A
-    // and B, token quad of D.
-    const uint32_t mt = lane & 15, mc = lane >> 4;
-    // V lane coordinates.
-    const uint32_t vsub = lane / kVLanesPerToken, vdl = lane % kVLanesPerToken;
-
-    // Query group as the B operand, unscaled, in its native 2-byte type; rows >= G are zero.
-    uint4 qb[kKSteps];
-    {
-        const uint16_t* q_row = q +
-                                ((uint64_t)q_token * a.hq + (uint64_t)kv_head * G + (mt < (uint32_t)G ? mt : 0)) * D +
-                                mc * 8;
-#pragma unroll
-        for (int i = 0; i < kKSteps; ++i) {
-            const uint4 v = *reinterpret_cast<const uint4*>(q_row + i * 32);
-            qb[i] = mt < (uint32_t)G ? v : make_uint4(0, 0, 0, 0);
-        }
-    }
-
-    const uint32_t log2p = 31 - __builtin_clz(a.walk.tokens_per_page);
-    const uint32_t page_mask = a.walk.tokens_per_page - 1;
-    const uint32_t* table_row = page_ids + ((uint64_t)req_slot * a.walk.num_layers + a.layer) *
-                                                      a.walk.num_blocks * a.walk.ids_per_block;
-    const uint64_t v_region = (uint64_t)a.walk.hkv * a.walk.tokens_per_page * D;
-
-    const uint32_t tile_begin = kv_begin / kTileTokens;
-    const uint32_t tile_end = (kv_end + kTileTokens - 1) / kTileTokens;
-
-    float run_max = -INFINITY, lane_sum = 0.0f;  // of query row mt, over this lane's tokens
-    float acc[G][8];
-#pragma unroll
-    for (int h = 0; h < G; ++h)
-#pragma unroll
-        for (int e = 0; e < 8; ++e) acc[h][e] = 0.0f;
-
-    auto load_page_id = [&](uint32_t tile) -> uint32_t {
-        return tile < tile_end ? table_row[(tile * kTileTokens) >> log2p] : 0u;
-    };
-    auto tile_k_base = [&](uint32_t tile, uint32_t page_id) -> const uint16_t* {
-        const uint32_t in_page = (tile * kTileTokens) & page_mask;
-        return pages + (uint64_t)page_id * a.walk.page_elems +
-               ((uint64_t)kv_head * a.walk.tokens_per_page + in_page) * D;
-    };
-
-    // One K and one V register buffer per wave.  A buffer entry is re-requested for the next tile
-    // as soon as its last use in the current tile has issued, so each load has about a whole tile
-    // period to land while the wave keeps only 16 KiB of tile data in registers.
-    uint4 kreg[kKSteps];  // lane (t = lane%16, c = lane/16): step i = dims [i*32 + c*8, +8) of token t
-    uint4 vreg[kVLoads];  // lane (sub, dl): load j = token j*kVTokensPerLoad + sub, dims [dl*8, +8)
-    auto issue_k = [&](uint32_t tile, uint32_t page_id) {
-        const uint16_t* k_lane = tile_k_base(tile, page_id) + mt * D + mc * 8;
-#pragma unroll
-        for (int i = 0; i < kKSteps; ++i) kreg[i] = *reinterpret_cast<const uint4*>(k_lane + i * 32);
-    };
-    auto v_lane_of = [&](uint32_t tile, uint32_t page_id) -> const uint16_t* {
-        return tile_k_base(tile, page_id) + v_region + vsub * D + vdl * 8;
-    };
-
-    float* my_p = p_lds[wave];
-    float* my_alpha = alpha_lds[wave];
-
-    // One 16-token tile.  `partial`: the tile holds tokens outside [kv_begin, kv_end).
-    // `has_next`: another tile of this wave follows; its K and V are requested on the way, each
-    // into the registers the current tile has just finished with.  Both flags are wave-uniform.
-    auto process_tile = [&](uint32_t tile, bool partial, auto has_next_tag, uint32_t next, uint32_t next_pid)
-                            __attribute__((always_inline)) {
-        // compile-time flag: the steady-state copy issues its refill loads unconditionally, which
-        // keeps the hardware load counter's order exact for the waits that follow
-        constexpr bool has_next = decltype(has_next_tag)::value;
-        // ---- logits of query rows x 16 tokens on the matrix cores
-        f32x4_t s0 = {0.0f, 0.0f, 0.0f, 0.0f}, s1 = {0.0f, 0.0f, 0.0f, 0.0f};
-#pragma unroll
-        for (int i = 0; i < kKSteps; i += 2) {
-            s0 = mfma_16x16x32<Tag>(kreg[i], qb[i], s0);
-            s1 = mfma_16x16x32<Tag>(kreg[i + 1], qb[i + 1], s1);
-        }
-        __builtin_amdgcn_sched_barrier(0);
-        if (has_next) issue_k(next, next_pid);
-        __builtin_amdgcn_sched_barrier(0);
-        // ---- online softmax of query row mt over this lane's tokens 4*mc + r
-        float v[4];
-        float m = -INFINITY;
-#pragma unroll
-        for (int r = 0; r < 4; ++r) {
-            const uint32_t token = tile * kTileTokens + mc * 4 + r;
-            const bool valid = token >= kv_begin && token < kv_end;
-            v[r] = valid ? (s0[r] + s1[r]) * a.scale_log2 : -INFINITY;
-            m = fmaxf(m, v[r]);
-        }
-        m = fmaxf(m, __shfl_xor(m, 16, 64));
-        m = fmaxf(m, __shfl_xor(m, 32, 64));
-        const float next_max = fmaxf(run_max, m);
-        const float alpha = __builtin_amdgcn_exp2f(run_max - next_max);  // 0 on the first tile
-        const bool rescale = __any(mt < (uint32_t)G && next_max != run_max);
-        run_max = next_max;
-        float p[4], tile_sum = 0.0f;
-#pragma unroll
-        for (int r = 0; r < 4; ++r) {
-            p[r] = __builtin_amdgcn_exp2f(v[r] - next_max);
-            tile_sum += p[r];
-        }
-        lane_sum = lane_sum * alpha + tile_sum;
-        wave_lds_fence();  // the previous tile's P reads are complete
-        if (mt < 8) {
-#pragma unroll
-            for (int r = 0; r < 4; ++r) my_p[(mc * 4 + r) * kPStride + mt] = p[r];
-            if (mc == 0) my_alpha[mt] = alpha;
-        }
-        wave_lds_fence();
-
-        // ---- acc[h][e] += P[token][h] * V[token][dl*8 + e] on the vector ALU
-        if (rescale) {
-            float al[8];
-            const float4 a0 = *reinterpret_cast<const float4*>(&my_alpha[0]);
-            al[0] = a0.x; al[1] = a0.y; al[2] = a0.z; al[3] = a0.w;
-            if (G > 4) {
-                const float4 a1 = *reinterpret_cast<const float4*>(&my_alpha[4]);
-                al[4] = a1.x; al[5] = a1.y; al[6] = a1.z; al[7] = a1.w;
-            }
-#pragma unroll
-            for (int h = 0; h < G; ++h)
-#pragma unroll
-                for (int e = 0; e < 8; ++e) acc[h][e] *= al[h];
-        }
-        if (partial) {
-            // tokens outside the split carry probability 0, but their V bytes may be NaN/Inf
-#pragma unroll
-            for (int j = 0; j < kVLoads; ++j) {
-                const uint32_t vtoken = tile * kTileTokens + j * kVTokensPerLoad + vsub;
-                if (vtoken < kv_begin || vtoken >= kv_end) vreg[j] = make_uint4(0, 0, 0, 0);
-            }
-        }
-        __builtin_amdgcn_sched_barrier(0);
-#pragma unroll
-        for (int j = 0; j < kVLoads; ++j) {
-            const uint32_t tok_in_tile = j * kVTokensPerLoad + vsub;
-            float pr[8];
-            {
-                const float4 p0 = *reinterpret_cast<const float4*>(&my_p[tok_in_tile * kPStride]);
-                pr[0] = p0.x; pr[1] = p0.y; pr[2] = p0.z; pr[3] = p0.w;
-                if (G > 4) {
-                    const float4 p1 = *reinterpret_cast<const float4*>(&my_p[tok_in_tile * kPStride + 4]);
-                    pr[4] = p1.x; pr[5] = p1.y; pr[6] = p1.z; pr[7] = p1.w;
-                }
-            }
-            float vf[8];
-            unpack2<Tag>(vreg[j].x, vf[0], vf[1]);
-            unpack2<Tag>(vreg[j].y, vf[2], vf[3]);
-            unpack2<Tag>(vreg[j].z, vf[4], vf[5]);
-            unpack2<Tag>(vreg[j].w, vf[6], vf[7]);
-#pragma unroll
-            for (int h = 0; h < G; ++h)
-#pragma unroll
-                for (int e = 0; e < 8; ++e) acc[h][e] = fmaf(pr[h], vf[e], acc[h][e]);
-            // keeps later P reads and V unpacks from being hoisted above this point (register budget)
-            __builtin_amdgcn_sched_barrier(0);
-        }
-        if (has_next) {
-            const uint16_t* v_next = v_lane_of(next, next_pid);
-#pragma unroll
-            for (int j = 0; j < kVLoads; ++j) vreg[j] = *reinterpret_cast<const uint4*>(v_next + j * kVTokensPerLoad * D);
-        }
-        __builtin_amdgcn_sched_barrier(0);
-    };
-
-    uint32_t tile = tile_begin + wave;
-    if (tile < tile_end) {
-        {
-            const uint32_t pid = load_page_id(tile);
-            issue_k(tile, pid);
-            const uint16_t* v_lane = v_lane_of(tile, pid);
-#pragma unroll
-            for (int j = 0; j < kVLoads; ++j) vreg[j] = *reinterpret_cast<const uint4*>(v_lane + j * kVTokensPerLoad * D);
-        }
-        uint32_t pid_next = load_page_id(tile + kWaves);
-        auto is_partial = [&](uint32_t t) { return t * kTileTokens < kv_begin || (t + 1) * kTileTokens > kv_end; };
-        while (tile + kWaves < tile_end) {
-            const uint32_t next = tile + kWaves;
-            const uint32_t pid_after = load_page_id(next + kWaves);
-            process_tile(tile, is_partial(tile), std::true_type(), next, pid_next);
-            pid_next = pid_after;
-            tile = next;
-        }
-        process_tile(tile, is_partial(tile), std::false_type(), 0u, 0u);  // the wave's last tile
-    }
-
-    // ---- wave epilogue: fold the V token sub-lanes together, reduce the per-lane sums.
-#pragma unroll
-    for (int h = 0; h < G; ++h)
-#pragma unroll
-        for (int e = 0; e < 8; ++e) {
-            float v = acc[h][e];
-            v += __shfl_xor(v, 32, 64);
-            if (kVTokensPerLoad == 4) v += __shfl_xor(v, 16, 64);
-            acc[h][e] = v;
-        }
-    lane_sum += __shfl_xor(lane_sum, 16, 64);
-    lane_sum += __shfl_xor(lane_sum, 32, 64);
-    if (lane < (uint32_t)kVLanesPerToken) {
-#pragma unroll
-        for (int h = 0; h < G; ++h) {
-            float4* dst = reinterpret_cast<float4*>(&merge_acc[wave][h * D + lane * 8]);
-            dst[0] = make_float4(acc[h][0], acc[h][1], acc[h][2], acc[h][3]);
-            dst[1] = make_float4(acc[h][4], acc[h][5], acc[h][6], acc[h][7]);
-        }
-    }
-    if (lane < (uint32_t)G) {  // mc == 0, mt = lane: one lane per query row
-        merge_max[wave][lane] = run_max;
-        merge_sum[wave][lane] = lane_sum;
-    }
-    __syncthreads();
-
-    // ---- merge the four wave states and emit the partial of (split, q_head).
-    for (uint32_t idx = tid; idx < (uint32_t)(G * D); idx += 256) {
-        const uint32_t h = idx / D, dim = idx % D;
-        float m = merge_max[0][h];
-#pragma unroll
-        for (int w = 1; w < kWaves; ++w) m = fmaxf(m, merge_max[w][h]);
-        float out = 0.0f, sum = 0.0f;
-#pragma unroll
-        for (int w = 0; w < kWaves; ++w) {
-            const float mw = merge_max[w][h];
-            const float f = mw > -INFINITY ? exp2f(mw - m) : 0.0f;
-            out = fmaf(f, merge_acc[w][idx], out);
-            sum = fmaf(f, merge_sum[w][h], sum);
-        }
-        const uint64_t row = (uint64_t)split * a.hq + (uint64_t)kv_head * G + h;
-        a.part_acc[row * D + dim] = out;
-        if (dim == 0) {
-            a.part_max[row] = m;
-            a.part_sum[row] = sum;
-        }
-    }
-}
+int launch_decode_map_bf16_d256(psi_hip_ctx* ctx, const Geometry& g, const MapArgs& a);
+int launch_decode_map_bf16_d128(psi_hip_ctx* ctx, const Geometry& g, const MapArgs& a);
+int launch_decode_map_f16_d256(psi_hip_ctx* ctx, const Geometry& g, const MapArgs& a);
+int launch_decode_map_f16_d128(psi_hip_ctx* ctx, const Geometry& g, const MapArgs& a);
 
 // Log-sum-exp combine: one wave per (token, q_head), lanes over head_dim.
 template <typename Tag, int D>
@@ -361,34 +38,12 @@ __global__ __launch_bounds__(256) void split_kv_reduce_fast(ReduceArgs a) {
     for (int e = 0; e < kPerLane; ++e) store_from_f32<Tag>(a.output, out_index + e, value[e] * inv);
 }
 
-template <typename Tag, int D>
-static int launch_map_g(psi_hip_ctx* ctx, const Geometry& g, const MapArgs& a) {
-    const dim3 grid(a.num_total_kv_splits * g.hkv), block(256);
-    switch (g.group) {
-#define PSI_CASE(G)                                                                              \
-    case G:                                                                                      \
-        hipLaunchKernelGGL((split_kv_decode_map<Tag, D, G>), grid, block, 0, ctx->stream, a,      \
-                           a.walk.page_ids, a.kv_splits, a.req_slots,                                \
-                           reinterpret_cast<const uint16_t*>(a.q),                                   \
-                           reinterpret_cast<const uint16_t*>(a.kv_pages));                           \
-        return PSI_HIP_OK;
-        PSI_CASE(1)
-        PSI_CASE(2)
-        PSI_CASE(3)
-        PSI_CASE(4)
-        PSI_CASE(5)
-        PSI_CASE(6)
-        PSI_CASE(7)
-        PSI_CASE(8)
-#undef PSI_CASE
-        default:
-            return PSI_HIP_ERR_UNSUPPORTED;
-    }
-}
-
 int launch_decode_map_fast(psi_hip_ctx* ctx, const Geometry& g, const MapArgs& a) {
     if (ctx->force_generic) return PSI_HIP_ERR_UNSUPPORTED;
-    if (ctx->decode_valu_qk) return launch_decode_map_valu(ctx, g, a);
+    if (ctx->decode_valu_qk) {
+        if (a.worker_cu != nullptr) return PSI_HIP_ERR_UNSUPPORTED;  // the comparison variant is row-per-workgroup
+        return launch_decode_map_valu(ctx, g, a);
+    }
     const bool two_byte = g.dtype == PSI_HIP_BF16 || g.dtype == PSI_HIP_F16;
     const uint32_t p = g.tokens_per_page;
     const bool page_ok = p >= 16 && (p & (p - 1)) == 0;
@@ -396,8 +51,8 @@ int launch_decode_map_fast(psi_hip_ctx* ctx, const Geometry& g, const MapArgs& a
     if (!two_byte || !page_ok || !aligned || g.group > 8 || (g.d != 256 && g.d != 128)) return PSI_HIP_ERR_UNSUPPORTED;
     if ((uint64_t)a.num_total_kv_splits * g.hkv > 0x7fffffffull) return PSI_HIP_ERR_UNSUPPORTED;
     if (g.dtype == PSI_HIP_BF16)
-        return g.d == 256 ? launch_map_g<BF16Tag, 256>(ctx, g, a) : launch_map_g<BF16Tag, 128>(ctx, g, a);
-    return g.d == 256 ? launch_map_g<F16Tag, 256>(ctx, g, a) : launch_map_g<F16Tag, 128>(ctx, g, a);
+        return g.d == 256 ? launch_decode_map_bf16_d256(ctx, g, a) : launch_decode_map_bf16_d128(ctx, g, a);
+    return g.d == 256 ? launch_decode_map_f16_d256(ctx, g, a) : launch_decode_map_f16_d128(ctx, g, a);
 }
 
 int launch_reduce_fast(psi_hip_ctx* ctx, const Geometry& g, const ReduceArgs& a) {

@@ -41,14 +41,12 @@ extern "C" int psi_hip_split_kv_single_q_scratch_bytes(const psi_hip_gqa_config*
     return PSI_HIP_OK;
 }
 
-extern "C" int psi_hip_split_kv_single_q_map(psi_hip_ctx* ctx, const psi_hip_gqa_config* cfg,
-                                             const psi_hip_page_table_layout* layout, const void* q,
-                                             const void* kv_pages, uint64_t kv_pages_bytes,
-                                             const uint32_t* req_slots, const uint32_t* page_ids,
-                                             const uint32_t* kv_splits, void* scratch, uint64_t scratch_bytes,
-                                             uint32_t gqa_layer_index, uint32_t num_total_tokens,
-                                             uint32_t num_total_kv_splits, uint32_t num_active_tokens,
-                                             uint32_t num_active_kv_splits) {
+static int single_q_map_impl(psi_hip_ctx* ctx, const psi_hip_gqa_config* cfg, const psi_hip_page_table_layout* layout,
+                             const void* q, const void* kv_pages, uint64_t kv_pages_bytes, const uint32_t* req_slots,
+                             const uint32_t* page_ids, const uint32_t* kv_splits, const uint32_t* worker_cu,
+                             uint32_t num_workers, void* scratch, uint64_t scratch_bytes, uint32_t gqa_layer_index,
+                             uint32_t num_total_tokens, uint32_t num_total_kv_splits, uint32_t num_active_tokens,
+                             uint32_t num_active_kv_splits) {
     PSI_REQUIRE(ctx != nullptr, "ctx must not be null");
     Geometry g;
     int rc = make_geometry(cfg, &g);
@@ -87,18 +85,49 @@ extern "C" int psi_hip_split_kv_single_q_map(psi_hip_ctx* ctx, const psi_hip_gqa
     a.num_active_tokens = num_active_tokens;
     a.num_active_kv_splits = num_active_kv_splits;
     a.scale_log2 = g.scale * kLog2e;
+    a.worker_cu = worker_cu;
+    a.num_workers = num_workers;
 
     LaunchScope scope(ctx, "split_kv_map");
     rc = launch_decode_map_fast(ctx, g, a);
     if (rc == PSI_HIP_ERR_UNSUPPORTED) {
         const uint64_t grid = (uint64_t)num_total_kv_splits * g.hq * ((g.d + 63) / 64);
         PSI_REQUIRE(grid <= 0x7fffffffull, "GQA SDPA map threads exceeds the shader u32 count domain");
+        a.worker_cu = nullptr;  // the generic kernel launches one workgroup per row
         launch_map_generic(ctx, g, a);
         rc = PSI_HIP_OK;
     }
     if (rc != PSI_HIP_OK) return rc;
     PSI_HIP_CHECK(hipGetLastError());
     return PSI_HIP_OK;
+}
+
+extern "C" int psi_hip_split_kv_single_q_map(psi_hip_ctx* ctx, const psi_hip_gqa_config* cfg,
+                                             const psi_hip_page_table_layout* layout, const void* q,
+                                             const void* kv_pages, uint64_t kv_pages_bytes,
+                                             const uint32_t* req_slots, const uint32_t* page_ids,
+                                             const uint32_t* kv_splits, void* scratch, uint64_t scratch_bytes,
+                                             uint32_t gqa_layer_index, uint32_t num_total_tokens,
+                                             uint32_t num_total_kv_splits, uint32_t num_active_tokens,
+                                             uint32_t num_active_kv_splits) {
+    return single_q_map_impl(ctx, cfg, layout, q, kv_pages, kv_pages_bytes, req_slots, page_ids, kv_splits, nullptr, 0,
+                             scratch, scratch_bytes, gqa_layer_index, num_total_tokens, num_total_kv_splits,
+                             num_active_tokens, num_active_kv_splits);
+}
+
+extern "C" int psi_hip_split_kv_single_q_map_balanced(psi_hip_ctx* ctx, const psi_hip_gqa_config* cfg,
+                                                      const psi_hip_page_table_layout* layout, const void* q,
+                                                      const void* kv_pages, uint64_t kv_pages_bytes,
+                                                      const uint32_t* req_slots, const uint32_t* page_ids,
+                                                      const uint32_t* kv_splits, const uint32_t* worker_cu,
+                                                      uint32_t num_workers, void* scratch, uint64_t scratch_bytes,
+                                                      uint32_t gqa_layer_index, uint32_t num_total_tokens,
+                                                      uint32_t num_total_kv_splits, uint32_t num_active_tokens,
+                                                      uint32_t num_active_kv_splits) {
+    PSI_REQUIRE(worker_cu != nullptr && num_workers > 0, "balanced map needs a worker table");
+    return single_q_map_impl(ctx, cfg, layout, q, kv_pages, kv_pages_bytes, req_slots, page_ids, kv_splits, worker_cu,
+                             num_workers, scratch, scratch_bytes, gqa_layer_index, num_total_tokens,
+                             num_total_kv_splits, num_active_tokens, num_active_kv_splits);
 }
 
 extern "C" int psi_hip_split_kv_single_q_reduce(psi_hip_ctx* ctx, const psi_hip_gqa_config* cfg, const void* scratch,

@@ -94,6 +94,10 @@ class Device:
         """Decode map variant with QK^T on the vector ALU instead of MFMA (for comparisons)."""
         L.check(self.lib.psi_hip_ctx_set_flag(self.ctx, L.FLAG_DECODE_VALU_QK, int(on)))
 
+    def decode_waves(self, waves: int):
+        """Waves per decode-map workgroup: 1, 2 or 4; 0 = chosen from the grid size."""
+        L.check(self.lib.psi_hip_ctx_set_flag(self.ctx, L.FLAG_DECODE_WAVES, int(waves)))
+
     def f32_output(self, on: bool):
         """Combine kernels then store f32 outputs (for checking the result before output rounding)."""
         L.check(self.lib.psi_hip_ctx_set_flag(self.ctx, L.FLAG_F32_OUTPUT, int(on)))
@@ -339,6 +343,13 @@ class GQAReplayBucketPolicy:
         return self.kv_splits.capacity(num_kv_splits)
 
 
+def balanced_workers(config: "GQASplitKVConfig") -> int:
+    """Decode-map workers per KV head that fill the device exactly once."""
+    out, cfg = ctypes.c_uint32(), config.struct()
+    L.check(L.load().psi_hip_split_kv_balanced_workers(ctypes.byref(cfg), ctypes.byref(out)))
+    return out.value
+
+
 def select_split_kv_variant(split_kv: GQASplitKV, max_tokens: int, replay_policy: Optional[GQAReplayBucketPolicy],
                             token_indices: Sequence[int], cu_tokens: Sequence[int]) -> GQASplitKVVariant:
     """`select_split_kv_variant` (attn/gqa/mod.rs:64-94); the (256, 8) work model applies by itself."""
@@ -434,6 +445,33 @@ class GQAMetadataBuffers:
         """Fixed-length KV partitions (not in the reference): ceil(ctx / partition) splits per row."""
         return self._update(req_slots, token_indices, cu_tokens, split_kv_variant, L.CAPACITY_FIXED_PARTITION,
                             partition_tokens=partition_tokens)
+
+    def balance(self, num_workers: int):
+        """Re-cuts the current SingleQ plan into rows grouped for `num_workers` equal-work decode
+        workgroups per KV head (psi_hip_split_kv_balance_plan); returns the new replay shape."""
+        s = self._shape
+        assert s is not None and not self._variant.is_tiled()
+        rows_in = s.num_sdpa_map_task_templates
+        cap = rows_in + num_workers
+        out_splits = np.full(cap * 3, L.SENTINEL, np.uint32)
+        out_cu = np.zeros(self._max_tokens + 1, np.uint32)
+        worker_cu = np.zeros(num_workers + 1, np.uint32)
+        n_out = ctypes.c_uint32()
+
+        def p(a):
+            return a.ctypes.data_as(ctypes.POINTER(ctypes.c_uint32))
+
+        L.check(L.load().psi_hip_split_kv_balance_plan(p(self.h_kv_splits), rows_in, p(self.h_cu_kv_splits),
+                                                       s.num_tokens, num_workers, p(out_splits), cap, p(out_cu),
+                                                       p(worker_cu), ctypes.byref(n_out)))
+        self.h_kv_splits, self.h_cu_kv_splits, self.h_worker_cu = out_splits, out_cu, worker_cu
+        self.num_workers = num_workers
+        self._shape = GQAReplayShape(s.num_tokens, s.num_total_tokens, s.num_q_token_tiles,
+                                     s.num_total_q_token_tiles, n_out.value, n_out.value, True)
+        if self.device is not None:
+            self.upload()
+            self.d_worker_cu = self.device.from_numpy(worker_cu)
+        return self._shape
 
     def replay_shape(self) -> GQAReplayShape:
         assert self._shape is not None, "GQA batch metadata must be updated before recording"
@@ -570,6 +608,17 @@ class GQASplitKVSingleQKernels:
             _ptr(req_slots), _ptr(page_ids), _ptr(sdpa_map_task_templates), _ptr(scratch.buffer), scratch.bytes,
             page_table_index, self.shape.num_total_tokens, self.shape.num_total_sdpa_map_task_templates,
             num_active_tokens, num_active_kv_splits))
+
+    def invoke_map_balanced(self, q, kv_pages, req_slots, page_ids, sdpa_map_task_templates, worker_cu,
+                            num_workers: int, scratch, page_table_index: int, num_active_tokens: int,
+                            num_active_kv_splits: int):
+        """The map over a balanced plan: one workgroup per (worker, KV head) walks its row range."""
+        cfg, layout = self.config.struct(), self.config.page_table_layout.struct()
+        L.check(self.device.lib.psi_hip_split_kv_single_q_map_balanced(
+            self.device.ctx, ctypes.byref(cfg), ctypes.byref(layout), _ptr(q), _ptr(kv_pages), _nbytes(kv_pages),
+            _ptr(req_slots), _ptr(page_ids), _ptr(sdpa_map_task_templates), _ptr(worker_cu), num_workers,
+            _ptr(scratch.buffer), scratch.bytes, page_table_index, self.shape.num_total_tokens,
+            self.shape.num_total_sdpa_map_task_templates, num_active_tokens, num_active_kv_splits))
 
     def invoke_reduce(self, scratch, cu_sdpa_partial_outputs, output):
         self.invoke_reduce_bucketed(scratch, cu_sdpa_partial_outputs, output, self.shape.num_total_tokens)

@@ -87,7 +87,7 @@ def make_workload(seed: int, context_lens: Sequence[int], num_q_heads: int, num_
                   dtype: G.Dtype, tokens_per_page: int = 16, q_lens=1, scale: Optional[float] = None,
                   input_scale: float = 1.0, num_gqa_layers: int = 1, layer: int = 0, num_page_ids_per_block: int = 1,
                   spare_pages: int = 3, host_pages: bool = True, outlier_rate: float = 0.0,
-                  outlier_sigma: float = 8.0, shuffle_slots: bool = True) -> Workload:
+                  outlier_sigma: float = 8.0, shuffle_slots: bool = True, shuffle_pages: bool = True) -> Workload:
     """`context_lens[r]` counts the tokens of request r after this step's append."""
     rng = np.random.default_rng(seed)
     context_lens = np.asarray(context_lens, dtype=np.int64)
@@ -104,6 +104,8 @@ def make_workload(seed: int, context_lens: Sequence[int], num_q_heads: int, num_
     req_slots = (rng.permutation(num_req_slots)[:batch] if shuffle_slots else np.arange(batch)).astype(np.uint32)
     num_pages = int(pages_per_req.sum()) + spare_pages
     pool = rng.permutation(num_pages).astype(np.uint32)
+    if not shuffle_pages:
+        pool = np.arange(num_pages, dtype=np.uint32)  # identity table, as the reference's own benches use
     table = np.zeros(layout.num_page_ids(), dtype=np.uint32)
     # rows of other layers stay zero on purpose: a kernel that walks the wrong layer reads page 0
     cursor = 0
@@ -143,7 +145,7 @@ class DeviceWorkload:
 
     def __init__(self, device: G.Device, w: Workload, partition_tokens: Optional[int] = None,
                  max_tokens: Optional[int] = None, variant: Optional[G.GQASplitKVVariant] = None,
-                 f32_output: bool = False):
+                 f32_output: bool = False, balanced: bool = False):
         import torch
 
         self.device, self.w = device, w
@@ -186,6 +188,11 @@ class DeviceWorkload:
         else:
             self.meta = G.GQAMetadataBuffers(device, max_tokens or max(w.num_tokens, 1))
             self.shape = self.meta.update(w.req_slots, w.token_indices, w.cu_tokens, variant)
+        self.balanced = balanced and not variant.is_tiled()
+        if self.balanced:
+            workers = G.balanced_workers(G.GQASplitKVConfig(w.dtype, w.page_bytes, w.num_q_heads, w.num_kv_heads,
+                                                            w.head_dim))
+            self.shape = self.meta.balance(workers)
         s = self.shape
         self.write = G.GQAKVPageWrite(device, G.GQAKVPageWriteConfig(w.num_kv_heads, w.head_dim, w.page_bytes,
                                                                      w.dtype))
@@ -225,6 +232,10 @@ class DeviceWorkload:
             self.kernels.invoke_map_bucketed(self.q, self.pages, m.d_req_slots, self.page_ids,
                                              m.d_flat_token_indices, m.d_q_token_tiles, m.d_kv_splits, self.scratch,
                                              self.w.layer, s.num_tokens, s.num_q_token_tiles,
+                                             s.num_sdpa_map_task_templates)
+        elif self.balanced:
+            self.kernels.invoke_map_balanced(self.q, self.pages, m.d_req_slots, self.page_ids, m.d_kv_splits,
+                                             m.d_worker_cu, m.num_workers, self.scratch, self.w.layer, s.num_tokens,
                                              s.num_sdpa_map_task_templates)
         else:
             self.kernels.invoke_map_bucketed(self.q, self.pages, m.d_req_slots, self.page_ids, m.d_kv_splits,
@@ -277,8 +288,10 @@ def config_c2_context_lens(seed: int = 2, batch: int = 32, lo: int = 1024, hi: i
     return rng.integers(lo, hi + 1, size=batch)
 
 
-def config_c2(seed: int = 2, batch: int = 32, host_pages: bool = False, lo: int = 1024, hi: int = 8192) -> Workload:
+def config_c2(seed: int = 2, batch: int = 32, host_pages: bool = False, lo: int = 1024, hi: int = 8192,
+              shuffle_pages: bool = True) -> Workload:
     """Batched ragged decode: contexts uniform in [lo, hi] (before the append), 24 Q / 4 KV heads,
     D=256, bf16, 16-token pages from a shuffled pool; each step appends one token per sequence."""
     ctx = config_c2_context_lens(seed, batch, lo, hi) + 1
-    return make_workload(seed, ctx, 24, 4, 256, G.Dtype.Bfloat16, 16, host_pages=host_pages)
+    return make_workload(seed, ctx, 24, 4, 256, G.Dtype.Bfloat16, 16, host_pages=host_pages,
+                         shuffle_pages=shuffle_pages)

@@ -74,3 +74,29 @@ def test_fast_and_generic_variants_agree(psi, oracle, device):
     finally:
         device.force_generic(False)
     assert np.abs(a - b).max() < 1e-5
+
+
+@pytest.mark.parametrize("waves", [1, 2, 4])
+def test_workgroup_widths_agree_with_oracle(psi, oracle, device, waves):
+    """The decode map with 1, 2 and 4 waves per workgroup (chosen from the grid size in production)."""
+    wl = importlib_workloads(psi)
+    w = wl.make_workload(19, [1500, 31, 530, 512], 24, 4, 256, psi.Dtype.Bfloat16, 16)
+    device.decode_waves(waves)
+    try:
+        run_and_check(psi, oracle, device, w, f"waves={waves}", partition_tokens=512, check_rounded=False)
+    finally:
+        device.decode_waves(0)
+
+
+def test_balanced_plan_matches_oracle(psi, oracle, device):
+    """Equal-work worker plan: rows re-cut at tile boundaries, several rows per workgroup."""
+    wl = importlib_workloads(psi)
+    ctx = [3000, 17, 1025, 2048, 700, 1]
+    w = wl.make_workload(29, ctx, 24, 4, 256, psi.Dtype.Bfloat16, 16)
+    stats, dw = run_and_check(psi, oracle, device, w, "balanced", partition_tokens=512, balanced=True)
+    m = dw.meta
+    rows = m.h_kv_splits[: dw.shape.num_sdpa_map_task_templates * 3].reshape(-1, 3)
+    tiles = (rows[:, 2] + 15) // 16 - rows[:, 1] // 16
+    per_worker = [int(tiles[m.h_worker_cu[i]:m.h_worker_cu[i + 1]].sum()) for i in range(m.num_workers)]
+    assert max(per_worker) - min(per_worker) <= 1
+    assert sum(per_worker) == sum(-(-c // 16) for c in ctx)
