@@ -295,6 +295,122 @@ int psi_hip_page_table_start_index(const psi_hip_page_table_layout* layout, uint
 int psi_hip_page_ids_by_layer(const uint32_t* block_ids, uint32_t block_ids_len, uint32_t num_gqa_layers,
                               uint32_t num_page_ids_per_block, uint32_t* out_by_layer);
 
+/* ---------------------------------------------------------------------------------------------
+ * Cache ownership on the host: page-ID allocator and the per-request token window.  No device work.
+ * ------------------------------------------------------------------------------------------- */
+
+/* `U32IDAllocator` (crates/inference-runtime-core/src/memory/u32_id_allocator.rs:40-173): IDs in
+ * [0, capacity); freed IDs are re-issued first, in the order they were freed, before never-used
+ * ones; a bitmap records what is allocated.  Thread-safe.  Exhaustion returns
+ * PSI_HIP_ERR_RESOURCE_EXHAUSTED ("not enough ID") and leaves the allocator unchanged apart from
+ * the order of the free queue (popped IDs go back to its tail, as in the reference).  Ownership is
+ * shared like the reference's Arc: destroy drops the creator's handle, the allocator itself lives
+ * until every decoder-blocks object created on it has been destroyed. */
+typedef struct psi_hip_id_allocator psi_hip_id_allocator;
+int psi_hip_id_allocator_create(uint64_t capacity, psi_hip_id_allocator** out);
+int psi_hip_id_allocator_destroy(psi_hip_id_allocator* allocator);
+int psi_hip_id_allocator_alloc_one(psi_hip_id_allocator* allocator, uint32_t* id);
+int psi_hip_id_allocator_alloc_many(psi_hip_id_allocator* allocator, size_t count, uint32_t* ids);
+int psi_hip_id_allocator_free_one(psi_hip_id_allocator* allocator, uint32_t id);
+int psi_hip_id_allocator_free_many(psi_hip_id_allocator* allocator, const uint32_t* ids, size_t count);
+/* `used` / `free` / `capacity` (u32_id_allocator.rs:143-153); any out pointer may be null. */
+int psi_hip_id_allocator_counts(psi_hip_id_allocator* allocator, uint64_t* used, uint64_t* free_count,
+                                uint64_t* capacity);
+/* `allocated_ids_bitmap_iter` (u32_id_allocator.rs:62-66): num_words must be ceil(capacity / 64). */
+int psi_hip_id_allocator_bitmap(psi_hip_id_allocator* allocator, uint64_t* words, size_t num_words);
+/* Runs of set bits as [begin, end) pairs, the scan the reference's hibernation uses to copy only
+ * allocated pages (crates/inference-runtime-core/src/runtime/scheduler/executor_hibernate.rs:15-47).
+ * ranges may be null to count only. */
+int psi_hip_bitmap_allocated_ranges(const uint64_t* words, size_t num_words, uint32_t* ranges, size_t capacity_pairs,
+                                    size_t* num_pairs);
+
+/* `TrieDecoderBlocks<N, P, L, BC>` (crates/inference-runtime-core/src/runtime/decoder/trie_cache/blocks/trie/
+ * mod.rs:17-39, api.rs:34-571) without prefix sharing: one request's tokens move
+ * queued -> ready -> scheduled -> cached through blocks of `tokens_per_block` tokens; each block owns
+ * `pages_per_kv_block` page IDs per cache lane (`TPKVBlockAllocator::allocate`,
+ * .../decoder/allocator/tp_kv_block_allocator.rs:24-36), drawn lane by lane and released when the
+ * block is.  Lane 0 is the main model, lanes 1.. the MTP modules, each one token ahead of the last.
+ * Not thread-safe (the allocator it draws from is). */
+typedef struct psi_hip_decoder_blocks psi_hip_decoder_blocks;
+typedef struct psi_hip_decoder_blocks_config {
+    uint32_t tokens_per_block;   /* N */
+    uint32_t num_cache_lanes;    /* L >= 1 */
+    uint32_t pages_per_kv_block; /* layers * N / tokens_per_page */
+} psi_hip_decoder_blocks_config;
+
+enum { PSI_HIP_QUERY_PREFILL = 0, PSI_HIP_QUERY_DECODE = 1 };
+/* `QueryTokens` (crates/inference-runtime-core/src/compute/request/decoder/query_tokens.rs:4-17).
+ * The token buffers belong to the caller; prepare fills them and the counts. */
+typedef struct psi_hip_query_tokens {
+    uint32_t kind;        /* PSI_HIP_QUERY_* */
+    uint32_t window;      /* prefill only: tokens that advance the cache (= num_tokens - (L - 1)) */
+    uint64_t epoch;
+    uint64_t token_index; /* absolute position of tokens[0] */
+    uint32_t* tokens;
+    size_t num_tokens, tokens_capacity;
+    uint32_t* spec_tokens; /* decode only: drafts to verify after `tokens` */
+    size_t num_spec_tokens, spec_tokens_capacity;
+} psi_hip_query_tokens;
+/* `SampledTokens` (.../request/decoder/sample_tokens.rs:6-20) minus the probabilities, which the
+ * token window never reads. */
+typedef struct psi_hip_sampled_tokens {
+    uint32_t kind; /* must equal the query's */
+    uint32_t sampled_token;
+    uint64_t epoch;
+    const uint32_t* validated_tokens; /* accepted prefix of the query's spec_tokens */
+    size_t num_validated_tokens;
+    const uint32_t* spec_tokens; /* drafts for the next step */
+    size_t num_spec_tokens;
+} psi_hip_sampled_tokens;
+enum {
+    PSI_HIP_TOKENS_CACHED = 0,
+    PSI_HIP_TOKENS_SCHEDULED = 1,
+    PSI_HIP_TOKENS_READY = 2,
+    PSI_HIP_TOKENS_QUEUED = 3,
+    PSI_HIP_TOKENS_SPEC = 4
+};
+
+/* `TrieDecoderBlocks::new` (mod.rs:47-82): history, prompt and sampled tokens concatenated. */
+int psi_hip_decoder_blocks_create(psi_hip_id_allocator* allocator, const psi_hip_decoder_blocks_config* cfg,
+                                  const uint32_t* tokens, size_t num_tokens, psi_hip_decoder_blocks** out);
+/* Drop (mod.rs:299-311): releases mutable then semi-immutable blocks, last to first; with no trie
+ * to keep them, committed blocks are released as well. */
+int psi_hip_decoder_blocks_destroy(psi_hip_decoder_blocks* blocks);
+/* `ready_token_slots` (api.rs:35-46). */
+int psi_hip_decoder_blocks_ready_token_slots(const psi_hip_decoder_blocks* blocks, size_t* out);
+/* `init_block_once` (api.rs:48-136): adds one block and moves up to N queued tokens into it.
+ * PSI_HIP_ERR_RESOURCE_EXHAUSTED (state unchanged) when the allocator cannot cover every lane. */
+int psi_hip_decoder_blocks_init_block_once(psi_hip_decoder_blocks* blocks, size_t* ready_token_slots);
+/* `uninit_block_once` (api.rs:138-153): releases the last block, its tokens return to the queue. */
+int psi_hip_decoder_blocks_uninit_block_once(psi_hip_decoder_blocks* blocks, size_t* cached_token_slots);
+/* Stored drafts as a resumed request would carry them (the reference's tests assign the field). */
+int psi_hip_decoder_blocks_set_spec_tokens(psi_hip_decoder_blocks* blocks, const uint32_t* spec_tokens, size_t count);
+/* `prepare` (api.rs:184-273): schedules up to `token_budget` ready tokens; a budget below
+ * ready + queued yields a prefill chunk, otherwise a decode step whose spare budget selects stored
+ * drafts (the rest are dropped). */
+int psi_hip_decoder_blocks_prepare(psi_hip_decoder_blocks* blocks, size_t token_budget, psi_hip_query_tokens* out);
+/* `cancel` (api.rs:276-331): un-schedules the newest outstanding query. */
+int psi_hip_decoder_blocks_cancel(psi_hip_decoder_blocks* blocks, const psi_hip_query_tokens* query);
+/* `commit` (api.rs:334-549): the query's window becomes cached; for a decode step the validated
+ * drafts and the sampled token are appended, and as many of them as every lane has seen go to the
+ * cache directly.  validated_tokens must be a prefix of the query's spec_tokens. */
+int psi_hip_decoder_blocks_commit(psi_hip_decoder_blocks* blocks, const psi_hip_query_tokens* query,
+                                  const psi_hip_sampled_tokens* sampled);
+/* `prepare_blocks` (mod.rs:176-229) -> `DecoderSyncBlocks` (.../request/decoder/decoder_sync_blocks.rs:2-6):
+ * page IDs of the blocks the executor has not seen yet, kv_page_ids[lane][block][pages_per_kv_block];
+ * with kv_page_ids null only the counts are returned and nothing is marked as synced. */
+int psi_hip_decoder_blocks_prepare_blocks(psi_hip_decoder_blocks* blocks, size_t* block_index, size_t* num_blocks,
+                                          uint32_t* kv_page_ids, size_t capacity_ids);
+/* `cancel_blocks` (mod.rs:231-233). */
+int psi_hip_decoder_blocks_cancel_blocks(psi_hip_decoder_blocks* blocks, size_t block_index);
+/* Block counts by kind and the number already synced; any out pointer may be null. */
+int psi_hip_decoder_blocks_counts(const psi_hip_decoder_blocks* blocks, size_t* immutable_blocks,
+                                  size_t* semi_immutable_blocks, size_t* mutable_blocks, size_t* in_sync_blocks);
+/* Lane-0 view of one token class (PSI_HIP_TOKENS_*), `cached_tokens()` .. `spec_tokens()`
+ * (blocks/trie/token.rs:10-181); out may be null to count only. */
+int psi_hip_decoder_blocks_tokens(const psi_hip_decoder_blocks* blocks, uint32_t which, uint32_t* out,
+                                  size_t capacity, size_t* count);
+
 #ifdef __cplusplus
 }
 #endif

@@ -5,7 +5,7 @@ missing, `load()` raises with the build command.
 """
 import ctypes
 import os
-from ctypes import POINTER, c_char_p, c_double, c_float, c_int, c_uint32, c_uint64, c_void_p
+from ctypes import POINTER, c_char_p, c_double, c_float, c_int, c_size_t, c_uint32, c_uint64, c_void_p
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_HERE, "lib", "libpsi_hip.so")
@@ -77,7 +77,40 @@ class ReplayShapeStruct(ctypes.Structure):
     ]
 
 
+class DecoderBlocksConfigStruct(ctypes.Structure):
+    _fields_ = [("tokens_per_block", c_uint32), ("num_cache_lanes", c_uint32), ("pages_per_kv_block", c_uint32)]
+
+
+class QueryTokensStruct(ctypes.Structure):
+    _fields_ = [
+        ("kind", c_uint32),
+        ("window", c_uint32),
+        ("epoch", c_uint64),
+        ("token_index", c_uint64),
+        ("tokens", POINTER(c_uint32)),
+        ("num_tokens", c_size_t),
+        ("tokens_capacity", c_size_t),
+        ("spec_tokens", POINTER(c_uint32)),
+        ("num_spec_tokens", c_size_t),
+        ("spec_tokens_capacity", c_size_t),
+    ]
+
+
+class SampledTokensStruct(ctypes.Structure):
+    _fields_ = [
+        ("kind", c_uint32),
+        ("sampled_token", c_uint32),
+        ("epoch", c_uint64),
+        ("validated_tokens", POINTER(c_uint32)),
+        ("num_validated_tokens", c_size_t),
+        ("spec_tokens", POINTER(c_uint32)),
+        ("num_spec_tokens", c_size_t),
+    ]
+
+
 _U32P = POINTER(c_uint32)
+_U64P = POINTER(c_uint64)
+_SZP = POINTER(c_size_t)
 _CFG = POINTER(GQAConfigStruct)
 _LAYOUT = POINTER(PageTableLayoutStruct)
 _VARIANT = POINTER(VariantStruct)
@@ -142,6 +175,30 @@ PROTOTYPES = {
     "psi_hip_page_table_reset_req_slot": (c_int, [c_void_p, _LAYOUT, c_void_p, c_uint32]),
     "psi_hip_page_table_start_index": (c_int, [_LAYOUT, c_uint32, c_uint32, c_uint32, POINTER(c_uint64)]),
     "psi_hip_page_ids_by_layer": (c_int, [_U32P, c_uint32, c_uint32, c_uint32, _U32P]),
+    "psi_hip_id_allocator_create": (c_int, [c_uint64, POINTER(c_void_p)]),
+    "psi_hip_id_allocator_destroy": (c_int, [c_void_p]),
+    "psi_hip_id_allocator_alloc_one": (c_int, [c_void_p, _U32P]),
+    "psi_hip_id_allocator_alloc_many": (c_int, [c_void_p, c_size_t, _U32P]),
+    "psi_hip_id_allocator_free_one": (c_int, [c_void_p, c_uint32]),
+    "psi_hip_id_allocator_free_many": (c_int, [c_void_p, _U32P, c_size_t]),
+    "psi_hip_id_allocator_counts": (c_int, [c_void_p, _U64P, _U64P, _U64P]),
+    "psi_hip_id_allocator_bitmap": (c_int, [c_void_p, _U64P, c_size_t]),
+    "psi_hip_bitmap_allocated_ranges": (c_int, [_U64P, c_size_t, _U32P, c_size_t, _SZP]),
+    "psi_hip_decoder_blocks_create": (
+        c_int, [c_void_p, POINTER(DecoderBlocksConfigStruct), _U32P, c_size_t, POINTER(c_void_p)]),
+    "psi_hip_decoder_blocks_destroy": (c_int, [c_void_p]),
+    "psi_hip_decoder_blocks_ready_token_slots": (c_int, [c_void_p, _SZP]),
+    "psi_hip_decoder_blocks_init_block_once": (c_int, [c_void_p, _SZP]),
+    "psi_hip_decoder_blocks_uninit_block_once": (c_int, [c_void_p, _SZP]),
+    "psi_hip_decoder_blocks_set_spec_tokens": (c_int, [c_void_p, _U32P, c_size_t]),
+    "psi_hip_decoder_blocks_prepare": (c_int, [c_void_p, c_size_t, POINTER(QueryTokensStruct)]),
+    "psi_hip_decoder_blocks_cancel": (c_int, [c_void_p, POINTER(QueryTokensStruct)]),
+    "psi_hip_decoder_blocks_commit": (
+        c_int, [c_void_p, POINTER(QueryTokensStruct), POINTER(SampledTokensStruct)]),
+    "psi_hip_decoder_blocks_prepare_blocks": (c_int, [c_void_p, _SZP, _SZP, _U32P, c_size_t]),
+    "psi_hip_decoder_blocks_cancel_blocks": (c_int, [c_void_p, c_size_t]),
+    "psi_hip_decoder_blocks_counts": (c_int, [c_void_p, _SZP, _SZP, _SZP, _SZP]),
+    "psi_hip_decoder_blocks_tokens": (c_int, [c_void_p, c_uint32, _U32P, c_size_t, _SZP]),
 }
 
 _lib = None

@@ -1,0 +1,441 @@
+"""Host-side planning (capacity buckets, variant selection, KV-split plans, page-table index math):
+the library through its C ABI and the Python oracle, both against the vectors the reference's own
+tests hold, then against each other on random batches.
+
+  buckets            crates/inference-executor-core/src/replay.rs:94-180
+  selector matrix    crates/inference-backend-metal/src/components/gqa_split_kv.rs:177-231
+  measured selector  crates/inference-executor-metal/src/attn/gqa/mod.rs:370-454
+  split plans        crates/inference-executor-metal/src/attn/gqa/batch_metadata.rs:535-680
+  page table         crates/inference-executor-metal/src/attn/gqa/request_page_table.rs:112-117,141-174
+  layer split        crates/inference-executor-metal/src/model/qwen/v3_x/state/gqa.rs:250-277
+"""
+import ctypes
+import random
+
+import numpy as np
+import pytest
+
+MAX = 0xFFFFFFFF
+
+
+def bf16_config(psi, head_dim, group, tokens_per_page, num_kv_heads=2, dtype=None):
+    dtype = psi.Dtype.Bfloat16 if dtype is None else dtype
+    return psi.GQASplitKVConfig(
+        io_dtype=dtype, page_bytes=2 * num_kv_heads * head_dim * tokens_per_page * dtype.item_size(),
+        num_q_heads=num_kv_heads * group, num_kv_heads=num_kv_heads, head_dim=head_dim)
+
+
+def as_tuple(v):
+    if v.is_tiled():
+        return ("TiledQ", v.q_token_tile_size, v.kv_token_tile_size, v.q_head_tile_size)
+    return ("SingleQ", v.kv_token_tile_size, v.num_threads_per_threadblock, v.q_head_tile_size)
+
+
+def from_tuple(psi, t):
+    if t[0] == "TiledQ":
+        return psi.GQASplitKVVariant.TiledQ(t[1], t[2], t[3])
+    return psi.GQASplitKVVariant.SingleQ(t[1], t[2], t[3])
+
+
+# ------------------------------------------------------------------ buckets
+
+
+@pytest.fixture(params=["oracle", "library"])
+def bucket_policy(request, host_oracle, psi):
+    if request.param == "oracle":
+        def make(cap, boundaries=()):
+            p = host_oracle.ReplayBucketPolicy(cap, boundaries)
+            return p.buckets, p.capacity
+    else:
+        def make(cap, boundaries=()):
+            p = psi.ReplayBucketPolicy(cap, boundaries)
+            return p.buckets(), p.capacity
+    return make
+
+
+def test_default_buckets(bucket_policy):
+    base = [1, 2, 4, 6, 8, 12, 16, 20, 24, 32, 40, 48, 56, 64]
+    assert bucket_policy(64)[0] == base
+    assert bucket_policy(128)[0] == base + [80, 96, 112, 128]
+    assert bucket_policy(70)[0][-1] == 70
+    assert bucket_policy(6)[0] == [1, 2, 4, 6]
+
+
+@pytest.mark.parametrize("cap", [65, 79, 80, 81, 127, 128, 129, MAX])
+def test_buckets_ordered_at_extension_boundaries(bucket_policy, cap):
+    buckets, capacity = bucket_policy(cap)
+    assert buckets[-1] == cap and capacity(cap) == cap
+    assert all(a < b for a, b in zip(buckets, buckets[1:]))
+
+
+def test_bucket_capacity(bucket_policy):
+    _, capacity = bucket_policy(64)
+    assert [capacity(a) for a in (1, 3, 5, 9, 25, 64)] == [1, 4, 6, 12, 32, 64]
+
+
+def test_topology_boundaries(bucket_policy):
+    buckets, capacity = bucket_policy(64, [5, 6, 10, 12, 18])
+    assert 0 not in buckets
+    assert [capacity(a) for a in (5, 9, 10, 11, 17, 18)] == [5, 9, 11, 11, 17, 20]
+    assert bucket_policy(6, [1])[0] == [1, 2, 4, 6]
+    buckets, capacity = bucket_policy(8, [6])
+    assert buckets == [1, 2, 4, 5, 6, 8]
+    assert [capacity(a) for a in (5, 6, 7)] == [5, 6, 8]
+
+
+def test_padding_stays_within_a_quarter(bucket_policy):
+    _, capacity = bucket_policy(256)
+    for active in range(1, 257):
+        total = capacity(active)
+        assert (total - active) * 4 <= total, (active, total)
+
+
+def test_capacity_rejects_overflow_and_zero(psi, host_oracle):
+    with pytest.raises(psi.PsiHipError, match="replay active work exceeds capacity"):
+        psi.ReplayBucketPolicy(6).capacity(7)
+    with pytest.raises(psi.PsiHipError, match="replay bucket requires active work"):
+        psi.ReplayBucketPolicy(6).capacity(0)
+    assert psi.ReplayBucketPolicy(6).capacity_allow_zero(0) == 0
+    with pytest.raises(AssertionError):
+        host_oracle.ReplayBucketPolicy(6).capacity(7)
+
+
+def test_buckets_agree_for_every_capacity_up_to_600(psi, host_oracle):
+    for cap in range(1, 600):
+        assert psi.ReplayBucketPolicy(cap).buckets() == host_oracle.ReplayBucketPolicy(cap).buckets, cap
+
+
+# ------------------------------------------------------------------ selector
+
+
+def test_selector_matrix_library(psi):
+    t256 = psi.GQASplitKV.new(bf16_config(psi, 256, 6, 16))
+    t256p8 = psi.GQASplitKV.new(bf16_config(psi, 256, 6, 8))
+    t128 = psi.GQASplitKV.new(bf16_config(psi, 128, 8, 8))
+    unsupported = psi.GQASplitKV.new(bf16_config(psi, 256, 8, 4))
+    single_partial = psi.GQASplitKV.new_dspark_history(bf16_config(psi, 128, 8, 8))
+    assert t256.max_q_tokens_per_partial_output() == 8
+    assert t256p8.max_q_tokens_per_partial_output() == 8
+    assert as_tuple(t256.select(4, 4)) == ("SingleQ", 256, 256, 6)
+    assert as_tuple(t256.select(8, 4)) == ("TiledQ", 8, 16, 3)
+    assert as_tuple(t256.select(16, 4)) == ("TiledQ", 8, 16, 6)
+    assert as_tuple(t256p8.select(16, 4)) == ("TiledQ", 8, 16, 6)
+    assert as_tuple(t128.select(8, 4)) == ("TiledQ", 8, 16, 8)
+    for s in (unsupported, single_partial):
+        assert s.max_q_tokens_per_partial_output() == 1
+        assert as_tuple(s.select(16, 4))[0] == "SingleQ"
+
+
+def test_selector_matrix_oracle(host_oracle):
+    S = host_oracle.SplitKVSelector
+    t256, t256p8, t128 = S(True, 256, 16, 6), S(True, 256, 8, 6), S(True, 128, 8, 8)
+    assert t256.max_q_tokens_per_partial_output() == 8
+    assert t256.select(4, 4) == ("SingleQ", 256, 256, 6)
+    assert t256.select(8, 4) == ("TiledQ", 8, 16, 3)
+    assert t256.select(16, 4) == ("TiledQ", 8, 16, 6)
+    assert t256p8.select(16, 4) == ("TiledQ", 8, 16, 6)
+    assert t128.select(8, 4) == ("TiledQ", 8, 16, 8)
+    for s in (S(True, 256, 4, 8), S(True, 128, 8, 8, dspark_history=True)):
+        assert s.max_q_tokens_per_partial_output() == 1
+        assert s.select(16, 4)[0] == "SingleQ"
+
+
+def test_selector_f32_and_wide_groups_stay_single_q(psi, host_oracle):
+    f32 = psi.GQASplitKV.new(bf16_config(psi, 256, 6, 16, dtype=psi.Dtype.Float32))
+    assert as_tuple(f32.select(64, 8))[0] == "SingleQ"
+    wide = psi.GQASplitKV.new(bf16_config(psi, 128, 16, 8))
+    assert as_tuple(wide.select(64, 8))[0] == "SingleQ"
+    assert host_oracle.SplitKVSelector(False, 256, 16, 6).select(64, 8)[0] == "SingleQ"
+    assert host_oracle.SplitKVSelector(True, 128, 8, 16).select(64, 8)[0] == "SingleQ"
+
+
+def test_selector_agrees_over_a_grid(psi, host_oracle):
+    for (d, g, p) in [(256, 6, 16), (256, 6, 8), (128, 8, 8), (256, 8, 4), (128, 4, 16), (64, 2, 32), (256, 1, 16)]:
+        lib = psi.GQASplitKV.new(bf16_config(psi, d, g, p))
+        ora = host_oracle.SplitKVSelector(True, d, p, g)
+        for tiles in (1, 2, 3, 7, 32):
+            for tokens in sorted({tiles, tiles + 1, 2 * tiles - 1, 2 * tiles, 3 * tiles, 4 * tiles - 1, 4 * tiles,
+                                  8 * tiles}):
+                if tokens < tiles:
+                    continue
+                assert as_tuple(lib.select(tokens, tiles)) == ora.select(tokens, tiles), (d, g, p, tokens, tiles)
+
+
+def _select_256_8(psi, host_oracle, token_indices, request_tokens, bucketed):
+    cu = [0]
+    for n in request_tokens:
+        cu.append(cu[-1] + n)
+    lib = psi.select_split_kv_variant(psi.GQASplitKV.new(bf16_config(psi, 256, 6, 8)), 128,
+                                      psi.GQAReplayBucketPolicy(128) if bucketed else None, token_indices, cu)
+    ora = host_oracle.select_split_kv_variant(host_oracle.SplitKVSelector(True, 256, 8, 6), True, 128,
+                                              128 if bucketed else 0, token_indices, cu)
+    assert as_tuple(lib) == ora
+    return ora[0]
+
+
+@pytest.mark.parametrize("bucketed", [False, True])
+def test_d256_page8_selector_measured_crossovers(psi, host_oracle, bucketed):
+    for tokens, context in [(1, 65536), (2, 65536), (4, 128), (8, 128), (25, 32)]:
+        assert _select_256_8(psi, host_oracle, [context], [tokens], bucketed) == "SingleQ", (tokens, context)
+    for tokens, context in [(4, 512), (8, 512), (16, 128), (25, 128), (64, 0)]:
+        assert _select_256_8(psi, host_oracle, [context], [tokens], bucketed) == "TiledQ", (tokens, context)
+
+
+def test_d256_page8_selector_prices_request_local_tail_tiles(psi, host_oracle):
+    assert _select_256_8(psi, host_oracle, [65536] * 8, [1] * 8, False) == "SingleQ"
+    assert _select_256_8(psi, host_oracle, [1024, 65536], [64, 1], False) == "SingleQ"
+    assert _select_256_8(psi, host_oracle, [65536, 1024], [1, 8], False) == "SingleQ"
+    assert _select_256_8(psi, host_oracle, [65536, 65536], [8, 1], False) == "TiledQ"
+
+
+def test_d256_page8_work_model_matches_the_materialised_plan(psi, host_oracle):
+    sel = host_oracle.SplitKVSelector(True, 256, 8, 6)
+    tiled = sel.select(65, 9)
+    work = host_oracle.tiled_q_selection_work(tiled, 6, 128, None, [1024, 65536], [0, 64, 65])
+    assert (work["num_kv_splits"], work["active_partial_states"], work["padded_replay_work"]) == (72, 128, 1024)
+    md = psi.GQAMetadataBuffers(None, 128)
+    shape = md.update([0, 1], [1024, 65536], [0, 64, 65], from_tuple(psi, tiled))
+    assert shape.num_sdpa_map_task_templates == 72
+    assert shape.num_total_sdpa_map_task_templates * 8 == 1024
+    tiles = md.h_q_token_tiles[:2 * shape.num_q_token_tiles].reshape(-1, 2)
+    cu = md.h_cu_kv_splits[:shape.num_q_token_tiles + 1]
+    assert int(((tiles[:, 1] - tiles[:, 0]) * (cu[1:] - cu[:-1])).sum()) == 128
+
+    work = host_oracle.tiled_q_selection_work(tiled, 6, 128, None, [65536] * 8, list(range(9)))
+    assert (work["num_kv_splits"], work["active_partial_states"], work["padded_replay_work"]) == (128, 128, 1024)
+
+    policy = host_oracle.ReplayBucketPolicy(128)
+    tiled = sel.select(25, 4)
+    work = host_oracle.tiled_q_selection_work(tiled, 6, 128, policy, [65536], [0, 25])
+    assert (work["num_kv_splits"], work["active_partial_states"], work["padded_replay_work"]) == (23, 128, 24 * 8)
+    shape = md.update_bucketed([0], [65536], [0, 25], from_tuple(psi, tiled), psi.GQAReplayBucketPolicy(128))
+    assert shape.num_sdpa_map_task_templates == 23 and shape.num_total_sdpa_map_task_templates == 24
+
+
+# ------------------------------------------------------------------ split plans
+
+SINGLE = ("SingleQ", 8, 32, 1)
+TILED = ("TiledQ", 8, 4, 1)
+KAT = dict(req_slots=[2, 5], token_indices=[7, 20], cu_tokens=[0, 2, 5])
+
+
+def shape_tuple(s):
+    return (s.num_tokens, s.num_total_tokens, s.num_q_token_tiles, s.num_total_q_token_tiles,
+            s.num_sdpa_map_task_templates, s.num_total_sdpa_map_task_templates, s.reduce_sdpa_partial_outputs)
+
+
+def test_metadata_kat_library(psi):
+    md = psi.GQAMetadataBuffers(None, 8)
+    s = md.update(KAT["req_slots"], KAT["token_indices"], KAT["cu_tokens"], from_tuple(psi, SINGLE))
+    assert md.h_req_slots[:5].tolist() == [2, 2, 5, 5, 5]
+    assert md.h_flat_token_indices[:5].tolist() == [7, 8, 20, 21, 22]
+    assert md.h_kv_splits[:24].tolist() == [0, 0, 8, 1, 0, 9, 2, 0, 8, 2, 8, 21, 3, 0, 8, 3, 8, 22, 4, 0, 8, 4, 8, 23]
+    assert md.h_cu_kv_splits[:6].tolist() == [0, 1, 2, 4, 6, 8]
+    assert shape_tuple(s) == (5, 5, 5, 5, 8, 8, True)
+
+    s = md.update(KAT["req_slots"], KAT["token_indices"], KAT["cu_tokens"], from_tuple(psi, TILED))
+    assert md.h_q_token_tiles[:4].tolist() == [0, 2, 2, 5]
+    assert md.h_kv_splits[:12].tolist() == [0, 0, 9, 1, 0, 12, 1, 12, 23, MAX, MAX, MAX]
+    assert md.h_cu_kv_splits[:3].tolist() == [0, 1, 3]
+    assert shape_tuple(s) == (5, 5, 2, 2, 3, 4, True)
+
+    policy = psi.GQAReplayBucketPolicy(8)
+    s = md.update_bucketed(KAT["req_slots"], KAT["token_indices"], KAT["cu_tokens"], from_tuple(psi, TILED), policy)
+    assert shape_tuple(s) == (5, 6, 2, 2, 3, 4, True)
+    s = md.update_bucketed_with_token_capacity(KAT["req_slots"], KAT["token_indices"], KAT["cu_tokens"],
+                                               from_tuple(psi, TILED), policy, 5)
+    assert shape_tuple(s) == (5, 5, 2, 2, 3, 4, True)
+    assert shape_tuple(md.replay_shape()) == shape_tuple(s)
+    assert as_tuple(md.split_kv_variant()) == TILED
+
+
+def test_metadata_kat_oracle(host_oracle):
+    m = host_oracle.metadata_update(8, variant=SINGLE, **KAT)
+    assert m["req_slots"] == [2, 2, 5, 5, 5] and m["flat_token_indices"] == [7, 8, 20, 21, 22]
+    assert m["kv_splits"] == [0, 0, 8, 1, 0, 9, 2, 0, 8, 2, 8, 21, 3, 0, 8, 3, 8, 22, 4, 0, 8, 4, 8, 23]
+    assert m["cu_kv_splits"] == [0, 1, 2, 4, 6, 8] and m["shape"] == (5, 5, 5, 5, 8, 8, True)
+    m = host_oracle.metadata_update(8, variant=TILED, **KAT)
+    assert m["q_token_tiles"] == [0, 2, 2, 5]
+    assert m["kv_splits"] == [0, 0, 9, 1, 0, 12, 1, 12, 23, MAX, MAX, MAX]
+    assert m["cu_kv_splits"] == [0, 1, 3] and m["shape"] == (5, 5, 2, 2, 3, 4, True)
+    assert host_oracle.metadata_update(8, variant=TILED, mode="bucketed", **KAT)["shape"] == (5, 6, 2, 2, 3, 4, True)
+    assert host_oracle.metadata_update(8, variant=TILED, mode="caller", caller_tokens=5, **KAT)["shape"] == \
+        (5, 5, 2, 2, 3, 4, True)
+    m = host_oracle.metadata_update(12, [2, 5, 7], [0, 0, 0], [0, 4, 8, 9], TILED, mode="bucketed")
+    assert m["shape"] == (9, 12, 3, 4, 3, 4, True)
+
+
+def test_bucketed_update_leaves_poisoned_tails_alone(psi):
+    md = psi.GQAMetadataBuffers(None, 12)
+    md.h_q_token_tiles[:] = 0xA5A5A5A5
+    md.h_kv_splits[:] = 0xB6B6B6B6
+    md.h_cu_kv_splits[:] = 0xC7C7C7C7
+    s = md.update_bucketed([2, 5, 7], [0, 0, 0], [0, 4, 8, 9], from_tuple(psi, TILED), psi.GQAReplayBucketPolicy(12))
+    assert shape_tuple(s) == (9, 12, 3, 4, 3, 4, True)
+    assert md.h_q_token_tiles[6:8].tolist() == [0xA5A5A5A5] * 2
+    assert md.h_kv_splits[9:12].tolist() == [MAX] * 3
+    assert md.h_kv_splits[12] == 0xB6B6B6B6
+    assert md.h_cu_kv_splits[4] == 0xC7C7C7C7
+
+
+def test_metadata_contract_violations(psi):
+    md = psi.GQAMetadataBuffers(None, 12)
+    policy = psi.GQAReplayBucketPolicy(12)
+    single = from_tuple(psi, SINGLE)
+    with pytest.raises(psi.PsiHipError, match="must not exceed the caller-owned token capacity"):
+        md.update_bucketed_with_token_capacity([0], [0], [0, 9], single, policy, 8)
+    with pytest.raises(psi.PsiHipError, match="must not exceed the metadata capacity"):
+        md.update_bucketed_with_token_capacity([0], [0], [0, 9], single, policy, 13)
+    with pytest.raises(psi.PsiHipError, match="nondecreasing"):
+        md.update([0, 1], [0, 0], [0, 3, 2], single)
+    with pytest.raises(psi.PsiHipError):
+        md.update([0], [0], [0, 13], single)  # more tokens than capacity
+    with pytest.raises(psi.PsiHipError):
+        md.update([0], [0], [0, 0], single)  # empty batch
+    with pytest.raises(psi.PsiHipError):
+        md.update([0], [MAX], [0, 2], single)  # position overflows u32
+
+
+def test_fixed_partition_plan(psi, host_oracle):
+    md = psi.GQAMetadataBuffers(None, 4, max_kv_splits=64)
+    single = psi.GQASplitKVVariant.SingleQ(256, 256, 6)
+    s = md.update_fixed_partition([0, 1, 2], [1023, 511, 1300], [0, 1, 2, 3], single, 512)
+    splits, cu = host_oracle.fixed_partition_splits([1023, 511, 1300], 512)
+    assert splits == [0, 0, 512, 0, 512, 1024, 1, 0, 512, 2, 0, 512, 2, 512, 1024, 2, 1024, 1301]
+    assert md.h_kv_splits[:len(splits)].tolist() == splits
+    assert md.h_cu_kv_splits[:4].tolist() == cu == [0, 2, 3, 6]
+    assert s.num_sdpa_map_task_templates == 6 and s.num_total_sdpa_map_task_templates == 6
+    with pytest.raises(psi.PsiHipError):
+        psi.GQAMetadataBuffers(None, 4, max_kv_splits=5).update_fixed_partition(
+            [0, 1, 2], [1023, 511, 1300], [0, 1, 2, 3], single, 512)
+
+
+def random_batch(rng, max_tokens):
+    n_req = rng.randint(1, min(6, max_tokens))
+    budget = max_tokens
+    counts = []
+    for r in range(n_req):
+        left = n_req - r - 1
+        c = rng.randint(0 if r else 1, max(1, min(20, budget - left)))
+        c = min(c, budget - left) if budget - left > 0 else 0
+        counts.append(max(c, 0))
+        budget -= counts[-1]
+    if sum(counts) == 0:
+        counts[0] = 1
+    cu = [0]
+    for c in counts:
+        cu.append(cu[-1] + c)
+    starts = [rng.choice([0, 1, 7, 63, 64, 500, 4095, rng.randrange(0, 70000)]) for _ in range(n_req)]
+    slots = [rng.randrange(0, 16) for _ in range(n_req)]
+    return slots, starts, cu
+
+
+@pytest.mark.parametrize("seed", range(40))
+def test_plans_agree_on_random_batches(psi, host_oracle, seed):
+    rng = random.Random(seed)
+    max_tokens = rng.choice([8, 12, 33, 64, 128])
+    slots, starts, cu = random_batch(rng, max_tokens)
+    variant = rng.choice([("SingleQ", rng.choice([8, 64, 256]), 256, 6), ("TiledQ", 8, rng.choice([4, 16]), 3)])
+    mode = rng.choice(["exact", "bucketed", "caller"])
+    boundaries = rng.choice([(), (5,), (6, 10, 18)])
+    caller = min(max_tokens, cu[-1] + rng.randint(0, 3))
+    exp = host_oracle.metadata_update(max_tokens, slots, starts, cu, variant, mode=mode, caller_tokens=caller,
+                                      boundaries=boundaries)
+    md = psi.GQAMetadataBuffers(None, max_tokens)
+    v = from_tuple(psi, variant)
+    if mode == "exact":
+        s = md.update(slots, starts, cu, v)
+    elif mode == "bucketed":
+        s = md.update_bucketed(slots, starts, cu, v, psi.GQAReplayBucketPolicy(max_tokens, boundaries))
+    else:
+        s = md.update_bucketed_with_token_capacity(slots, starts, cu, v,
+                                                   psi.GQAReplayBucketPolicy(max_tokens, boundaries), caller)
+    assert shape_tuple(s) == exp["shape"]
+    t = cu[-1]
+    assert md.h_req_slots[:t].tolist() == exp["req_slots"]
+    assert md.h_flat_token_indices[:t].tolist() == exp["flat_token_indices"]
+    assert md.h_q_token_tiles[:len(exp["q_token_tiles"])].tolist() == exp["q_token_tiles"]
+    assert md.h_kv_splits[:len(exp["kv_splits"])].tolist() == exp["kv_splits"]
+    assert md.h_cu_kv_splits[:len(exp["cu_kv_splits"])].tolist() == exp["cu_kv_splits"]
+
+
+@pytest.mark.parametrize("seed", range(10))
+def test_plan_invariants(psi, seed):
+    """What any valid plan satisfies, whatever the greedy order: every row's splits tile [0, ctx)
+    on KV-tile boundaries, in order, and the budget is respected."""
+    rng = random.Random(100 + seed)
+    max_tokens = rng.choice([16, 64, 128])
+    slots, starts, cu = random_batch(rng, max_tokens)
+    tile = rng.choice([8, 256])
+    md = psi.GQAMetadataBuffers(None, max_tokens)
+    s = md.update(slots, starts, cu, psi.GQASplitKVVariant.SingleQ(tile, 256, 6))
+    assert s.num_sdpa_map_task_templates <= max_tokens
+    ks = md.h_kv_splits[:3 * s.num_sdpa_map_task_templates].reshape(-1, 3)
+    cu_s = md.h_cu_kv_splits[:s.num_tokens + 1]
+    for row in range(s.num_tokens):
+        part = ks[cu_s[row]:cu_s[row + 1]]
+        ctx = int(md.h_flat_token_indices[row]) + 1
+        assert len(part) >= 1 and (part[:, 0] == row).all()
+        assert part[0, 1] == 0 and part[-1, 2] == ctx
+        assert (part[1:, 1] == part[:-1, 2]).all() and (part[:, 1] < part[:, 2]).all()
+        assert (part[:, 1] % tile == 0).all()
+    assert (md.h_kv_splits[3 * s.num_sdpa_map_task_templates:3 * s.num_total_sdpa_map_task_templates] == MAX).all()
+
+
+# ------------------------------------------------------------------ page table index math (no device)
+
+
+def _start_index(psi, layout, slot, layer, block):
+    lib = psi.load()
+    out = ctypes.c_uint64()
+    st = psi.GQAPageTableLayout(*layout).struct()
+    rc = lib.psi_hip_page_table_start_index(ctypes.byref(st), slot, layer, block, ctypes.byref(out))
+    return rc, out.value
+
+
+def test_page_table_start_index(psi, host_oracle):
+    layout = (4, 3, 6, 2)
+    for slot, layer, block in [(0, 0, 0), (1, 2, 5), (3, 0, 4), (3, 2, 5)]:
+        rc, idx = _start_index(psi, layout, slot, layer, block)
+        assert rc == 0
+        assert idx == ((slot * 3 + layer) * 6 + block) * 2 == host_oracle.page_table_start_index(layout, slot, layer, block)
+    for bad in [(4, 0, 0), (0, 3, 0), (0, 0, 6)]:
+        assert _start_index(psi, layout, *bad)[0] != 0
+        with pytest.raises(AssertionError):
+            host_oracle.page_table_start_index(layout, *bad)
+
+
+def test_page_ids_by_layer(psi, host_oracle):
+    lib = psi.load()
+    block = (ctypes.c_uint32 * 4)(10, 11, 20, 21)
+    out = (ctypes.c_uint32 * 4)()
+    assert lib.psi_hip_page_ids_by_layer(block, 4, 2, 2, out) == 0
+    assert [list(out[0:2]), list(out[2:4])] == [[10, 11], [20, 21]] == host_oracle.page_ids_by_layer([10, 11, 20, 21], 2, 2)
+    assert lib.psi_hip_page_ids_by_layer(block, 3, 2, 2, out) != 0
+
+
+def test_tokens_per_page(psi, oracle):
+    for dtype, es, odt in ((psi.Dtype.Float32, 4, oracle.F32), (psi.Dtype.Bfloat16, 2, oracle.BF16),
+                          (psi.Dtype.Float16, 2, oracle.F16)):
+        for hkv, d, p in [(1, 2, 2), (2, 256, 16), (4, 256, 16), (4, 128, 8), (8, 64, 32)]:
+            cfg = psi.GQAKVPageWriteConfig(dtype=dtype, page_bytes=2 * hkv * d * p * es, num_kv_heads=hkv, head_dim=d)
+            assert cfg.num_tokens_per_page() == p == oracle.tokens_per_page(hkv, d, 2 * hkv * d * p * es, odt)
+    bad = psi.GQAKVPageWriteConfig(dtype=psi.Dtype.Bfloat16, page_bytes=1000, num_kv_heads=2, head_dim=256)
+    with pytest.raises(psi.PsiHipError):
+        bad.num_tokens_per_page()
+
+
+def test_balance_plan_covers_the_same_ranges(psi):
+    md = psi.GQAMetadataBuffers(None, 8, max_kv_splits=256)
+    single = psi.GQASplitKVVariant.SingleQ(256, 256, 6)
+    ctx = [5000, 300, 8192, 1024, 17]
+    md.update_fixed_partition(list(range(5)), [c - 1 for c in ctx], list(range(6)), single, 512)
+    s = md.balance(24)
+    ks = md.h_kv_splits[:3 * s.num_sdpa_map_task_templates].reshape(-1, 3)
+    cu = md.h_cu_kv_splits[:6]
+    for row, c in enumerate(ctx):
+        part = ks[cu[row]:cu[row + 1]]
+        assert part[0, 1] == 0 and part[-1, 2] == c and (part[1:, 1] == part[:-1, 2]).all()
+        assert (part[:, 0] == row).all()
+    w = md.h_worker_cu
+    assert w[0] == 0 and w[-1] == s.num_sdpa_map_task_templates and (np.diff(w.astype(np.int64)) >= 0).all()
