@@ -41,6 +41,9 @@ def parse_args():
     p.add_argument("--decode-waves", type=int, default=0, help="waves per decode workgroup (0 = automatic)")
     p.add_argument("--balance", action="store_true", help="equal-tile worker plan instead of one workgroup per partition")
     p.add_argument("--kernel-only", action="store_true", help="time only the map kernel (for profiling runs)")
+    p.add_argument("--calibrate-copy", action="store_true",
+                   help="run only the plain copy / read probes of known size (counter calibration, practical ceiling)")
+    p.add_argument("--probe-mib", type=int, default=1024)
     return p.parse_args()
 
 
@@ -102,6 +105,31 @@ def cpu_baseline(psi, wl, w, dw, budget_s):
     }
 
 
+def calibrate_copy(device, args):
+    """Copies (and separately just reads) a buffer of known size with the library's probe kernels.
+    Under `rocprofv3 --pmc FETCH_SIZE` / `WRITE_SIZE` the counter value of these launches against the
+    known byte count gives the scale factor applied to the attention kernels' counter readings."""
+    import torch
+
+    nbytes = args.probe_mib << 20
+    src = torch.empty(nbytes, dtype=torch.uint8, device="cuda").random_(0, 255)
+    dst = torch.empty_like(src)
+    out = {"probe_bytes": nbytes, "launches": args.steps}
+    for name, read_only in (("copy_probe", False), ("read_probe", True)):
+        for _ in range(args.warmup):
+            device.copy_probe(dst, src, nbytes, read_only)
+        device.set_timing(True)
+        device.reset_timing()
+        for _ in range(args.steps):
+            device.copy_probe(dst, src, nbytes, read_only)
+        ms, n = device.kernel_time_ms(name)
+        device.set_timing(False)
+        moved = nbytes if read_only else 2 * nbytes
+        out[name] = {"avg_launch_us": ms / n * 1e3, "bytes_moved_per_launch": moved,
+                     "GB/s": moved / (ms / n / 1e3) / 1e9}
+    print(json.dumps(out))
+
+
 def main():
     args = parse_args()
     if args.gpus != 1:
@@ -118,6 +146,9 @@ def main():
         sys.exit(1)
     device = psi.Device(0)
     device.decode_waves(args.decode_waves)
+    if args.calibrate_copy:
+        calibrate_copy(device, args)
+        return
 
     arenas = []
     for i in range(max(1, args.arenas)):

@@ -295,6 +295,11 @@ int psi_hip_page_table_start_index(const psi_hip_page_table_layout* layout, uint
 int psi_hip_page_ids_by_layer(const uint32_t* block_ids, uint32_t block_ids_len, uint32_t num_gqa_layers,
                               uint32_t num_page_ids_per_block, uint32_t* out_by_layer);
 
+/* Measurement aid with no counterpart in the reference: a plain copy (read_only = 0: `bytes` read and
+ * `bytes` written) or a pure read (read_only = 1) of known size, timed under the names "copy_probe" /
+ * "read_probe".  HBM traffic counters are calibrated against it.  bytes must be a multiple of 16. */
+int psi_hip_copy_probe(psi_hip_ctx* ctx, void* dst, const void* src, uint64_t bytes, int read_only);
+
 /* ---------------------------------------------------------------------------------------------
  * Cache ownership on the host: page-ID allocator and the per-request token window.  No device work.
  * ------------------------------------------------------------------------------------------- */

@@ -87,6 +87,10 @@ class Device:
                                                     ctypes.byref(launches)))
         return total.value, launches.value
 
+    def copy_probe(self, dst, src, nbytes: int, read_only: bool = False):
+        """Plain copy (or pure read) of `nbytes`: the calibration load for HBM traffic counters."""
+        L.check(self.lib.psi_hip_copy_probe(self.ctx, _ptr(dst), _ptr(src), nbytes, int(read_only)))
+
     def force_generic(self, on: bool):
         L.check(self.lib.psi_hip_ctx_set_flag(self.ctx, L.FLAG_FORCE_GENERIC, int(on)))
 
