@@ -1,0 +1,207 @@
+"""GPU parity of the multi-query path (speculative verify with 2 or 4 tokens per sequence, prefill
+chunks, mixed batches) against the CPU oracle through the C ABI, and the verify -> accept -> roll
+back cycle driven by the library's own token-window bookkeeping.  Same tolerance as the decode
+path: 2e-3 max-abs / 1e-3 relative RMS on f32 outputs, pages bit-exact."""
+import importlib
+
+import numpy as np
+import pytest
+
+from parity_util import assert_outputs_close, importlib_workloads, oracle_step, run_and_check
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.mark.parametrize("q_len,expected_head_tile", [(2, 3), (4, 6)])
+def test_verify_batches(psi, oracle, device, q_len, expected_head_tile):
+    """C4's geometry (24 Q / 4 KV, D=256, bf16, 16-token pages) at oracle-sized contexts."""
+    wl = importlib_workloads(psi)
+    rng = np.random.default_rng(40 + q_len)
+    ctx = rng.integers(40, 1500, size=8).tolist() + [q_len, 16, 17, 513]
+    w = wl.make_workload(41 + q_len, ctx, 24, 4, 256, psi.Dtype.Bfloat16, 16, q_lens=q_len)
+    stats, dw = run_and_check(psi, oracle, device, w, f"verify q_len={q_len}", max_tokens=4 * len(ctx) * q_len)
+    assert dw.variant.is_tiled() and dw.variant.q_head_tile_size == expected_head_tile
+    print("verify q_len", q_len, "max_abs %.3e rel_rms %.3e" % stats, dw.shape)
+
+
+@pytest.mark.parametrize("partition", [None, 256])
+def test_prefill_chunk_on_prefix(psi, oracle, device, partition):
+    """A 200-token chunk on a 300-token prefix next to decode-sized requests, one variant for all."""
+    wl = importlib_workloads(psi)
+    q_lens = [200, 1, 1, 3, 8, 9]
+    ctx = [500, 700, 33, 64, 8, 40]
+    w = wl.make_workload(51, ctx, 24, 4, 256, psi.Dtype.Bfloat16, 16, q_lens=q_lens)
+    stats, dw = run_and_check(psi, oracle, device, w, "prefill chunk", partition_tokens=partition, max_tokens=512)
+    assert dw.variant.is_tiled()
+    print("prefill chunk max_abs %.3e rel_rms %.3e" % stats, dw.shape)
+
+
+@pytest.mark.parametrize("dtype_name,hq,hkv,d,p,q_len", [
+    ("Bfloat16", 32, 4, 128, 8, 4),
+    ("Bfloat16", 12, 2, 256, 8, 2),
+    ("Float16", 16, 2, 256, 16, 5),
+    ("Bfloat16", 4, 4, 256, 16, 8),
+    ("Float32", 4, 2, 64, 4, 3),
+])
+def test_tiled_geometries(psi, oracle, device, dtype_name, hq, hkv, d, p, q_len):
+    wl = importlib_workloads(psi)
+    dtype = getattr(psi.Dtype, dtype_name)
+    w = wl.make_workload(61, [300, 31, 129, q_len], hq, hkv, d, dtype, p, q_lens=q_len, num_page_ids_per_block=2)
+    variant = psi.GQASplitKVVariant.TiledQ(8, 16 if p >= 8 else 4, min(hq // hkv, 8))
+    run_and_check(psi, oracle, device, w, f"tiled {dtype_name} {hq}/{hkv}/{d} P={p} q={q_len}", max_tokens=64,
+                  variant=variant)
+
+
+def test_sentinel_split_rows_are_skipped(psi, oracle, device):
+    """The split list is padded to its capacity with 0xFFFFFFFF rows; they must not touch anything:
+    the scratch behind the active rows keeps its fill pattern."""
+    import torch
+
+    wl = importlib_workloads(psi)
+    w = wl.make_workload(71, [90, 200, 45], 24, 4, 256, psi.Dtype.Bfloat16, 16, q_lens=[2, 2, 1])
+    dw = wl.DeviceWorkload(device, w, max_tokens=32, f32_output=True,
+                           variant=psi.GQASplitKVVariant.TiledQ(8, 16, 6))
+    assert dw.shape.num_total_sdpa_map_task_templates > dw.shape.num_sdpa_map_task_templates
+    dw.scratch.buffer.view(torch.int32).fill_(0x5A5A5A5A)
+    dw.step()
+    got = dw.output_f32()
+    _, exp = oracle_step(oracle, w)
+    assert_outputs_close(got, exp, "padded")
+    raw = dw.scratch.buffer.view(torch.int32).cpu().numpy()
+    assert (raw == 0x5A5A5A5A).sum() > 0, "padded rows of the scratch were overwritten"
+
+
+def test_verify_accept_rollback_cycle(psi, oracle, device):
+    """Two verify steps with drafts: step 1 writes K/V for [token, d1, d2, d3]; the host accepts a
+    prefix; step 2 starts at the first rejected position and overwrites it.  Attention of step 2
+    must see the accepted history only, and the page table / lengths come from the library's
+    allocator and token window."""
+    import torch
+
+    rt = importlib.import_module("psi-dec_amd.runtime")
+    wl = importlib_workloads(psi)
+    rng = np.random.default_rng(81)
+    hq, hkv, d, p, dtype = 24, 4, 256, 16, psi.Dtype.Bfloat16
+    odt = oracle.BF16
+    n_req, spec = 5, 3
+    prompts = [int(x) for x in rng.integers(20, 200, size=n_req)]
+    page_elems = 2 * hkv * p * d
+    num_pages = sum(-(-(n + 16) // p) for n in prompts) + 8
+    alloc = rt.U32IDAllocator(num_pages)
+    max_blocks = max(-(-(n + 16) // p) for n in prompts)
+    layout = psi.GQAPageTableLayout(n_req, 1, max_blocks, 1)
+    table = psi.GQARequestPageTable(device, layout)
+    host_table = np.zeros(layout.num_page_ids(), np.uint32)
+    pages = np.zeros(num_pages * page_elems, np.uint16)  # host mirror maintained by the oracle
+    dev_pages = device.from_numpy(pages)
+    cfg_w = psi.GQAKVPageWriteConfig(hkv, d, page_elems * 2, dtype)
+    blocks = []
+    # per-token K/V/Q are a pure function of (request, position, token id) so that both sides agree
+
+    def kvq(r, pos, tok):
+        g = np.random.default_rng([r, pos, tok])
+        return (wl.to_storage(g.standard_normal((hkv, d), dtype=np.float32), dtype),
+                wl.to_storage(g.standard_normal((hkv, d), dtype=np.float32), dtype),
+                wl.to_storage(g.standard_normal((hq, d), dtype=np.float32), dtype))
+
+    def sync(r, b):
+        s = b.prepare_blocks()
+        for i, ids in enumerate(s.kv_page_ids[0]):
+            table.write_page_ids(r, 0, s.block_index + i, ids, num_cache_pages=num_pages)
+            host_table[(r * max_blocks + s.block_index + i)] = ids[0]
+
+    def run_step(queries):
+        """queries[r] = (token_index, [token ids incl. drafts]); appends then attends."""
+        slots = list(range(n_req))
+        starts = [q[0] for q in queries]
+        cu = np.concatenate([[0], np.cumsum([len(q[1]) for q in queries])]).astype(np.uint32)
+        fk, fv, fq = [], [], []
+        for r, (start, toks) in enumerate(queries):
+            for i, t in enumerate(toks):
+                k, v, q = kvq(r, start + i, t)
+                fk.append(k), fv.append(v), fq.append(q)
+        fk, fv, fq = np.stack(fk), np.stack(fv), np.stack(fq)
+        total = int(cu[-1])
+        split = psi.GQASplitKV.new(psi.GQASplitKVConfig(dtype, page_elems * 2, hq, hkv, d))
+        variant = split.select(total, n_req)
+        assert variant.is_tiled()
+        meta = psi.GQAMetadataBuffers(device, 64)
+        shape = meta.update(slots, starts, cu.tolist(), variant)
+        write = psi.GQAKVPageWrite(device, cfg_w)
+        write.invoke_bucketed(psi.GQAKVPageWriteShape(shape.num_total_tokens, layout),
+                              psi.GQAKVPageWriteBuffers(dev_pages, device.from_numpy(fk.reshape(-1)),
+                                                        device.from_numpy(fv.reshape(-1)), meta.d_req_slots,
+                                                        meta.d_flat_token_indices, table.page_ids_buffer()),
+                              shape.num_tokens, 0)
+        cfg = psi.GQASplitKVTiledQConfig(hq, hkv, d, variant.q_head_tile_size, variant.q_token_tile_size,
+                                         variant.kv_token_tile_size, 1.0 / 16.0, page_elems * 2, dtype, layout)
+        kshape = psi.GQASplitKVTiledQShape(shape.num_total_tokens, shape.num_total_q_token_tiles,
+                                           shape.num_total_sdpa_map_task_templates)
+        kern = psi.GQASplitKVTiledQKernels(device, cfg, kshape)
+        scratch = psi.GQASplitKVTiledQScratch(device, cfg, kshape)
+        out = torch.zeros(shape.num_total_tokens * hq * d, dtype=torch.float32, device=device.torch_device)
+        kern.invoke_map_bucketed(device.from_numpy(fq.reshape(-1)), dev_pages, meta.d_req_slots,
+                                 table.page_ids_buffer(), meta.d_flat_token_indices, meta.d_q_token_tiles,
+                                 meta.d_kv_splits, scratch, 0, shape.num_tokens, shape.num_q_token_tiles,
+                                 shape.num_sdpa_map_task_templates)
+        device.f32_output(True)
+        kern.invoke_reduce_bucketed(scratch, meta.d_q_token_tiles, meta.d_cu_kv_splits, out,
+                                    shape.num_q_token_tiles)
+        device.f32_output(False)
+        device.sync()
+        # oracle on the host mirror
+        lt = (n_req, 1, max_blocks, 1)
+        oracle.kv_page_write(pages, fk.reshape(-1), fv.reshape(-1), meta.h_req_slots[:total],
+                             meta.h_flat_token_indices[:total], host_table, total, 0, lt, hkv, d, page_elems * 2, odt)
+        exp = oracle.paged_gqa(hq, hkv, d, 1.0 / 16.0, page_elems * 2, odt, lt, 0, slots, starts, cu, fq.reshape(-1),
+                               pages, host_table, num_threads=8)
+        got = out[:total * hq * d].cpu().numpy()
+        assert_outputs_close(got, exp, "verify step")
+        assert np.array_equal(dev_pages.view(torch.int16).cpu().numpy().view(np.uint16), pages)
+
+    # prefill the prompts on the host side of the bookkeeping (K/V history written by the oracle path)
+    for r, n in enumerate(prompts):
+        toks = [1000 * r + i for i in range(n)]
+        b = rt.DecoderBlocks(alloc, p, 1, 1, toks)
+        blocks.append(b)
+        while b.ready_token_slots() < n - 1:
+            assert b.init_block_once() != "ResourceLimitExceeded"
+        q = b.prepare(n - 1)  # everything but the last prompt token
+        assert q.kind == "Prefill" and q.token_index == 0
+        sync(r, b)
+        fk = np.stack([kvq(r, i, toks[i])[0] for i in range(n - 1)])
+        fv = np.stack([kvq(r, i, toks[i])[1] for i in range(n - 1)])
+        oracle.kv_page_write(pages, fk.reshape(-1), fv.reshape(-1), [r] * (n - 1), list(range(n - 1)), host_table,
+                             n - 1, 0, (n_req, 1, max_blocks, 1), hkv, d, page_elems * 2, odt)
+        b.commit(q, rt.SampledTokens.prefill(q.epoch))
+        b.set_spec_tokens([50000 + 10 * r + j for j in range(spec)])
+    dev_pages.copy_(device.from_numpy(pages))
+
+    accepted_total = 0
+    for step in range(2):
+        queries, prepared = [], []
+        for r, b in enumerate(blocks):
+            budget = len(b.ready_tokens()) + len(b.queued_tokens()) + len(b.spec_tokens())
+            while b.ready_token_slots() < budget:
+                assert b.init_block_once() != "ResourceLimitExceeded"
+            budget = len(b.ready_tokens()) + len(b.queued_tokens()) + len(b.spec_tokens())
+            q = b.prepare(budget)
+            assert q.kind == "Decode" and len(q.tokens) == 1 and len(q.spec_tokens) == spec
+            assert q.token_index == len(b.cached_tokens())
+            sync(r, b)
+            prepared.append(q)
+            queries.append((q.token_index, q.tokens + q.spec_tokens))
+        run_step(queries)
+        for r, (b, q) in enumerate(zip(blocks, prepared)):
+            accept = int(rng.integers(0, spec + 1))  # seeded Bernoulli-prefix accept mask
+            accepted_total += accept
+            before = len(b.cached_tokens())
+            b.commit(q, rt.SampledTokens.decode(q.epoch, q.spec_tokens[:accept], 70000 + 100 * step + r,
+                                                [60000 + 100 * step + 10 * r + j for j in range(spec)]))
+            # the cache advanced by the input token plus the accepted drafts; rejected slots will be rewritten
+            assert len(b.cached_tokens()) == before + 1 + accept
+    assert 0 < accepted_total < 2 * n_req * spec
+    used = alloc.used()
+    for b in blocks:
+        b.close()
+    assert alloc.used() == 0 and used > 0
