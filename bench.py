@@ -41,6 +41,10 @@ def parse_args():
     p.add_argument("--decode-waves", type=int, default=0, help="waves per decode workgroup (0 = automatic)")
     p.add_argument("--balance", action="store_true", help="equal-tile worker plan instead of one workgroup per partition")
     p.add_argument("--kernel-only", action="store_true", help="time only the map kernel (for profiling runs)")
+    p.add_argument("--workload", choices=["decode", "verify"], default="decode",
+                   help="decode: one new token per sequence (the headline workload); verify: --q-len tokens per "
+                        "sequence through the multi-query kernels (batch 64, contexts 2048-16384 unless overridden)")
+    p.add_argument("--q-len", type=int, default=2)
     p.add_argument("--calibrate-copy", action="store_true",
                    help="run only the plain copy / read probes of known size (counter calibration, practical ceiling)")
     p.add_argument("--probe-mib", type=int, default=1024)
@@ -150,10 +154,19 @@ def main():
         calibrate_copy(device, args)
         return
 
+    verify = args.workload == "verify"
+    if verify and args.batch == 32 and args.ctx_lo == 1024 and args.ctx_hi == 8192:
+        args.batch, args.ctx_lo, args.ctx_hi = 64, 2048, 16384
+    map_kernel = "tiled_q_map" if verify else "split_kv_map"
     arenas = []
     for i in range(max(1, args.arenas)):
-        w = wl.config_c2(seed=args.seed, batch=args.batch, host_pages=False, lo=args.ctx_lo, hi=args.ctx_hi,
-                         shuffle_pages=not args.identity_pages)
+        if verify:
+            ctx = wl.config_c2_context_lens(args.seed, args.batch, args.ctx_lo, args.ctx_hi) + args.q_len
+            w = wl.make_workload(args.seed, ctx, 24, 4, 256, psi.Dtype.Bfloat16, 16, q_lens=args.q_len,
+                                 host_pages=False, shuffle_pages=not args.identity_pages)
+        else:
+            w = wl.config_c2(seed=args.seed, batch=args.batch, host_pages=False, lo=args.ctx_lo, hi=args.ctx_hi,
+                             shuffle_pages=not args.identity_pages)
         w.seed = args.seed + 1000 * i  # same geometry, different page contents
         arenas.append(wl.DeviceWorkload(device, w, partition_tokens=args.partition, balanced=args.balance))
     w = arenas[0].w
@@ -182,13 +195,13 @@ def main():
     device.set_timing(True)
     device.reset_timing()
     run_maps(min(args.steps, 100))
-    map_ms, map_launches = device.kernel_time_ms("split_kv_map")
+    map_ms, map_launches = device.kernel_time_ms(map_kernel)
     device.set_timing(False)
     map_avg_s = map_ms / max(map_launches, 1) / 1e3
     achieved = map_bytes / map_avg_s / 1e9
 
-    workload_key = (f"decode_b{args.batch}_ctx{args.ctx_lo}-{args.ctx_hi}_24q4kv_d256_bf16_p16_part{args.partition}"
-                    f"_seed{args.seed}")
+    workload_key = (f"{'verify_q%d' % args.q_len if verify else 'decode'}_b{args.batch}_ctx{args.ctx_lo}-{args.ctx_hi}"
+                    f"_24q4kv_d256_bf16_p16_part{args.partition}_seed{args.seed}")
     result = {
         "metric": "decode attn achieved HBM GB/s per layer-step (B=32, ctx 1k-8k); us/layer-step alongside",
         "value": (map_bytes if args.kernel_only else step_bytes) / (ms_per_step / 1e3) / 1e9,
@@ -215,7 +228,7 @@ def main():
         },
         "roofline": {
             "bound": "hbm",
-            "kernel": "split_kv_decode_map",
+            "kernel": "split_kv_tiled_map" if verify else "split_kv_decode_map",
             "achieved": achieved,
             "peak": HBM_PEAK_GBPS,
             "unit": "GB/s",

@@ -253,7 +253,10 @@ int psi_hip_split_kv_tiled_q_scratch_bytes(const psi_hip_gqa_config* cfg, uint32
 
 /* `GQASplitKVTiledQKernels::invoke_map_bucketed` (gqa_split_kv_tiled_q.rs:279-300; kernel
  * metal/gqa_split_kv_tiled_q.metal:49-319).  q_token_tiles: device u32[num_total_q_token_tiles][2];
- * kv_splits rows index q-token tiles.  Causal mask: key position > flat_token_indices[q] is hidden. */
+ * kv_splits rows index q-token tiles.  Causal mask: key position > flat_token_indices[q] is hidden.
+ * max_active_q_tile_tokens (no counterpart in the reference): the largest number of tokens any active
+ * tile holds, e.g. 2 for a verify step with one draft; it sizes the kernel's query-column blocks.
+ * 0 = unknown, any tile may hold q_token_tile_size tokens. */
 int psi_hip_split_kv_tiled_q_map(psi_hip_ctx* ctx, const psi_hip_gqa_config* cfg,
                                  const psi_hip_page_table_layout* layout, uint32_t q_token_tile_size,
                                  const void* q, const void* kv_pages, uint64_t kv_pages_bytes,
@@ -263,7 +266,7 @@ int psi_hip_split_kv_tiled_q_map(psi_hip_ctx* ctx, const psi_hip_gqa_config* cfg
                                  uint32_t gqa_layer_index, uint32_t num_total_tokens,
                                  uint32_t num_total_q_token_tiles, uint32_t num_total_kv_splits,
                                  uint32_t num_active_tokens, uint32_t num_active_q_token_tiles,
-                                 uint32_t num_active_kv_splits);
+                                 uint32_t num_active_kv_splits, uint32_t max_active_q_tile_tokens);
 
 /* `GQASplitKVTiledQKernels::invoke_reduce_bucketed` (gqa_split_kv_tiled_q.rs:314-327; kernel
  * metal/gqa_split_kv_tiled_q.metal:324-378). */

@@ -163,7 +163,8 @@ PROTOTYPES = {
     "psi_hip_split_kv_tiled_q_map": (
         c_int,
         [c_void_p, _CFG, _LAYOUT, c_uint32, c_void_p, c_void_p, c_uint64, c_void_p, c_void_p, c_void_p, c_void_p,
-         c_void_p, c_void_p, c_uint64, c_uint32, c_uint32, c_uint32, c_uint32, c_uint32, c_uint32, c_uint32],
+         c_void_p, c_void_p, c_uint64, c_uint32, c_uint32, c_uint32, c_uint32, c_uint32, c_uint32, c_uint32,
+         c_uint32],
     ),
     "psi_hip_split_kv_tiled_q_reduce": (
         c_int,

@@ -46,6 +46,7 @@ struct MapArgs {
     const uint32_t* flat_token_indices = nullptr;  // request-absolute position of each flat token
     uint32_t rows_per_split_head = 1;              // q_token_tile_size
     uint32_t num_active_q_token_tiles = 0;
+    uint32_t max_q_tile_tokens = 0;                // largest active tile (0: up to rows_per_split_head)
     // Balanced decode launch only: workgroup w of a KV head serves kv_splits rows
     // [worker_cu[w], worker_cu[w + 1]).
     const uint32_t* worker_cu = nullptr;

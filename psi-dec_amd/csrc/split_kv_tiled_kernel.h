@@ -1,0 +1,418 @@
+// gfx950 split-KV multi-query map (speculative verify, prefill chunks) for 2-byte K/V (bf16 / f16),
+// head_dim 128 or 256, pages of 16*k tokens.  Semantics of
+// crates/inference-backend-metal/src/components/metal/gqa_split_kv_tiled_q.metal:49-319.
+//
+// Work decomposition
+//   one workgroup (4 waves) = one (kv_split row, kv_head).  The row names a request-local tile of
+//   up to 8 query tokens; with the G query heads that share the KV head this gives up to 8*G
+//   query columns, column c = token_in_tile * G + head, handled as NB blocks of 16 columns.  Every
+//   K and V byte of the split is therefore fetched once for all of them.  One wave = every 4th
+//   16-token KV tile, with its own online-softmax state per column; wave states merge through LDS
+//   at the end.
+//
+// Per 16-token KV tile and wave
+//   QK^T  S[token][column] on v_mfma_f32_16x16x32: A = the K tile straight from the page (lane =
+//         token lane%16, 8 contiguous dims per 128-bit load), B = the query columns staged once
+//         per workgroup in LDS in operand order.
+//   softmax  the MFMA leaves each lane with 4 tokens of one column; causal / range masks per
+//         column; probabilities stay in registers: that register layout is exactly the A operand
+//         of v_mfma_f32_16x16x16 (row = column, k = 4 tokens).
+//   PV    O[column][dim] += P^T * V on v_mfma_f32_16x16x16.  The contraction runs over tokens, the
+//         strided axis of V, so the V tile goes through a per-wave LDS buffer: written with
+//         128-bit stores as loaded, read back as 4 tokens x 1 dim per lane.  bf16 probabilities
+//         are split into two bf16 terms (two MFMAs) so that P carries 16 mantissa bits; f16
+//         carries 11 in one.
+//   K and V loads run one tile ahead, as in the decode kernel.
+//
+// Algorithmic bytes per (kv token, kv head): 2 * head_dim * 2, read once per (Q tile, split).
+#pragma once
+#include <type_traits>
+
+#include "split_kv_decode_kernel.h"
+
+namespace psi {
+
+typedef __attribute__((ext_vector_type(4))) short s16x4_t;
+typedef __attribute__((ext_vector_type(4))) _Float16 f16x4_t;
+
+// D(16x16, f32) += A(16x16) * B(16x16).  Lane l holds A[row l%16][k 4*(l/16)..+4],
+// B[k 4*(l/16)..+4][col l%16] and D[row 4*(l/16)+r][col l%16], r = 0..3.
+template <typename Tag>
+__device__ __forceinline__ f32x4_t mfma_16x16x16(uint2 a, uint2 b, f32x4_t c);
+template <>
+__device__ __forceinline__ f32x4_t mfma_16x16x16<BF16Tag>(uint2 a, uint2 b, f32x4_t c) {
+    return __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(__builtin_bit_cast(s16x4_t, a), __builtin_bit_cast(s16x4_t, b), c,
+                                                     0, 0, 0);
+}
+template <>
+__device__ __forceinline__ f32x4_t mfma_16x16x16<F16Tag>(uint2 a, uint2 b, f32x4_t c) {
+    return __builtin_amdgcn_mfma_f32_16x16x16f16(__builtin_bit_cast(f16x4_t, a), __builtin_bit_cast(f16x4_t, b), c, 0,
+                                                 0, 0);
+}
+
+// Probabilities of 4 tokens -> A operand(s).  bf16: p = hi + lo with both terms truncated to bf16,
+// 16 mantissa bits in total; f16: one rounded term.
+template <typename Tag>
+struct ProbOperand;
+template <>
+struct ProbOperand<BF16Tag> {
+    static constexpr int kTerms = 2;
+    uint2 term[2];
+    __device__ __forceinline__ void set(const float (&p)[4]) {
+        uint32_t hi[4], lo[4];
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+            hi[r] = __float_as_uint(p[r]) & 0xffff0000u;
+            lo[r] = __float_as_uint(p[r] - __uint_as_float(hi[r])) & 0xffff0000u;
+        }
+        term[0] = make_uint2((hi[0] >> 16) | hi[1], (hi[2] >> 16) | hi[3]);
+        term[1] = make_uint2((lo[0] >> 16) | lo[1], (lo[2] >> 16) | lo[3]);
+    }
+};
+template <>
+struct ProbOperand<F16Tag> {
+    static constexpr int kTerms = 1;
+    uint2 term[1];
+    __device__ __forceinline__ void set(const float (&p)[4]) {
+        const f16x4_t h = {(_Float16)p[0], (_Float16)p[1], (_Float16)p[2], (_Float16)p[3]};
+        term[0] = __builtin_bit_cast(uint2, h);
+    }
+};
+
+constexpr int kTiledWaves = 4;
+
+template <int NB>
+struct TiledOccupancy {
+    static constexpr int value = NB == 1 ? 3 : (NB == 2 ? 2 : 1);
+};
+
+template <typename Tag, int D, int NB>
+__global__ __launch_bounds__(64 * kTiledWaves, TiledOccupancy<NB>::value) void split_kv_tiled_map(
+    MapArgs a, const uint32_t* __restrict__ page_ids, const uint32_t* __restrict__ kv_splits,
+    const uint32_t* __restrict__ req_slots, const uint16_t* __restrict__ q, const uint16_t* __restrict__ pages,
+    const uint32_t* __restrict__ q_token_tiles, const uint32_t* __restrict__ flat_token_indices) {
+    constexpr int kWaves = kTiledWaves;
+    constexpr int kVLanesPerToken = D / 8;                  // 32 (D=256) or 16 (D=128)
+    constexpr int kVTokensPerLoad = 64 / kVLanesPerToken;   // 2 or 4
+    constexpr int kVLoads = kTileTokens / kVTokensPerLoad;  // 8 or 4
+    constexpr int kKSteps = D / 32;                         // MFMA k-steps of QK^T
+    constexpr int kDimBlocks = D / 16;                      // 16-dim output blocks of PV
+    constexpr int kVStride = D + 8;                         // elements per token row of the V buffer (bank spread)
+    constexpr int kCols = NB * 16;
+    constexpr int kMergeStride = D + 4;                     // floats per column row of the merge buffer
+
+    // LDS: the main loop's V buffers and Q operands share their bytes with the epilogue's merge buffer.
+    constexpr int kVBytes = kWaves * kTileTokens * kVStride * 2;
+    constexpr int kQBytes = NB * kKSteps * 64 * 16;
+    constexpr int kMergeBytes = kCols * kMergeStride * 4;
+    constexpr int kUnionBytes = (kVBytes + kQBytes) > kMergeBytes ? (kVBytes + kQBytes) : kMergeBytes;
+    __shared__ __attribute__((aligned(16))) unsigned char lds_union[kUnionBytes];
+    __shared__ float wave_max_lds[kWaves][kCols];
+    __shared__ float col_max_lds[kCols];
+    __shared__ float col_sum_lds[kCols];
+    uint16_t* v_lds = reinterpret_cast<uint16_t*>(lds_union);
+    uint4* qb_lds = reinterpret_cast<uint4*>(lds_union + kVBytes);  // [NB][kKSteps][64]
+    float* merge = reinterpret_cast<float*>(lds_union);
+
+    const uint32_t G = a.group;
+    const uint32_t kv_head = blockIdx.x % a.walk.hkv;
+    const uint32_t split = blockIdx.x / a.walk.hkv;
+    const uint32_t tid = threadIdx.x;
+    const uint32_t lane = tid & 63;
+    const uint32_t wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const uint32_t mt = lane & 15, mc = lane >> 4;
+    const uint32_t vsub = lane / kVLanesPerToken, vdl = lane % kVLanesPerToken;
+
+    if (split >= a.num_active_kv_splits) return;
+    const uint32_t q_tile = kv_splits[split * 3];
+    if (q_tile >= a.num_active_q_token_tiles) return;  // sentinel padding
+    const uint32_t kv_begin = kv_splits[split * 3 + 1];
+    const uint32_t kv_end = kv_splits[split * 3 + 2];
+    const uint32_t flat_begin = q_token_tiles[q_tile * 2], flat_end = q_token_tiles[q_tile * 2 + 1];
+    if (flat_begin >= a.num_active_tokens || flat_end > a.num_active_tokens || flat_end <= flat_begin) return;
+    const uint32_t tile_tokens = flat_end - flat_begin;
+    const uint32_t ncols = tile_tokens * G;
+    if (ncols > (uint32_t)kCols) return;  // the launcher sizes NB from the largest tile; never taken
+    const uint32_t nb_active = (ncols + 15) / 16;
+    const uint32_t req_slot = req_slots[flat_begin];
+
+    // Column of this lane in block nb: c = 16*nb + mt; its query token, head and visible key range.
+    uint32_t lim[NB];  // keys [kv_begin, lim) are visible to the column (0: column unused)
+#pragma unroll
+    for (int nb = 0; nb < NB; ++nb) {
+        const uint32_t c = nb * 16 + mt;
+        lim[nb] = 0;
+        if (c < ncols) lim[nb] = min(kv_end, flat_token_indices[flat_begin + c / G] + 1);
+    }
+
+    // Query columns as MFMA B operands [nb][k-step][lane]; unused columns are zero.
+    for (uint32_t nb = wave; nb < nb_active; nb += kWaves) {
+        const uint32_t c = nb * 16 + mt;
+        const bool used = c < ncols;
+        const uint32_t cc = used ? c : 0;
+        const uint16_t* q_row =
+            q + ((uint64_t)(flat_begin + cc / G) * a.hq + (uint64_t)kv_head * G + cc % G) * D + mc * 8;
+#pragma unroll
+        for (int i = 0; i < kKSteps; ++i) {
+            const uint4 v = *reinterpret_cast<const uint4*>(q_row + i * 32);
+            qb_lds[(nb * kKSteps + i) * 64 + lane] = used ? v : make_uint4(0, 0, 0, 0);
+        }
+    }
+    __syncthreads();
+
+    const uint32_t log2p = 31 - __builtin_clz(a.walk.tokens_per_page);
+    const uint32_t page_mask = a.walk.tokens_per_page - 1;
+    const uint32_t* table_row = page_ids + ((uint64_t)req_slot * a.walk.num_layers + a.layer) *
+                                                      a.walk.num_blocks * a.walk.ids_per_block;
+    const uint64_t v_region = (uint64_t)a.walk.hkv * a.walk.tokens_per_page * D;
+    const uint32_t tile_begin = kv_begin / kTileTokens;
+    const uint32_t tile_end = (kv_end + kTileTokens - 1) / kTileTokens;
+
+    float run_max[NB], lane_sum[NB];
+    f32x4_t o[NB][kDimBlocks];
+#pragma unroll
+    for (int nb = 0; nb < NB; ++nb) {
+        run_max[nb] = -INFINITY;
+        lane_sum[nb] = 0.0f;
+#pragma unroll
+        for (int db = 0; db < kDimBlocks; ++db) o[nb][db] = f32x4_t{0.0f, 0.0f, 0.0f, 0.0f};
+    }
+
+    auto load_page_id = [&](uint32_t tile) -> uint32_t {
+        return tile < tile_end ? table_row[(tile * kTileTokens) >> log2p] : 0u;
+    };
+    auto tile_k_base = [&](uint32_t tile, uint32_t page_id) -> const uint16_t* {
+        const uint32_t in_page = (tile * kTileTokens) & page_mask;
+        return pages + (uint64_t)page_id * a.walk.page_elems +
+               ((uint64_t)kv_head * a.walk.tokens_per_page + in_page) * D;
+    };
+    uint4 kreg[kKSteps];
+    uint4 vreg[kVLoads];
+    auto issue_k = [&](uint32_t tile, uint32_t page_id) {
+        const uint16_t* k_lane = tile_k_base(tile, page_id) + mt * D + mc * 8;
+#pragma unroll
+        for (int i = 0; i < kKSteps; ++i) kreg[i] = *reinterpret_cast<const uint4*>(k_lane + i * 32);
+    };
+    auto issue_v = [&](uint32_t tile, uint32_t page_id) {
+        const uint16_t* v_lane = tile_k_base(tile, page_id) + v_region + vsub * D + vdl * 8;
+#pragma unroll
+        for (int j = 0; j < kVLoads; ++j) vreg[j] = *reinterpret_cast<const uint4*>(v_lane + j * kVTokensPerLoad * D);
+    };
+
+    uint16_t* my_v = v_lds + wave * kTileTokens * kVStride;
+    // B operand of PV for dim block db: 4 consecutive tokens of this lane's token quad, one dim.
+    const uint16_t* my_v_read = my_v + (mc * 4) * kVStride + mt;
+
+    auto process_tile = [&](uint32_t tile, bool partial, auto has_next_tag, uint32_t next, uint32_t next_pid)
+                            __attribute__((always_inline)) {
+        constexpr bool has_next = decltype(has_next_tag)::value;
+        // ---- logits S[token][column] on the matrix cores
+        f32x4_t s[NB];
+#pragma unroll
+        for (int nb = 0; nb < NB; ++nb) {
+            s[nb] = f32x4_t{0.0f, 0.0f, 0.0f, 0.0f};
+            if ((uint32_t)nb < nb_active) {
+#pragma unroll
+                for (int i = 0; i < kKSteps; ++i)
+                    s[nb] = mfma_16x16x32<Tag>(kreg[i], qb_lds[(nb * kKSteps + i) * 64 + lane], s[nb]);
+            }
+        }
+        __builtin_amdgcn_sched_barrier(0);
+        if (has_next) issue_k(next, next_pid);
+        __builtin_amdgcn_sched_barrier(0);
+
+        // ---- online softmax per column over this lane's tokens 4*mc + r
+        ProbOperand<Tag> pa[NB];
+        float alpha[NB];
+        bool moved = false;
+#pragma unroll
+        for (int nb = 0; nb < NB; ++nb) {
+            alpha[nb] = 1.0f;
+            if ((uint32_t)nb < nb_active) {
+                float v[4];
+                bool valid[4];
+                float m = -INFINITY;
+#pragma unroll
+                for (int r = 0; r < 4; ++r) {
+                    const uint32_t token = tile * kTileTokens + mc * 4 + r;
+                    valid[r] = token >= kv_begin && token < lim[nb];
+                    v[r] = valid[r] ? s[nb][r] * a.scale_log2 : -INFINITY;
+                    m = fmaxf(m, v[r]);
+                }
+                m = fmaxf(m, __shfl_xor(m, 16, 64));
+                m = fmaxf(m, __shfl_xor(m, 32, 64));
+                const float next_max = fmaxf(run_max[nb], m);
+                // a column with no visible key so far keeps max = -inf, sum = 0, O = 0
+                alpha[nb] = run_max[nb] > -INFINITY ? __builtin_amdgcn_exp2f(run_max[nb] - next_max) : 0.0f;
+                moved = moved || next_max != run_max[nb];
+                run_max[nb] = next_max;
+                float p[4], tile_sum = 0.0f;
+#pragma unroll
+                for (int r = 0; r < 4; ++r) {
+                    p[r] = valid[r] ? __builtin_amdgcn_exp2f(v[r] - next_max) : 0.0f;
+                    tile_sum += p[r];
+                }
+                lane_sum[nb] = lane_sum[nb] * alpha[nb] + tile_sum;
+                pa[nb].set(p);
+            }
+        }
+        const bool rescale = __any(moved);
+
+        // ---- V tile: registers -> this wave's LDS buffer (rows outside the split zeroed: their
+        // probability is 0 but their bytes may be NaN/Inf), then refill the registers for the next tile
+        wave_lds_fence();  // the previous tile's reads of the buffer are complete
+#pragma unroll
+        for (int j = 0; j < kVLoads; ++j) {
+            const uint32_t tok_in_tile = j * kVTokensPerLoad + vsub;
+            uint4 val = vreg[j];
+            if (partial) {
+                const uint32_t vtoken = tile * kTileTokens + tok_in_tile;
+                if (vtoken < kv_begin || vtoken >= kv_end) val = make_uint4(0, 0, 0, 0);
+            }
+            *reinterpret_cast<uint4*>(my_v + tok_in_tile * kVStride + vdl * 8) = val;
+        }
+        __builtin_amdgcn_sched_barrier(0);
+        if (has_next) issue_v(next, next_pid);
+        __builtin_amdgcn_sched_barrier(0);
+        wave_lds_fence();
+
+        // ---- O[column][dim] = alpha * O + P^T V
+        if (rescale) {
+#pragma unroll
+            for (int nb = 0; nb < NB; ++nb) {
+                if ((uint32_t)nb < nb_active) {
+                    float al[4];
+#pragma unroll
+                    for (int r = 0; r < 4; ++r) al[r] = __shfl(alpha[nb], mc * 4 + r, 64);
+#pragma unroll
+                    for (int db = 0; db < kDimBlocks; ++db)
+#pragma unroll
+                        for (int r = 0; r < 4; ++r) o[nb][db][r] *= al[r];
+                }
+            }
+        }
+#pragma unroll
+        for (int db = 0; db < kDimBlocks; ++db) {
+            const uint16_t* src = my_v_read + db * 16;
+            const uint32_t v0 = src[0], v1 = src[kVStride], v2 = src[2 * kVStride], v3 = src[3 * kVStride];
+            const uint2 b = make_uint2(v0 | (v1 << 16), v2 | (v3 << 16));
+#pragma unroll
+            for (int nb = 0; nb < NB; ++nb) {
+                if ((uint32_t)nb < nb_active) {
+#pragma unroll
+                    for (int t = 0; t < ProbOperand<Tag>::kTerms; ++t)
+                        o[nb][db] = mfma_16x16x16<Tag>(pa[nb].term[t], b, o[nb][db]);
+                }
+            }
+        }
+        __builtin_amdgcn_sched_barrier(0);
+    };
+
+    uint32_t tile = tile_begin + wave;
+    if (tile < tile_end) {
+        {
+            const uint32_t pid = load_page_id(tile);
+            issue_k(tile, pid);
+            issue_v(tile, pid);
+        }
+        uint32_t pid_next = load_page_id(tile + kWaves);
+        auto is_partial = [&](uint32_t t) { return t * kTileTokens < kv_begin || (t + 1) * kTileTokens > kv_end; };
+        while (tile + kWaves < tile_end) {
+            const uint32_t next = tile + kWaves;
+            const uint32_t pid_after = load_page_id(next + kWaves);
+            process_tile(tile, is_partial(tile), std::true_type(), next, pid_next);
+            pid_next = pid_after;
+            tile = next;
+        }
+        process_tile(tile, is_partial(tile), std::false_type(), 0u, 0u);
+    }
+
+    // ---- merge the four wave states.  Column statistics live in the S layout (lane <-> column mt),
+    // the accumulators in the MFMA output layout (lane <-> columns 4*mc + r, dim mt).
+#pragma unroll
+    for (int nb = 0; nb < NB; ++nb) {
+        lane_sum[nb] += __shfl_xor(lane_sum[nb], 16, 64);
+        lane_sum[nb] += __shfl_xor(lane_sum[nb], 32, 64);
+        if (mc == 0) wave_max_lds[wave][nb * 16 + mt] = run_max[nb];
+    }
+    __syncthreads();  // every wave has left the main loop: the V / Q bytes may now be reused
+#pragma unroll
+    for (int nb = 0; nb < NB; ++nb) {
+        const uint32_t c = nb * 16 + mt;
+        float gm = wave_max_lds[0][c];
+#pragma unroll
+        for (int w = 1; w < kWaves; ++w) gm = fmaxf(gm, wave_max_lds[w][c]);
+        const float f = run_max[nb] > -INFINITY ? __builtin_amdgcn_exp2f(run_max[nb] - gm) : 0.0f;
+        lane_sum[nb] *= f;
+        if (wave == 0 && mc == 0) col_max_lds[c] = gm;
+        float fr[4];
+#pragma unroll
+        for (int r = 0; r < 4; ++r) fr[r] = __shfl(f, mc * 4 + r, 64);
+#pragma unroll
+        for (int db = 0; db < kDimBlocks; ++db)
+#pragma unroll
+            for (int r = 0; r < 4; ++r) o[nb][db][r] *= fr[r];
+    }
+    for (uint32_t w = 0; w < (uint32_t)kWaves; ++w) {
+        if (wave == w) {
+#pragma unroll
+            for (int nb = 0; nb < NB; ++nb) {
+                if ((uint32_t)nb < nb_active) {
+                    if (mc == 0) {
+                        const uint32_t c = nb * 16 + mt;
+                        col_sum_lds[c] = (w == 0 ? 0.0f : col_sum_lds[c]) + lane_sum[nb];
+                    }
+#pragma unroll
+                    for (int db = 0; db < kDimBlocks; ++db)
+#pragma unroll
+                        for (int r = 0; r < 4; ++r) {
+                            float* dst = merge + (nb * 16 + mc * 4 + r) * kMergeStride + db * 16 + mt;
+                            *dst = (w == 0 ? 0.0f : *dst) + o[nb][db][r];
+                        }
+                }
+            }
+        }
+        __syncthreads();
+    }
+
+    // ---- emit: partial row of (split, q_head, token_in_tile); 1 KiB of contiguous f32 per wave store
+    const uint32_t rows = a.rows_per_split_head;
+    for (uint32_t idx = tid; idx < ncols * (D / 4); idx += 64 * kWaves) {
+        const uint32_t c = idx / (D / 4), d4 = idx % (D / 4);
+        const uint64_t row = ((uint64_t)split * a.hq + (uint64_t)kv_head * G + c % G) * rows + c / G;
+        const float4 val = *reinterpret_cast<const float4*>(merge + c * kMergeStride + d4 * 4);
+        *reinterpret_cast<float4*>(&a.part_acc[row * D + d4 * 4]) = val;
+    }
+    if (tid < ncols) {
+        const uint64_t row = ((uint64_t)split * a.hq + (uint64_t)kv_head * G + tid % G) * rows + tid / G;
+        a.part_max[row] = col_max_lds[tid];
+        a.part_sum[row] = col_sum_lds[tid];
+    }
+}
+
+// Column blocks needed for tiles of up to `max_tile_tokens` query tokens and `group` heads per KV head.
+inline int tiled_column_blocks(uint32_t max_tile_tokens, uint32_t group) { return (int)((max_tile_tokens * group + 15) / 16); }
+
+template <typename Tag, int D>
+inline int launch_tiled_map_typed(psi_hip_ctx* ctx, const Geometry& g, const MapArgs& a, uint32_t max_tile_tokens) {
+    const int nb = tiled_column_blocks(max_tile_tokens, g.group);
+    const dim3 grid(a.num_total_kv_splits * g.hkv), block(64 * kTiledWaves);
+    const uint16_t* q = reinterpret_cast<const uint16_t*>(a.q);
+    const uint16_t* pages = reinterpret_cast<const uint16_t*>(a.kv_pages);
+#define PSI_TILED_CASE(NB)                                                                                         \
+    case NB:                                                                                                        \
+        hipLaunchKernelGGL((split_kv_tiled_map<Tag, D, NB>), grid, block, 0, ctx->stream, a, a.walk.page_ids,       \
+                           a.kv_splits, a.req_slots, q, pages, a.q_token_tiles, a.flat_token_indices);              \
+        return PSI_HIP_OK;
+    switch (nb) {
+        PSI_TILED_CASE(1)
+        PSI_TILED_CASE(2)
+        PSI_TILED_CASE(3)
+        PSI_TILED_CASE(4)
+        default:
+            return PSI_HIP_ERR_UNSUPPORTED;
+    }
+#undef PSI_TILED_CASE
+}
+
+}  // namespace psi

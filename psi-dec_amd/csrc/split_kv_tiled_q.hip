@@ -50,7 +50,7 @@ extern "C" int psi_hip_split_kv_tiled_q_map(psi_hip_ctx* ctx, const psi_hip_gqa_
                                             uint32_t gqa_layer_index, uint32_t num_total_tokens,
                                             uint32_t num_total_q_token_tiles, uint32_t num_total_kv_splits,
                                             uint32_t num_active_tokens, uint32_t num_active_q_token_tiles,
-                                            uint32_t num_active_kv_splits) {
+                                            uint32_t num_active_kv_splits, uint32_t max_active_q_tile_tokens) {
     PSI_REQUIRE(ctx != nullptr, "ctx must not be null");
     Geometry g;
     int rc = make_geometry(cfg, &g);
@@ -93,6 +93,9 @@ extern "C" int psi_hip_split_kv_tiled_q_map(psi_hip_ctx* ctx, const psi_hip_gqa_
     a.flat_token_indices = flat_token_indices;
     a.rows_per_split_head = q_token_tile_size;
     a.num_active_q_token_tiles = num_active_q_token_tiles;
+    PSI_REQUIRE(max_active_q_tile_tokens <= q_token_tile_size,
+                "GQA SplitKV TiledQ largest active tile exceeds the Q-token tile size");
+    a.max_q_tile_tokens = max_active_q_tile_tokens;
 
     LaunchScope scope(ctx, "tiled_q_map");
     rc = launch_tiled_map_fast(ctx, g, a);

@@ -693,14 +693,17 @@ class GQASplitKVTiledQKernels:
 
     def invoke_map_bucketed(self, q, kv_pages, req_slots, page_ids, flat_token_indices, q_token_tiles,
                             sdpa_map_task_templates, scratch, page_table_index: int, num_active_tokens: int,
-                            num_active_q_token_tiles: int, num_active_kv_splits: int):
+                            num_active_q_token_tiles: int, num_active_kv_splits: int,
+                            max_active_q_tile_tokens: int = 0):
+        """`max_active_q_tile_tokens`: the largest tile of this batch (2 for a one-draft verify step);
+        0 = unknown, any tile may be full."""
         cfg, layout, s = self.config.struct(), self.config.page_table_layout.struct(), self.shape
         L.check(self.device.lib.psi_hip_split_kv_tiled_q_map(
             self.device.ctx, ctypes.byref(cfg), ctypes.byref(layout), self.config.q_token_tile_size, _ptr(q),
             _ptr(kv_pages), _nbytes(kv_pages), _ptr(req_slots), _ptr(page_ids), _ptr(flat_token_indices),
             _ptr(q_token_tiles), _ptr(sdpa_map_task_templates), _ptr(scratch.buffer), scratch.bytes,
             page_table_index, s.num_total_tokens, s.num_total_q_token_tiles, s.num_total_sdpa_map_task_templates,
-            num_active_tokens, num_active_q_token_tiles, num_active_kv_splits))
+            num_active_tokens, num_active_q_token_tiles, num_active_kv_splits, max_active_q_tile_tokens))
 
     def invoke_reduce(self, scratch, q_token_tiles, cu_sdpa_partial_outputs, output):
         self.invoke_reduce_bucketed(scratch, q_token_tiles, cu_sdpa_partial_outputs, output,

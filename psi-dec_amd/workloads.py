@@ -232,7 +232,9 @@ class DeviceWorkload:
             self.kernels.invoke_map_bucketed(self.q, self.pages, m.d_req_slots, self.page_ids,
                                              m.d_flat_token_indices, m.d_q_token_tiles, m.d_kv_splits, self.scratch,
                                              self.w.layer, s.num_tokens, s.num_q_token_tiles,
-                                             s.num_sdpa_map_task_templates)
+                                             s.num_sdpa_map_task_templates,
+                                             min(int(np.diff(self.w.cu_tokens).max()),
+                                                 self.variant.q_token_tile_size))
         elif self.balanced:
             self.kernels.invoke_map_balanced(self.q, self.pages, m.d_req_slots, self.page_ids, m.d_kv_splits,
                                              m.d_worker_cu, m.num_workers, self.scratch, self.w.layer, s.num_tokens,

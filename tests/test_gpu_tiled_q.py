@@ -205,3 +205,22 @@ def test_verify_accept_rollback_cycle(psi, oracle, device):
     for b in blocks:
         b.close()
     assert alloc.used() == 0 and used > 0
+
+
+def test_mfma_and_generic_kernels_agree_but_differ_in_rounding(psi, oracle, device):
+    """The gfx950 kernels and the shape-generic kernels on one verify batch: both within tolerance of
+    each other, and not bit-identical (which would mean the generic kernels served both runs)."""
+    wl = importlib_workloads(psi)
+    w = wl.make_workload(91, [900, 2048, 77, 300], 24, 4, 256, psi.Dtype.Bfloat16, 16, q_lens=4)
+    fast = wl.DeviceWorkload(device, w, partition_tokens=512, f32_output=True)
+    fast.step()
+    a = fast.output_f32()
+    device.force_generic(True)
+    try:
+        slow = wl.DeviceWorkload(device, w, partition_tokens=512, f32_output=True)
+        slow.step()
+        b = slow.output_f32()
+    finally:
+        device.force_generic(False)
+    assert np.abs(a - b).max() < 2e-4
+    assert not np.array_equal(a, b)
