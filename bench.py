@@ -41,10 +41,12 @@ def parse_args():
     p.add_argument("--decode-waves", type=int, default=0, help="waves per decode workgroup (0 = automatic)")
     p.add_argument("--balance", action="store_true", help="equal-tile worker plan instead of one workgroup per partition")
     p.add_argument("--kernel-only", action="store_true", help="time only the map kernel (for profiling runs)")
-    p.add_argument("--workload", choices=["decode", "verify"], default="decode",
+    p.add_argument("--workload", choices=["decode", "verify", "prefill"], default="decode",
                    help="decode: one new token per sequence (the headline workload); verify: --q-len tokens per "
                         "sequence through the multi-query kernels (batch 64, contexts 2048-16384 unless overridden)")
     p.add_argument("--q-len", type=int, default=2)
+    p.add_argument("--prefix", type=int, default=4096, help="prefill workload: cached tokens before the chunk")
+    p.add_argument("--chunk", type=int, default=2048, help="prefill workload: new tokens of the one sequence")
     p.add_argument("--calibrate-copy", action="store_true",
                    help="run only the plain copy / read probes of known size (counter calibration, practical ceiling)")
     p.add_argument("--probe-mib", type=int, default=1024)
@@ -154,14 +156,18 @@ def main():
         calibrate_copy(device, args)
         return
 
-    verify = args.workload == "verify"
+    verify = args.workload in ("verify", "prefill")
+    prefill = args.workload == "prefill"
+    if prefill:
+        args.batch, args.q_len = 1, args.chunk
     if verify and args.batch == 32 and args.ctx_lo == 1024 and args.ctx_hi == 8192:
         args.batch, args.ctx_lo, args.ctx_hi = 64, 2048, 16384
     map_kernel = "tiled_q_map" if verify else "split_kv_map"
     arenas = []
     for i in range(max(1, args.arenas)):
         if verify:
-            ctx = wl.config_c2_context_lens(args.seed, args.batch, args.ctx_lo, args.ctx_hi) + args.q_len
+            ctx = ([args.prefix + args.chunk] if prefill else
+                   wl.config_c2_context_lens(args.seed, args.batch, args.ctx_lo, args.ctx_hi) + args.q_len)
             w = wl.make_workload(args.seed, ctx, 24, 4, 256, psi.Dtype.Bfloat16, 16, q_lens=args.q_len,
                                  host_pages=False, shuffle_pages=not args.identity_pages)
         else:
@@ -239,6 +245,13 @@ def main():
             "launches_timed": int(map_launches),
         },
     }
+    if prefill:
+        # multi-query chunk: priced against the matrix cores as well (4 * Hq * D flops per visible (query, key) pair)
+        pairs = sum(args.prefix + i + 1 for i in range(args.chunk))
+        flops = 4 * w.num_q_heads * w.head_dim * pairs
+        result["config"]["workload"] = f"prefill_chunk{args.chunk}_on_prefix{args.prefix}_24q4kv_d256_bf16_p16_part{args.partition}"
+        result["mfma"] = {"bound": "mfma", "flops_per_launch": flops, "achieved": flops / map_avg_s / 1e12,
+                          "peak": 2500.0, "unit": "TFLOP/s", "frac": flops / map_avg_s / 1e12 / 2500.0}
     if not args.no_cpu_baseline:
         result["cpu_baseline"] = cpu_baseline(psi, wl, w, arenas[0], args.cpu_seconds)
     print(json.dumps(result))

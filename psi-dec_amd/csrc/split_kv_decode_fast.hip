@@ -38,6 +38,43 @@ __global__ __launch_bounds__(256) void split_kv_reduce_fast(ReduceArgs a) {
     for (int e = 0; e < kPerLane; ++e) store_from_f32<Tag>(a.output, out_index + e, value[e] * inv);
 }
 
+// The same combine for Q-token tiles: one wave per (tile, token in tile, q_head); the tile's partial
+// rows are cu_kv_splits[tile] .. cu_kv_splits[tile + 1].
+template <typename Tag, int D>
+__global__ __launch_bounds__(256) void split_kv_reduce_tiled_fast(ReduceArgs a) {
+    constexpr int kPerLane = D / 64;
+    const uint32_t lane = threadIdx.x & 63;
+    const uint64_t id = (uint64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
+    const uint32_t rows = a.rows_per_split_head;
+    const uint32_t q_head = (uint32_t)(id % a.hq);
+    const uint32_t tile_row = (uint32_t)((id / a.hq) % rows);
+    const uint64_t tile = id / ((uint64_t)a.hq * rows);
+    if (tile >= a.num_active_q_token_tiles) return;
+    const uint32_t flat_begin = a.q_token_tiles[tile * 2], flat_end = a.q_token_tiles[tile * 2 + 1];
+    const uint32_t token = flat_begin + tile_row;
+    if (token >= flat_end) return;
+    const uint32_t begin = a.cu_kv_splits[tile], end = a.cu_kv_splits[tile + 1];
+    float global_max = -INFINITY;
+    for (uint32_t p = begin; p < end; ++p)
+        global_max = fmaxf(global_max, a.part_max[((uint64_t)p * a.hq + q_head) * rows + tile_row]);
+    float weight_sum = 0.0f, value[kPerLane];
+#pragma unroll
+    for (int e = 0; e < kPerLane; ++e) value[e] = 0.0f;
+    for (uint32_t p = begin; p < end; ++p) {
+        const uint64_t row = ((uint64_t)p * a.hq + q_head) * rows + tile_row;
+        const float m = a.part_max[row];
+        const float w = m > -INFINITY ? exp2f(m - global_max) : 0.0f;
+        weight_sum = fmaf(w, a.part_sum[row], weight_sum);
+        const float* src = a.part_acc + row * D + lane * kPerLane;
+#pragma unroll
+        for (int e = 0; e < kPerLane; ++e) value[e] = fmaf(w, src[e], value[e]);
+    }
+    const float inv = weight_sum > 0.0f ? 1.0f / weight_sum : 0.0f;
+    const uint64_t out_index = ((uint64_t)token * a.hq + q_head) * D + lane * kPerLane;
+#pragma unroll
+    for (int e = 0; e < kPerLane; ++e) store_from_f32<Tag>(a.output, out_index + e, value[e] * inv);
+}
+
 int launch_decode_map_fast(psi_hip_ctx* ctx, const Geometry& g, const MapArgs& a) {
     if (ctx->force_generic) return PSI_HIP_ERR_UNSUPPORTED;
     if (ctx->decode_valu_qk) {
@@ -58,12 +95,20 @@ int launch_decode_map_fast(psi_hip_ctx* ctx, const Geometry& g, const MapArgs& a
 int launch_reduce_fast(psi_hip_ctx* ctx, const Geometry& g, const ReduceArgs& a) {
     if (ctx->force_generic) return PSI_HIP_ERR_UNSUPPORTED;
     if (g.d != 256 && g.d != 128) return PSI_HIP_ERR_UNSUPPORTED;
-    const uint64_t rows = (uint64_t)a.num_active_tokens * g.hq;
+    const bool tiled = a.q_token_tiles != nullptr;
+    const uint64_t rows = tiled ? (uint64_t)a.num_active_q_token_tiles * a.rows_per_split_head * g.hq
+                                : (uint64_t)a.num_active_tokens * g.hq;
+    if ((rows + 3) / 4 > 0x7fffffffull) return PSI_HIP_ERR_UNSUPPORTED;
     const dim3 grid((uint32_t)((rows + 3) / 4)), block(256);
-#define PSI_REDUCE(TAG)                                                                                       \
-    do {                                                                                                      \
-        if (g.d == 256) hipLaunchKernelGGL((split_kv_reduce_fast<TAG, 256>), grid, block, 0, ctx->stream, a); \
-        else hipLaunchKernelGGL((split_kv_reduce_fast<TAG, 128>), grid, block, 0, ctx->stream, a);            \
+#define PSI_REDUCE(TAG)                                                                                             \
+    do {                                                                                                            \
+        if (tiled) {                                                                                                \
+            if (g.d == 256) hipLaunchKernelGGL((split_kv_reduce_tiled_fast<TAG, 256>), grid, block, 0, ctx->stream, a); \
+            else hipLaunchKernelGGL((split_kv_reduce_tiled_fast<TAG, 128>), grid, block, 0, ctx->stream, a);       \
+        } else {                                                                                                    \
+            if (g.d == 256) hipLaunchKernelGGL((split_kv_reduce_fast<TAG, 256>), grid, block, 0, ctx->stream, a);  \
+            else hipLaunchKernelGGL((split_kv_reduce_fast<TAG, 128>), grid, block, 0, ctx->stream, a);             \
+        }                                                                                                           \
     } while (0)
     if (a.out_dtype == PSI_HIP_F32) PSI_REDUCE(F32Tag);
     else if (a.out_dtype == PSI_HIP_BF16) PSI_REDUCE(BF16Tag);

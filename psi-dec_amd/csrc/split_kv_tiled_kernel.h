@@ -5,10 +5,12 @@
 // Work decomposition
 //   one workgroup (4 waves) = one (kv_split row, kv_head).  The row names a request-local tile of
 //   up to 8 query tokens; with the G query heads that share the KV head this gives up to 8*G
-//   query columns, column c = token_in_tile * G + head, handled as NB blocks of 16 columns.  Every
-//   K and V byte of the split is therefore fetched once for all of them.  One wave = every 4th
-//   16-token KV tile, with its own online-softmax state per column; wave states merge through LDS
-//   at the end.
+//   query columns, column c = token_in_tile * G + head, handled as blocks of 16 columns.  Every
+//   K and V byte of the split is therefore fetched from HBM once for all of them.  One wave =
+//   every 4th 16-token KV tile for NB column blocks, with its own online-softmax state per column;
+//   wave states merge through LDS at the end.  Up to 32 columns fit one wave's registers (NB <= 2);
+//   wider tiles use a second group of four waves for columns 32..63 (CG = 2), which walks the same
+//   KV tiles a moment later and finds them in cache.
 //
 // Per 16-token KV tile and wave
 //   QK^T  S[token][column] on v_mfma_f32_16x16x32: A = the K tile straight from the page (lane =
@@ -79,39 +81,41 @@ struct ProbOperand<F16Tag> {
     }
 };
 
-constexpr int kTiledWaves = 4;
+constexpr int kTiledTileWaves = 4;  // waves that share the KV tiles of a split among them
 
-template <int NB>
+template <int NB, int CG>
 struct TiledOccupancy {
-    static constexpr int value = NB == 1 ? 3 : (NB == 2 ? 2 : 1);
+    static constexpr int value = CG == 2 ? 2 : (NB == 1 ? 3 : 2);
 };
 
-template <typename Tag, int D, int NB>
-__global__ __launch_bounds__(64 * kTiledWaves, TiledOccupancy<NB>::value) void split_kv_tiled_map(
+// NB: column blocks per wave (1 or 2); CG: column groups (1 or 2), each a set of four waves.
+template <typename Tag, int D, int NB, int CG>
+__global__ __launch_bounds__(64 * kTiledTileWaves * CG, (TiledOccupancy<NB, CG>::value)) void split_kv_tiled_map(
     MapArgs a, const uint32_t* __restrict__ page_ids, const uint32_t* __restrict__ kv_splits,
     const uint32_t* __restrict__ req_slots, const uint16_t* __restrict__ q, const uint16_t* __restrict__ pages,
     const uint32_t* __restrict__ q_token_tiles, const uint32_t* __restrict__ flat_token_indices) {
-    constexpr int kWaves = kTiledWaves;
+    constexpr int kTileWaves = kTiledTileWaves;
+    constexpr int kWaves = kTileWaves * CG;
     constexpr int kVLanesPerToken = D / 8;                  // 32 (D=256) or 16 (D=128)
     constexpr int kVTokensPerLoad = 64 / kVLanesPerToken;   // 2 or 4
     constexpr int kVLoads = kTileTokens / kVTokensPerLoad;  // 8 or 4
     constexpr int kKSteps = D / 32;                         // MFMA k-steps of QK^T
     constexpr int kDimBlocks = D / 16;                      // 16-dim output blocks of PV
     constexpr int kVStride = D + 8;                         // elements per token row of the V buffer (bank spread)
-    constexpr int kCols = NB * 16;
+    constexpr int kCols = CG * NB * 16;
     constexpr int kMergeStride = D + 4;                     // floats per column row of the merge buffer
 
     // LDS: the main loop's V buffers and Q operands share their bytes with the epilogue's merge buffer.
     constexpr int kVBytes = kWaves * kTileTokens * kVStride * 2;
-    constexpr int kQBytes = NB * kKSteps * 64 * 16;
+    constexpr int kQBytes = CG * NB * kKSteps * 64 * 16;
     constexpr int kMergeBytes = kCols * kMergeStride * 4;
     constexpr int kUnionBytes = (kVBytes + kQBytes) > kMergeBytes ? (kVBytes + kQBytes) : kMergeBytes;
     __shared__ __attribute__((aligned(16))) unsigned char lds_union[kUnionBytes];
-    __shared__ float wave_max_lds[kWaves][kCols];
+    __shared__ float wave_max_lds[kTileWaves][kCols];
     __shared__ float col_max_lds[kCols];
     __shared__ float col_sum_lds[kCols];
     uint16_t* v_lds = reinterpret_cast<uint16_t*>(lds_union);
-    uint4* qb_lds = reinterpret_cast<uint4*>(lds_union + kVBytes);  // [NB][kKSteps][64]
+    uint4* qb_lds = reinterpret_cast<uint4*>(lds_union + kVBytes);  // [CG * NB][kKSteps][64]
     float* merge = reinterpret_cast<float*>(lds_union);
 
     const uint32_t G = a.group;
@@ -120,6 +124,8 @@ __global__ __launch_bounds__(64 * kTiledWaves, TiledOccupancy<NB>::value) void s
     const uint32_t tid = threadIdx.x;
     const uint32_t lane = tid & 63;
     const uint32_t wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const uint32_t tile_wave = wave % kTileWaves;       // which KV tiles this wave takes
+    const uint32_t col_base = (wave / kTileWaves) * NB;  // first column block of this wave
     const uint32_t mt = lane & 15, mc = lane >> 4;
     const uint32_t vsub = lane / kVLanesPerToken, vdl = lane % kVLanesPerToken;
 
@@ -133,20 +139,23 @@ __global__ __launch_bounds__(64 * kTiledWaves, TiledOccupancy<NB>::value) void s
     const uint32_t tile_tokens = flat_end - flat_begin;
     const uint32_t ncols = tile_tokens * G;
     if (ncols > (uint32_t)kCols) return;  // the launcher sizes NB from the largest tile; never taken
-    const uint32_t nb_active = (ncols + 15) / 16;
+    const uint32_t nb_total = (ncols + 15) / 16;
+    // column blocks this wave works on: col_base + [0, nb_active)
+    const uint32_t nb_active = nb_total > col_base ? min(nb_total - col_base, (uint32_t)NB) : 0u;
     const uint32_t req_slot = req_slots[flat_begin];
 
-    // Column of this lane in block nb: c = 16*nb + mt; its query token, head and visible key range.
+    // Column of this lane in its block nb: c = 16*(col_base + nb) + mt; its query token, head and
+    // visible key range.
     uint32_t lim[NB];  // keys [kv_begin, lim) are visible to the column (0: column unused)
 #pragma unroll
     for (int nb = 0; nb < NB; ++nb) {
-        const uint32_t c = nb * 16 + mt;
+        const uint32_t c = (col_base + nb) * 16 + mt;
         lim[nb] = 0;
         if (c < ncols) lim[nb] = min(kv_end, flat_token_indices[flat_begin + c / G] + 1);
     }
 
     // Query columns as MFMA B operands [nb][k-step][lane]; unused columns are zero.
-    for (uint32_t nb = wave; nb < nb_active; nb += kWaves) {
+    for (uint32_t nb = wave; nb < nb_total; nb += kWaves) {
         const uint32_t c = nb * 16 + mt;
         const bool used = c < ncols;
         const uint32_t cc = used ? c : 0;
@@ -214,7 +223,7 @@ __global__ __launch_bounds__(64 * kTiledWaves, TiledOccupancy<NB>::value) void s
             if ((uint32_t)nb < nb_active) {
 #pragma unroll
                 for (int i = 0; i < kKSteps; ++i)
-                    s[nb] = mfma_16x16x32<Tag>(kreg[i], qb_lds[(nb * kKSteps + i) * 64 + lane], s[nb]);
+                    s[nb] = mfma_16x16x32<Tag>(kreg[i], qb_lds[((col_base + nb) * kKSteps + i) * 64 + lane], s[nb]);
             }
         }
         __builtin_amdgcn_sched_barrier(0);
@@ -308,18 +317,18 @@ __global__ __launch_bounds__(64 * kTiledWaves, TiledOccupancy<NB>::value) void s
         __builtin_amdgcn_sched_barrier(0);
     };
 
-    uint32_t tile = tile_begin + wave;
-    if (tile < tile_end) {
+    uint32_t tile = tile_begin + tile_wave;
+    if (tile < tile_end && nb_active != 0) {
         {
             const uint32_t pid = load_page_id(tile);
             issue_k(tile, pid);
             issue_v(tile, pid);
         }
-        uint32_t pid_next = load_page_id(tile + kWaves);
+        uint32_t pid_next = load_page_id(tile + kTileWaves);
         auto is_partial = [&](uint32_t t) { return t * kTileTokens < kv_begin || (t + 1) * kTileTokens > kv_end; };
-        while (tile + kWaves < tile_end) {
-            const uint32_t next = tile + kWaves;
-            const uint32_t pid_after = load_page_id(next + kWaves);
+        while (tile + kTileWaves < tile_end) {
+            const uint32_t next = tile + kTileWaves;
+            const uint32_t pid_after = load_page_id(next + kTileWaves);
             process_tile(tile, is_partial(tile), std::true_type(), next, pid_next);
             pid_next = pid_after;
             tile = next;
@@ -327,24 +336,24 @@ __global__ __launch_bounds__(64 * kTiledWaves, TiledOccupancy<NB>::value) void s
         process_tile(tile, is_partial(tile), std::false_type(), 0u, 0u);
     }
 
-    // ---- merge the four wave states.  Column statistics live in the S layout (lane <-> column mt),
-    // the accumulators in the MFMA output layout (lane <-> columns 4*mc + r, dim mt).
+    // ---- merge the four wave states of each column group.  Column statistics live in the S layout
+    // (lane <-> column mt), the accumulators in the MFMA output layout (lane <-> columns 4*mc + r, dim mt).
 #pragma unroll
     for (int nb = 0; nb < NB; ++nb) {
         lane_sum[nb] += __shfl_xor(lane_sum[nb], 16, 64);
         lane_sum[nb] += __shfl_xor(lane_sum[nb], 32, 64);
-        if (mc == 0) wave_max_lds[wave][nb * 16 + mt] = run_max[nb];
+        if (mc == 0) wave_max_lds[tile_wave][(col_base + nb) * 16 + mt] = run_max[nb];
     }
     __syncthreads();  // every wave has left the main loop: the V / Q bytes may now be reused
 #pragma unroll
     for (int nb = 0; nb < NB; ++nb) {
-        const uint32_t c = nb * 16 + mt;
+        const uint32_t c = (col_base + nb) * 16 + mt;
         float gm = wave_max_lds[0][c];
 #pragma unroll
-        for (int w = 1; w < kWaves; ++w) gm = fmaxf(gm, wave_max_lds[w][c]);
+        for (int w = 1; w < kTileWaves; ++w) gm = fmaxf(gm, wave_max_lds[w][c]);
         const float f = run_max[nb] > -INFINITY ? __builtin_amdgcn_exp2f(run_max[nb] - gm) : 0.0f;
         lane_sum[nb] *= f;
-        if (wave == 0 && mc == 0) col_max_lds[c] = gm;
+        if (tile_wave == 0 && mc == 0) col_max_lds[c] = gm;
         float fr[4];
 #pragma unroll
         for (int r = 0; r < 4; ++r) fr[r] = __shfl(f, mc * 4 + r, 64);
@@ -353,20 +362,20 @@ __global__ __launch_bounds__(64 * kTiledWaves, TiledOccupancy<NB>::value) void s
 #pragma unroll
             for (int r = 0; r < 4; ++r) o[nb][db][r] *= fr[r];
     }
-    for (uint32_t w = 0; w < (uint32_t)kWaves; ++w) {
-        if (wave == w) {
+    for (uint32_t w = 0; w < (uint32_t)kTileWaves; ++w) {
+        if (tile_wave == w) {
 #pragma unroll
             for (int nb = 0; nb < NB; ++nb) {
                 if ((uint32_t)nb < nb_active) {
                     if (mc == 0) {
-                        const uint32_t c = nb * 16 + mt;
+                        const uint32_t c = (col_base + nb) * 16 + mt;
                         col_sum_lds[c] = (w == 0 ? 0.0f : col_sum_lds[c]) + lane_sum[nb];
                     }
 #pragma unroll
                     for (int db = 0; db < kDimBlocks; ++db)
 #pragma unroll
                         for (int r = 0; r < 4; ++r) {
-                            float* dst = merge + (nb * 16 + mc * 4 + r) * kMergeStride + db * 16 + mt;
+                            float* dst = merge + ((col_base + nb) * 16 + mc * 4 + r) * kMergeStride + db * 16 + mt;
                             *dst = (w == 0 ? 0.0f : *dst) + o[nb][db][r];
                         }
                 }
@@ -396,23 +405,18 @@ inline int tiled_column_blocks(uint32_t max_tile_tokens, uint32_t group) { retur
 template <typename Tag, int D>
 inline int launch_tiled_map_typed(psi_hip_ctx* ctx, const Geometry& g, const MapArgs& a, uint32_t max_tile_tokens) {
     const int nb = tiled_column_blocks(max_tile_tokens, g.group);
-    const dim3 grid(a.num_total_kv_splits * g.hkv), block(64 * kTiledWaves);
+    const dim3 grid(a.num_total_kv_splits * g.hkv);
     const uint16_t* q = reinterpret_cast<const uint16_t*>(a.q);
     const uint16_t* pages = reinterpret_cast<const uint16_t*>(a.kv_pages);
-#define PSI_TILED_CASE(NB)                                                                                         \
-    case NB:                                                                                                        \
-        hipLaunchKernelGGL((split_kv_tiled_map<Tag, D, NB>), grid, block, 0, ctx->stream, a, a.walk.page_ids,       \
-                           a.kv_splits, a.req_slots, q, pages, a.q_token_tiles, a.flat_token_indices);              \
-        return PSI_HIP_OK;
-    switch (nb) {
-        PSI_TILED_CASE(1)
-        PSI_TILED_CASE(2)
-        PSI_TILED_CASE(3)
-        PSI_TILED_CASE(4)
-        default:
-            return PSI_HIP_ERR_UNSUPPORTED;
-    }
-#undef PSI_TILED_CASE
+#define PSI_TILED_LAUNCH(NB, CG)                                                                                      \
+    hipLaunchKernelGGL((split_kv_tiled_map<Tag, D, NB, CG>), grid, dim3(64 * kTiledTileWaves * CG), 0, ctx->stream, a, \
+                       a.walk.page_ids, a.kv_splits, a.req_slots, q, pages, a.q_token_tiles, a.flat_token_indices)
+    if (nb == 1) PSI_TILED_LAUNCH(1, 1);
+    else if (nb == 2) PSI_TILED_LAUNCH(2, 1);
+    else if (nb <= 4) PSI_TILED_LAUNCH(2, 2);
+    else return PSI_HIP_ERR_UNSUPPORTED;
+#undef PSI_TILED_LAUNCH
+    return PSI_HIP_OK;
 }
 
 }  // namespace psi

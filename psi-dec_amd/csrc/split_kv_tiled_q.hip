@@ -144,7 +144,7 @@ extern "C" int psi_hip_split_kv_tiled_q_reduce(psi_hip_ctx* ctx, const psi_hip_g
     a.num_active_q_token_tiles = num_active_q_token_tiles;
 
     LaunchScope scope(ctx, "tiled_q_reduce");
-    launch_reduce_generic(ctx, g, a, num_active_q_token_tiles);
+    if (launch_reduce_fast(ctx, g, a) == PSI_HIP_ERR_UNSUPPORTED) launch_reduce_generic(ctx, g, a, num_active_q_token_tiles);
     PSI_HIP_CHECK(hipGetLastError());
     return PSI_HIP_OK;
 }
