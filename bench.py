@@ -54,19 +54,23 @@ def parse_args():
 
 
 def read_profile_traffic(workload_key):
-    """HBM bytes per map launch measured with rocprofv3 --pmc (FETCH_SIZE + WRITE_SIZE), if the
-    committed summary covers this workload."""
-    path = os.path.join(ROOT, "profiles", "split_kv_decode_map_c2_pmc.txt")
+    """HBM bytes per launch of the dominant kernel measured with rocprofv3 --pmc (FETCH_SIZE +
+    WRITE_SIZE, scaled by the copy calibration), if a committed summary covers this workload."""
+    folder = os.path.join(ROOT, "profiles")
     try:
-        with open(path) as f:
-            text = f.read()
+        names = sorted(os.listdir(folder))
     except OSError:
         return None
-    if f"workload={workload_key}" not in text:
-        return None
-    for line in text.splitlines():
-        if line.startswith("traffic_bytes_per_launch="):
-            return float(line.split("=", 1)[1])
+    for name in names:
+        if not name.endswith(".txt"):
+            continue
+        with open(os.path.join(folder, name)) as f:
+            text = f.read()
+        if f"workload={workload_key}" not in text:
+            continue
+        for line in text.splitlines():
+            if line.startswith("traffic_bytes_per_launch="):
+                return float(line.split("=", 1)[1])
     return None
 
 

@@ -9,28 +9,45 @@ int launch_decode_map_bf16_d128(psi_hip_ctx* ctx, const Geometry& g, const MapAr
 int launch_decode_map_f16_d256(psi_hip_ctx* ctx, const Geometry& g, const MapArgs& a);
 int launch_decode_map_f16_d128(psi_hip_ctx* ctx, const Geometry& g, const MapArgs& a);
 
-// Log-sum-exp combine: one wave per (token, q_head), lanes over head_dim.
+// Log-sum-exp combine: one wave per (token, q_head), lanes over head_dim.  The row maxima are
+// fetched lane-parallel first; the accumulator rows are then read four at a time so that a wave
+// keeps several 1 KiB reads in flight instead of one.
 template <typename Tag, int D>
 __global__ __launch_bounds__(256) void split_kv_reduce_fast(ReduceArgs a) {
     constexpr int kPerLane = D / 64;  // 4 or 2
+    constexpr int kUnroll = 4;
     const uint32_t lane = threadIdx.x & 63;
     const uint64_t row_out = (uint64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
     if (row_out >= (uint64_t)a.num_active_tokens * a.hq) return;
     const uint32_t token = (uint32_t)(row_out / a.hq), q_head = (uint32_t)(row_out % a.hq);
     const uint32_t begin = a.cu_kv_splits[token], end = a.cu_kv_splits[token + 1];
     float global_max = -INFINITY;
-    for (uint32_t p = begin; p < end; ++p) global_max = fmaxf(global_max, a.part_max[(uint64_t)p * a.hq + q_head]);
+    for (uint32_t p = begin + lane; p < end; p += 64)
+        global_max = fmaxf(global_max, a.part_max[(uint64_t)p * a.hq + q_head]);
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) global_max = fmaxf(global_max, __shfl_xor(global_max, off, 64));
     float weight_sum = 0.0f, value[kPerLane];
 #pragma unroll
     for (int e = 0; e < kPerLane; ++e) value[e] = 0.0f;
-    for (uint32_t p = begin; p < end; ++p) {
-        const uint64_t row = (uint64_t)p * a.hq + q_head;
-        const float m = a.part_max[row];
-        const float w = m > -INFINITY ? exp2f(m - global_max) : 0.0f;
-        weight_sum = fmaf(w, a.part_sum[row], weight_sum);
-        const float* src = a.part_acc + row * D + lane * kPerLane;
+    for (uint32_t p0 = begin; p0 < end; p0 += kUnroll) {
+        float w[kUnroll], sums[kUnroll], part[kUnroll][kPerLane];
 #pragma unroll
-        for (int e = 0; e < kPerLane; ++e) value[e] = fmaf(w, src[e], value[e]);
+        for (int u = 0; u < kUnroll; ++u) {
+            const bool live = p0 + u < end;
+            const uint64_t row = (uint64_t)(live ? p0 + u : begin) * a.hq + q_head;
+            const float m = a.part_max[row];
+            sums[u] = a.part_sum[row];
+            w[u] = live && m > -INFINITY ? exp2f(m - global_max) : 0.0f;
+            const float* src = a.part_acc + row * D + lane * kPerLane;
+#pragma unroll
+            for (int e = 0; e < kPerLane; ++e) part[u][e] = src[e];
+        }
+#pragma unroll
+        for (int u = 0; u < kUnroll; ++u) {
+            weight_sum = fmaf(w[u], sums[u], weight_sum);
+#pragma unroll
+            for (int e = 0; e < kPerLane; ++e) value[e] = fmaf(w[u], part[u][e], value[e]);
+        }
     }
     const float inv = weight_sum > 0.0f ? 1.0f / weight_sum : 0.0f;
     const uint64_t out_index = row_out * D + lane * kPerLane;
@@ -54,20 +71,34 @@ __global__ __launch_bounds__(256) void split_kv_reduce_tiled_fast(ReduceArgs a) 
     const uint32_t token = flat_begin + tile_row;
     if (token >= flat_end) return;
     const uint32_t begin = a.cu_kv_splits[tile], end = a.cu_kv_splits[tile + 1];
+    constexpr int kUnroll = 4;
     float global_max = -INFINITY;
-    for (uint32_t p = begin; p < end; ++p)
+    for (uint32_t p = begin + lane; p < end; p += 64)
         global_max = fmaxf(global_max, a.part_max[((uint64_t)p * a.hq + q_head) * rows + tile_row]);
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) global_max = fmaxf(global_max, __shfl_xor(global_max, off, 64));
     float weight_sum = 0.0f, value[kPerLane];
 #pragma unroll
     for (int e = 0; e < kPerLane; ++e) value[e] = 0.0f;
-    for (uint32_t p = begin; p < end; ++p) {
-        const uint64_t row = ((uint64_t)p * a.hq + q_head) * rows + tile_row;
-        const float m = a.part_max[row];
-        const float w = m > -INFINITY ? exp2f(m - global_max) : 0.0f;
-        weight_sum = fmaf(w, a.part_sum[row], weight_sum);
-        const float* src = a.part_acc + row * D + lane * kPerLane;
+    for (uint32_t p0 = begin; p0 < end; p0 += kUnroll) {
+        float w[kUnroll], sums[kUnroll], part[kUnroll][kPerLane];
 #pragma unroll
-        for (int e = 0; e < kPerLane; ++e) value[e] = fmaf(w, src[e], value[e]);
+        for (int u = 0; u < kUnroll; ++u) {
+            const bool live = p0 + u < end;
+            const uint64_t row = ((uint64_t)(live ? p0 + u : begin) * a.hq + q_head) * rows + tile_row;
+            const float m = a.part_max[row];
+            sums[u] = a.part_sum[row];
+            w[u] = live && m > -INFINITY ? exp2f(m - global_max) : 0.0f;
+            const float* src = a.part_acc + row * D + lane * kPerLane;
+#pragma unroll
+            for (int e = 0; e < kPerLane; ++e) part[u][e] = src[e];
+        }
+#pragma unroll
+        for (int u = 0; u < kUnroll; ++u) {
+            weight_sum = fmaf(w[u], sums[u], weight_sum);
+#pragma unroll
+            for (int e = 0; e < kPerLane; ++e) value[e] = fmaf(w[u], part[u][e], value[e]);
+        }
     }
     const float inv = weight_sum > 0.0f ? 1.0f / weight_sum : 0.0f;
     const uint64_t out_index = ((uint64_t)token * a.hq + q_head) * D + lane * kPerLane;
