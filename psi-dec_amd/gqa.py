@@ -75,6 +75,11 @@ class Device:
     def sync(self):
         L.check(self.lib.psi_hip_sync(self.ctx))
 
+    def use_stream(self, stream):
+        """Launch on another torch stream from now on (e.g. the stream a graph is captured on)."""
+        self.stream = stream
+        L.check(self.lib.psi_hip_ctx_set_stream(self.ctx, ctypes.c_void_p(stream.cuda_stream)))
+
     def set_timing(self, enabled: bool):
         L.check(self.lib.psi_hip_ctx_set_timing(self.ctx, int(enabled)))
 
