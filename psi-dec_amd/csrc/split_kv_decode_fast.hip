@@ -109,12 +109,13 @@ __global__ __launch_bounds__(256) void split_kv_reduce_tiled_fast(ReduceArgs a) 
 int launch_decode_map_fast(psi_hip_ctx* ctx, const Geometry& g, const MapArgs& a) {
     if (ctx->force_generic) return PSI_HIP_ERR_UNSUPPORTED;
     if (ctx->decode_valu_qk) {
-        if (a.worker_cu != nullptr) return PSI_HIP_ERR_UNSUPPORTED;  // the comparison variant is row-per-workgroup
+        // the comparison variant is row-per-workgroup and needs a tile inside one page
+        if (a.worker_cu != nullptr || g.tokens_per_page < 16) return PSI_HIP_ERR_UNSUPPORTED;
         return launch_decode_map_valu(ctx, g, a);
     }
     const bool two_byte = g.dtype == PSI_HIP_BF16 || g.dtype == PSI_HIP_F16;
     const uint32_t p = g.tokens_per_page;
-    const bool page_ok = p >= 16 && (p & (p - 1)) == 0;
+    const bool page_ok = p >= 8 && (p & (p - 1)) == 0;
     const bool aligned = reinterpret_cast<uintptr_t>(a.q) % 16 == 0 && reinterpret_cast<uintptr_t>(a.kv_pages) % 16 == 0;
     if (!two_byte || !page_ok || !aligned || g.group > 8 || (g.d != 256 && g.d != 128)) return PSI_HIP_ERR_UNSUPPORTED;
     if ((uint64_t)a.num_total_kv_splits * g.hkv > 0x7fffffffull) return PSI_HIP_ERR_UNSUPPORTED;

@@ -1,5 +1,5 @@
 // gfx950 split-KV grouped-query decode map for 2-byte K/V (bf16 / f16),
-// head_dim 128 or 256, pages of 16*k tokens.
+// head_dim 128 or 256, pages of 8 or 16*2^k tokens.
 //
 // Work decomposition
 //   one workgroup (W = 1, 2 or 4 waves) = one (kv_split, kv_head); it serves all G query heads of
@@ -73,7 +73,13 @@ __device__ __forceinline__ void wave_lds_fence() { asm volatile("s_waitcnt lgkmc
 
 constexpr int kTileTokens = 16;
 
-template <typename Tag, int D, int G, int kWaves>
+// Page IDs behind one 16-token tile: one page when a page holds at least 16 tokens, two when it
+// holds 8 (tokens 0..7 of the tile in `a`, 8..15 in `b`).
+struct TilePages {
+    uint32_t a, b;
+};
+
+template <typename Tag, int D, int G, int kWaves, bool kHalfPage>
 __global__ __launch_bounds__(64 * kWaves, PSI_DECODE_WAVES_PER_SIMD) void split_kv_decode_map(
     MapArgs a, const uint32_t* __restrict__ page_ids, const uint32_t* __restrict__ kv_splits,
     const uint32_t* __restrict__ req_slots, const uint16_t* __restrict__ q, const uint16_t* __restrict__ pages,
@@ -153,13 +159,19 @@ __global__ __launch_bounds__(64 * kWaves, PSI_DECODE_WAVES_PER_SIMD) void split_
 #pragma unroll
         for (int e = 0; e < 8; ++e) acc[h][e] = 0.0f;
 
-    auto load_page_id = [&](uint32_t tile) -> uint32_t {
-        return tile < tile_end ? table_row[(tile * kTileTokens) >> log2p] : 0u;
+    const uint32_t last_page = (kv_end - 1) >> log2p;
+    auto load_page_id = [&](uint32_t tile) -> TilePages {
+        TilePages p{0u, 0u};
+        if (tile < tile_end) {
+            const uint32_t first = (tile * kTileTokens) >> log2p;
+            p.a = table_row[first];
+            if (kHalfPage) p.b = table_row[min(first + 1, last_page)];
+        }
+        return p;
     };
-    auto tile_k_base = [&](uint32_t tile, uint32_t page_id) -> const uint16_t* {
-        const uint32_t in_page = (tile * kTileTokens) & page_mask;
-        return pages + (uint64_t)page_id * a.walk.page_elems +
-               ((uint64_t)kv_head * a.walk.tokens_per_page + in_page) * D;
+    // K line 0 of (page, kv_head); the V lines follow v_region elements later.
+    auto head_base = [&](uint32_t page_id) -> const uint16_t* {
+        return pages + (uint64_t)page_id * a.walk.page_elems + (uint64_t)kv_head * a.walk.tokens_per_page * D;
     };
 
     // One K and one V register buffer per wave.  A buffer entry is re-requested for the next tile
@@ -167,13 +179,27 @@ __global__ __launch_bounds__(64 * kWaves, PSI_DECODE_WAVES_PER_SIMD) void split_
     // period to land while the wave keeps only 16 KiB of tile data in registers.
     uint4 kreg[kKSteps];  // lane (t = lane%16, c = lane/16): step i = dims [i*32 + c*8, +8) of token t
     uint4 vreg[kVLoads];  // lane (sub, dl): load j = token j*kVTokensPerLoad + sub, dims [dl*8, +8)
-    auto issue_k = [&](uint32_t tile, uint32_t page_id) {
-        const uint16_t* k_lane = tile_k_base(tile, page_id) + mt * D + mc * 8;
+    auto issue_k = [&](uint32_t tile, TilePages p) {
+        const uint16_t* k_lane;
+        if (kHalfPage)
+            k_lane = head_base(mt < 8 ? p.a : p.b) + (mt & 7) * D + mc * 8;
+        else
+            k_lane = head_base(p.a) + (((tile * kTileTokens) & page_mask) + mt) * D + mc * 8;
 #pragma unroll
         for (int i = 0; i < kKSteps; ++i) kreg[i] = *reinterpret_cast<const uint4*>(k_lane + i * 32);
     };
-    auto v_lane_of = [&](uint32_t tile, uint32_t page_id) -> const uint16_t* {
-        return tile_k_base(tile, page_id) + v_region + vsub * D + vdl * 8;
+    auto issue_v = [&](uint32_t tile, TilePages p) {
+#pragma unroll
+        for (int j = 0; j < kVLoads; ++j) {
+            const uint16_t* v_lane;
+            if (kHalfPage)  // load j covers tokens j*kVTokensPerLoad .. +kVTokensPerLoad-1: one half of the tile
+                v_lane = head_base(j * kVTokensPerLoad < 8 ? p.a : p.b) + v_region +
+                         ((j * kVTokensPerLoad + vsub) & 7) * D + vdl * 8;
+            else
+                v_lane = head_base(p.a) + v_region +
+                         (((tile * kTileTokens) & page_mask) + j * kVTokensPerLoad + vsub) * D + vdl * 8;
+            vreg[j] = *reinterpret_cast<const uint4*>(v_lane);
+        }
     };
 
     float* my_p = p_lds[wave];
@@ -182,7 +208,7 @@ __global__ __launch_bounds__(64 * kWaves, PSI_DECODE_WAVES_PER_SIMD) void split_
     // One 16-token tile.  `partial`: the tile holds tokens outside [kv_begin, kv_end).
     // `has_next`: another tile of this wave follows; its K and V are requested on the way, each
     // into the registers the current tile has just finished with.  Both flags are wave-uniform.
-    auto process_tile = [&](uint32_t tile, bool partial, auto has_next_tag, uint32_t next, uint32_t next_pid)
+    auto process_tile = [&](uint32_t tile, bool partial, auto has_next_tag, uint32_t next, TilePages next_pid)
                             __attribute__((always_inline)) {
         // compile-time flag: the steady-state copy issues its refill loads unconditionally, which
         // keeps the hardware load counter's order exact for the waits that follow
@@ -275,33 +301,27 @@ __global__ __launch_bounds__(64 * kWaves, PSI_DECODE_WAVES_PER_SIMD) void split_
             // keeps later P reads and V unpacks from being hoisted above this point (register budget)
             __builtin_amdgcn_sched_barrier(0);
         }
-        if (has_next) {
-            const uint16_t* v_next = v_lane_of(next, next_pid);
-#pragma unroll
-            for (int j = 0; j < kVLoads; ++j) vreg[j] = *reinterpret_cast<const uint4*>(v_next + j * kVTokensPerLoad * D);
-        }
+        if (has_next) issue_v(next, next_pid);
         __builtin_amdgcn_sched_barrier(0);
     };
 
     uint32_t tile = tile_begin + wave;
     if (tile < tile_end) {
         {
-            const uint32_t pid = load_page_id(tile);
+            const TilePages pid = load_page_id(tile);
             issue_k(tile, pid);
-            const uint16_t* v_lane = v_lane_of(tile, pid);
-#pragma unroll
-            for (int j = 0; j < kVLoads; ++j) vreg[j] = *reinterpret_cast<const uint4*>(v_lane + j * kVTokensPerLoad * D);
+            issue_v(tile, pid);
         }
-        uint32_t pid_next = load_page_id(tile + kWaves);
+        TilePages pid_next = load_page_id(tile + kWaves);
         auto is_partial = [&](uint32_t t) { return t * kTileTokens < kv_begin || (t + 1) * kTileTokens > kv_end; };
         while (tile + kWaves < tile_end) {
             const uint32_t next = tile + kWaves;
-            const uint32_t pid_after = load_page_id(next + kWaves);
+            const TilePages pid_after = load_page_id(next + kWaves);
             process_tile(tile, is_partial(tile), std::true_type(), next, pid_next);
             pid_next = pid_after;
             tile = next;
         }
-        process_tile(tile, is_partial(tile), std::false_type(), 0u, 0u);  // the wave's last tile
+        process_tile(tile, is_partial(tile), std::false_type(), 0u, TilePages{0u, 0u});  // the wave's last tile
     }
 
 #ifdef PSI_DECODE_TIMESTAMPS
@@ -391,15 +411,18 @@ inline void launch_decode_map_w(psi_hip_ctx* ctx, const Geometry& g, const MapAr
     const dim3 grid((a.worker_cu ? a.num_workers : a.num_total_kv_splits) * g.hkv);
     const uint16_t* q = reinterpret_cast<const uint16_t*>(a.q);
     const uint16_t* pages = reinterpret_cast<const uint16_t*>(a.kv_pages);
-    if (waves == 4)
-        hipLaunchKernelGGL((split_kv_decode_map<Tag, D, G, 4>), grid, dim3(256), 0, ctx->stream, a, a.walk.page_ids,
-                           a.kv_splits, a.req_slots, q, pages, a.worker_cu);
+    if (g.tokens_per_page == 8)  // a tile spans two pages; one workgroup width is built for this case
+        hipLaunchKernelGGL((split_kv_decode_map<Tag, D, G, 4, true>), grid, dim3(256), 0, ctx->stream, a,
+                           a.walk.page_ids, a.kv_splits, a.req_slots, q, pages, a.worker_cu);
+    else if (waves == 4)
+        hipLaunchKernelGGL((split_kv_decode_map<Tag, D, G, 4, false>), grid, dim3(256), 0, ctx->stream, a,
+                           a.walk.page_ids, a.kv_splits, a.req_slots, q, pages, a.worker_cu);
     else if (waves == 2)
-        hipLaunchKernelGGL((split_kv_decode_map<Tag, D, G, 2>), grid, dim3(128), 0, ctx->stream, a, a.walk.page_ids,
-                           a.kv_splits, a.req_slots, q, pages, a.worker_cu);
+        hipLaunchKernelGGL((split_kv_decode_map<Tag, D, G, 2, false>), grid, dim3(128), 0, ctx->stream, a,
+                           a.walk.page_ids, a.kv_splits, a.req_slots, q, pages, a.worker_cu);
     else
-        hipLaunchKernelGGL((split_kv_decode_map<Tag, D, G, 1>), grid, dim3(64), 0, ctx->stream, a, a.walk.page_ids,
-                           a.kv_splits, a.req_slots, q, pages, a.worker_cu);
+        hipLaunchKernelGGL((split_kv_decode_map<Tag, D, G, 1, false>), grid, dim3(64), 0, ctx->stream, a,
+                           a.walk.page_ids, a.kv_splits, a.req_slots, q, pages, a.worker_cu);
 }
 
 // One translation unit per (element type, head_dim) instantiates every group size 1..8.

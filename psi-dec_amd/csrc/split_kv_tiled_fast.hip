@@ -13,7 +13,7 @@ int launch_tiled_map_fast(psi_hip_ctx* ctx, const Geometry& g, const MapArgs& a)
     if (ctx->force_generic) return PSI_HIP_ERR_UNSUPPORTED;
     const bool two_byte = g.dtype == PSI_HIP_BF16 || g.dtype == PSI_HIP_F16;
     const uint32_t p = g.tokens_per_page;
-    const bool page_ok = p >= 16 && (p & (p - 1)) == 0;
+    const bool page_ok = p >= 8 && (p & (p - 1)) == 0;
     const bool aligned = reinterpret_cast<uintptr_t>(a.q) % 16 == 0 && reinterpret_cast<uintptr_t>(a.kv_pages) % 16 == 0;
     // partial rows are laid out for 8-token tiles; the kernels hold at most 64 query columns
     if (!two_byte || !page_ok || !aligned || (g.d != 256 && g.d != 128) || a.rows_per_split_head > 8) return PSI_HIP_ERR_UNSUPPORTED;

@@ -1,5 +1,5 @@
 // gfx950 split-KV multi-query map (speculative verify, prefill chunks) for 2-byte K/V (bf16 / f16),
-// head_dim 128 or 256, pages of 16*k tokens.  Semantics of
+// head_dim 128 or 256, pages of 8 or 16*2^k tokens.  Semantics of
 // crates/inference-backend-metal/src/components/metal/gqa_split_kv_tiled_q.metal:49-319.
 //
 // Work decomposition
@@ -89,7 +89,7 @@ struct TiledOccupancy {
 };
 
 // NB: column blocks per wave (1 or 2); CG: column groups (1 or 2), each a set of four waves.
-template <typename Tag, int D, int NB, int CG>
+template <typename Tag, int D, int NB, int CG, bool kHalfPage>
 __global__ __launch_bounds__(64 * kTiledTileWaves * CG, (TiledOccupancy<NB, CG>::value)) void split_kv_tiled_map(
     MapArgs a, const uint32_t* __restrict__ page_ids, const uint32_t* __restrict__ kv_splits,
     const uint32_t* __restrict__ req_slots, const uint16_t* __restrict__ q, const uint16_t* __restrict__ pages,
@@ -187,32 +187,49 @@ __global__ __launch_bounds__(64 * kTiledTileWaves * CG, (TiledOccupancy<NB, CG>:
         for (int db = 0; db < kDimBlocks; ++db) o[nb][db] = f32x4_t{0.0f, 0.0f, 0.0f, 0.0f};
     }
 
-    auto load_page_id = [&](uint32_t tile) -> uint32_t {
-        return tile < tile_end ? table_row[(tile * kTileTokens) >> log2p] : 0u;
+    const uint32_t last_page = (kv_end - 1) >> log2p;
+    auto load_page_id = [&](uint32_t tile) -> TilePages {
+        TilePages p{0u, 0u};
+        if (tile < tile_end) {
+            const uint32_t first = (tile * kTileTokens) >> log2p;
+            p.a = table_row[first];
+            if (kHalfPage) p.b = table_row[min(first + 1, last_page)];
+        }
+        return p;
     };
-    auto tile_k_base = [&](uint32_t tile, uint32_t page_id) -> const uint16_t* {
-        const uint32_t in_page = (tile * kTileTokens) & page_mask;
-        return pages + (uint64_t)page_id * a.walk.page_elems +
-               ((uint64_t)kv_head * a.walk.tokens_per_page + in_page) * D;
+    auto head_base = [&](uint32_t page_id) -> const uint16_t* {
+        return pages + (uint64_t)page_id * a.walk.page_elems + (uint64_t)kv_head * a.walk.tokens_per_page * D;
     };
     uint4 kreg[kKSteps];
     uint4 vreg[kVLoads];
-    auto issue_k = [&](uint32_t tile, uint32_t page_id) {
-        const uint16_t* k_lane = tile_k_base(tile, page_id) + mt * D + mc * 8;
+    auto issue_k = [&](uint32_t tile, TilePages p) {
+        const uint16_t* k_lane;
+        if (kHalfPage)
+            k_lane = head_base(mt < 8 ? p.a : p.b) + (mt & 7) * D + mc * 8;
+        else
+            k_lane = head_base(p.a) + (((tile * kTileTokens) & page_mask) + mt) * D + mc * 8;
 #pragma unroll
         for (int i = 0; i < kKSteps; ++i) kreg[i] = *reinterpret_cast<const uint4*>(k_lane + i * 32);
     };
-    auto issue_v = [&](uint32_t tile, uint32_t page_id) {
-        const uint16_t* v_lane = tile_k_base(tile, page_id) + v_region + vsub * D + vdl * 8;
+    auto issue_v = [&](uint32_t tile, TilePages p) {
 #pragma unroll
-        for (int j = 0; j < kVLoads; ++j) vreg[j] = *reinterpret_cast<const uint4*>(v_lane + j * kVTokensPerLoad * D);
+        for (int j = 0; j < kVLoads; ++j) {
+            const uint16_t* v_lane;
+            if (kHalfPage)
+                v_lane = head_base(j * kVTokensPerLoad < 8 ? p.a : p.b) + v_region +
+                         ((j * kVTokensPerLoad + vsub) & 7) * D + vdl * 8;
+            else
+                v_lane = head_base(p.a) + v_region +
+                         (((tile * kTileTokens) & page_mask) + j * kVTokensPerLoad + vsub) * D + vdl * 8;
+            vreg[j] = *reinterpret_cast<const uint4*>(v_lane);
+        }
     };
 
     uint16_t* my_v = v_lds + wave * kTileTokens * kVStride;
     // B operand of PV for dim block db: 4 consecutive tokens of this lane's token quad, one dim.
     const uint16_t* my_v_read = my_v + (mc * 4) * kVStride + mt;
 
-    auto process_tile = [&](uint32_t tile, bool partial, auto has_next_tag, uint32_t next, uint32_t next_pid)
+    auto process_tile = [&](uint32_t tile, bool partial, auto has_next_tag, uint32_t next, TilePages next_pid)
                             __attribute__((always_inline)) {
         constexpr bool has_next = decltype(has_next_tag)::value;
         // ---- logits S[token][column] on the matrix cores
@@ -320,20 +337,20 @@ __global__ __launch_bounds__(64 * kTiledTileWaves * CG, (TiledOccupancy<NB, CG>:
     uint32_t tile = tile_begin + tile_wave;
     if (tile < tile_end && nb_active != 0) {
         {
-            const uint32_t pid = load_page_id(tile);
+            const TilePages pid = load_page_id(tile);
             issue_k(tile, pid);
             issue_v(tile, pid);
         }
-        uint32_t pid_next = load_page_id(tile + kTileWaves);
+        TilePages pid_next = load_page_id(tile + kTileWaves);
         auto is_partial = [&](uint32_t t) { return t * kTileTokens < kv_begin || (t + 1) * kTileTokens > kv_end; };
         while (tile + kTileWaves < tile_end) {
             const uint32_t next = tile + kTileWaves;
-            const uint32_t pid_after = load_page_id(next + kTileWaves);
+            const TilePages pid_after = load_page_id(next + kTileWaves);
             process_tile(tile, is_partial(tile), std::true_type(), next, pid_next);
             pid_next = pid_after;
             tile = next;
         }
-        process_tile(tile, is_partial(tile), std::false_type(), 0u, 0u);
+        process_tile(tile, is_partial(tile), std::false_type(), 0u, TilePages{0u, 0u});
     }
 
     // ---- merge the four wave states of each column group.  Column statistics live in the S layout
@@ -408,9 +425,17 @@ inline int launch_tiled_map_typed(psi_hip_ctx* ctx, const Geometry& g, const Map
     const dim3 grid(a.num_total_kv_splits * g.hkv);
     const uint16_t* q = reinterpret_cast<const uint16_t*>(a.q);
     const uint16_t* pages = reinterpret_cast<const uint16_t*>(a.kv_pages);
-#define PSI_TILED_LAUNCH(NB, CG)                                                                                      \
-    hipLaunchKernelGGL((split_kv_tiled_map<Tag, D, NB, CG>), grid, dim3(64 * kTiledTileWaves * CG), 0, ctx->stream, a, \
-                       a.walk.page_ids, a.kv_splits, a.req_slots, q, pages, a.q_token_tiles, a.flat_token_indices)
+#define PSI_TILED_LAUNCH(NB, CG)                                                                                       \
+    do {                                                                                                               \
+        if (g.tokens_per_page == 8)                                                                                    \
+            hipLaunchKernelGGL((split_kv_tiled_map<Tag, D, NB, CG, true>), grid, dim3(64 * kTiledTileWaves * CG), 0,    \
+                               ctx->stream, a, a.walk.page_ids, a.kv_splits, a.req_slots, q, pages, a.q_token_tiles,   \
+                               a.flat_token_indices);                                                                  \
+        else                                                                                                           \
+            hipLaunchKernelGGL((split_kv_tiled_map<Tag, D, NB, CG, false>), grid, dim3(64 * kTiledTileWaves * CG), 0,   \
+                               ctx->stream, a, a.walk.page_ids, a.kv_splits, a.req_slots, q, pages, a.q_token_tiles,   \
+                               a.flat_token_indices);                                                                  \
+    } while (0)
     if (nb == 1) PSI_TILED_LAUNCH(1, 1);
     else if (nb == 2) PSI_TILED_LAUNCH(2, 1);
     else if (nb <= 4) PSI_TILED_LAUNCH(2, 2);

@@ -36,6 +36,9 @@ def test_c2_shape_small_batch_bf16(psi, oracle, device, partition):
     ("Bfloat16", 5, 1, 256, 64),
     ("Bfloat16", 6, 2, 256, 16),
     ("Float16", 14, 2, 256, 16),
+    ("Bfloat16", 24, 4, 256, 8),   # 8-token pages: every 16-token tile spans two pages
+    ("Bfloat16", 32, 4, 128, 8),
+    ("Float16", 12, 2, 256, 8),
 ])
 def test_fast_path_geometries(psi, oracle, device, dtype_name, hq, hkv, d, p):
     wl = importlib_workloads(psi)

@@ -42,6 +42,8 @@ def test_prefill_chunk_on_prefix(psi, oracle, device, partition):
     ("Float16", 16, 2, 256, 16, 5),
     ("Bfloat16", 4, 4, 256, 16, 8),
     ("Float32", 4, 2, 64, 4, 3),
+    ("Bfloat16", 24, 4, 256, 8, 8),  # the reference's (256, 8) profile, full tiles
+    ("Float16", 8, 1, 128, 8, 3),
 ])
 def test_tiled_geometries(psi, oracle, device, dtype_name, hq, hkv, d, p, q_len):
     wl = importlib_workloads(psi)
