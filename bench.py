@@ -39,6 +39,8 @@ def parse_args():
     p.add_argument("--no-cpu-baseline", action="store_true")
     p.add_argument("--identity-pages", action="store_true", help="unshuffled page pool (diagnostic)")
     p.add_argument("--decode-waves", type=int, default=0, help="waves per decode workgroup (0 = automatic)")
+    p.add_argument("--plan-order", action="store_true",
+                   help="dispatch the split rows in plan order instead of longest first")
     p.add_argument("--balance", action="store_true", help="equal-tile worker plan instead of one workgroup per partition")
     p.add_argument("--kernel-only", action="store_true", help="time only the map kernel (for profiling runs)")
     p.add_argument("--graph", action="store_true",
@@ -181,7 +183,8 @@ def main():
             w = wl.config_c2(seed=args.seed, batch=args.batch, host_pages=False, lo=args.ctx_lo, hi=args.ctx_hi,
                              shuffle_pages=not args.identity_pages)
         w.seed = args.seed + 1000 * i  # same geometry, different page contents
-        arenas.append(wl.DeviceWorkload(device, w, partition_tokens=args.partition, balanced=args.balance))
+        arenas.append(wl.DeviceWorkload(device, w, partition_tokens=args.partition, balanced=args.balance,
+                                        longest_first=not args.plan_order))
     w = arenas[0].w
     shape = arenas[0].shape
     step_bytes = w.algorithmic_bytes()
@@ -190,6 +193,8 @@ def main():
     def run_steps(n):
         for i in range(n):
             arenas[i % len(arenas)].step()
+
+    run_steps_direct = run_steps
 
     def run_maps(n):
         for i in range(n):
@@ -236,6 +241,15 @@ def main():
     map_ms, map_launches = device.kernel_time_ms(map_kernel)
     device.set_timing(False)
     map_avg_s = map_ms / max(map_launches, 1) / 1e3
+    # the other two kernels of the step, for the record
+    device.set_timing(True)
+    device.reset_timing()
+    run_steps_direct(min(args.steps, 50))
+    kernels_us = {}
+    for name in ("kv_page_write", map_kernel, "tiled_q_reduce" if verify else "split_kv_reduce"):
+        ms, n = device.kernel_time_ms(name)
+        kernels_us[name] = ms / max(n, 1) * 1e3
+    device.set_timing(False)
     achieved = map_bytes / map_avg_s / 1e9
 
     workload_key = (f"{'verify_q%d' % args.q_len if verify else 'decode'}_b{args.batch}_ctx{args.ctx_lo}-{args.ctx_hi}"
@@ -264,6 +278,8 @@ def main():
             "kv_splits": shape.num_sdpa_map_task_templates,
             "algorithmic_bytes_per_step": step_bytes,
             "arenas_rotated": len(arenas),
+            "kernel_us_in_step": kernels_us,
+            "dispatch_order": "plan order" if args.plan_order or args.balance else "longest split first",
         },
         "roofline": {
             "bound": "hbm",

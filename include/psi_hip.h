@@ -174,6 +174,15 @@ int psi_hip_gqa_metadata_update(uint32_t max_tokens, const uint32_t* req_slots, 
                                 uint32_t* q_token_tiles, uint32_t* kv_splits, uint32_t* cu_kv_splits,
                                 psi_hip_gqa_replay_shape* out_shape);
 
+/* Dispatch order (no counterpart in the reference, which launches rows in plan order): sorts the
+ * first num_kv_splits rows of kv_splits in place by descending length (stable; padding rows last) so
+ * that the map's longest workgroups start first and the short ones fill the end of the launch.  The
+ * rows of a token are then no longer adjacent: partial_row_index[i] (host u32[num_kv_splits]) is the
+ * new position of original row i.  Upload it and pass it to the combine entry points as
+ * `partial_row_index`; cu_kv_splits keeps indexing the original order.  The map entry points need
+ * nothing: they treat rows independently. */
+int psi_hip_split_kv_order_longest_first(uint32_t* kv_splits, uint32_t num_kv_splits, uint32_t* partial_row_index);
+
 /* Balanced decode plan (no counterpart in the reference, whose planner budgets partial states, not
  * device occupancy).  Cuts the rows of an existing SingleQ plan at tile boundaries so that
  * `num_workers` consecutive groups of rows hold equal numbers of 16-token tiles; a decode-map
@@ -239,10 +248,12 @@ int psi_hip_split_kv_single_q_map_balanced(psi_hip_ctx* ctx, const psi_hip_gqa_c
 /* `GQASplitKVSingleQKernels::invoke_reduce_bucketed` (gqa_split_kv_single_q.rs:353-383; kernel
  * metal/gqa_split_kv_single_q_reduce.metal:10-49).  cu_kv_splits: device u32[num_total_tokens + 1];
  * output: device [num_total_tokens, Hq, D]; rows >= num_active_tokens keep their bytes. */
+/* partial_row_index: device u32[num_total_kv_splits] from psi_hip_split_kv_order_longest_first, or null
+ * when the rows of a token are adjacent as planned. */
 int psi_hip_split_kv_single_q_reduce(psi_hip_ctx* ctx, const psi_hip_gqa_config* cfg, const void* scratch,
                                      uint64_t scratch_bytes, const uint32_t* cu_kv_splits, void* output,
                                      uint32_t num_total_tokens, uint32_t num_total_kv_splits,
-                                     uint32_t num_active_tokens);
+                                     uint32_t num_active_tokens, const uint32_t* partial_row_index);
 
 /* ------------------------------------------------------------------ split-KV verify / prefill (TiledQ) */
 
@@ -274,7 +285,7 @@ int psi_hip_split_kv_tiled_q_reduce(psi_hip_ctx* ctx, const psi_hip_gqa_config* 
                                     const void* scratch, uint64_t scratch_bytes, const uint32_t* q_token_tiles,
                                     const uint32_t* cu_kv_splits, void* output, uint32_t num_total_tokens,
                                     uint32_t num_total_q_token_tiles, uint32_t num_total_kv_splits,
-                                    uint32_t num_active_q_token_tiles);
+                                    uint32_t num_active_q_token_tiles, const uint32_t* partial_row_index);
 
 /* ------------------------------------------------------------------ request page table */
 

@@ -158,7 +158,8 @@ PROTOTYPES = {
          c_uint32, c_uint32, c_uint32, c_uint32, c_uint32],
     ),
     "psi_hip_split_kv_single_q_reduce": (
-        c_int, [c_void_p, _CFG, c_void_p, c_uint64, c_void_p, c_void_p, c_uint32, c_uint32, c_uint32]),
+        c_int, [c_void_p, _CFG, c_void_p, c_uint64, c_void_p, c_void_p, c_uint32, c_uint32, c_uint32, c_void_p]),
+    "psi_hip_split_kv_order_longest_first": (c_int, [_U32P, c_uint32, _U32P]),
     "psi_hip_split_kv_tiled_q_scratch_bytes": (c_int, [_CFG, c_uint32, c_uint32, POINTER(c_uint64)]),
     "psi_hip_split_kv_tiled_q_map": (
         c_int,
@@ -169,7 +170,7 @@ PROTOTYPES = {
     "psi_hip_split_kv_tiled_q_reduce": (
         c_int,
         [c_void_p, _CFG, c_uint32, c_void_p, c_uint64, c_void_p, c_void_p, c_void_p, c_uint32, c_uint32, c_uint32,
-         c_uint32],
+         c_uint32, c_void_p],
     ),
     "psi_hip_page_table_write_page_ids": (
         c_int, [c_void_p, _LAYOUT, c_void_p, c_uint32, c_uint32, c_uint32, _U32P, c_uint32, c_uint32]),

@@ -569,3 +569,23 @@ extern "C" int psi_hip_split_kv_balance_plan(const uint32_t* kv_splits_in, uint3
     *out_num_rows = out_rows;
     return PSI_HIP_OK;
 }
+
+extern "C" int psi_hip_split_kv_order_longest_first(uint32_t* kv_splits, uint32_t num_kv_splits,
+                                                    uint32_t* partial_row_index) {
+    PSI_REQUIRE(kv_splits != nullptr && partial_row_index != nullptr, "split arrays must not be null");
+    std::vector<uint32_t> order(num_kv_splits);
+    for (uint32_t i = 0; i < num_kv_splits; ++i) order[i] = i;
+    auto length = [&](uint32_t row) -> uint64_t {
+        const uint32_t* r = kv_splits + (size_t)row * 3;
+        if (r[0] == PSI_HIP_SENTINEL) return 0;  // padding rows stay last
+        return (uint64_t)r[2] - r[1] + 1;
+    };
+    std::stable_sort(order.begin(), order.end(), [&](uint32_t x, uint32_t y) { return length(x) > length(y); });
+    std::vector<uint32_t> sorted((size_t)num_kv_splits * 3);
+    for (uint32_t pos = 0; pos < num_kv_splits; ++pos) {
+        std::copy(kv_splits + (size_t)order[pos] * 3, kv_splits + (size_t)order[pos] * 3 + 3, sorted.begin() + (size_t)pos * 3);
+        partial_row_index[order[pos]] = pos;
+    }
+    std::copy(sorted.begin(), sorted.end(), kv_splits);
+    return PSI_HIP_OK;
+}

@@ -62,6 +62,9 @@ struct ReduceArgs {
     uint32_t hq, d;
     uint32_t num_active_tokens;
     uint32_t out_dtype = PSI_HIP_F32;  // element type of `output`
+    // Optional: the partial rows of token / tile t are row_index[cu[t] .. cu[t + 1]) instead of
+    // cu[t] .. cu[t + 1] themselves (plans whose rows were re-ordered for dispatch).
+    const uint32_t* row_index = nullptr;
     // TiledQ only: cu_kv_splits is indexed by Q-token tile.
     const uint32_t* q_token_tiles = nullptr;
     uint32_t rows_per_split_head = 1;

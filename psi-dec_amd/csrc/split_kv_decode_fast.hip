@@ -12,7 +12,7 @@ int launch_decode_map_f16_d128(psi_hip_ctx* ctx, const Geometry& g, const MapArg
 // Log-sum-exp combine: one wave per (token, q_head), lanes over head_dim.  The row maxima are
 // fetched lane-parallel first; the accumulator rows are then read four at a time so that a wave
 // keeps several 1 KiB reads in flight instead of one.
-template <typename Tag, int D>
+template <typename Tag, int D, bool kIndexed>
 __global__ __launch_bounds__(256) void split_kv_reduce_fast(ReduceArgs a) {
     constexpr int kPerLane = D / 64;  // 4 or 2
     constexpr int kUnroll = 4;
@@ -22,8 +22,9 @@ __global__ __launch_bounds__(256) void split_kv_reduce_fast(ReduceArgs a) {
     const uint32_t token = (uint32_t)(row_out / a.hq), q_head = (uint32_t)(row_out % a.hq);
     const uint32_t begin = a.cu_kv_splits[token], end = a.cu_kv_splits[token + 1];
     float global_max = -INFINITY;
+    const uint32_t* row_index = a.row_index;
     for (uint32_t p = begin + lane; p < end; p += 64)
-        global_max = fmaxf(global_max, a.part_max[(uint64_t)p * a.hq + q_head]);
+        global_max = fmaxf(global_max, a.part_max[(uint64_t)(kIndexed ? row_index[p] : p) * a.hq + q_head]);
 #pragma unroll
     for (int off = 32; off > 0; off >>= 1) global_max = fmaxf(global_max, __shfl_xor(global_max, off, 64));
     float weight_sum = 0.0f, value[kPerLane];
@@ -34,7 +35,8 @@ __global__ __launch_bounds__(256) void split_kv_reduce_fast(ReduceArgs a) {
 #pragma unroll
         for (int u = 0; u < kUnroll; ++u) {
             const bool live = p0 + u < end;
-            const uint64_t row = (uint64_t)(live ? p0 + u : begin) * a.hq + q_head;
+            const uint32_t p = live ? p0 + u : begin;
+            const uint64_t row = (uint64_t)(kIndexed ? row_index[p] : p) * a.hq + q_head;
             const float m = a.part_max[row];
             sums[u] = a.part_sum[row];
             w[u] = live && m > -INFINITY ? exp2f(m - global_max) : 0.0f;
@@ -57,7 +59,7 @@ __global__ __launch_bounds__(256) void split_kv_reduce_fast(ReduceArgs a) {
 
 // The same combine for Q-token tiles: one wave per (tile, token in tile, q_head); the tile's partial
 // rows are cu_kv_splits[tile] .. cu_kv_splits[tile + 1].
-template <typename Tag, int D>
+template <typename Tag, int D, bool kIndexed>
 __global__ __launch_bounds__(256) void split_kv_reduce_tiled_fast(ReduceArgs a) {
     constexpr int kPerLane = D / 64;
     const uint32_t lane = threadIdx.x & 63;
@@ -73,8 +75,10 @@ __global__ __launch_bounds__(256) void split_kv_reduce_tiled_fast(ReduceArgs a) 
     const uint32_t begin = a.cu_kv_splits[tile], end = a.cu_kv_splits[tile + 1];
     constexpr int kUnroll = 4;
     float global_max = -INFINITY;
+    const uint32_t* row_index = a.row_index;
     for (uint32_t p = begin + lane; p < end; p += 64)
-        global_max = fmaxf(global_max, a.part_max[((uint64_t)p * a.hq + q_head) * rows + tile_row]);
+        global_max = fmaxf(global_max,
+                           a.part_max[((uint64_t)(kIndexed ? row_index[p] : p) * a.hq + q_head) * rows + tile_row]);
 #pragma unroll
     for (int off = 32; off > 0; off >>= 1) global_max = fmaxf(global_max, __shfl_xor(global_max, off, 64));
     float weight_sum = 0.0f, value[kPerLane];
@@ -85,7 +89,8 @@ __global__ __launch_bounds__(256) void split_kv_reduce_tiled_fast(ReduceArgs a) 
 #pragma unroll
         for (int u = 0; u < kUnroll; ++u) {
             const bool live = p0 + u < end;
-            const uint64_t row = ((uint64_t)(live ? p0 + u : begin) * a.hq + q_head) * rows + tile_row;
+            const uint32_t p = live ? p0 + u : begin;
+            const uint64_t row = ((uint64_t)(kIndexed ? row_index[p] : p) * a.hq + q_head) * rows + tile_row;
             const float m = a.part_max[row];
             sums[u] = a.part_sum[row];
             w[u] = live && m > -INFINITY ? exp2f(m - global_max) : 0.0f;
@@ -132,19 +137,25 @@ int launch_reduce_fast(psi_hip_ctx* ctx, const Geometry& g, const ReduceArgs& a)
                                 : (uint64_t)a.num_active_tokens * g.hq;
     if ((rows + 3) / 4 > 0x7fffffffull) return PSI_HIP_ERR_UNSUPPORTED;
     const dim3 grid((uint32_t)((rows + 3) / 4)), block(256);
-#define PSI_REDUCE(TAG)                                                                                             \
-    do {                                                                                                            \
-        if (tiled) {                                                                                                \
-            if (g.d == 256) hipLaunchKernelGGL((split_kv_reduce_tiled_fast<TAG, 256>), grid, block, 0, ctx->stream, a); \
-            else hipLaunchKernelGGL((split_kv_reduce_tiled_fast<TAG, 128>), grid, block, 0, ctx->stream, a);       \
-        } else {                                                                                                    \
-            if (g.d == 256) hipLaunchKernelGGL((split_kv_reduce_fast<TAG, 256>), grid, block, 0, ctx->stream, a);  \
-            else hipLaunchKernelGGL((split_kv_reduce_fast<TAG, 128>), grid, block, 0, ctx->stream, a);             \
-        }                                                                                                           \
+#define PSI_REDUCE_D(TAG, DIM, INDEXED)                                                                          \
+    do {                                                                                                         \
+        if (tiled) hipLaunchKernelGGL((split_kv_reduce_tiled_fast<TAG, DIM, INDEXED>), grid, block, 0, ctx->stream, a); \
+        else hipLaunchKernelGGL((split_kv_reduce_fast<TAG, DIM, INDEXED>), grid, block, 0, ctx->stream, a);     \
+    } while (0)
+#define PSI_REDUCE(TAG)                                                   \
+    do {                                                                  \
+        if (g.d == 256) {                                                 \
+            if (a.row_index) PSI_REDUCE_D(TAG, 256, true);                \
+            else PSI_REDUCE_D(TAG, 256, false);                           \
+        } else {                                                          \
+            if (a.row_index) PSI_REDUCE_D(TAG, 128, true);                \
+            else PSI_REDUCE_D(TAG, 128, false);                           \
+        }                                                                 \
     } while (0)
     if (a.out_dtype == PSI_HIP_F32) PSI_REDUCE(F32Tag);
     else if (a.out_dtype == PSI_HIP_BF16) PSI_REDUCE(BF16Tag);
     else PSI_REDUCE(F16Tag);
+#undef PSI_REDUCE_D
 #undef PSI_REDUCE
     return PSI_HIP_OK;
 }

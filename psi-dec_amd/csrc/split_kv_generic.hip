@@ -128,11 +128,14 @@ __global__ __launch_bounds__(256) void split_kv_reduce_generic(ReduceArgs a, uin
         end = a.cu_kv_splits[tile + 1];
     }
     float global_max = -INFINITY;
-    for (uint32_t p = begin; p < end; ++p)
-        global_max = fmaxf(global_max, a.part_max[((uint64_t)p * a.hq + q_head) * a.rows_per_split_head + tile_row]);
+    for (uint32_t p = begin; p < end; ++p) {
+        const uint32_t phys = a.row_index ? a.row_index[p] : p;
+        global_max = fmaxf(global_max, a.part_max[((uint64_t)phys * a.hq + q_head) * a.rows_per_split_head + tile_row]);
+    }
     float weight_sum = 0.0f, value = 0.0f;
     for (uint32_t p = begin; p < end; ++p) {
-        const uint64_t row = ((uint64_t)p * a.hq + q_head) * a.rows_per_split_head + tile_row;
+        const uint32_t phys = a.row_index ? a.row_index[p] : p;
+        const uint64_t row = ((uint64_t)phys * a.hq + q_head) * a.rows_per_split_head + tile_row;
         const float m = a.part_max[row];
         const float w = m > -INFINITY ? exp2f(m - global_max) : 0.0f;
         weight_sum += w * a.part_sum[row];

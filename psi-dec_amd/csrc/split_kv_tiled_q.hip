@@ -115,7 +115,8 @@ extern "C" int psi_hip_split_kv_tiled_q_reduce(psi_hip_ctx* ctx, const psi_hip_g
                                                uint64_t scratch_bytes, const uint32_t* q_token_tiles,
                                                const uint32_t* cu_kv_splits, void* output, uint32_t num_total_tokens,
                                                uint32_t num_total_q_token_tiles, uint32_t num_total_kv_splits,
-                                               uint32_t num_active_q_token_tiles) {
+                                               uint32_t num_active_q_token_tiles,
+                                               const uint32_t* partial_row_index) {
     PSI_REQUIRE(ctx != nullptr, "ctx must not be null");
     Geometry g;
     int rc = make_geometry(cfg, &g);
@@ -134,6 +135,7 @@ extern "C" int psi_hip_split_kv_tiled_q_reduce(psi_hip_ctx* ctx, const psi_hip_g
     a.part_sum = reinterpret_cast<const float*>(static_cast<const char*>(scratch) + pl.sum_offset);
     a.part_acc = reinterpret_cast<const float*>(static_cast<const char*>(scratch) + pl.acc_offset);
     a.cu_kv_splits = cu_kv_splits;
+    a.row_index = partial_row_index;
     a.output = output;
     a.hq = g.hq;
     a.d = g.d;

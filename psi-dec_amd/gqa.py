@@ -400,6 +400,7 @@ class GQAMetadataBuffers:
         self._shape, self._variant = None, None
         self.d_req_slots = self.d_flat_token_indices = self.d_q_token_tiles = None
         self.d_kv_splits = self.d_cu_kv_splits = None
+        self.h_partial_row_index = self.d_partial_row_index = None
 
     def max_tokens(self) -> int:
         return self._max_tokens
@@ -422,6 +423,7 @@ class GQAMetadataBuffers:
                                      shape.num_total_q_token_tiles, shape.num_kv_splits, shape.num_total_kv_splits,
                                      bool(shape.reduce_sdpa_partial_outputs))
         self._variant = variant
+        self.h_partial_row_index = self.d_partial_row_index = None  # rows are in plan order again
         if self.device is not None:
             self.upload()
         return self._shape
@@ -454,6 +456,23 @@ class GQAMetadataBuffers:
         """Fixed-length KV partitions (not in the reference): ceil(ctx / partition) splits per row."""
         return self._update(req_slots, token_indices, cu_tokens, split_kv_variant, L.CAPACITY_FIXED_PARTITION,
                             partition_tokens=partition_tokens)
+
+    def order_longest_first(self):
+        """Re-orders the planned rows for dispatch (psi_hip_split_kv_order_longest_first): longest
+        rows first.  `d_partial_row_index` must then be passed to the combine."""
+        s = self._shape
+        n = s.num_sdpa_map_task_templates
+        self.h_partial_row_index = np.zeros(max(len(self.h_kv_splits) // 3, 1), np.uint32)
+        self.h_partial_row_index[:] = np.arange(len(self.h_partial_row_index), dtype=np.uint32)
+
+        def p(a):
+            return a.ctypes.data_as(ctypes.POINTER(ctypes.c_uint32))
+
+        L.check(L.load().psi_hip_split_kv_order_longest_first(p(self.h_kv_splits), n, p(self.h_partial_row_index)))
+        if self.device is not None:
+            self.upload()
+            self.d_partial_row_index = self.device.from_numpy(self.h_partial_row_index)
+        return self.h_partial_row_index
 
     def balance(self, num_workers: int):
         """Re-cuts the current SingleQ plan into rows grouped for `num_workers` equal-work decode
@@ -632,12 +651,13 @@ class GQASplitKVSingleQKernels:
     def invoke_reduce(self, scratch, cu_sdpa_partial_outputs, output):
         self.invoke_reduce_bucketed(scratch, cu_sdpa_partial_outputs, output, self.shape.num_total_tokens)
 
-    def invoke_reduce_bucketed(self, scratch, cu_sdpa_partial_outputs, output, num_active_tokens: int):
+    def invoke_reduce_bucketed(self, scratch, cu_sdpa_partial_outputs, output, num_active_tokens: int,
+                               partial_row_index=None):
         cfg = self.config.struct()
         L.check(self.device.lib.psi_hip_split_kv_single_q_reduce(
             self.device.ctx, ctypes.byref(cfg), _ptr(scratch.buffer), scratch.bytes, _ptr(cu_sdpa_partial_outputs),
             _ptr(output), self.shape.num_total_tokens, self.shape.num_total_sdpa_map_task_templates,
-            num_active_tokens))
+            num_active_tokens, _ptr(partial_row_index)))
 
 
 # ------------------------------------------------------------------ TiledQ verify / prefill
@@ -715,9 +735,10 @@ class GQASplitKVTiledQKernels:
                                     self.shape.num_total_q_token_tiles)
 
     def invoke_reduce_bucketed(self, scratch, q_token_tiles, cu_sdpa_partial_outputs, output,
-                               num_active_q_token_tiles: int):
+                               num_active_q_token_tiles: int, partial_row_index=None):
         cfg, s = self.config.struct(), self.shape
         L.check(self.device.lib.psi_hip_split_kv_tiled_q_reduce(
             self.device.ctx, ctypes.byref(cfg), self.config.q_token_tile_size, _ptr(scratch.buffer), scratch.bytes,
             _ptr(q_token_tiles), _ptr(cu_sdpa_partial_outputs), _ptr(output), s.num_total_tokens,
-            s.num_total_q_token_tiles, s.num_total_sdpa_map_task_templates, num_active_q_token_tiles))
+            s.num_total_q_token_tiles, s.num_total_sdpa_map_task_templates, num_active_q_token_tiles,
+            _ptr(partial_row_index)))

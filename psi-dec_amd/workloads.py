@@ -145,7 +145,7 @@ class DeviceWorkload:
 
     def __init__(self, device: G.Device, w: Workload, partition_tokens: Optional[int] = None,
                  max_tokens: Optional[int] = None, variant: Optional[G.GQASplitKVVariant] = None,
-                 f32_output: bool = False, balanced: bool = False):
+                 f32_output: bool = False, balanced: bool = False, longest_first: bool = False):
         import torch
 
         self.device, self.w = device, w
@@ -188,6 +188,8 @@ class DeviceWorkload:
         else:
             self.meta = G.GQAMetadataBuffers(device, max_tokens or max(w.num_tokens, 1))
             self.shape = self.meta.update(w.req_slots, w.token_indices, w.cu_tokens, variant)
+        if longest_first and not balanced:
+            self.meta.order_longest_first()
         self.balanced = balanced and not variant.is_tiled()
         if self.balanced:
             workers = G.balanced_workers(G.GQASplitKVConfig(w.dtype, w.page_bytes, w.num_q_heads, w.num_kv_heads,
@@ -249,9 +251,10 @@ class DeviceWorkload:
         self.device.f32_output(self.f32_output)
         if self.variant.is_tiled():
             self.kernels.invoke_reduce_bucketed(self.scratch, m.d_q_token_tiles, m.d_cu_kv_splits, self.output,
-                                                s.num_q_token_tiles)
+                                                s.num_q_token_tiles, partial_row_index=m.d_partial_row_index)
         else:
-            self.kernels.invoke_reduce_bucketed(self.scratch, m.d_cu_kv_splits, self.output, s.num_tokens)
+            self.kernels.invoke_reduce_bucketed(self.scratch, m.d_cu_kv_splits, self.output, s.num_tokens,
+                                                partial_row_index=m.d_partial_row_index)
         self.device.f32_output(False)
 
     def step(self):

@@ -103,3 +103,22 @@ def test_balanced_plan_matches_oracle(psi, oracle, device):
     per_worker = [int(tiles[m.h_worker_cu[i]:m.h_worker_cu[i + 1]].sum()) for i in range(m.num_workers)]
     assert max(per_worker) - min(per_worker) <= 1
     assert sum(per_worker) == sum(-(-c // 16) for c in ctx)
+
+
+@pytest.mark.parametrize("q_len", [1, 3])
+def test_longest_first_dispatch_order(psi, oracle, device, q_len):
+    """Rows re-ordered for dispatch (longest first): the combine follows them through its row index,
+    and the result is bit-identical to the plan-order launch."""
+    wl = importlib_workloads(psi)
+    ctx = [3000, 17, 1025, 2048, 700, 5, 513]
+    w = wl.make_workload(37, ctx, 24, 4, 256, psi.Dtype.Bfloat16, 16, q_lens=q_len)
+    stats, dw = run_and_check(psi, oracle, device, w, "longest first", partition_tokens=512, longest_first=True)
+    m = dw.meta
+    n = dw.shape.num_sdpa_map_task_templates
+    rows = m.h_kv_splits[: n * 3].reshape(-1, 3).astype(np.int64)
+    lengths = rows[:, 2] - rows[:, 1]
+    assert (np.diff(lengths) <= 0).all() and lengths[0] == 512
+    assert sorted(m.h_partial_row_index[:n].tolist()) == list(range(n))
+    plain = wl.DeviceWorkload(device, w, partition_tokens=512, f32_output=True)
+    plain.step()
+    assert np.array_equal(plain.output_f32(), dw.output_f32())

@@ -439,3 +439,16 @@ def test_balance_plan_covers_the_same_ranges(psi):
         assert (part[:, 0] == row).all()
     w = md.h_worker_cu
     assert w[0] == 0 and w[-1] == s.num_sdpa_map_task_templates and (np.diff(w.astype(np.int64)) >= 0).all()
+
+
+def test_longest_first_order(psi):
+    lib = psi.load()
+    rows = np.array([0, 0, 512, 0, 512, 700, 1, 0, 40, 2, 0, 512, 2, 512, 1024, 2, 1024, 1030,
+                     MAX, MAX, MAX, MAX, MAX, MAX], np.uint32)
+    index = np.zeros(8, np.uint32)
+    p = lambda a: a.ctypes.data_as(ctypes.POINTER(ctypes.c_uint32))  # noqa: E731
+    assert lib.psi_hip_split_kv_order_longest_first(p(rows), 8, p(index)) == 0
+    got = rows.reshape(-1, 3).tolist()
+    assert got[:6] == [[0, 0, 512], [2, 0, 512], [2, 512, 1024], [0, 512, 700], [1, 0, 40], [2, 1024, 1030]]
+    assert got[6:] == [[MAX, MAX, MAX]] * 2
+    assert index.tolist() == [0, 3, 4, 1, 2, 5, 6, 7]
