@@ -52,6 +52,8 @@ def parse_args():
     p.add_argument("--q-len", type=int, default=2)
     p.add_argument("--prefix", type=int, default=4096, help="prefill workload: cached tokens before the chunk")
     p.add_argument("--chunk", type=int, default=2048, help="prefill workload: new tokens of the one sequence")
+    p.add_argument("--no-row-groups", action="store_true",
+                   help="prefill workload: one workgroup per (row, KV head) instead of the row-group map")
     p.add_argument("--calibrate-copy", action="store_true",
                    help="run only the plain copy / read probes of known size (counter calibration, practical ceiling)")
     p.add_argument("--probe-mib", type=int, default=1024)
@@ -184,7 +186,8 @@ def main():
                              shuffle_pages=not args.identity_pages)
         w.seed = args.seed + 1000 * i  # same geometry, different page contents
         arenas.append(wl.DeviceWorkload(device, w, partition_tokens=args.partition, balanced=args.balance,
-                                        longest_first=not args.plan_order))
+                                        longest_first=not args.plan_order,
+                                        grouped=prefill and not args.no_row_groups))
     w = arenas[0].w
     shape = arenas[0].shape
     step_bytes = w.algorithmic_bytes()
@@ -299,6 +302,7 @@ def main():
         pairs = sum(args.prefix + i + 1 for i in range(args.chunk))
         flops = 4 * w.num_q_heads * w.head_dim * pairs
         result["config"]["workload"] = f"prefill_chunk{args.chunk}_on_prefix{args.prefix}_24q4kv_d256_bf16_p16_part{args.partition}"
+        result["config"]["row_groups"] = arenas[0].meta.num_row_groups
         result["mfma"] = {"bound": "mfma", "flops_per_launch": flops, "achieved": flops / map_avg_s / 1e12,
                           "peak": 2500.0, "unit": "TFLOP/s", "frac": flops / map_avg_s / 1e12 / 2500.0}
     if not args.no_cpu_baseline:

@@ -279,6 +279,39 @@ int psi_hip_split_kv_tiled_q_map(psi_hip_ctx* ctx, const psi_hip_gqa_config* cfg
                                  uint32_t num_active_tokens, uint32_t num_active_q_token_tiles,
                                  uint32_t num_active_kv_splits, uint32_t max_active_q_tile_tokens);
 
+/* Row groups for prefill chunks (no counterpart in the reference, whose TiledQ map launches one
+ * threadgroup per (row, Q-head tile), gqa_split_kv_tiled_q.rs:402-409).  Host helper: gathers the
+ * kv_split rows of consecutive Q-token tiles of one request that start at the same key (the rows of one
+ * KV partition of a fixed-partition plan) into groups of up to *out_group_tiles rows, heaviest group
+ * first.  row_groups: host u32[row_groups_capacity], written as [*out_num_groups][*out_group_tiles] row
+ * indices padded with PSI_HIP_SENTINEL; capacity of num_kv_splits * 32 words always suffices.  req_slots
+ * is the per-token slot array of psi_hip_gqa_metadata_update.  Every non-padding row lands in exactly
+ * one group.  *out_group_tiles = 0 when the geometry has no grouped kernel (use the plain map then). */
+int psi_hip_split_kv_tiled_q_group_rows(const psi_hip_gqa_config* cfg, uint32_t q_token_tile_size,
+                                        const uint32_t* kv_splits, uint32_t num_kv_splits,
+                                        const uint32_t* q_token_tiles, uint32_t num_q_token_tiles,
+                                        const uint32_t* req_slots, uint32_t* row_groups,
+                                        uint64_t row_groups_capacity, uint32_t* out_group_tiles,
+                                        uint32_t* out_num_groups);
+
+/* psi_hip_split_kv_tiled_q_map with one workgroup per (row group, KV head [, half of the Q heads]):
+ * the group's K/V tiles are staged once in LDS for up to 128 query columns and both contractions run
+ * on the matrix cores.  Same arguments, scratch layout and results (within rounding) as the plain map;
+ * row_groups: device copy of the table of psi_hip_split_kv_tiled_q_group_rows for the same kv_splits.
+ * Geometries outside the grouped kernel (other than bf16 / f16, head_dim 256, pages of 16*2^k tokens)
+ * run the plain map. */
+int psi_hip_split_kv_tiled_q_map_grouped(psi_hip_ctx* ctx, const psi_hip_gqa_config* cfg,
+                                         const psi_hip_page_table_layout* layout, uint32_t q_token_tile_size,
+                                         const void* q, const void* kv_pages, uint64_t kv_pages_bytes,
+                                         const uint32_t* req_slots, const uint32_t* page_ids,
+                                         const uint32_t* flat_token_indices, const uint32_t* q_token_tiles,
+                                         const uint32_t* kv_splits, void* scratch, uint64_t scratch_bytes,
+                                         uint32_t gqa_layer_index, uint32_t num_total_tokens,
+                                         uint32_t num_total_q_token_tiles, uint32_t num_total_kv_splits,
+                                         uint32_t num_active_tokens, uint32_t num_active_q_token_tiles,
+                                         uint32_t num_active_kv_splits, uint32_t max_active_q_tile_tokens,
+                                         const uint32_t* row_groups, uint32_t group_tiles, uint32_t num_groups);
+
 /* `GQASplitKVTiledQKernels::invoke_reduce_bucketed` (gqa_split_kv_tiled_q.rs:314-327; kernel
  * metal/gqa_split_kv_tiled_q.metal:324-378). */
 int psi_hip_split_kv_tiled_q_reduce(psi_hip_ctx* ctx, const psi_hip_gqa_config* cfg, uint32_t q_token_tile_size,

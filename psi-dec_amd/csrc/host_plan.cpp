@@ -8,7 +8,7 @@
 #include <algorithm>
 #include <queue>
 
-#include "common.h"
+#include "split_kv.h"
 
 namespace psi {
 
@@ -587,5 +587,78 @@ extern "C" int psi_hip_split_kv_order_longest_first(uint32_t* kv_splits, uint32_
         partial_row_index[order[pos]] = pos;
     }
     std::copy(sorted.begin(), sorted.end(), kv_splits);
+    return PSI_HIP_OK;
+}
+
+// Row groups for the prefill-chunk map.  Rows are sorted by (request slot, first key, Q-token tile); a
+// group is a run of rows of consecutive, contiguous tiles of one request that start at the same key,
+// every tile but the last one full, at most `max_tiles` of them.
+extern "C" int psi_hip_split_kv_tiled_q_group_rows(const psi_hip_gqa_config* cfg, uint32_t q_token_tile_size,
+                                                   const uint32_t* kv_splits, uint32_t num_kv_splits,
+                                                   const uint32_t* q_token_tiles, uint32_t num_q_token_tiles,
+                                                   const uint32_t* req_slots, uint32_t* row_groups,
+                                                   uint64_t row_groups_capacity, uint32_t* out_group_tiles,
+                                                   uint32_t* out_num_groups) {
+    Geometry g;
+    int rc = make_geometry(cfg, &g);
+    if (rc != PSI_HIP_OK) return rc;
+    PSI_REQUIRE(kv_splits && q_token_tiles && req_slots && row_groups && out_group_tiles && out_num_groups,
+                "row-group arrays must not be null");
+    PSI_REQUIRE(q_token_tile_size > 0 && q_token_tile_size <= 64, "GQA Q-token tile size must be in 1..64");
+    *out_group_tiles = 0;
+    *out_num_groups = 0;
+    if (!chunk_map_supported(g, q_token_tile_size)) return PSI_HIP_OK;  // no grouped kernel for this shape
+    const uint32_t max_tiles = chunk_group_tiles(g.group, q_token_tile_size);
+
+    struct Row {
+        uint32_t slot, kv_begin, tile, row, kv_end;
+    };
+    std::vector<Row> rows;
+    rows.reserve(num_kv_splits);
+    for (uint32_t r = 0; r < num_kv_splits; ++r) {
+        const uint32_t* s = kv_splits + (size_t)r * 3;
+        if (s[0] == PSI_HIP_SENTINEL) continue;
+        PSI_REQUIRE(s[0] < num_q_token_tiles, "kv_split row %u names Q-token tile %u of %u", r, s[0], num_q_token_tiles);
+        PSI_REQUIRE(s[2] > s[1], "kv_split row %u is empty", r);
+        const uint32_t flat_begin = q_token_tiles[(size_t)s[0] * 2];
+        rows.push_back(Row{req_slots[flat_begin], s[1], s[0], r, s[2]});
+    }
+    std::sort(rows.begin(), rows.end(), [](const Row& x, const Row& y) {
+        if (x.slot != y.slot) return x.slot < y.slot;
+        if (x.kv_begin != y.kv_begin) return x.kv_begin < y.kv_begin;
+        if (x.tile != y.tile) return x.tile < y.tile;
+        return x.row < y.row;
+    });
+    struct Group {
+        uint32_t first, count;  // range of `rows`
+        uint64_t work;          // query tokens x keys, the dispatch-order key
+    };
+    std::vector<Group> groups;
+    auto tile_tokens = [&](uint32_t tile) { return q_token_tiles[(size_t)tile * 2 + 1] - q_token_tiles[(size_t)tile * 2]; };
+    for (uint32_t i = 0; i < rows.size(); ++i) {
+        bool join = false;
+        if (!groups.empty()) {
+            const Group& cur = groups.back();
+            const Row& prev = rows[i - 1];
+            join = cur.count < max_tiles && prev.slot == rows[i].slot && prev.kv_begin == rows[i].kv_begin &&
+                   prev.tile + 1 == rows[i].tile && tile_tokens(prev.tile) == q_token_tile_size &&
+                   q_token_tiles[(size_t)prev.tile * 2 + 1] == q_token_tiles[(size_t)rows[i].tile * 2];
+        }
+        if (!join) groups.push_back(Group{i, 0, 0});
+        groups.back().count += 1;
+        groups.back().work += (uint64_t)tile_tokens(rows[i].tile) * (rows[i].kv_end - rows[i].kv_begin);
+    }
+    PSI_REQUIRE((uint64_t)groups.size() * max_tiles <= row_groups_capacity,
+                "row-group table too small: %llu groups of %u rows, capacity %llu words",
+                (unsigned long long)groups.size(), max_tiles, (unsigned long long)row_groups_capacity);
+    // heaviest groups first, so that the light ones fill the end of the launch
+    std::stable_sort(groups.begin(), groups.end(), [](const Group& x, const Group& y) { return x.work > y.work; });
+    for (size_t gi = 0; gi < groups.size(); ++gi) {
+        uint32_t* out = row_groups + gi * max_tiles;
+        for (uint32_t m = 0; m < max_tiles; ++m)
+            out[m] = m < groups[gi].count ? rows[groups[gi].first + m].row : PSI_HIP_SENTINEL;
+    }
+    *out_group_tiles = max_tiles;
+    *out_num_groups = (uint32_t)groups.size();
     return PSI_HIP_OK;
 }

@@ -71,6 +71,24 @@ struct ReduceArgs {
     uint32_t num_active_q_token_tiles = 0;
 };
 
+// Prefill-chunk map: a workgroup serves up to kChunkCols query columns (tokens of a row group x
+// heads).  The heads of one KV head are dealt to chunk_head_subsets() workgroups, and a row group
+// holds up to chunk_group_tiles() Q-token tiles (0: the shape does not fit the kernel).
+constexpr int kChunkCols = 128;
+inline uint32_t chunk_head_subsets(uint32_t group) { return group > 5 ? 2u : 1u; }
+inline uint32_t chunk_group_tiles(uint32_t group, uint32_t q_token_tile_size) {
+    const uint32_t subsets = chunk_head_subsets(group);
+    const uint32_t heads = (group + subsets - 1) / subsets;
+    const uint32_t tiles = (uint32_t)kChunkCols / (heads * q_token_tile_size);
+    return tiles > 32 ? 32u : tiles;
+}
+// True when the prefill-chunk map covers the geometry (2-byte elements, head_dim 256, pages of 16*2^k tokens).
+inline bool chunk_map_supported(const Geometry& g, uint32_t q_token_tile_size) {
+    const uint32_t p = g.tokens_per_page;
+    return (g.dtype == PSI_HIP_BF16 || g.dtype == PSI_HIP_F16) && g.d == 256 && p >= 16 && (p & (p - 1)) == 0 &&
+           q_token_tile_size > 0 && chunk_group_tiles(g.group, q_token_tile_size) >= 1;
+}
+
 // Shape-generic kernels (any head_dim / page size / element type), SingleQ and TiledQ layouts.
 void launch_map_generic(psi_hip_ctx* ctx, const Geometry& g, const MapArgs& a);
 void launch_reduce_generic(psi_hip_ctx* ctx, const Geometry& g, const ReduceArgs& a, uint32_t num_total_tokens);
@@ -84,5 +102,8 @@ int launch_reduce_fast(psi_hip_ctx* ctx, const Geometry& g, const ReduceArgs& a)
 int launch_decode_map_valu(psi_hip_ctx* ctx, const Geometry& g, const MapArgs& a);
 // MFMA TiledQ map for bf16 / f16, head_dim 256 / 128; PSI_HIP_ERR_UNSUPPORTED outside its domain.
 int launch_tiled_map_fast(psi_hip_ctx* ctx, const Geometry& g, const MapArgs& a);
+// MFMA prefill-chunk map over row groups; PSI_HIP_ERR_UNSUPPORTED outside chunk_map_supported().
+int launch_chunk_map(psi_hip_ctx* ctx, const Geometry& g, const MapArgs& a, const uint32_t* row_groups,
+                     uint32_t group_tiles, uint32_t num_groups);
 
 }  // namespace psi

@@ -1,0 +1,451 @@
+// gfx950 split-KV map for prefill chunks: many query tokens of one request against one KV range,
+// 2-byte K/V (bf16 / f16), head_dim 256, pages of 16*2^k tokens.  Same results as the
+// multi-query map (semantics of
+// crates/inference-backend-metal/src/components/metal/gqa_split_kv_tiled_q.metal:49-319), other
+// decomposition: the matrix cores are the bound here, not HBM.
+//
+// Work decomposition
+//   one workgroup (4 waves) = one (row group, kv_head).  A row group is a run of consecutive
+//   Q-token tiles of one request whose kv_split rows start at the same key (the rows of one KV
+//   partition).  With more than 5 query heads per KV head the heads are dealt to two workgroups.
+//   The workgroup's query columns, column c = token_in_group * heads + head, are dealt out 32 per
+//   wave: a wave keeps the online-softmax state and the accumulators of its columns for the whole
+//   KV range, so wave states never merge.  The four waves walk the KV range together in tiles of
+//   32 keys which they load once, together, into LDS (two buffers, one barrier per tile).
+//
+// Per 32-key tile and wave (2 column blocks of 16)
+//   QK^T  S[key][column] on v_mfma_f32_16x16x32: A = K rows from LDS, B = the query columns, staged
+//         once in LDS in operand order.  Row i of key block b is key 8*(i/4) + 4*b + i%4, so
+//         that a lane ends up with keys 8*(lane/16) .. +7 of its column: the B-operand layout of
+//         the next contraction.
+//   softmax  per column, in-lane over 8 keys plus two cross-lane steps; masks only on tiles that
+//         touch the start of the range or a column's causal limit.  The reference maximum of a
+//         column moves only when a tile exceeds it by more than 2^8, so the accumulators are
+//         rescaled a handful of times per range; probabilities stay below 2^8.
+//   PV    O^T[dim][column] += V^T[dim][key] * P^T[key][column] on v_mfma_f32_16x16x32: A = V^T
+//         from LDS (the tile is transposed once, on its way into LDS, so that a lane reads its 8
+//         keys of one dim as one 128-bit word), B = the probabilities from registers.  The
+//         accumulators keep a column per lane, so rescaling needs no cross-lane traffic.  bf16
+//         probabilities are two truncated bf16 terms (two MFMAs), f16 one rounded term.
+//
+// Registers: 128 accumulators + operands stay inside the 256 architectural VGPRs, so every MFMA
+// reads and writes them in place.
+//
+// LDS layout per buffer
+//   K    [32 keys][D] elements, 16-byte chunk index XOR (key%4 + 4*((key/8)%2)): conflict-free for
+//        both the row-wise stores and the operand reads.
+//   V^T  [D dims][32 keys] elements, 16 bytes of padding after every 8 rows.
+#pragma once
+#include "split_kv_tiled_kernel.h"
+
+namespace psi {
+
+constexpr int kChunkKeys = 32;         // keys per KV tile
+constexpr int kChunkWaves = 4;
+constexpr int kChunkColBlocks = 2;     // 16-column blocks per wave
+constexpr int kChunkWaveCols = 16 * kChunkColBlocks;
+static_assert(kChunkWaves * kChunkWaveCols == kChunkCols, "128 query columns per workgroup");
+constexpr uint32_t kNoRow = 0xffffffffu;
+typedef __attribute__((ext_vector_type(4))) uint32_t u32x4_t;  // 128-bit word that stays in registers
+
+// Probabilities of 8 keys -> B operand(s) of the 16x16x32 contraction.
+template <typename Tag>
+struct ProbOperand8;
+template <>
+struct ProbOperand8<BF16Tag> {
+    static constexpr int kTerms = 2;
+    uint4 term[2];
+    __device__ __forceinline__ void set(const float (&p)[8]) {
+        uint32_t hi[8], lo[8];
+#pragma unroll
+        for (int j = 0; j < 8; ++j) {
+            hi[j] = __float_as_uint(p[j]) & 0xffff0000u;
+            lo[j] = __float_as_uint(p[j] - __uint_as_float(hi[j]));
+        }
+        term[0] = make_uint4((hi[0] >> 16) | hi[1], (hi[2] >> 16) | hi[3], (hi[4] >> 16) | hi[5], (hi[6] >> 16) | hi[7]);
+        term[1] = make_uint4((lo[0] >> 16) | (lo[1] & 0xffff0000u), (lo[2] >> 16) | (lo[3] & 0xffff0000u),
+                             (lo[4] >> 16) | (lo[5] & 0xffff0000u), (lo[6] >> 16) | (lo[7] & 0xffff0000u));
+    }
+};
+template <>
+struct ProbOperand8<F16Tag> {
+    static constexpr int kTerms = 1;
+    uint4 term[1];
+    __device__ __forceinline__ void set(const float (&p)[8]) {
+        const f16x8_t h = {(_Float16)p[0], (_Float16)p[1], (_Float16)p[2], (_Float16)p[3],
+                           (_Float16)p[4], (_Float16)p[5], (_Float16)p[6], (_Float16)p[7]};
+        term[0] = __builtin_bit_cast(uint4, h);
+    }
+};
+
+__device__ __forceinline__ uint32_t wave_min_u32(uint32_t v) {
+#pragma unroll
+    for (int s = 1; s < 64; s <<= 1) v = min(v, (uint32_t)__shfl_xor((int)v, s, 64));
+    return v;
+}
+__device__ __forceinline__ uint32_t wave_max_u32(uint32_t v) {
+#pragma unroll
+    for (int s = 1; s < 64; s <<= 1) v = max(v, (uint32_t)__shfl_xor((int)v, s, 64));
+    return v;
+}
+
+template <int D>
+struct ChunkLds {
+    static constexpr int kKBytes = kChunkKeys * D * 2;
+    static constexpr int kVtBytes = D * kChunkKeys * 2 + (D / 8) * 16;
+    static constexpr int kQBytes = kChunkCols * D * 2;
+    static constexpr int bytes = 2 * (kKBytes + kVtBytes) + kQBytes;
+};
+
+template <typename Tag, int D>
+__global__ __launch_bounds__(64 * kChunkWaves, 2) void split_kv_chunk_map(
+    MapArgs a, const uint32_t* __restrict__ page_ids, const uint32_t* __restrict__ kv_splits,
+    const uint32_t* __restrict__ req_slots, const uint16_t* __restrict__ q, const uint16_t* __restrict__ pages,
+    const uint32_t* __restrict__ q_token_tiles, const uint32_t* __restrict__ flat_token_indices,
+    const uint32_t* __restrict__ row_groups, uint32_t group_tiles, uint32_t num_groups, uint32_t head_subsets) {
+    static_assert(D == 256, "the tile loaders are laid out for head_dim 256");
+    constexpr int kKSteps = D / 32;              // MFMA k-steps of QK^T
+    constexpr int kDimBlocks = D / 16;           // 16-dim output blocks of PV
+    constexpr int kRowChunks = D / 8;            // 16-byte chunks per K row
+    constexpr int kLoads = kChunkKeys * kRowChunks / (64 * kChunkWaves);  // 128-bit loads per thread and operand (4)
+    constexpr int kKBytes = ChunkLds<D>::kKBytes;
+    constexpr int kVtBytes = ChunkLds<D>::kVtBytes;
+    constexpr int kBufBytes = kKBytes + kVtBytes;
+    constexpr int CB = kChunkColBlocks;
+    constexpr float kSlack = 8.0f;
+    // Dynamic LDS (the launcher passes ChunkLds<D>::bytes): with a static size the compiler sees
+    // that one workgroup fills the CU and lifts the register cap that keeps the accumulators in
+    // architectural VGPRs.
+    extern __shared__ __attribute__((aligned(16))) unsigned char lds[];
+    uint4* qb_lds = reinterpret_cast<uint4*>(lds + 2 * kBufBytes);  // [wave][cb][ks][lane]
+
+    const uint32_t TS = a.rows_per_split_head;  // Q tokens per tile
+    // heads of the KV head served here: head_first + [0, G)
+    const uint32_t subset = blockIdx.x % head_subsets;
+    const uint32_t kv_head = (blockIdx.x / head_subsets) % a.walk.hkv;
+    const uint32_t group = blockIdx.x / (head_subsets * a.walk.hkv);
+    const uint32_t heads_per_subset = (a.group + head_subsets - 1) / head_subsets;
+    const uint32_t head_first = kv_head * a.group + subset * heads_per_subset;
+    const uint32_t G = min(heads_per_subset, a.group - subset * heads_per_subset);
+    const uint32_t tid = threadIdx.x;
+    const uint32_t lane = tid & 63;
+    const uint32_t wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const uint32_t mt = lane & 15, mc = lane >> 4;
+    if (group >= num_groups) return;
+
+    // ---- the group: rows[m] is the kv_split row of its m-th Q-token tile
+    const uint32_t* rows = row_groups + (uint64_t)group * group_tiles;
+    const uint32_t my_row = lane < group_tiles ? rows[lane] : kNoRow;
+    const bool my_row_ok = my_row != kNoRow && my_row < a.num_active_kv_splits;
+    const uint32_t num_tiles = __builtin_amdgcn_readfirstlane(__popcll(__ballot(my_row_ok)));
+    if (num_tiles == 0) return;
+    const uint32_t row0 = __builtin_amdgcn_readfirstlane(rows[0]);
+    if (row0 >= a.num_active_kv_splits) return;
+    const uint32_t q_tile0 = kv_splits[row0 * 3];
+    if (q_tile0 >= a.num_active_q_token_tiles || q_tile0 + num_tiles > a.num_active_q_token_tiles) return;
+    const uint32_t kv_begin = kv_splits[row0 * 3 + 1];
+    const uint32_t kv_end_max = wave_max_u32(my_row_ok && lane < num_tiles ? kv_splits[my_row * 3 + 2] : 0u);
+    const uint32_t flat_begin = q_token_tiles[q_tile0 * 2];
+    const uint32_t flat_end = q_token_tiles[(q_tile0 + num_tiles - 1) * 2 + 1];
+    if (flat_end <= flat_begin || flat_end > a.num_active_tokens || kv_end_max <= kv_begin) return;
+    const uint32_t ncols = (flat_end - flat_begin) * G;
+    if (ncols > (uint32_t)kChunkCols || flat_end - flat_begin > num_tiles * TS) return;  // the planner never builds such a group
+    const uint32_t req_slot = req_slots[flat_begin];
+
+    // ---- this lane's columns: c = 32 * wave + 16 * cb + mt; their query rows go to LDS as B operands
+    // (dims 32 * ks + 8 * mc .. +8), zero for unused columns.  Only this wave reads them back.
+    uint32_t lim[CB];        // keys [kv_begin, lim) are visible to the column; 0: column unused
+    uint64_t part_row[CB];   // partial-state row of the column
+    uint4* my_q = qb_lds + wave * (CB * kKSteps * 64) + lane;
+    uint32_t lo_lim = 0xffffffffu, hi_lim = 0;
+#pragma unroll
+    for (int cb = 0; cb < CB; ++cb) {
+        const uint32_t c = wave * kChunkWaveCols + cb * 16 + mt;
+        const bool used = c < ncols;
+        const uint32_t t = used ? c / G : 0u, h = used ? c % G : 0u;
+        const uint32_t m = t / TS, r = t % TS;
+        const uint32_t row = rows[m];
+        lim[cb] = 0;
+        part_row[cb] = 0;
+        if (used) {
+            lim[cb] = min(kv_splits[row * 3 + 2], flat_token_indices[flat_begin + t] + 1);
+            part_row[cb] = ((uint64_t)row * a.hq + head_first + h) * TS + r;
+            lo_lim = min(lo_lim, lim[cb]);
+            hi_lim = max(hi_lim, lim[cb]);
+        }
+        const uint16_t* q_row = q + ((uint64_t)(flat_begin + t) * a.hq + head_first + h) * D + mc * 8;
+#pragma unroll
+        for (int ks = 0; ks < kKSteps; ++ks)
+            my_q[(cb * kKSteps + ks) * 64] = used ? *reinterpret_cast<const uint4*>(q_row + ks * 32) : make_uint4(0, 0, 0, 0);
+    }
+    // Tiles at or beyond wave_hi hold no visible key for this wave; tiles inside [kv_begin, wave_lo)
+    // need no mask.
+    const uint32_t wave_lo = __builtin_amdgcn_readfirstlane(wave_min_u32(lo_lim));
+    const uint32_t wave_hi = __builtin_amdgcn_readfirstlane(wave_max_u32(hi_lim));
+
+    // ---- page walk and the cooperative tile loaders
+    const uint32_t log2p = 31 - __builtin_clz(a.walk.tokens_per_page);
+    const uint32_t page_mask = a.walk.tokens_per_page - 1;
+    const uint32_t* table_row = page_ids + ((uint64_t)req_slot * a.walk.num_layers + a.layer) *
+                                                      a.walk.num_blocks * a.walk.ids_per_block;
+    const uint64_t v_region = (uint64_t)a.walk.hkv * a.walk.tokens_per_page * D;
+    const uint32_t last_page = (kv_end_max - 1) >> log2p;
+    const uint32_t key_base0 = kv_begin & ~(uint32_t)(kChunkKeys - 1);
+    const uint32_t num_kv_tiles = (kv_end_max - key_base0 + kChunkKeys - 1) / kChunkKeys;
+
+    struct TileIds {
+        uint32_t a, b;  // page of keys 0..15 and of keys 16..31 of the tile
+    };
+    auto load_ids = [&](uint32_t it) -> TileIds {
+        TileIds p{0u, 0u};
+        if (it < num_kv_tiles) {
+            const uint32_t kb = key_base0 + it * kChunkKeys;
+            p.a = table_row[min(kb >> log2p, last_page)];
+            p.b = table_row[min((kb + 16) >> log2p, last_page)];
+        }
+        return p;
+    };
+    const uint32_t ld_chunk = tid % kRowChunks;   // 16-byte chunk of a row (8 dims)
+    const uint32_t ld_sub = tid / kRowChunks;     // 0..7
+    struct Staging {
+        u32x4_t k[kLoads], v[kLoads];
+    };
+    // K: load j takes key 8 * j + ld_sub; V: load j takes key 4 * ld_sub + j (4 keys of one chunk).
+    auto issue_loads = [&](uint32_t it, TileIds p) __attribute__((always_inline)) -> Staging {
+        Staging st;
+        const uint32_t kb = key_base0 + it * kChunkKeys;
+#pragma unroll
+        for (int j = 0; j < kLoads; ++j) {
+            const uint32_t key = 8 * j + ld_sub;
+            const uint32_t page = j < kLoads / 2 ? p.a : p.b;
+            const uint16_t* src = pages + (uint64_t)page * a.walk.page_elems +
+                                  ((uint64_t)kv_head * a.walk.tokens_per_page + ((kb + key) & page_mask)) * D + ld_chunk * 8;
+            st.k[j] = *reinterpret_cast<const u32x4_t*>(src);
+        }
+        const uint32_t vpage = ld_sub < 4 ? p.a : p.b;
+#pragma unroll
+        for (int j = 0; j < kLoads; ++j) {
+            const uint32_t key = 4 * ld_sub + j;
+            const uint16_t* src = pages + (uint64_t)vpage * a.walk.page_elems + v_region +
+                                  ((uint64_t)kv_head * a.walk.tokens_per_page + ((kb + key) & page_mask)) * D + ld_chunk * 8;
+            st.v[j] = *reinterpret_cast<const u32x4_t*>(src);
+        }
+        return st;
+    };
+    // Registers -> LDS buffer `buf`.  V rows outside [kv_begin, kv_end_max) are zeroed: their
+    // probability is 0 but their bytes may be NaN / Inf.
+    auto store_tile = [&](uint32_t it, uint32_t buf, const Staging& st) __attribute__((always_inline)) {
+        unsigned char* kbuf = lds + buf * kBufBytes;
+        unsigned char* vbuf = kbuf + kKBytes;
+        const uint32_t kb = key_base0 + it * kChunkKeys;
+#pragma unroll
+        for (int j = 0; j < kLoads; ++j) {
+            const uint32_t key = 8 * j + ld_sub;
+            const uint32_t swz = (ld_sub & 3) + 4 * (j & 1);
+            *reinterpret_cast<u32x4_t*>(kbuf + key * (D * 2) + ((ld_chunk ^ swz) * 16)) = st.k[j];
+        }
+        uint32_t w[kLoads][4];
+#pragma unroll
+        for (int j = 0; j < kLoads; ++j) {
+            const uint32_t token = kb + 4 * ld_sub + j;
+            const bool live = token >= kv_begin && token < kv_end_max;
+            w[j][0] = live ? st.v[j][0] : 0u;
+            w[j][1] = live ? st.v[j][1] : 0u;
+            w[j][2] = live ? st.v[j][2] : 0u;
+            w[j][3] = live ? st.v[j][3] : 0u;
+        }
+        static_assert(kLoads == 4, "the transposing store packs 4 keys per 64-bit word");
+#pragma unroll
+        for (int e = 0; e < 8; ++e) {
+            const int word = e / 2;
+            uint2 out;
+            if (e % 2 == 0) {
+                out.x = (w[0][word] & 0xffffu) | (w[1][word] << 16);
+                out.y = (w[2][word] & 0xffffu) | (w[3][word] << 16);
+            } else {
+                out.x = (w[0][word] >> 16) | (w[1][word] & 0xffff0000u);
+                out.y = (w[2][word] >> 16) | (w[3][word] & 0xffff0000u);
+            }
+            // row = 8 * ld_chunk + e; 64 bytes per row, 16 bytes of padding per 8 rows
+            *reinterpret_cast<uint2*>(vbuf + (8 * ld_chunk + e) * 64 + ld_chunk * 16 + ld_sub * 8) = out;
+        }
+    };
+
+    // ---- operand read addresses of this lane
+    // K row of (block b, lane row mt): key 8 * (mt / 4) + 4 * b + mt % 4, chunk (4 * ks + mc) ^ swizzle
+    const uint32_t k_swz = (mt & 3) + 4 * ((mt >> 2) & 1);
+    const uint32_t k_row0 = (8 * (mt >> 2) + (mt & 3)) * (D * 2);
+    // V^T row of (dim block db, lane row mt): dim 16 * db + mt, keys 8 * mc .. +7
+    const uint32_t vt_row0 = mt * 64 + (mt >> 3) * 16 + mc * 16;
+
+    float run_max[CB], lane_sum[CB];
+    f32x4_t o[CB][kDimBlocks];
+#pragma unroll
+    for (int cb = 0; cb < CB; ++cb) {
+        run_max[cb] = -INFINITY;
+        lane_sum[cb] = 0.0f;
+#pragma unroll
+        for (int db = 0; db < kDimBlocks; ++db) o[cb][db] = f32x4_t{0.0f, 0.0f, 0.0f, 0.0f};
+    }
+    const bool wave_has_cols = wave * kChunkWaveCols < ncols;
+
+    // `masked`: the tile touches the start of the range or a causal limit of this wave (wave-uniform).
+    // One instantiation on purpose: two copies of this body under an if / else made the register
+    // allocator spill half of the accumulators.
+    auto compute_tile = [&](uint32_t it, uint32_t buf, bool masked) __attribute__((always_inline)) {
+        const unsigned char* kbuf = lds + buf * kBufBytes;
+        const unsigned char* vbuf = kbuf + kKBytes;
+        const uint32_t kb = key_base0 + it * kChunkKeys;
+        // ---- logits S[key][column]: two key blocks x CB column blocks
+        f32x4_t s[2][CB];
+#pragma unroll
+        for (int b = 0; b < 2; ++b)
+#pragma unroll
+            for (int cb = 0; cb < CB; ++cb) s[b][cb] = f32x4_t{0.0f, 0.0f, 0.0f, 0.0f};
+        // operand reads run one step ahead of the MFMAs that use them; the scheduling fences keep
+        // the compiler from hoisting every read of the tile to its start (register pressure)
+        auto read_k = [&](int ks, uint4& k0, uint4& k1) {
+            const uint32_t off = k_row0 + (((4 * ks + mc) ^ k_swz) * 16);
+            k0 = *reinterpret_cast<const uint4*>(kbuf + off);
+            k1 = *reinterpret_cast<const uint4*>(kbuf + off + 4 * (D * 2));
+        };
+        uint4 kc0, kc1, qc[CB];
+        read_k(0, kc0, kc1);
+#pragma unroll
+        for (int cb = 0; cb < CB; ++cb) qc[cb] = my_q[cb * kKSteps * 64];
+#pragma unroll
+        for (int ks = 0; ks < kKSteps; ++ks) {
+            uint4 kn0 = kc0, kn1 = kc1, qn[CB];
+#pragma unroll
+            for (int cb = 0; cb < CB; ++cb) qn[cb] = qc[cb];
+            if (ks + 1 < kKSteps) {
+                read_k(ks + 1, kn0, kn1);
+#pragma unroll
+                for (int cb = 0; cb < CB; ++cb) qn[cb] = my_q[(cb * kKSteps + ks + 1) * 64];
+            }
+#pragma unroll
+            for (int cb = 0; cb < CB; ++cb) {
+                s[0][cb] = mfma_16x16x32<Tag>(kc0, qc[cb], s[0][cb]);
+                s[1][cb] = mfma_16x16x32<Tag>(kc1, qc[cb], s[1][cb]);
+            }
+            __builtin_amdgcn_sched_barrier(0);
+            kc0 = kn0;
+            kc1 = kn1;
+#pragma unroll
+            for (int cb = 0; cb < CB; ++cb) qc[cb] = qn[cb];
+        }
+        // ---- online softmax; this lane holds keys kb + 8 * mc + j, j = 4 * b + r, of column mt
+        ProbOperand8<Tag> pb[CB];
+        float alpha[CB];
+        bool moved = false;
+#pragma unroll
+        for (int cb = 0; cb < CB; ++cb) {
+            float v[8];
+            bool valid[8];
+            float m = -INFINITY;
+#pragma unroll
+            for (int j = 0; j < 8; ++j) {
+                const uint32_t token = kb + 8 * mc + j;
+                valid[j] = !masked || (token >= kv_begin && token < lim[cb]);
+                v[j] = valid[j] ? s[j / 4][cb][j % 4] * a.scale_log2 : -INFINITY;
+                m = fmaxf(m, v[j]);
+            }
+            m = fmaxf(m, __shfl_xor(m, 16, 64));
+            m = fmaxf(m, __shfl_xor(m, 32, 64));
+            // The reference maximum follows the tile maximum only when that exceeds it by more than
+            // kSlack (log2 domain); a column with no visible key so far keeps max = -inf, sum = 0, O = 0.
+            const bool bump = m > run_max[cb] + kSlack;
+            const float next_max = bump ? m : run_max[cb];
+            alpha[cb] = !bump ? 1.0f : (run_max[cb] > -INFINITY ? __builtin_amdgcn_exp2f(run_max[cb] - next_max) : 0.0f);
+            moved = moved || bump;
+            run_max[cb] = next_max;
+            float p[8], tile_sum = 0.0f;
+#pragma unroll
+            for (int j = 0; j < 8; ++j) {
+                p[j] = valid[j] ? __builtin_amdgcn_exp2f(v[j] - next_max) : 0.0f;
+                tile_sum += p[j];
+            }
+            lane_sum[cb] = lane_sum[cb] * alpha[cb] + tile_sum;
+            pb[cb].set(p);
+        }
+        if (__any(moved)) {
+#pragma unroll
+            for (int cb = 0; cb < CB; ++cb)
+#pragma unroll
+                for (int db = 0; db < kDimBlocks; ++db)
+#pragma unroll
+                    for (int r = 0; r < 4; ++r) o[cb][db][r] *= alpha[cb];
+        }
+        // ---- O^T[dim][column] += V^T * P^T
+        auto read_vt = [&](int db) { return *reinterpret_cast<const uint4*>(vbuf + vt_row0 + db * (16 * 64 + 32)); };
+        uint4 vc = read_vt(0);
+        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+        for (int db = 0; db < kDimBlocks; ++db) {
+            uint4 vn = vc;
+            if (db + 1 < kDimBlocks) vn = read_vt(db + 1);
+#pragma unroll
+            for (int t = 0; t < ProbOperand8<Tag>::kTerms; ++t)
+#pragma unroll
+                for (int cb = 0; cb < CB; ++cb) o[cb][db] = mfma_16x16x32<Tag>(vc, pb[cb].term[t], o[cb][db]);
+            __builtin_amdgcn_sched_barrier(0);
+            vc = vn;
+        }
+    };
+
+    // ---- main loop: tile it in buffer it % 2
+    {
+        const TileIds p0 = load_ids(0);
+        const Staging st = issue_loads(0, p0);
+        store_tile(0, 0, st);
+    }
+    TileIds ids_next = load_ids(1);
+    __syncthreads();
+    for (uint32_t it = 0; it < num_kv_tiles; ++it) {
+        const bool has_next = it + 1 < num_kv_tiles;
+        const TileIds ids_after = load_ids(it + 2);
+        Staging st;
+        if (has_next) st = issue_loads(it + 1, ids_next);
+        const uint32_t kb = key_base0 + it * kChunkKeys;
+        if (wave_has_cols && kb < wave_hi) {
+            compute_tile(it, it & 1, !(kb >= kv_begin && kb + kChunkKeys <= wave_lo));
+        }
+        if (has_next) store_tile(it + 1, (it + 1) & 1, st);
+        ids_next = ids_after;
+        __syncthreads();
+    }
+
+    // ---- emit this wave's columns: un-normalised accumulators, log2-domain maximum, sum
+#pragma unroll
+    for (int cb = 0; cb < CB; ++cb) {
+        lane_sum[cb] += __shfl_xor(lane_sum[cb], 16, 64);
+        lane_sum[cb] += __shfl_xor(lane_sum[cb], 32, 64);
+        if (lim[cb] != 0) {
+            if (mc == 0) {
+                a.part_max[part_row[cb]] = run_max[cb];
+                a.part_sum[part_row[cb]] = lane_sum[cb];
+            }
+            float* dst = a.part_acc + part_row[cb] * D + mc * 4;
+#pragma unroll
+            for (int db = 0; db < kDimBlocks; ++db)
+                *reinterpret_cast<float4*>(dst + db * 16) = make_float4(o[cb][db][0], o[cb][db][1], o[cb][db][2], o[cb][db][3]);
+        }
+    }
+}
+
+template <typename Tag, int D>
+inline int launch_chunk_map_typed(psi_hip_ctx* ctx, const Geometry& g, const MapArgs& a, const uint32_t* row_groups,
+                                  uint32_t group_tiles, uint32_t num_groups) {
+    const uint32_t subsets = chunk_head_subsets(g.group);
+    const dim3 grid(num_groups * g.hkv * subsets);
+    static const hipError_t lds_ok = hipFuncSetAttribute(reinterpret_cast<const void*>(&split_kv_chunk_map<Tag, D>),
+                                                         hipFuncAttributeMaxDynamicSharedMemorySize, ChunkLds<D>::bytes);
+    if (lds_ok != hipSuccess) return PSI_HIP_ERR_UNSUPPORTED;
+    hipLaunchKernelGGL((split_kv_chunk_map<Tag, D>), grid, dim3(64 * kChunkWaves), ChunkLds<D>::bytes, ctx->stream, a, a.walk.page_ids,
+                       a.kv_splits, a.req_slots, reinterpret_cast<const uint16_t*>(a.q),
+                       reinterpret_cast<const uint16_t*>(a.kv_pages), a.q_token_tiles, a.flat_token_indices, row_groups,
+                       group_tiles, num_groups, subsets);
+    return PSI_HIP_OK;
+}
+
+}  // namespace psi

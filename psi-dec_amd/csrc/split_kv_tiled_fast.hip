@@ -9,6 +9,21 @@ int launch_tiled_map_bf16_d128(psi_hip_ctx* ctx, const Geometry& g, const MapArg
 int launch_tiled_map_f16_d256(psi_hip_ctx* ctx, const Geometry& g, const MapArgs& a, uint32_t max_tile_tokens);
 int launch_tiled_map_f16_d128(psi_hip_ctx* ctx, const Geometry& g, const MapArgs& a, uint32_t max_tile_tokens);
 
+int launch_chunk_map_bf16_d256(psi_hip_ctx* ctx, const Geometry& g, const MapArgs& a, const uint32_t* row_groups,
+                               uint32_t group_tiles, uint32_t num_groups);
+int launch_chunk_map_f16_d256(psi_hip_ctx* ctx, const Geometry& g, const MapArgs& a, const uint32_t* row_groups,
+                              uint32_t group_tiles, uint32_t num_groups);
+
+int launch_chunk_map(psi_hip_ctx* ctx, const Geometry& g, const MapArgs& a, const uint32_t* row_groups,
+                     uint32_t group_tiles, uint32_t num_groups) {
+    if (ctx->force_generic || !chunk_map_supported(g, a.rows_per_split_head)) return PSI_HIP_ERR_UNSUPPORTED;
+    const bool aligned = reinterpret_cast<uintptr_t>(a.q) % 16 == 0 && reinterpret_cast<uintptr_t>(a.kv_pages) % 16 == 0;
+    if (!aligned || group_tiles == 0 || group_tiles > chunk_group_tiles(g.group, a.rows_per_split_head)) return PSI_HIP_ERR_UNSUPPORTED;
+    if ((uint64_t)num_groups * g.hkv * chunk_head_subsets(g.group) > 0x7fffffffull) return PSI_HIP_ERR_UNSUPPORTED;
+    return g.dtype == PSI_HIP_BF16 ? launch_chunk_map_bf16_d256(ctx, g, a, row_groups, group_tiles, num_groups)
+                                   : launch_chunk_map_f16_d256(ctx, g, a, row_groups, group_tiles, num_groups);
+}
+
 int launch_tiled_map_fast(psi_hip_ctx* ctx, const Geometry& g, const MapArgs& a) {
     if (ctx->force_generic) return PSI_HIP_ERR_UNSUPPORTED;
     const bool two_byte = g.dtype == PSI_HIP_BF16 || g.dtype == PSI_HIP_F16;

@@ -401,6 +401,8 @@ class GQAMetadataBuffers:
         self.d_req_slots = self.d_flat_token_indices = self.d_q_token_tiles = None
         self.d_kv_splits = self.d_cu_kv_splits = None
         self.h_partial_row_index = self.d_partial_row_index = None
+        self.h_row_groups = self.d_row_groups = None
+        self.group_tiles = self.num_row_groups = 0
 
     def max_tokens(self) -> int:
         return self._max_tokens
@@ -424,6 +426,8 @@ class GQAMetadataBuffers:
                                      bool(shape.reduce_sdpa_partial_outputs))
         self._variant = variant
         self.h_partial_row_index = self.d_partial_row_index = None  # rows are in plan order again
+        self.h_row_groups = self.d_row_groups = None
+        self.group_tiles = self.num_row_groups = 0
         if self.device is not None:
             self.upload()
         return self._shape
@@ -473,6 +477,30 @@ class GQAMetadataBuffers:
             self.upload()
             self.d_partial_row_index = self.device.from_numpy(self.h_partial_row_index)
         return self.h_partial_row_index
+
+    def group_rows(self, config) -> int:
+        """Row groups of the current TiledQ plan for the prefill-chunk map
+        (psi_hip_split_kv_tiled_q_group_rows); `config` is the kernels' GQASplitKVTiledQConfig.
+        Returns the number of groups, 0 when the geometry has no grouped kernel.  Call after any
+        re-ordering of the rows: the table holds row positions."""
+        s = self._shape
+        assert s is not None and self._variant.is_tiled()
+        n = s.num_sdpa_map_task_templates
+        table = np.full(max(n, 1) * 32, L.SENTINEL, np.uint32)
+        tiles, groups = ctypes.c_uint32(), ctypes.c_uint32()
+        cfg = config.struct()
+
+        def p(a):
+            return a.ctypes.data_as(ctypes.POINTER(ctypes.c_uint32))
+
+        L.check(L.load().psi_hip_split_kv_tiled_q_group_rows(
+            ctypes.byref(cfg), config.q_token_tile_size, p(self.h_kv_splits), n, p(self.h_q_token_tiles),
+            s.num_q_token_tiles, p(self.h_req_slots), p(table), len(table), ctypes.byref(tiles), ctypes.byref(groups)))
+        self.group_tiles, self.num_row_groups = tiles.value, groups.value
+        self.h_row_groups = table[:max(tiles.value * groups.value, 1)].copy()
+        if self.device is not None and groups.value:
+            self.d_row_groups = self.device.from_numpy(self.h_row_groups)
+        return groups.value
 
     def balance(self, num_workers: int):
         """Re-cuts the current SingleQ plan into rows grouped for `num_workers` equal-work decode
@@ -729,6 +757,21 @@ class GQASplitKVTiledQKernels:
             _ptr(q_token_tiles), _ptr(sdpa_map_task_templates), _ptr(scratch.buffer), scratch.bytes,
             page_table_index, s.num_total_tokens, s.num_total_q_token_tiles, s.num_total_sdpa_map_task_templates,
             num_active_tokens, num_active_q_token_tiles, num_active_kv_splits, max_active_q_tile_tokens))
+
+    def invoke_map_grouped(self, q, kv_pages, req_slots, page_ids, flat_token_indices, q_token_tiles,
+                           sdpa_map_task_templates, scratch, page_table_index: int, num_active_tokens: int,
+                           num_active_q_token_tiles: int, num_active_kv_splits: int, row_groups, group_tiles: int,
+                           num_groups: int, max_active_q_tile_tokens: int = 0):
+        """The map with one workgroup per row group (prefill chunks); `row_groups` is the device copy
+        of GQAMetadataBuffers.group_rows()."""
+        cfg, layout, s = self.config.struct(), self.config.page_table_layout.struct(), self.shape
+        L.check(self.device.lib.psi_hip_split_kv_tiled_q_map_grouped(
+            self.device.ctx, ctypes.byref(cfg), ctypes.byref(layout), self.config.q_token_tile_size, _ptr(q),
+            _ptr(kv_pages), _nbytes(kv_pages), _ptr(req_slots), _ptr(page_ids), _ptr(flat_token_indices),
+            _ptr(q_token_tiles), _ptr(sdpa_map_task_templates), _ptr(scratch.buffer), scratch.bytes,
+            page_table_index, s.num_total_tokens, s.num_total_q_token_tiles, s.num_total_sdpa_map_task_templates,
+            num_active_tokens, num_active_q_token_tiles, num_active_kv_splits, max_active_q_tile_tokens,
+            _ptr(row_groups), group_tiles, num_groups))
 
     def invoke_reduce(self, scratch, q_token_tiles, cu_sdpa_partial_outputs, output):
         self.invoke_reduce_bucketed(scratch, q_token_tiles, cu_sdpa_partial_outputs, output,

@@ -145,7 +145,8 @@ class DeviceWorkload:
 
     def __init__(self, device: G.Device, w: Workload, partition_tokens: Optional[int] = None,
                  max_tokens: Optional[int] = None, variant: Optional[G.GQASplitKVVariant] = None,
-                 f32_output: bool = False, balanced: bool = False, longest_first: bool = False):
+                 f32_output: bool = False, balanced: bool = False, longest_first: bool = False,
+                 grouped: bool = False):
         import torch
 
         self.device, self.w = device, w
@@ -219,6 +220,9 @@ class DeviceWorkload:
             self.kernels = G.GQASplitKVSingleQKernels(device, self.cfg, self.kshape)
             self.scratch = G.GQASplitKVSingleQScratch(device, self.cfg, self.kshape)
         self._rows = rows
+        self.grouped = bool(grouped) and variant.is_tiled()
+        if self.grouped:
+            self.meta.group_rows(self.cfg)
 
     def append(self):
         m = self.meta
@@ -230,7 +234,15 @@ class DeviceWorkload:
 
     def map(self):
         m, s = self.meta, self.shape
-        if self.variant.is_tiled():
+        if self.variant.is_tiled() and self.grouped and m.num_row_groups:
+            self.kernels.invoke_map_grouped(self.q, self.pages, m.d_req_slots, self.page_ids,
+                                            m.d_flat_token_indices, m.d_q_token_tiles, m.d_kv_splits, self.scratch,
+                                            self.w.layer, s.num_tokens, s.num_q_token_tiles,
+                                            s.num_sdpa_map_task_templates, m.d_row_groups, m.group_tiles,
+                                            m.num_row_groups,
+                                            min(int(np.diff(self.w.cu_tokens).max()),
+                                                self.variant.q_token_tile_size))
+        elif self.variant.is_tiled():
             self.kernels.invoke_map_bucketed(self.q, self.pages, m.d_req_slots, self.page_ids,
                                              m.d_flat_token_indices, m.d_q_token_tiles, m.d_kv_splits, self.scratch,
                                              self.w.layer, s.num_tokens, s.num_q_token_tiles,

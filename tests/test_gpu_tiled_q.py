@@ -226,3 +226,54 @@ def test_mfma_and_generic_kernels_agree_but_differ_in_rounding(psi, oracle, devi
         device.force_generic(False)
     assert np.abs(a - b).max() < 2e-4
     assert not np.array_equal(a, b)
+
+
+@pytest.mark.parametrize("partition,prefix,chunk", [(256, 300, 200), (512, 0, 77), (128, 1000, 64), (2048, 37, 300)])
+def test_grouped_prefill_chunk(psi, oracle, device, partition, prefix, chunk):
+    """The row-group map (K/V tiles staged once in LDS for up to 128 query columns) on a chunk next to
+    decode-sized requests: same tolerance against the oracle as every other path."""
+    wl = importlib_workloads(psi)
+    q_lens = [chunk, 1, 3, 8]
+    ctx = [prefix + chunk, 700, 64, 8]
+    w = wl.make_workload(91, ctx, 24, 4, 256, psi.Dtype.Bfloat16, 16, q_lens=q_lens)
+    stats, dw = run_and_check(psi, oracle, device, w, f"grouped chunk {chunk} on {prefix}", partition_tokens=partition,
+                              max_tokens=512, grouped=True, variant=psi.GQASplitKVVariant.TiledQ(8, 16, 6))
+    assert dw.meta.num_row_groups > 0 and dw.meta.group_tiles == 5
+    print("grouped chunk max_abs %.3e rel_rms %.3e" % stats, dw.shape, dw.meta.num_row_groups)
+
+
+@pytest.mark.parametrize("dtype_name,hq,hkv,p,q_len", [
+    ("Float16", 16, 2, 16, 50),    # 8 heads per KV head: two head subsets of 4, f16 single-term P
+    ("Bfloat16", 4, 4, 32, 130),   # one head per KV head: 16 tiles per group, 32-token pages
+    ("Bfloat16", 10, 2, 64, 41),   # 5 heads per KV head: one subset, 3 tiles per group
+    ("Bfloat16", 14, 2, 16, 23),   # 7 heads: subsets of 4 and 3
+])
+def test_grouped_geometries(psi, oracle, device, dtype_name, hq, hkv, p, q_len):
+    wl = importlib_workloads(psi)
+    dtype = getattr(psi.Dtype, dtype_name)
+    w = wl.make_workload(93, [300, 31 + q_len, q_len], hq, hkv, 256, dtype, p, q_lens=[q_len, q_len, q_len],
+                         num_page_ids_per_block=2)
+    variant = psi.GQASplitKVVariant.TiledQ(8, 16, min(hq // hkv, 8))
+    _, dw = run_and_check(psi, oracle, device, w, f"grouped {dtype_name} {hq}/{hkv} P={p} q={q_len}", max_tokens=512,
+                          variant=variant, partition_tokens=128, grouped=True)
+    assert dw.meta.num_row_groups > 0
+
+
+def test_grouped_and_plain_maps_agree(psi, oracle, device):
+    """Same plan through both maps: the outputs differ only in rounding, the grouped table falls
+    back to the plain map where the geometry has no grouped kernel (8-token pages)."""
+    wl = importlib_workloads(psi)
+    for p, expect_groups in [(16, True), (8, False)]:
+        w = wl.make_workload(95, [900, 450], 24, 4, 256, psi.Dtype.Bfloat16, p, q_lens=[300, 450])
+        outs = []
+        for grouped in (False, True):
+            dw = wl.DeviceWorkload(device, w, partition_tokens=256, max_tokens=1024, f32_output=True, grouped=grouped,
+                                   variant=psi.GQASplitKVVariant.TiledQ(8, 16, 6))
+            dw.step()
+            outs.append(dw.output_f32())
+            if grouped:
+                assert (dw.meta.num_row_groups > 0) == expect_groups
+        diff = np.abs(outs[0] - outs[1]).max()
+        assert diff < 1e-3, diff
+        if not expect_groups:
+            assert diff == 0.0

@@ -452,3 +452,100 @@ def test_longest_first_order(psi):
     assert got[:6] == [[0, 0, 512], [2, 0, 512], [2, 512, 1024], [0, 512, 700], [1, 0, 40], [2, 1024, 1030]]
     assert got[6:] == [[MAX, MAX, MAX]] * 2
     assert index.tolist() == [0, 3, 4, 1, 2, 5, 6, 7]
+
+
+# ------------------------------------------------------------------ row groups of prefill chunks
+
+
+def tiled_config(psi, hq, hkv, d=256, p=16, dtype=None):
+    dtype = psi.Dtype.Bfloat16 if dtype is None else dtype
+    layout = psi.GQAPageTableLayout(8, 1, 64, 1)
+    return psi.GQASplitKVTiledQConfig(hq, hkv, d, hq // hkv, 8, 16, 1.0 / 16, 2 * hkv * d * p * dtype.item_size(),
+                                      dtype, layout)
+
+
+def check_groups(meta, shape, tile_size, max_tiles):
+    """Every planned row sits in exactly one group; a group is a run of consecutive full tiles of one
+    request that start at the same key."""
+    rows = meta.h_kv_splits.reshape(-1, 3)
+    tiles = meta.h_q_token_tiles.reshape(-1, 2)
+    table = meta.h_row_groups.reshape(meta.num_row_groups, meta.group_tiles)
+    assert meta.group_tiles == max_tiles
+    seen = []
+    work = []
+    for g in table:
+        members = [int(r) for r in g if r != MAX]
+        assert members and [int(r) for r in g[:len(members)]] == members, "padding only at the end"
+        seen += members
+        first = rows[members[0]]
+        slot = meta.h_req_slots[tiles[first[0]][0]]
+        w = 0
+        for i, r in enumerate(members):
+            tile, begin, end = (int(x) for x in rows[r])
+            assert begin == first[1] and tile == first[0] + i
+            assert meta.h_req_slots[tiles[tile][0]] == slot
+            if i + 1 < len(members):
+                assert tiles[tile][1] - tiles[tile][0] == tile_size and tiles[tile][1] == tiles[tile + 1][0]
+            w += int(tiles[tile][1] - tiles[tile][0]) * (end - begin)
+        work.append(w)
+    assert sorted(seen) == list(range(shape.num_sdpa_map_task_templates)), "rows lost or duplicated"
+    assert work == sorted(work, reverse=True), "heaviest group first"
+    return table
+
+
+def test_row_groups_of_a_prefill_chunk(psi):
+    """A 70-token chunk on a 300-token prefix, 256-token partitions, next to two decode requests:
+    24 Q / 4 KV heads deal 3 heads to a workgroup, so a group holds 5 tiles of 8 tokens."""
+    meta = psi.GQAMetadataBuffers(None, 128, max_kv_splits=64)
+    variant = psi.GQASplitKVVariant.TiledQ(8, 16, 6)
+    shape = meta.update_fixed_partition([3, 1, 5], [300, 40, 999], [0, 70, 71, 72], variant, 256)
+    assert meta.group_rows(tiled_config(psi, 24, 4)) == meta.num_row_groups > 0
+    table = check_groups(meta, shape, 8, 5)
+    rows = meta.h_kv_splits.reshape(-1, 3)
+    # the chunk has 9 tiles; partition 0 is seen by all of them -> groups of 5 + 4
+    sizes = sorted(int((g != MAX).sum()) for g in table if rows[g[0]][1] == 0 and rows[g[0]][0] < 9)
+    assert sizes == [4, 5]
+    # the groups survive a re-ordering of the rows (positions change, membership does not)
+    meta.order_longest_first()
+    meta.group_rows(tiled_config(psi, 24, 4))
+    check_groups(meta, shape, 8, 5)
+
+
+@pytest.mark.parametrize("hq,hkv,expected", [(16, 2, 4), (8, 2, 4), (4, 4, 16), (10, 2, 3), (14, 2, 4)])
+def test_row_group_size_follows_the_head_group(psi, hq, hkv, expected):
+    meta = psi.GQAMetadataBuffers(None, 256, max_kv_splits=256)
+    shape = meta.update_fixed_partition([0], [0], [0, 200], psi.GQASplitKVVariant.TiledQ(8, 16, min(hq // hkv, 8)), 128)
+    assert meta.group_rows(tiled_config(psi, hq, hkv)) > 0
+    check_groups(meta, shape, 8, expected)
+
+
+def test_row_groups_unsupported_geometry_and_greedy_plan(psi):
+    meta = psi.GQAMetadataBuffers(None, 64)
+    variant = psi.GQASplitKVVariant.TiledQ(8, 16, 4)
+    shape = meta.update([0, 1], [100, 7], [0, 20, 24], variant)
+    # head_dim 128 and 8-token pages have no grouped kernel
+    assert meta.group_rows(tiled_config(psi, 8, 2, d=128)) == 0 and meta.group_tiles == 0
+    assert meta.group_rows(tiled_config(psi, 8, 2, p=8)) == 0
+    # the reference's greedy plan cuts every tile differently: groups degenerate but stay complete
+    assert meta.group_rows(tiled_config(psi, 8, 2)) > 0
+    check_groups(meta, shape, 8, 4)
+
+
+def test_row_group_table_capacity_is_checked(psi):
+    lib = psi.load()
+    cfg = tiled_config(psi, 24, 4).struct()
+    rows = np.array([0, 0, 16, 1, 0, 16], np.uint32)
+    tiles = np.array([0, 8, 8, 10], np.uint32)
+    slots = np.zeros(10, np.uint32)
+    slots[8:] = 1
+    table = np.zeros(5, np.uint32)
+    n_tiles, n_groups = ctypes.c_uint32(), ctypes.c_uint32()
+    p = lambda a: a.ctypes.data_as(ctypes.POINTER(ctypes.c_uint32))  # noqa: E731
+    rc = lib.psi_hip_split_kv_tiled_q_group_rows(ctypes.byref(cfg), 8, p(rows), 2, p(tiles), 2, p(slots), p(table), 5,
+                                                 ctypes.byref(n_tiles), ctypes.byref(n_groups))
+    assert rc != 0 and b"row-group table too small" in lib.psi_hip_last_error()
+    table = np.zeros(10, np.uint32)
+    assert lib.psi_hip_split_kv_tiled_q_group_rows(ctypes.byref(cfg), 8, p(rows), 2, p(tiles), 2, p(slots), p(table),
+                                                   10, ctypes.byref(n_tiles), ctypes.byref(n_groups)) == 0
+    assert (n_tiles.value, n_groups.value) == (5, 2)  # two requests never share a group
+    assert table.tolist() == [0, MAX, MAX, MAX, MAX, 1, MAX, MAX, MAX, MAX]
