@@ -32,17 +32,21 @@
 // reads and writes them in place.
 //
 // LDS layout per buffer
-//   K    [32 keys][D] elements, 16-byte chunk index XOR (key%4 + 4*((key/8)%2)): conflict-free for
-//        both the row-wise stores and the operand reads.
-//   V^T  [D dims][32 keys] elements, 16 bytes of padding after every 8 rows.
+//   K    [32 keys][D] elements, 16-byte chunk index XOR (key%4 + 4*(key/8)): the 16 lanes of an
+//        operand read (16 rows, one chunk) then hit 16 different bank groups, and a row-wise store
+//        stays a permutation of its row.
+//   V^T  [D dims][32 keys] elements: 64-byte rows, 64 bytes of padding after every 8 rows, the 16-byte
+//        slot of keys 8s .. 8s+7 at position s XOR (row/4)%4.  Operand reads (16 consecutive rows, one
+//        slot) and transposing stores (4 rows 8 apart, all 16 key pairs) both cover 256 bytes of
+//        distinct banks.
 #pragma once
 #include "split_kv_tiled_kernel.h"
 
 namespace psi {
 
 constexpr int kChunkKeys = 32;         // keys per KV tile
-constexpr int kChunkWaves = 4;
-constexpr int kChunkColBlocks = 2;     // 16-column blocks per wave
+constexpr int kChunkWaves = 8;
+constexpr int kChunkColBlocks = 1;     // 16-column blocks per wave
 constexpr int kChunkWaveCols = 16 * kChunkColBlocks;
 static_assert(kChunkWaves * kChunkWaveCols == kChunkCols, "128 query columns per workgroup");
 constexpr uint32_t kNoRow = 0xffffffffu;
@@ -92,7 +96,7 @@ __device__ __forceinline__ uint32_t wave_max_u32(uint32_t v) {
 template <int D>
 struct ChunkLds {
     static constexpr int kKBytes = kChunkKeys * D * 2;
-    static constexpr int kVtBytes = D * kChunkKeys * 2 + (D / 8) * 16;
+    static constexpr int kVtBytes = D * kChunkKeys * 2 + (D / 8) * 64;
     static constexpr int kQBytes = kChunkCols * D * 2;
     static constexpr int bytes = 2 * (kKBytes + kVtBytes) + kQBytes;
 };
@@ -144,7 +148,9 @@ __global__ __launch_bounds__(64 * kChunkWaves, 2) void split_kv_chunk_map(
     const uint32_t q_tile0 = kv_splits[row0 * 3];
     if (q_tile0 >= a.num_active_q_token_tiles || q_tile0 + num_tiles > a.num_active_q_token_tiles) return;
     const uint32_t kv_begin = kv_splits[row0 * 3 + 1];
-    const uint32_t kv_end_max = wave_max_u32(my_row_ok && lane < num_tiles ? kv_splits[my_row * 3 + 2] : 0u);
+    // wave-uniform by construction; said explicitly so that the page-ID reads below stay scalar loads
+    const uint32_t kv_end_max = __builtin_amdgcn_readfirstlane(
+        wave_max_u32(my_row_ok && lane < num_tiles ? kv_splits[my_row * 3 + 2] : 0u));
     const uint32_t flat_begin = q_token_tiles[q_tile0 * 2];
     const uint32_t flat_end = q_token_tiles[(q_tile0 + num_tiles - 1) * 2 + 1];
     if (flat_end <= flat_begin || flat_end > a.num_active_tokens || kv_end_max <= kv_begin) return;
@@ -152,7 +158,7 @@ __global__ __launch_bounds__(64 * kChunkWaves, 2) void split_kv_chunk_map(
     if (ncols > (uint32_t)kChunkCols || flat_end - flat_begin > num_tiles * TS) return;  // the planner never builds such a group
     const uint32_t req_slot = req_slots[flat_begin];
 
-    // ---- this lane's columns: c = 32 * wave + 16 * cb + mt; their query rows go to LDS as B operands
+    // ---- this lane's columns: c = 16 * wave + 16 * cb + mt; their query rows go to LDS as B operands
     // (dims 32 * ks + 8 * mc .. +8), zero for unused columns.  Only this wave reads them back.
     uint32_t lim[CB];        // keys [kv_begin, lim) are visible to the column; 0: column unused
     uint64_t part_row[CB];   // partial-state row of the column
@@ -205,29 +211,34 @@ __global__ __launch_bounds__(64 * kChunkWaves, 2) void split_kv_chunk_map(
         }
         return p;
     };
+    constexpr int kSubs = 64 * kChunkWaves / kRowChunks;  // threads per 16-byte column of the tile (16)
     const uint32_t ld_chunk = tid % kRowChunks;   // 16-byte chunk of a row (8 dims)
-    const uint32_t ld_sub = tid / kRowChunks;     // 0..7
+    const uint32_t ld_sub = tid / kRowChunks;     // 0 .. kSubs - 1
+    // V goes the other way round: 16 adjacent lanes take the 16 key pairs of one chunk, so that a
+    // transposing store instruction covers whole 64-byte rows of V^T.
+    const uint32_t v_pair = tid % kSubs;          // keys kLoads * v_pair .. +kLoads - 1
+    const uint32_t v_chunk = tid / kSubs;
     struct Staging {
         u32x4_t k[kLoads], v[kLoads];
     };
-    // K: load j takes key 8 * j + ld_sub; V: load j takes key 4 * ld_sub + j (4 keys of one chunk).
+    // K: load j takes key kSubs * j + ld_sub; V: load j takes key kLoads * ld_sub + j (adjacent keys of one chunk).
     auto issue_loads = [&](uint32_t it, TileIds p) __attribute__((always_inline)) -> Staging {
         Staging st;
         const uint32_t kb = key_base0 + it * kChunkKeys;
 #pragma unroll
         for (int j = 0; j < kLoads; ++j) {
-            const uint32_t key = 8 * j + ld_sub;
-            const uint32_t page = j < kLoads / 2 ? p.a : p.b;
+            const uint32_t key = kSubs * j + ld_sub;
+            const uint32_t page = key < 16 ? p.a : p.b;
             const uint16_t* src = pages + (uint64_t)page * a.walk.page_elems +
                                   ((uint64_t)kv_head * a.walk.tokens_per_page + ((kb + key) & page_mask)) * D + ld_chunk * 8;
             st.k[j] = *reinterpret_cast<const u32x4_t*>(src);
         }
-        const uint32_t vpage = ld_sub < 4 ? p.a : p.b;
+        const uint32_t vpage = kLoads * v_pair < 16 ? p.a : p.b;
 #pragma unroll
         for (int j = 0; j < kLoads; ++j) {
-            const uint32_t key = 4 * ld_sub + j;
+            const uint32_t key = kLoads * v_pair + j;
             const uint16_t* src = pages + (uint64_t)vpage * a.walk.page_elems + v_region +
-                                  ((uint64_t)kv_head * a.walk.tokens_per_page + ((kb + key) & page_mask)) * D + ld_chunk * 8;
+                                  ((uint64_t)kv_head * a.walk.tokens_per_page + ((kb + key) & page_mask)) * D + v_chunk * 8;
             st.v[j] = *reinterpret_cast<const u32x4_t*>(src);
         }
         return st;
@@ -240,43 +251,38 @@ __global__ __launch_bounds__(64 * kChunkWaves, 2) void split_kv_chunk_map(
         const uint32_t kb = key_base0 + it * kChunkKeys;
 #pragma unroll
         for (int j = 0; j < kLoads; ++j) {
-            const uint32_t key = 8 * j + ld_sub;
-            const uint32_t swz = (ld_sub & 3) + 4 * (j & 1);
+            const uint32_t key = kSubs * j + ld_sub;
+            const uint32_t swz = (key & 3) + 4 * (key >> 3);
             *reinterpret_cast<u32x4_t*>(kbuf + key * (D * 2) + ((ld_chunk ^ swz) * 16)) = st.k[j];
         }
         uint32_t w[kLoads][4];
 #pragma unroll
         for (int j = 0; j < kLoads; ++j) {
-            const uint32_t token = kb + 4 * ld_sub + j;
+            const uint32_t token = kb + kLoads * v_pair + j;
             const bool live = token >= kv_begin && token < kv_end_max;
             w[j][0] = live ? st.v[j][0] : 0u;
             w[j][1] = live ? st.v[j][1] : 0u;
             w[j][2] = live ? st.v[j][2] : 0u;
             w[j][3] = live ? st.v[j][3] : 0u;
         }
-        static_assert(kLoads == 4, "the transposing store packs 4 keys per 64-bit word");
+        static_assert(kLoads == 2, "the transposing store packs 2 keys per 32-bit word");
 #pragma unroll
         for (int e = 0; e < 8; ++e) {
             const int word = e / 2;
-            uint2 out;
-            if (e % 2 == 0) {
-                out.x = (w[0][word] & 0xffffu) | (w[1][word] << 16);
-                out.y = (w[2][word] & 0xffffu) | (w[3][word] << 16);
-            } else {
-                out.x = (w[0][word] >> 16) | (w[1][word] & 0xffff0000u);
-                out.y = (w[2][word] >> 16) | (w[3][word] & 0xffff0000u);
-            }
-            // row = 8 * ld_chunk + e; 64 bytes per row, 16 bytes of padding per 8 rows
-            *reinterpret_cast<uint2*>(vbuf + (8 * ld_chunk + e) * 64 + ld_chunk * 16 + ld_sub * 8) = out;
+            const uint32_t out = e % 2 == 0 ? ((w[0][word] & 0xffffu) | (w[1][word] << 16))
+                                            : ((w[0][word] >> 16) | (w[1][word] & 0xffff0000u));
+            // row = 8 * v_chunk + e; its 16-byte slot v_pair / 4 is swizzled with (row / 4) % 4
+            const uint32_t slot = (v_pair >> 2) ^ ((2 * v_chunk + e / 4) & 3);
+            *reinterpret_cast<uint32_t*>(vbuf + (8 * v_chunk + e) * 64 + v_chunk * 64 + slot * 16 + (v_pair & 3) * 4) = out;
         }
     };
 
     // ---- operand read addresses of this lane
     // K row of (block b, lane row mt): key 8 * (mt / 4) + 4 * b + mt % 4, chunk (4 * ks + mc) ^ swizzle
-    const uint32_t k_swz = (mt & 3) + 4 * ((mt >> 2) & 1);
+    const uint32_t k_swz = mt;  // = key % 4 + 4 * (key / 8) for both key blocks
     const uint32_t k_row0 = (8 * (mt >> 2) + (mt & 3)) * (D * 2);
     // V^T row of (dim block db, lane row mt): dim 16 * db + mt, keys 8 * mc .. +7
-    const uint32_t vt_row0 = mt * 64 + (mt >> 3) * 16 + mc * 16;
+    const uint32_t vt_row0 = mt * 64 + (mt >> 3) * 64 + ((mc ^ ((mt >> 2) & 3)) * 16);
 
     float run_max[CB], lane_sum[CB];
     f32x4_t o[CB][kDimBlocks];
@@ -328,7 +334,6 @@ __global__ __launch_bounds__(64 * kChunkWaves, 2) void split_kv_chunk_map(
                 s[0][cb] = mfma_16x16x32<Tag>(kc0, qc[cb], s[0][cb]);
                 s[1][cb] = mfma_16x16x32<Tag>(kc1, qc[cb], s[1][cb]);
             }
-            __builtin_amdgcn_sched_barrier(0);
             kc0 = kn0;
             kc1 = kn1;
 #pragma unroll
@@ -377,9 +382,8 @@ __global__ __launch_bounds__(64 * kChunkWaves, 2) void split_kv_chunk_map(
                     for (int r = 0; r < 4; ++r) o[cb][db][r] *= alpha[cb];
         }
         // ---- O^T[dim][column] += V^T * P^T
-        auto read_vt = [&](int db) { return *reinterpret_cast<const uint4*>(vbuf + vt_row0 + db * (16 * 64 + 32)); };
+        auto read_vt = [&](int db) { return *reinterpret_cast<const uint4*>(vbuf + vt_row0 + db * (16 * 64 + 2 * 64)); };
         uint4 vc = read_vt(0);
-        __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
         for (int db = 0; db < kDimBlocks; ++db) {
             uint4 vn = vc;
@@ -388,7 +392,6 @@ __global__ __launch_bounds__(64 * kChunkWaves, 2) void split_kv_chunk_map(
             for (int t = 0; t < ProbOperand8<Tag>::kTerms; ++t)
 #pragma unroll
                 for (int cb = 0; cb < CB; ++cb) o[cb][db] = mfma_16x16x32<Tag>(vc, pb[cb].term[t], o[cb][db]);
-            __builtin_amdgcn_sched_barrier(0);
             vc = vn;
         }
     };
