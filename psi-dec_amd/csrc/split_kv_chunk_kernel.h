@@ -97,8 +97,7 @@ template <int D>
 struct ChunkLds {
     static constexpr int kKBytes = kChunkKeys * D * 2;
     static constexpr int kVtBytes = D * kChunkKeys * 2 + (D / 8) * 64;
-    static constexpr int kQBytes = kChunkCols * D * 2;
-    static constexpr int bytes = 2 * (kKBytes + kVtBytes) + kQBytes;
+    static constexpr int bytes = 2 * (kKBytes + kVtBytes);
 };
 
 template <typename Tag, int D>
@@ -111,17 +110,17 @@ __global__ __launch_bounds__(64 * kChunkWaves, 2) void split_kv_chunk_map(
     constexpr int kKSteps = D / 32;              // MFMA k-steps of QK^T
     constexpr int kDimBlocks = D / 16;           // 16-dim output blocks of PV
     constexpr int kRowChunks = D / 8;            // 16-byte chunks per K row
-    constexpr int kLoads = kChunkKeys * kRowChunks / (64 * kChunkWaves);  // 128-bit loads per thread and operand (4)
+    constexpr int kLoads = kChunkKeys * kRowChunks / (64 * kChunkWaves);  // 128-bit loads per thread and operand (2)
     constexpr int kKBytes = ChunkLds<D>::kKBytes;
     constexpr int kVtBytes = ChunkLds<D>::kVtBytes;
     constexpr int kBufBytes = kKBytes + kVtBytes;
     constexpr int CB = kChunkColBlocks;
     constexpr float kSlack = 8.0f;
+    constexpr int kIdTiles = 32;  // KV tiles per block of page IDs held in one register (<= 64 pages)
+    static_assert(kLoads == 2 && CB == 1, "loader and softmax are written for 8 waves of 16 columns");
     // Dynamic LDS (the launcher passes ChunkLds<D>::bytes): with a static size the compiler sees
-    // that one workgroup fills the CU and lifts the register cap that keeps the accumulators in
-    // architectural VGPRs.
+    // that one workgroup fills the CU and lifts the register cap.
     extern __shared__ __attribute__((aligned(16))) unsigned char lds[];
-    uint4* qb_lds = reinterpret_cast<uint4*>(lds + 2 * kBufBytes);  // [wave][cb][ks][lane]
 
     const uint32_t TS = a.rows_per_split_head;  // Q tokens per tile
     // heads of the KV head served here: head_first + [0, G)
@@ -148,7 +147,7 @@ __global__ __launch_bounds__(64 * kChunkWaves, 2) void split_kv_chunk_map(
     const uint32_t q_tile0 = kv_splits[row0 * 3];
     if (q_tile0 >= a.num_active_q_token_tiles || q_tile0 + num_tiles > a.num_active_q_token_tiles) return;
     const uint32_t kv_begin = kv_splits[row0 * 3 + 1];
-    // wave-uniform by construction; said explicitly so that the page-ID reads below stay scalar loads
+    // wave-uniform by construction; said explicitly so that everything derived from it stays scalar
     const uint32_t kv_end_max = __builtin_amdgcn_readfirstlane(
         wave_max_u32(my_row_ok && lane < num_tiles ? kv_splits[my_row * 3 + 2] : 0u));
     const uint32_t flat_begin = q_token_tiles[q_tile0 * 2];
@@ -158,119 +157,108 @@ __global__ __launch_bounds__(64 * kChunkWaves, 2) void split_kv_chunk_map(
     if (ncols > (uint32_t)kChunkCols || flat_end - flat_begin > num_tiles * TS) return;  // the planner never builds such a group
     const uint32_t req_slot = req_slots[flat_begin];
 
-    // ---- this lane's columns: c = 16 * wave + 16 * cb + mt; their query rows go to LDS as B operands
-    // (dims 32 * ks + 8 * mc .. +8), zero for unused columns.  Only this wave reads them back.
-    uint32_t lim[CB];        // keys [kv_begin, lim) are visible to the column; 0: column unused
-    uint64_t part_row[CB];   // partial-state row of the column
-    uint4* my_q = qb_lds + wave * (CB * kKSteps * 64) + lane;
-    uint32_t lo_lim = 0xffffffffu, hi_lim = 0;
-#pragma unroll
-    for (int cb = 0; cb < CB; ++cb) {
-        const uint32_t c = wave * kChunkWaveCols + cb * 16 + mt;
-        const bool used = c < ncols;
+    // ---- this lane's column c = 16 * wave + mt: visible range, partial-state row, query row as B
+    // operands (dims 32 * ks + 8 * mc .. +8; zero for an unused column)
+    const uint32_t c = wave * kChunkWaveCols + mt;
+    const bool used = c < ncols;
+    uint32_t lim = 0;        // keys [kv_begin, lim) are visible to the column; 0: column unused
+    uint64_t part_row = 0;   // partial-state row of the column
+    uint4 qreg[kKSteps];
+    {
         const uint32_t t = used ? c / G : 0u, h = used ? c % G : 0u;
         const uint32_t m = t / TS, r = t % TS;
         const uint32_t row = rows[m];
-        lim[cb] = 0;
-        part_row[cb] = 0;
         if (used) {
-            lim[cb] = min(kv_splits[row * 3 + 2], flat_token_indices[flat_begin + t] + 1);
-            part_row[cb] = ((uint64_t)row * a.hq + head_first + h) * TS + r;
-            lo_lim = min(lo_lim, lim[cb]);
-            hi_lim = max(hi_lim, lim[cb]);
+            lim = min(kv_splits[row * 3 + 2], flat_token_indices[flat_begin + t] + 1);
+            part_row = ((uint64_t)row * a.hq + head_first + h) * TS + r;
         }
         const uint16_t* q_row = q + ((uint64_t)(flat_begin + t) * a.hq + head_first + h) * D + mc * 8;
 #pragma unroll
         for (int ks = 0; ks < kKSteps; ++ks)
-            my_q[(cb * kKSteps + ks) * 64] = used ? *reinterpret_cast<const uint4*>(q_row + ks * 32) : make_uint4(0, 0, 0, 0);
+            qreg[ks] = used ? *reinterpret_cast<const uint4*>(q_row + ks * 32) : make_uint4(0, 0, 0, 0);
     }
     // Tiles at or beyond wave_hi hold no visible key for this wave; tiles inside [kv_begin, wave_lo)
     // need no mask.
-    const uint32_t wave_lo = __builtin_amdgcn_readfirstlane(wave_min_u32(lo_lim));
-    const uint32_t wave_hi = __builtin_amdgcn_readfirstlane(wave_max_u32(hi_lim));
+    const uint32_t wave_lo = __builtin_amdgcn_readfirstlane(wave_min_u32(used ? lim : 0xffffffffu));
+    const uint32_t wave_hi = __builtin_amdgcn_readfirstlane(wave_max_u32(lim));
 
-    // ---- page walk and the cooperative tile loaders
+    // ---- page walk.  Page IDs of kIdTiles tiles at a time sit in one register (lane l: the l-th page
+    // of the block) and are picked out with v_readlane: no memory access on the per-tile path.
     const uint32_t log2p = 31 - __builtin_clz(a.walk.tokens_per_page);
     const uint32_t page_mask = a.walk.tokens_per_page - 1;
     const uint32_t* table_row = page_ids + ((uint64_t)req_slot * a.walk.num_layers + a.layer) *
                                                       a.walk.num_blocks * a.walk.ids_per_block;
-    const uint64_t v_region = (uint64_t)a.walk.hkv * a.walk.tokens_per_page * D;
     const uint32_t last_page = (kv_end_max - 1) >> log2p;
     const uint32_t key_base0 = kv_begin & ~(uint32_t)(kChunkKeys - 1);
     const uint32_t num_kv_tiles = (kv_end_max - key_base0 + kChunkKeys - 1) / kChunkKeys;
+    auto load_id_block = [&](uint32_t first_tile) -> uint32_t {
+        const uint32_t page0 = (key_base0 + first_tile * kChunkKeys) >> log2p;
+        return table_row[min(page0 + lane, last_page)];
+    };
+    struct TileBases {
+        const unsigned char* a;  // page of keys 0..15 of the tile, advanced to the tile's first token
+        const unsigned char* b;  // page of keys 16..31
+    };
+    const uint64_t page_bytes = a.walk.page_elems * 2;
+    auto tile_bases = [&](uint32_t it, uint32_t id_block) -> TileBases {
+        const uint32_t kb = key_base0 + it * kChunkKeys;
+        const uint32_t page0 = (key_base0 + (it & ~(uint32_t)(kIdTiles - 1)) * kChunkKeys) >> log2p;
+        const uint32_t ia = min(kb >> log2p, last_page) - page0, ib = min((kb + 16) >> log2p, last_page) - page0;
+        const uint32_t pa = __builtin_amdgcn_readlane(id_block, ia), pb = __builtin_amdgcn_readlane(id_block, ib);
+        const uint64_t in_page = (uint64_t)(kb & page_mask) * (D * 2);
+        const unsigned char* base = reinterpret_cast<const unsigned char*>(pages);
+        return TileBases{base + pa * page_bytes + in_page, base + pb * page_bytes + in_page};
+    };
 
-    struct TileIds {
-        uint32_t a, b;  // page of keys 0..15 and of keys 16..31 of the tile
-    };
-    auto load_ids = [&](uint32_t it) -> TileIds {
-        TileIds p{0u, 0u};
-        if (it < num_kv_tiles) {
-            const uint32_t kb = key_base0 + it * kChunkKeys;
-            p.a = table_row[min(kb >> log2p, last_page)];
-            p.b = table_row[min((kb + 16) >> log2p, last_page)];
-        }
-        return p;
-    };
-    constexpr int kSubs = 64 * kChunkWaves / kRowChunks;  // threads per 16-byte column of the tile (16)
-    const uint32_t ld_chunk = tid % kRowChunks;   // 16-byte chunk of a row (8 dims)
-    const uint32_t ld_sub = tid / kRowChunks;     // 0 .. kSubs - 1
+    // ---- cooperative tile loaders: per-thread byte offsets inside a page are fixed for the kernel
+    constexpr int kSubs = 64 * kChunkWaves / kRowChunks;  // 16
+    const uint32_t ld_chunk = tid % kRowChunks;   // K: 16-byte chunk of a row (8 dims)
+    const uint32_t ld_sub = tid / kRowChunks;     // K: load j takes key kSubs * j + ld_sub
     // V goes the other way round: 16 adjacent lanes take the 16 key pairs of one chunk, so that a
     // transposing store instruction covers whole 64-byte rows of V^T.
-    const uint32_t v_pair = tid % kSubs;          // keys kLoads * v_pair .. +kLoads - 1
+    const uint32_t v_pair = tid % kSubs;          // V: load j takes key 2 * v_pair + j
     const uint32_t v_chunk = tid / kSubs;
+    const bool small_page = a.walk.tokens_per_page == 16;  // keys 16..31 of a tile then start their own page
+    uint32_t k_off[kLoads], v_off[kLoads];
+#pragma unroll
+    for (int j = 0; j < kLoads; ++j) {
+        const uint32_t k_key = kSubs * j + ld_sub, v_key = kLoads * v_pair + j;
+        k_off[j] = ((kv_head * a.walk.tokens_per_page + (small_page ? (k_key & 15) : k_key)) * D + ld_chunk * 8) * 2;
+        v_off[j] = (((a.walk.hkv + kv_head) * a.walk.tokens_per_page + (small_page ? (v_key & 15) : v_key)) * D + v_chunk * 8) * 2;
+    }
     struct Staging {
         u32x4_t k[kLoads], v[kLoads];
     };
-    // K: load j takes key kSubs * j + ld_sub; V: load j takes key kLoads * ld_sub + j (adjacent keys of one chunk).
-    auto issue_loads = [&](uint32_t it, TileIds p) __attribute__((always_inline)) -> Staging {
+    auto issue_loads = [&](TileBases tb) __attribute__((always_inline)) -> Staging {
         Staging st;
-        const uint32_t kb = key_base0 + it * kChunkKeys;
+        st.k[0] = *reinterpret_cast<const u32x4_t*>(tb.a + k_off[0]);  // keys 0..15
+        st.k[1] = *reinterpret_cast<const u32x4_t*>(tb.b + k_off[1]);  // keys 16..31
+        const unsigned char* vb = v_pair < 8 ? tb.a : tb.b;
 #pragma unroll
-        for (int j = 0; j < kLoads; ++j) {
-            const uint32_t key = kSubs * j + ld_sub;
-            const uint32_t page = key < 16 ? p.a : p.b;
-            const uint16_t* src = pages + (uint64_t)page * a.walk.page_elems +
-                                  ((uint64_t)kv_head * a.walk.tokens_per_page + ((kb + key) & page_mask)) * D + ld_chunk * 8;
-            st.k[j] = *reinterpret_cast<const u32x4_t*>(src);
-        }
-        const uint32_t vpage = kLoads * v_pair < 16 ? p.a : p.b;
-#pragma unroll
-        for (int j = 0; j < kLoads; ++j) {
-            const uint32_t key = kLoads * v_pair + j;
-            const uint16_t* src = pages + (uint64_t)vpage * a.walk.page_elems + v_region +
-                                  ((uint64_t)kv_head * a.walk.tokens_per_page + ((kb + key) & page_mask)) * D + v_chunk * 8;
-            st.v[j] = *reinterpret_cast<const u32x4_t*>(src);
-        }
+        for (int j = 0; j < kLoads; ++j) st.v[j] = *reinterpret_cast<const u32x4_t*>(vb + v_off[j]);
         return st;
     };
     // Registers -> LDS buffer `buf`.  V rows outside [kv_begin, kv_end_max) are zeroed: their
     // probability is 0 but their bytes may be NaN / Inf.
+    const uint32_t k_store0 = ld_sub * (D * 2) + ((ld_chunk ^ ((ld_sub & 3) + 4 * (ld_sub >> 3))) * 16);
+    const uint32_t k_store1 = (kSubs + ld_sub) * (D * 2) + ((ld_chunk ^ ((ld_sub & 3) + 4 * ((kSubs + ld_sub) >> 3))) * 16);
     auto store_tile = [&](uint32_t it, uint32_t buf, const Staging& st) __attribute__((always_inline)) {
         unsigned char* kbuf = lds + buf * kBufBytes;
         unsigned char* vbuf = kbuf + kKBytes;
         const uint32_t kb = key_base0 + it * kChunkKeys;
-#pragma unroll
-        for (int j = 0; j < kLoads; ++j) {
-            const uint32_t key = kSubs * j + ld_sub;
-            const uint32_t swz = (key & 3) + 4 * (key >> 3);
-            *reinterpret_cast<u32x4_t*>(kbuf + key * (D * 2) + ((ld_chunk ^ swz) * 16)) = st.k[j];
+        *reinterpret_cast<u32x4_t*>(kbuf + k_store0) = st.k[0];
+        *reinterpret_cast<u32x4_t*>(kbuf + k_store1) = st.k[1];
+        u32x4_t w0 = st.v[0], w1 = st.v[1];
+        if (kb < kv_begin || kb + kChunkKeys > kv_end_max) {  // first or last tile of the range
+            const uint32_t token = kb + kLoads * v_pair;
+            if (token < kv_begin || token >= kv_end_max) w0 = u32x4_t{0u, 0u, 0u, 0u};
+            if (token + 1 < kv_begin || token + 1 >= kv_end_max) w1 = u32x4_t{0u, 0u, 0u, 0u};
         }
-        uint32_t w[kLoads][4];
-#pragma unroll
-        for (int j = 0; j < kLoads; ++j) {
-            const uint32_t token = kb + kLoads * v_pair + j;
-            const bool live = token >= kv_begin && token < kv_end_max;
-            w[j][0] = live ? st.v[j][0] : 0u;
-            w[j][1] = live ? st.v[j][1] : 0u;
-            w[j][2] = live ? st.v[j][2] : 0u;
-            w[j][3] = live ? st.v[j][3] : 0u;
-        }
-        static_assert(kLoads == 2, "the transposing store packs 2 keys per 32-bit word");
 #pragma unroll
         for (int e = 0; e < 8; ++e) {
             const int word = e / 2;
-            const uint32_t out = e % 2 == 0 ? ((w[0][word] & 0xffffu) | (w[1][word] << 16))
-                                            : ((w[0][word] >> 16) | (w[1][word] & 0xffff0000u));
+            const uint32_t out = e % 2 == 0 ? ((w0[word] & 0xffffu) | (w1[word] << 16))
+                                            : ((w0[word] >> 16) | (w1[word] & 0xffff0000u));
             // row = 8 * v_chunk + e; its 16-byte slot v_pair / 4 is swizzled with (row / 4) % 4
             const uint32_t slot = (v_pair >> 2) ^ ((2 * v_chunk + e / 4) & 3);
             *reinterpret_cast<uint32_t*>(vbuf + (8 * v_chunk + e) * 64 + v_chunk * 64 + slot * 16 + (v_pair & 3) * 4) = out;
@@ -284,155 +272,107 @@ __global__ __launch_bounds__(64 * kChunkWaves, 2) void split_kv_chunk_map(
     // V^T row of (dim block db, lane row mt): dim 16 * db + mt, keys 8 * mc .. +7
     const uint32_t vt_row0 = mt * 64 + (mt >> 3) * 64 + ((mc ^ ((mt >> 2) & 3)) * 16);
 
-    float run_max[CB], lane_sum[CB];
-    f32x4_t o[CB][kDimBlocks];
+    float run_max = -INFINITY, lane_sum = 0.0f;
+    f32x4_t o[kDimBlocks];
 #pragma unroll
-    for (int cb = 0; cb < CB; ++cb) {
-        run_max[cb] = -INFINITY;
-        lane_sum[cb] = 0.0f;
-#pragma unroll
-        for (int db = 0; db < kDimBlocks; ++db) o[cb][db] = f32x4_t{0.0f, 0.0f, 0.0f, 0.0f};
-    }
+    for (int db = 0; db < kDimBlocks; ++db) o[db] = f32x4_t{0.0f, 0.0f, 0.0f, 0.0f};
     const bool wave_has_cols = wave * kChunkWaveCols < ncols;
 
     // `masked`: the tile touches the start of the range or a causal limit of this wave (wave-uniform).
-    // One instantiation on purpose: two copies of this body under an if / else made the register
-    // allocator spill half of the accumulators.
     auto compute_tile = [&](uint32_t it, uint32_t buf, bool masked) __attribute__((always_inline)) {
         const unsigned char* kbuf = lds + buf * kBufBytes;
         const unsigned char* vbuf = kbuf + kKBytes;
         const uint32_t kb = key_base0 + it * kChunkKeys;
-        // ---- logits S[key][column]: two key blocks x CB column blocks
-        f32x4_t s[2][CB];
-#pragma unroll
-        for (int b = 0; b < 2; ++b)
-#pragma unroll
-            for (int cb = 0; cb < CB; ++cb) s[b][cb] = f32x4_t{0.0f, 0.0f, 0.0f, 0.0f};
-        // operand reads run one step ahead of the MFMAs that use them; the scheduling fences keep
-        // the compiler from hoisting every read of the tile to its start (register pressure)
-        auto read_k = [&](int ks, uint4& k0, uint4& k1) {
-            const uint32_t off = k_row0 + (((4 * ks + mc) ^ k_swz) * 16);
-            k0 = *reinterpret_cast<const uint4*>(kbuf + off);
-            k1 = *reinterpret_cast<const uint4*>(kbuf + off + 4 * (D * 2));
-        };
-        uint4 kc0, kc1, qc[CB];
-        read_k(0, kc0, kc1);
-#pragma unroll
-        for (int cb = 0; cb < CB; ++cb) qc[cb] = my_q[cb * kKSteps * 64];
+        // ---- logits S[key][column]: two key blocks
+        f32x4_t s0 = f32x4_t{0.0f, 0.0f, 0.0f, 0.0f}, s1 = s0;
 #pragma unroll
         for (int ks = 0; ks < kKSteps; ++ks) {
-            uint4 kn0 = kc0, kn1 = kc1, qn[CB];
-#pragma unroll
-            for (int cb = 0; cb < CB; ++cb) qn[cb] = qc[cb];
-            if (ks + 1 < kKSteps) {
-                read_k(ks + 1, kn0, kn1);
-#pragma unroll
-                for (int cb = 0; cb < CB; ++cb) qn[cb] = my_q[(cb * kKSteps + ks + 1) * 64];
-            }
-#pragma unroll
-            for (int cb = 0; cb < CB; ++cb) {
-                s[0][cb] = mfma_16x16x32<Tag>(kc0, qc[cb], s[0][cb]);
-                s[1][cb] = mfma_16x16x32<Tag>(kc1, qc[cb], s[1][cb]);
-            }
-            kc0 = kn0;
-            kc1 = kn1;
-#pragma unroll
-            for (int cb = 0; cb < CB; ++cb) qc[cb] = qn[cb];
+            const uint32_t off = k_row0 + (((4 * ks + mc) ^ k_swz) * 16);
+            const uint4 k0 = *reinterpret_cast<const uint4*>(kbuf + off);
+            const uint4 k1 = *reinterpret_cast<const uint4*>(kbuf + off + 4 * (D * 2));
+            s0 = mfma_16x16x32<Tag>(k0, qreg[ks], s0);
+            s1 = mfma_16x16x32<Tag>(k1, qreg[ks], s1);
         }
-        // ---- online softmax; this lane holds keys kb + 8 * mc + j, j = 4 * b + r, of column mt
-        ProbOperand8<Tag> pb[CB];
-        float alpha[CB];
-        bool moved = false;
+        // ---- online softmax; this lane holds keys kb + 8 * mc + j, j = 4 * b + r, of column mt.
+        // Logits relative to the column's reference maximum; masked keys at -inf.
+        float v[8];
 #pragma unroll
-        for (int cb = 0; cb < CB; ++cb) {
-            float v[8];
-            bool valid[8];
-            float m = -INFINITY;
+        for (int j = 0; j < 8; ++j) v[j] = (j < 4 ? s0[j] : s1[j - 4]) * a.scale_log2;
+        if (masked) {
 #pragma unroll
             for (int j = 0; j < 8; ++j) {
                 const uint32_t token = kb + 8 * mc + j;
-                valid[j] = !masked || (token >= kv_begin && token < lim[cb]);
-                v[j] = valid[j] ? s[j / 4][cb][j % 4] * a.scale_log2 : -INFINITY;
-                m = fmaxf(m, v[j]);
+                if (token < kv_begin || token >= lim) v[j] = -INFINITY;
             }
+        }
+        float m = fmaxf(fmaxf(fmaxf(v[0], v[1]), fmaxf(v[2], v[3])), fmaxf(fmaxf(v[4], v[5]), fmaxf(v[6], v[7])));
+        // The reference maximum moves only when some key exceeds it by more than kSlack (log2 domain):
+        // rare after the first tiles, so the cross-lane maximum and the rescaling sit behind a
+        // wave-wide test.  A column with no visible key so far keeps max = -inf, sum = 0, O = 0.
+        if (__any(m > run_max + kSlack)) {
             m = fmaxf(m, __shfl_xor(m, 16, 64));
             m = fmaxf(m, __shfl_xor(m, 32, 64));
-            // The reference maximum follows the tile maximum only when that exceeds it by more than
-            // kSlack (log2 domain); a column with no visible key so far keeps max = -inf, sum = 0, O = 0.
-            const bool bump = m > run_max[cb] + kSlack;
-            const float next_max = bump ? m : run_max[cb];
-            alpha[cb] = !bump ? 1.0f : (run_max[cb] > -INFINITY ? __builtin_amdgcn_exp2f(run_max[cb] - next_max) : 0.0f);
-            moved = moved || bump;
-            run_max[cb] = next_max;
-            float p[8], tile_sum = 0.0f;
-#pragma unroll
-            for (int j = 0; j < 8; ++j) {
-                p[j] = valid[j] ? __builtin_amdgcn_exp2f(v[j] - next_max) : 0.0f;
-                tile_sum += p[j];
-            }
-            lane_sum[cb] = lane_sum[cb] * alpha[cb] + tile_sum;
-            pb[cb].set(p);
-        }
-        if (__any(moved)) {
-#pragma unroll
-            for (int cb = 0; cb < CB; ++cb)
+            if (m > run_max + kSlack) {
+                const float alpha = run_max > -INFINITY ? __builtin_amdgcn_exp2f(run_max - m) : 0.0f;
+                run_max = m;
+                lane_sum *= alpha;
 #pragma unroll
                 for (int db = 0; db < kDimBlocks; ++db)
 #pragma unroll
-                    for (int r = 0; r < 4; ++r) o[cb][db][r] *= alpha[cb];
+                    for (int r = 0; r < 4; ++r) o[db][r] *= alpha;
+            }
         }
+        float p[8], tile_sum = 0.0f;
+#pragma unroll
+        for (int j = 0; j < 8; ++j) {
+            // -inf - (-inf) only when the column has seen no key at all: such a key is masked
+            p[j] = v[j] > -INFINITY ? __builtin_amdgcn_exp2f(v[j] - run_max) : 0.0f;
+            tile_sum += p[j];
+        }
+        lane_sum += tile_sum;
+        ProbOperand8<Tag> pb;
+        pb.set(p);
         // ---- O^T[dim][column] += V^T * P^T
-        auto read_vt = [&](int db) { return *reinterpret_cast<const uint4*>(vbuf + vt_row0 + db * (16 * 64 + 2 * 64)); };
-        uint4 vc = read_vt(0);
 #pragma unroll
         for (int db = 0; db < kDimBlocks; ++db) {
-            uint4 vn = vc;
-            if (db + 1 < kDimBlocks) vn = read_vt(db + 1);
+            const uint4 vt = *reinterpret_cast<const uint4*>(vbuf + vt_row0 + db * (16 * 64 + 2 * 64));
 #pragma unroll
-            for (int t = 0; t < ProbOperand8<Tag>::kTerms; ++t)
-#pragma unroll
-                for (int cb = 0; cb < CB; ++cb) o[cb][db] = mfma_16x16x32<Tag>(vc, pb[cb].term[t], o[cb][db]);
-            vc = vn;
+            for (int t = 0; t < ProbOperand8<Tag>::kTerms; ++t) o[db] = mfma_16x16x32<Tag>(vt, pb.term[t], o[db]);
         }
     };
 
-    // ---- main loop: tile it in buffer it % 2
+    // ---- main loop: tile `it` lives in LDS buffer it % 2; its loads were issued one tile earlier
+    uint32_t id_block = load_id_block(0), id_block_next = 0;
     {
-        const TileIds p0 = load_ids(0);
-        const Staging st = issue_loads(0, p0);
+        const Staging st = issue_loads(tile_bases(0, id_block));
         store_tile(0, 0, st);
     }
-    TileIds ids_next = load_ids(1);
     __syncthreads();
     for (uint32_t it = 0; it < num_kv_tiles; ++it) {
-        const bool has_next = it + 1 < num_kv_tiles;
-        const TileIds ids_after = load_ids(it + 2);
+        const uint32_t nt = it + 1;  // the tile to fetch now
+        const bool has_next = nt < num_kv_tiles;
+        if ((nt & (kIdTiles - 1)) == kIdTiles / 2) id_block_next = load_id_block((nt & ~(uint32_t)(kIdTiles - 1)) + kIdTiles);
+        if ((nt & (kIdTiles - 1)) == 0) id_block = id_block_next;
         Staging st;
-        if (has_next) st = issue_loads(it + 1, ids_next);
+        if (has_next) st = issue_loads(tile_bases(nt, id_block));
         const uint32_t kb = key_base0 + it * kChunkKeys;
-        if (wave_has_cols && kb < wave_hi) {
-            compute_tile(it, it & 1, !(kb >= kv_begin && kb + kChunkKeys <= wave_lo));
-        }
-        if (has_next) store_tile(it + 1, (it + 1) & 1, st);
-        ids_next = ids_after;
+        if (wave_has_cols && kb < wave_hi) compute_tile(it, it & 1, !(kb >= kv_begin && kb + kChunkKeys <= wave_lo));
+        if (has_next) store_tile(nt, nt & 1, st);
         __syncthreads();
     }
 
     // ---- emit this wave's columns: un-normalised accumulators, log2-domain maximum, sum
-#pragma unroll
-    for (int cb = 0; cb < CB; ++cb) {
-        lane_sum[cb] += __shfl_xor(lane_sum[cb], 16, 64);
-        lane_sum[cb] += __shfl_xor(lane_sum[cb], 32, 64);
-        if (lim[cb] != 0) {
-            if (mc == 0) {
-                a.part_max[part_row[cb]] = run_max[cb];
-                a.part_sum[part_row[cb]] = lane_sum[cb];
-            }
-            float* dst = a.part_acc + part_row[cb] * D + mc * 4;
-#pragma unroll
-            for (int db = 0; db < kDimBlocks; ++db)
-                *reinterpret_cast<float4*>(dst + db * 16) = make_float4(o[cb][db][0], o[cb][db][1], o[cb][db][2], o[cb][db][3]);
+    lane_sum += __shfl_xor(lane_sum, 16, 64);
+    lane_sum += __shfl_xor(lane_sum, 32, 64);
+    if (lim != 0) {
+        if (mc == 0) {
+            a.part_max[part_row] = run_max;
+            a.part_sum[part_row] = lane_sum;
         }
+        float* dst = a.part_acc + part_row * D + mc * 4;
+#pragma unroll
+        for (int db = 0; db < kDimBlocks; ++db)
+            *reinterpret_cast<float4*>(dst + db * 16) = make_float4(o[db][0], o[db][1], o[db][2], o[db][3]);
     }
 }
 
