@@ -97,7 +97,8 @@ template <int D>
 struct ChunkLds {
     static constexpr int kKBytes = kChunkKeys * D * 2;
     static constexpr int kVtBytes = D * kChunkKeys * 2 + (D / 8) * 64;
-    static constexpr int bytes = 2 * (kKBytes + kVtBytes);
+    static constexpr int kIdCap = 4096;  // page IDs of a stretch of the KV range kept in LDS (+8: two tiles of look-ahead)
+    static constexpr int bytes = 2 * (kKBytes + kVtBytes) + (kIdCap + 8) * 4;
 };
 
 template <typename Tag, int D>
@@ -116,7 +117,7 @@ __global__ __launch_bounds__(64 * kChunkWaves, 2) void split_kv_chunk_map(
     constexpr int kBufBytes = kKBytes + kVtBytes;
     constexpr int CB = kChunkColBlocks;
     constexpr float kSlack = 8.0f;
-    constexpr int kIdTiles = 32;  // KV tiles per block of page IDs held in one register (<= 64 pages)
+    constexpr int kIdCap = ChunkLds<D>::kIdCap;
     static_assert(kLoads == 2 && CB == 1, "loader and softmax are written for 8 waves of 16 columns");
     // Dynamic LDS (the launcher passes ChunkLds<D>::bytes): with a static size the compiler sees
     // that one workgroup fills the CU and lifts the register cap.
@@ -182,8 +183,9 @@ __global__ __launch_bounds__(64 * kChunkWaves, 2) void split_kv_chunk_map(
     const uint32_t wave_lo = __builtin_amdgcn_readfirstlane(wave_min_u32(used ? lim : 0xffffffffu));
     const uint32_t wave_hi = __builtin_amdgcn_readfirstlane(wave_max_u32(lim));
 
-    // ---- page walk.  Page IDs of kIdTiles tiles at a time sit in one register (lane l: the l-th page
-    // of the block) and are picked out with v_readlane: no memory access on the per-tile path.
+    // ---- page walk.  The page IDs of a stretch of the KV range (kIdCap pages) sit in LDS, so the
+    // per-tile path has no dependent global access; a tile's two IDs are read one step before they
+    // are needed.
     const uint32_t log2p = 31 - __builtin_clz(a.walk.tokens_per_page);
     const uint32_t page_mask = a.walk.tokens_per_page - 1;
     const uint32_t* table_row = page_ids + ((uint64_t)req_slot * a.walk.num_layers + a.layer) *
@@ -191,23 +193,33 @@ __global__ __launch_bounds__(64 * kChunkWaves, 2) void split_kv_chunk_map(
     const uint32_t last_page = (kv_end_max - 1) >> log2p;
     const uint32_t key_base0 = kv_begin & ~(uint32_t)(kChunkKeys - 1);
     const uint32_t num_kv_tiles = (kv_end_max - key_base0 + kChunkKeys - 1) / kChunkKeys;
-    auto load_id_block = [&](uint32_t first_tile) -> uint32_t {
-        const uint32_t page0 = (key_base0 + first_tile * kChunkKeys) >> log2p;
-        return table_row[min(page0 + lane, last_page)];
+    const uint32_t stretch_tiles = ((uint32_t)kIdCap << log2p) / kChunkKeys;  // tiles per refill of the ID table
+    uint32_t* id_lds = reinterpret_cast<uint32_t*>(lds + 2 * kBufBytes);
+    uint32_t id_page0 = 0;  // page behind id_lds[0]
+    auto refill_ids = [&](uint32_t first_tile) {
+        id_page0 = (key_base0 + first_tile * kChunkKeys) >> log2p;
+        for (uint32_t i = tid; i < (uint32_t)kIdCap + 8; i += 64 * kChunkWaves) id_lds[i] = table_row[min(id_page0 + i, last_page)];
+    };
+    struct TileIds {
+        uint32_t a, b;  // page of keys 0..15 and of keys 16..31 of a tile (the same value in every lane)
+    };
+    // Tiles past the end of the range are clamped to the last one: loads and stores stay
+    // unconditional, which keeps the compiler's count of outstanding loads exact.
+    auto read_ids = [&](uint32_t t) -> TileIds {
+        const uint32_t kb = key_base0 + min(t, num_kv_tiles - 1) * kChunkKeys;
+        return TileIds{id_lds[min(kb >> log2p, last_page) - id_page0], id_lds[min((kb + 16) >> log2p, last_page) - id_page0]};
     };
     struct TileBases {
         const unsigned char* a;  // page of keys 0..15 of the tile, advanced to the tile's first token
         const unsigned char* b;  // page of keys 16..31
     };
     const uint64_t page_bytes = a.walk.page_elems * 2;
-    auto tile_bases = [&](uint32_t it, uint32_t id_block) -> TileBases {
-        const uint32_t kb = key_base0 + it * kChunkKeys;
-        const uint32_t page0 = (key_base0 + (it & ~(uint32_t)(kIdTiles - 1)) * kChunkKeys) >> log2p;
-        const uint32_t ia = min(kb >> log2p, last_page) - page0, ib = min((kb + 16) >> log2p, last_page) - page0;
-        const uint32_t pa = __builtin_amdgcn_readlane(id_block, ia), pb = __builtin_amdgcn_readlane(id_block, ib);
+    auto tile_bases = [&](uint32_t t, TileIds ids) -> TileBases {
+        const uint32_t kb = key_base0 + min(t, num_kv_tiles - 1) * kChunkKeys;
         const uint64_t in_page = (uint64_t)(kb & page_mask) * (D * 2);
         const unsigned char* base = reinterpret_cast<const unsigned char*>(pages);
-        return TileBases{base + pa * page_bytes + in_page, base + pb * page_bytes + in_page};
+        return TileBases{base + __builtin_amdgcn_readfirstlane(ids.a) * page_bytes + in_page,
+                         base + __builtin_amdgcn_readfirstlane(ids.b) * page_bytes + in_page};
     };
 
     // ---- cooperative tile loaders: per-thread byte offsets inside a page are fixed for the kernel
@@ -245,7 +257,7 @@ __global__ __launch_bounds__(64 * kChunkWaves, 2) void split_kv_chunk_map(
     auto store_tile = [&](uint32_t it, uint32_t buf, const Staging& st) __attribute__((always_inline)) {
         unsigned char* kbuf = lds + buf * kBufBytes;
         unsigned char* vbuf = kbuf + kKBytes;
-        const uint32_t kb = key_base0 + it * kChunkKeys;
+        const uint32_t kb = key_base0 + min(it, num_kv_tiles - 1) * kChunkKeys;
         *reinterpret_cast<u32x4_t*>(kbuf + k_store0) = st.k[0];
         *reinterpret_cast<u32x4_t*>(kbuf + k_store1) = st.k[1];
         u32x4_t w0 = st.v[0], w1 = st.v[1];
@@ -295,9 +307,9 @@ __global__ __launch_bounds__(64 * kChunkWaves, 2) void split_kv_chunk_map(
         }
         // ---- online softmax; this lane holds keys kb + 8 * mc + j, j = 4 * b + r, of column mt.
         // Logits relative to the column's reference maximum; masked keys at -inf.
-        float v[8];
+        float v[8];  // raw logits; masked keys at -inf
 #pragma unroll
-        for (int j = 0; j < 8; ++j) v[j] = (j < 4 ? s0[j] : s1[j - 4]) * a.scale_log2;
+        for (int j = 0; j < 8; ++j) v[j] = j < 4 ? s0[j] : s1[j - 4];
         if (masked) {
 #pragma unroll
             for (int j = 0; j < 8; ++j) {
@@ -305,7 +317,8 @@ __global__ __launch_bounds__(64 * kChunkWaves, 2) void split_kv_chunk_map(
                 if (token < kv_begin || token >= lim) v[j] = -INFINITY;
             }
         }
-        float m = fmaxf(fmaxf(fmaxf(v[0], v[1]), fmaxf(v[2], v[3])), fmaxf(fmaxf(v[4], v[5]), fmaxf(v[6], v[7])));
+        // scale > 0: the maximum of the scaled logits is the scaled maximum
+        float m = fmaxf(fmaxf(fmaxf(v[0], v[1]), fmaxf(v[2], v[3])), fmaxf(fmaxf(v[4], v[5]), fmaxf(v[6], v[7]))) * a.scale_log2;
         // The reference maximum moves only when some key exceeds it by more than kSlack (log2 domain):
         // rare after the first tiles, so the cross-lane maximum and the rescaling sit behind a
         // wave-wide test.  A column with no visible key so far keeps max = -inf, sum = 0, O = 0.
@@ -322,11 +335,13 @@ __global__ __launch_bounds__(64 * kChunkWaves, 2) void split_kv_chunk_map(
                     for (int r = 0; r < 4; ++r) o[db][r] *= alpha;
             }
         }
+        // exp2(logit * scale - reference); a column that has seen no key at all (reference -inf) has
+        // only masked keys here: -inf - 0 keeps them at probability 0
+        const float neg_ref = run_max > -INFINITY ? -run_max : 0.0f;
         float p[8], tile_sum = 0.0f;
 #pragma unroll
         for (int j = 0; j < 8; ++j) {
-            // -inf - (-inf) only when the column has seen no key at all: such a key is masked
-            p[j] = v[j] > -INFINITY ? __builtin_amdgcn_exp2f(v[j] - run_max) : 0.0f;
+            p[j] = __builtin_amdgcn_exp2f(__builtin_fmaf(v[j], a.scale_log2, neg_ref));
             tile_sum += p[j];
         }
         lane_sum += tile_sum;
@@ -341,24 +356,35 @@ __global__ __launch_bounds__(64 * kChunkWaves, 2) void split_kv_chunk_map(
         }
     };
 
-    // ---- main loop: tile `it` lives in LDS buffer it % 2; its loads were issued one tile earlier
-    uint32_t id_block = load_id_block(0), id_block_next = 0;
-    {
-        const Staging st = issue_loads(tile_bases(0, id_block));
-        store_tile(0, 0, st);
-    }
-    __syncthreads();
-    for (uint32_t it = 0; it < num_kv_tiles; ++it) {
-        const uint32_t nt = it + 1;  // the tile to fetch now
-        const bool has_next = nt < num_kv_tiles;
-        if ((nt & (kIdTiles - 1)) == kIdTiles / 2) id_block_next = load_id_block((nt & ~(uint32_t)(kIdTiles - 1)) + kIdTiles);
-        if ((nt & (kIdTiles - 1)) == 0) id_block = id_block_next;
-        Staging st;
-        if (has_next) st = issue_loads(tile_bases(nt, id_block));
+    // ---- main loop: tile `it` lives in LDS buffer it % 2.  Its global loads are issued two tiles
+    // earlier into one of two register sets and parked in LDS one tile earlier, so a load has two
+    // tile times to arrive.  The loop body is written twice so that the register sets keep their names.
+    auto step = [&](uint32_t it, Staging& incoming, const Staging& parked, TileIds& ids) __attribute__((always_inline)) {
+        incoming = issue_loads(tile_bases(it + 2, ids));
+        ids = read_ids(it + 3);
         const uint32_t kb = key_base0 + it * kChunkKeys;
-        if (wave_has_cols && kb < wave_hi) compute_tile(it, it & 1, !(kb >= kv_begin && kb + kChunkKeys <= wave_lo));
-        if (has_next) store_tile(nt, nt & 1, st);
+        if (it < num_kv_tiles && wave_has_cols && kb < wave_hi)
+            compute_tile(it, it & 1, !(kb >= kv_begin && kb + kChunkKeys <= wave_lo));
+        store_tile(it + 1, (it + 1) & 1, parked);
         __syncthreads();
+    };
+    refill_ids(0);
+    __syncthreads();
+    Staging st_a, st_b;
+    st_a = issue_loads(tile_bases(0, read_ids(0)));
+    store_tile(0, 0, st_a);
+    st_a = issue_loads(tile_bases(1, read_ids(1)));
+    TileIds ids = read_ids(2);
+    uint32_t next_refill = stretch_tiles;
+    __syncthreads();
+    for (uint32_t it = 0; it < num_kv_tiles; it += 2) {
+        if (it >= next_refill) {  // rare: the range is longer than the ID table
+            refill_ids(it);
+            next_refill += stretch_tiles;
+            __syncthreads();
+        }
+        step(it, st_b, st_a, ids);
+        step(it + 1, st_a, st_b, ids);
     }
 
     // ---- emit this wave's columns: un-normalised accumulators, log2-domain maximum, sum
