@@ -32,7 +32,8 @@ def parse_args():
     p.add_argument("--batch", type=int, default=32)
     p.add_argument("--ctx-lo", type=int, default=1024)
     p.add_argument("--ctx-hi", type=int, default=8192)
-    p.add_argument("--partition", type=int, default=512, help="split-KV partition length in tokens")
+    p.add_argument("--partition", type=int, default=None,
+                   help="split-KV partition length in tokens (default 512; 2048 for the prefill workload)")
     p.add_argument("--arenas", type=int, default=2, help="independent page arenas rotated between steps")
     p.add_argument("--seed", type=int, default=2)
     p.add_argument("--cpu-seconds", type=float, default=12.0, help="budget of the CPU baseline sample")
@@ -169,6 +170,8 @@ def main():
 
     verify = args.workload in ("verify", "prefill")
     prefill = args.workload == "prefill"
+    if args.partition is None:
+        args.partition = 2048 if prefill else 512
     if prefill:
         args.batch, args.q_len = 1, args.chunk
     if verify and args.batch == 32 and args.ctx_lo == 1024 and args.ctx_hi == 8192:

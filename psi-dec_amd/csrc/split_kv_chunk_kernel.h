@@ -2,34 +2,37 @@
 // 2-byte K/V (bf16 / f16), head_dim 256, pages of 16*2^k tokens.  Same results as the
 // multi-query map (semantics of
 // crates/inference-backend-metal/src/components/metal/gqa_split_kv_tiled_q.metal:49-319), other
-// decomposition: the matrix cores are the bound here, not HBM.
+// decomposition: here the matrix cores and the LDS are the bound, not HBM.
 //
 // Work decomposition
-//   one workgroup (4 waves) = one (row group, kv_head).  A row group is a run of consecutive
-//   Q-token tiles of one request whose kv_split rows start at the same key (the rows of one KV
-//   partition).  With more than 5 query heads per KV head the heads are dealt to two workgroups.
-//   The workgroup's query columns, column c = token_in_group * heads + head, are dealt out 32 per
-//   wave: a wave keeps the online-softmax state and the accumulators of its columns for the whole
-//   KV range, so wave states never merge.  The four waves walk the KV range together in tiles of
-//   32 keys which they load once, together, into LDS (two buffers, one barrier per tile).
+//   one workgroup (8 waves) = one (row group, kv_head [, half of the query heads]).  A row group is
+//   a run of consecutive Q-token tiles of one request whose kv_split rows start at the same key
+//   (the rows of one KV partition).  With more than 5 query heads per KV head the heads are dealt
+//   to two workgroups.  The workgroup's query columns, column c = token_in_group * heads + head,
+//   are dealt out 16 per wave: a wave keeps the online-softmax state and the accumulators of its
+//   columns for the whole KV range, so wave states never merge.  The eight waves walk the KV range
+//   together in tiles of 32 keys which they load once, together, into LDS (two buffers, one
+//   barrier per tile; global loads run two tiles ahead in two register sets).
 //
-// Per 32-key tile and wave (2 column blocks of 16)
-//   QK^T  S[key][column] on v_mfma_f32_16x16x32: A = K rows from LDS, B = the query columns, staged
-//         once in LDS in operand order.  Row i of key block b is key 8*(i/4) + 4*b + i%4, so
+// Per 32-key tile and wave (16 columns)
+//   QK^T  S[key][column] on v_mfma_f32_16x16x32: A = K rows from LDS, B = the query columns, held
+//         in registers for the whole kernel.  Row i of key block b is key 8*(i/4) + 4*b + i%4, so
 //         that a lane ends up with keys 8*(lane/16) .. +7 of its column: the B-operand layout of
 //         the next contraction.
-//   softmax  per column, in-lane over 8 keys plus two cross-lane steps; masks only on tiles that
-//         touch the start of the range or a column's causal limit.  The reference maximum of a
-//         column moves only when a tile exceeds it by more than 2^8, so the accumulators are
-//         rescaled a handful of times per range; probabilities stay below 2^8.
+//   softmax  per column, in-lane over 8 keys; masks only on tiles that touch the start of the range
+//         or a column's causal limit.  The reference maximum of a column moves only when a tile
+//         exceeds it by more than 2^8; a wave-wide vote guards the cross-lane maximum and the
+//         rescaling of the accumulators, which therefore run a handful of times per range.
+//         Probabilities stay below 2^8.
 //   PV    O^T[dim][column] += V^T[dim][key] * P^T[key][column] on v_mfma_f32_16x16x32: A = V^T
 //         from LDS (the tile is transposed once, on its way into LDS, so that a lane reads its 8
 //         keys of one dim as one 128-bit word), B = the probabilities from registers.  The
 //         accumulators keep a column per lane, so rescaling needs no cross-lane traffic.  bf16
 //         probabilities are two truncated bf16 terms (two MFMAs), f16 one rounded term.
 //
-// Registers: 128 accumulators + operands stay inside the 256 architectural VGPRs, so every MFMA
-// reads and writes them in place.
+// What bounds it: every wave reads the whole K and V^T tile from LDS (8 x 32 KB per 32 keys), which is
+// about as long as the MFMA work of the tile; 16 columns per wave is what fits next to the query
+// operands in 256 registers.
 //
 // LDS layout per buffer
 //   K    [32 keys][D] elements, 16-byte chunk index XOR (key%4 + 4*(key/8)): the 16 lanes of an
@@ -39,6 +42,7 @@
 //        slot of keys 8s .. 8s+7 at position s XOR (row/4)%4.  Operand reads (16 consecutive rows, one
 //        slot) and transposing stores (4 rows 8 apart, all 16 key pairs) both cover 256 bytes of
 //        distinct banks.
+//   page IDs of up to 4096 pages of the range, refilled for longer ranges.
 #pragma once
 #include "split_kv_tiled_kernel.h"
 
@@ -348,11 +352,16 @@ __global__ __launch_bounds__(64 * kChunkWaves, 2) void split_kv_chunk_map(
         ProbOperand8<Tag> pb;
         pb.set(p);
         // ---- O^T[dim][column] += V^T * P^T
+        // four dim blocks at a time: four independent accumulators between the two terms of one block
 #pragma unroll
-        for (int db = 0; db < kDimBlocks; ++db) {
-            const uint4 vt = *reinterpret_cast<const uint4*>(vbuf + vt_row0 + db * (16 * 64 + 2 * 64));
+        for (int g = 0; g < kDimBlocks; g += 4) {
+            uint4 vt[4];
 #pragma unroll
-            for (int t = 0; t < ProbOperand8<Tag>::kTerms; ++t) o[db] = mfma_16x16x32<Tag>(vt, pb.term[t], o[db]);
+            for (int i = 0; i < 4; ++i) vt[i] = *reinterpret_cast<const uint4*>(vbuf + vt_row0 + (g + i) * (16 * 64 + 2 * 64));
+#pragma unroll
+            for (int t = 0; t < ProbOperand8<Tag>::kTerms; ++t)
+#pragma unroll
+                for (int i = 0; i < 4; ++i) o[g + i] = mfma_16x16x32<Tag>(vt[i], pb.term[t], o[g + i]);
         }
     };
 
