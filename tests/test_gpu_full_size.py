@@ -115,3 +115,48 @@ def test_verify_full_batch_split_and_placement(psi, device):
         del dw
     assert np.isfinite(outs[0]).all()
     assert np.abs(outs[0] - outs[1]).max() < 2e-5
+
+
+def test_c5_prefill_chunk_full_size(psi, oracle, device):
+    """C5's chunk: 2048 new tokens on a 4096-token prefix, 24 Q / 4 KV heads.  The row-group map and
+    the plain multi-query map agree to rounding on the whole chunk, partition lengths do not matter,
+    and sampled query tokens (first, a partition boundary, middle, last) match the scalar oracle run
+    on the device's own pages."""
+    wl = importlib_workloads(psi)
+    w = wl.make_workload(5, [4096 + 2048], 24, 4, 256, psi.Dtype.Bfloat16, 16, q_lens=2048, host_pages=False)
+    variant = psi.GQASplitKVVariant.TiledQ(8, 16, 6)
+    outs = {}
+    for name, partition, grouped in (("grouped 2048", 2048, True), ("grouped 512", 512, True), ("plain 2048", 2048, False)):
+        dw = wl.DeviceWorkload(device, w, partition_tokens=partition, f32_output=True, grouped=grouped, variant=variant)
+        assert (dw.meta.num_row_groups > 0) == grouped
+        dw.step()
+        outs[name] = dw.output_f32().reshape(2048, -1)
+        if name == "grouped 2048":
+            pages = dw.pages_host()
+        del dw
+    assert np.isfinite(outs["grouped 2048"]).all()
+    assert np.abs(outs["grouped 2048"] - outs["grouped 512"]).max() < 1e-4
+    assert np.abs(outs["grouped 2048"] - outs["plain 2048"]).max() < 1e-4
+    picks = np.array([0, 1, 511, 512, 1023, 2040, 2047])
+    dt = oracle_dtype(oracle, w)
+    exp = oracle.paged_gqa(w.num_q_heads, w.num_kv_heads, w.head_dim, w.scale, w.page_bytes, dt, layout_tuple(w),
+                           w.layer, np.repeat(w.req_slots, len(picks)), (w.token_indices[0] + picks).astype(np.uint32),
+                           np.arange(len(picks) + 1, dtype=np.uint32), w.q.reshape(2048, -1)[picks].reshape(-1), pages,
+                           w.page_ids, num_threads=16)
+    assert_outputs_close(outs["grouped 2048"][picks].reshape(-1), exp, "C5 chunk sampled")
+
+
+def test_c5_decode_batch_full_size(psi, device):
+    """C5's decode side: 128 sequences with contexts 512..32768 (about 8.7 GB of K/V), split-count
+    invariance between 512- and 4096-token partitions."""
+    wl = importlib_workloads(psi)
+    ctx = wl.config_c2_context_lens(55, 128, 512, 32768)
+    w = wl.make_workload(55, ctx, 24, 4, 256, psi.Dtype.Bfloat16, 16, host_pages=False)
+    outs = []
+    for partition in (512, 4096):
+        dw = wl.DeviceWorkload(device, w, partition_tokens=partition, f32_output=True)
+        dw.step()
+        outs.append(dw.output_f32())
+        del dw
+    assert np.isfinite(outs[0]).all()
+    assert np.abs(outs[0] - outs[1]).max() < 2e-5
