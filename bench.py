@@ -35,6 +35,8 @@ def parse_args():
     p.add_argument("--partition", type=int, default=None,
                    help="split-KV partition length in tokens (default 512; 2048 for the prefill workload)")
     p.add_argument("--arenas", type=int, default=2, help="independent page arenas rotated between steps")
+    p.add_argument("--q-heads", type=int, default=24, help="decode workload: query heads (24; 16 for the long-context shape)")
+    p.add_argument("--kv-heads", type=int, default=4, help="decode workload: KV heads (4; 2 for the long-context shape)")
     p.add_argument("--seed", type=int, default=2)
     p.add_argument("--cpu-seconds", type=float, default=12.0, help="budget of the CPU baseline sample")
     p.add_argument("--no-cpu-baseline", action="store_true")
@@ -185,8 +187,9 @@ def main():
             w = wl.make_workload(args.seed, ctx, 24, 4, 256, psi.Dtype.Bfloat16, 16, q_lens=args.q_len,
                                  host_pages=False, shuffle_pages=not args.identity_pages)
         else:
-            w = wl.config_c2(seed=args.seed, batch=args.batch, host_pages=False, lo=args.ctx_lo, hi=args.ctx_hi,
-                             shuffle_pages=not args.identity_pages)
+            ctx = wl.config_c2_context_lens(args.seed, args.batch, args.ctx_lo, args.ctx_hi) + 1
+            w = wl.make_workload(args.seed, ctx, args.q_heads, args.kv_heads, 256, psi.Dtype.Bfloat16, 16,
+                                 host_pages=False, shuffle_pages=not args.identity_pages)
         w.seed = args.seed + 1000 * i  # same geometry, different page contents
         arenas.append(wl.DeviceWorkload(device, w, partition_tokens=args.partition, balanced=args.balance,
                                         longest_first=not args.plan_order,
@@ -259,7 +262,7 @@ def main():
     achieved = map_bytes / map_avg_s / 1e9
 
     workload_key = (f"{'verify_q%d' % args.q_len if verify else 'decode'}_b{args.batch}_ctx{args.ctx_lo}-{args.ctx_hi}"
-                    f"_24q4kv_d256_bf16_p16_part{args.partition}_seed{args.seed}")
+                    f"_{w.num_q_heads}q{w.num_kv_heads}kv_d256_bf16_p16_part{args.partition}_seed{args.seed}")
     result = {
         "metric": "decode attn achieved HBM GB/s per layer-step (B=32, ctx 1k-8k); us/layer-step alongside",
         "value": (map_bytes if args.kernel_only else step_bytes) / (ms_per_step / 1e3) / 1e9,
