@@ -61,6 +61,7 @@ struct ReduceArgs {
     void* output;
     uint32_t hq, d;
     uint32_t num_active_tokens;
+    uint32_t num_total_kv_splits = 0;  // capacity of the split list (sizes the combine's parallelism)
     uint32_t out_dtype = PSI_HIP_F32;  // element type of `output`
     // Optional: the partial rows of token / tile t are row_index[cu[t] .. cu[t + 1]) instead of
     // cu[t] .. cu[t + 1] themselves (plans whose rows were re-ordered for dispatch).

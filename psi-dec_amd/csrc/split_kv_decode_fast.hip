@@ -57,6 +57,75 @@ __global__ __launch_bounds__(256) void split_kv_reduce_fast(ReduceArgs a) {
     for (int e = 0; e < kPerLane; ++e) store_from_f32<Tag>(a.output, out_index + e, value[e] * inv);
 }
 
+// The combine for long split lists (long contexts, few tokens): one workgroup of eight waves per
+// (token, q_head); wave w takes the rows begin + w, begin + w + 8, ... four at a time, and the wave
+// results, all relative to the same maximum, are added through LDS.
+constexpr int kWideWaves = 8;
+template <typename Tag, int D, bool kIndexed>
+__global__ __launch_bounds__(64 * kWideWaves) void split_kv_reduce_wide(ReduceArgs a) {
+    constexpr int kPerLane = D / 64;
+    constexpr int kUnroll = 4;
+    __shared__ float wave_max[kWideWaves];
+    __shared__ float wave_sum[kWideWaves];
+    __shared__ float wave_val[kWideWaves][D];
+    const uint32_t lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const uint64_t row_out = blockIdx.x;
+    const uint32_t token = (uint32_t)(row_out / a.hq), q_head = (uint32_t)(row_out % a.hq);
+    const uint32_t begin = a.cu_kv_splits[token], end = a.cu_kv_splits[token + 1];
+    const uint32_t* row_index = a.row_index;
+    float global_max = -INFINITY;
+    for (uint32_t p = begin + threadIdx.x; p < end; p += 64 * kWideWaves)
+        global_max = fmaxf(global_max, a.part_max[(uint64_t)(kIndexed ? row_index[p] : p) * a.hq + q_head]);
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) global_max = fmaxf(global_max, __shfl_xor(global_max, off, 64));
+    if (lane == 0) wave_max[wave] = global_max;
+    __syncthreads();
+#pragma unroll
+    for (int w = 0; w < kWideWaves; ++w) global_max = fmaxf(global_max, wave_max[w]);
+    float weight_sum = 0.0f, value[kPerLane];
+#pragma unroll
+    for (int e = 0; e < kPerLane; ++e) value[e] = 0.0f;
+    for (uint32_t p0 = begin + wave; p0 < end; p0 += kWideWaves * kUnroll) {
+        float w[kUnroll], sums[kUnroll], part[kUnroll][kPerLane];
+#pragma unroll
+        for (int u = 0; u < kUnroll; ++u) {
+            const bool live = p0 + u * kWideWaves < end;
+            const uint32_t p = live ? p0 + u * kWideWaves : begin;
+            const uint64_t row = (uint64_t)(kIndexed ? row_index[p] : p) * a.hq + q_head;
+            const float m = a.part_max[row];
+            sums[u] = a.part_sum[row];
+            w[u] = live && m > -INFINITY ? exp2f(m - global_max) : 0.0f;
+            const float* src = a.part_acc + row * D + lane * kPerLane;
+#pragma unroll
+            for (int e = 0; e < kPerLane; ++e) part[u][e] = src[e];
+        }
+#pragma unroll
+        for (int u = 0; u < kUnroll; ++u) {
+            weight_sum = fmaf(w[u], sums[u], weight_sum);
+#pragma unroll
+            for (int e = 0; e < kPerLane; ++e) value[e] = fmaf(w[u], part[u][e], value[e]);
+        }
+    }
+    if (lane == 0) wave_sum[wave] = weight_sum;
+#pragma unroll
+    for (int e = 0; e < kPerLane; ++e) wave_val[wave][lane * kPerLane + e] = value[e];
+    __syncthreads();
+    if (wave != 0) return;
+    weight_sum = 0.0f;
+#pragma unroll
+    for (int e = 0; e < kPerLane; ++e) value[e] = 0.0f;
+#pragma unroll
+    for (int w = 0; w < kWideWaves; ++w) {
+        weight_sum += wave_sum[w];
+#pragma unroll
+        for (int e = 0; e < kPerLane; ++e) value[e] += wave_val[w][lane * kPerLane + e];
+    }
+    const float inv = weight_sum > 0.0f ? 1.0f / weight_sum : 0.0f;
+    const uint64_t out_index = row_out * D + lane * kPerLane;
+#pragma unroll
+    for (int e = 0; e < kPerLane; ++e) store_from_f32<Tag>(a.output, out_index + e, value[e] * inv);
+}
+
 // The same combine for Q-token tiles: one wave per (tile, token in tile, q_head); the tile's partial
 // rows are cu_kv_splits[tile] .. cu_kv_splits[tile + 1].
 template <typename Tag, int D, bool kIndexed>
@@ -137,9 +206,13 @@ int launch_reduce_fast(psi_hip_ctx* ctx, const Geometry& g, const ReduceArgs& a)
                                 : (uint64_t)a.num_active_tokens * g.hq;
     if ((rows + 3) / 4 > 0x7fffffffull) return PSI_HIP_ERR_UNSUPPORTED;
     const dim3 grid((uint32_t)((rows + 3) / 4)), block(256);
+    // long split lists on few tokens: a workgroup per output row instead of a wave
+    const bool wide = !tiled && a.num_active_tokens != 0 && a.num_total_kv_splits / a.num_active_tokens >= 32 &&
+                      rows <= 0x7fffffffull;
 #define PSI_REDUCE_D(TAG, DIM, INDEXED)                                                                          \
     do {                                                                                                         \
         if (tiled) hipLaunchKernelGGL((split_kv_reduce_tiled_fast<TAG, DIM, INDEXED>), grid, block, 0, ctx->stream, a); \
+        else if (wide) hipLaunchKernelGGL((split_kv_reduce_wide<TAG, DIM, INDEXED>), dim3((uint32_t)rows), dim3(64 * kWideWaves), 0, ctx->stream, a); \
         else hipLaunchKernelGGL((split_kv_reduce_fast<TAG, DIM, INDEXED>), grid, block, 0, ctx->stream, a);     \
     } while (0)
 #define PSI_REDUCE(TAG)                                                   \

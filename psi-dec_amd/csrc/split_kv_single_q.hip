@@ -158,6 +158,7 @@ extern "C" int psi_hip_split_kv_single_q_reduce(psi_hip_ctx* ctx, const psi_hip_
     a.d = g.d;
     a.out_dtype = ctx->f32_output ? PSI_HIP_F32 : g.dtype;
     a.num_active_tokens = num_active_tokens;
+    a.num_total_kv_splits = num_total_kv_splits;
 
     LaunchScope scope(ctx, "split_kv_reduce");
     rc = launch_reduce_fast(ctx, g, a);

@@ -122,3 +122,17 @@ def test_longest_first_dispatch_order(psi, oracle, device, q_len):
     plain = wl.DeviceWorkload(device, w, partition_tokens=512, f32_output=True)
     plain.step()
     assert np.array_equal(plain.output_f32(), dw.output_f32())
+
+
+@pytest.mark.parametrize("longest_first", [False, True])
+def test_long_split_lists_use_the_wide_combine(psi, oracle, device, longest_first):
+    """Two sequences of 6000 and 3000 tokens cut into 16-token partitions: 375 and 188 rows per token,
+    merged by the workgroup-per-row combine; one-token and many-token partitions must agree too."""
+    wl = importlib_workloads(psi)
+    w = wl.make_workload(77, [6000, 3000], 16, 2, 256, psi.Dtype.Bfloat16, 16)
+    variant = psi.GQASplitKVVariant.SingleQ(16, 256, 8)
+    stats, dw = run_and_check(psi, oracle, device, w, "wide combine", partition_tokens=16, variant=variant,
+                              longest_first=longest_first)
+    assert dw.shape.num_sdpa_map_task_templates == 375 + 188
+    _, dw2 = run_and_check(psi, oracle, device, w, "narrow combine", partition_tokens=1024, variant=variant)
+    assert np.abs(dw.output_f32() - dw2.output_f32()).max() < 2e-5
