@@ -197,6 +197,81 @@ int psi_hip_split_kv_balance_plan(const uint32_t* kv_splits_in, uint32_t num_row
 /* Workers per KV head that fill the device exactly once with decode-map workgroups. */
 int psi_hip_split_kv_balanced_workers(const psi_hip_gqa_config* cfg, uint32_t* out_num_workers);
 
+/* ------------------------------------------------------------------ projections around the attention
+ *
+ * The kernels a gated GQA layer records before and after the attention proper
+ * (crates/inference-executor-metal/src/attn/gqa/backend.rs:394-658): QGKV split, Q / K RMSNorm + RoPE, sigmoid
+ * gate.  Each has a stand-alone entry point with the reference component's meaning; the K side is also fused
+ * into the append (psi_hip_kv_page_write_norm_rope) and the gate into the combine (`gate` argument of the two
+ * reduce entry points), which removes a global round trip of K and of the attention output.  Inputs may be
+ * strided views of the projection output, so the split itself is optional. */
+
+#define PSI_HIP_ROPE_DEFAULT 0u
+#define PSI_HIP_ROPE_YARN 1u
+
+/* `RopeScaling` (crates/inference-backend-metal/src/components/rms_norm_rope.rs:16-27). */
+typedef struct psi_hip_rope_scaling {
+    uint32_t kind; /* PSI_HIP_ROPE_DEFAULT: the other fields are ignored */
+    float factor;
+    float attention_factor;
+    float beta_fast;
+    float beta_slow;
+    uint32_t original_max_position_embeddings;
+    uint32_t truncate;
+} psi_hip_rope_scaling;
+
+/* `RMSNormRopeConfig` (rms_norm_rope.rs:40-49; validate :81-96).  dtype: f32 or bf16 like the reference, or f16. */
+typedef struct psi_hip_rms_norm_rope_config {
+    uint32_t num_heads;
+    uint32_t head_dim;
+    uint32_t rope_dim; /* even, 2 .. min(head_dim, 256) */
+    float eps;
+    float rope_theta;
+    psi_hip_rope_scaling scaling;
+    uint32_t dtype;
+} psi_hip_rms_norm_rope_config;
+
+/* Attention-output gate for the combine: gates in the IO dtype, element (token, q_head, d) at
+ * gates[token * token_stride + q_head * head_stride + d].  [T][Hq][D] from a split: strides Hq*D and D; the
+ * projection output in place: pointer qgkv + D, strides 2*(Hq+Hkv)*D and 2*D. */
+typedef struct psi_hip_output_gate {
+    const void* gates;
+    uint64_t token_stride;
+    uint64_t head_stride;
+} psi_hip_output_gate;
+
+/* Host helper: `RopeScaling::kernel_parameters` (rms_norm_rope.rs:170-238): the f32 inverse frequencies
+ * [rope_dim / 2] the kernels use (theta^(-d / half), Yarn ramp applied), the attention factor, and the Yarn
+ * correction range (low, high) when out_correction is not null and the scaling is Yarn. */
+int psi_hip_rope_parameters(const psi_hip_rms_norm_rope_config* cfg, float* out_inverse_frequencies,
+                            float* out_attention_factor, float* out_correction);
+
+/* `RMSNormRopeKernel::invoke_bucketed` (rms_norm_rope.rs:273-296; kernel metal/rms_norm_rope.metal:7-82).
+ * input: device, row (token, head) at input + (token * input_token_stride + head * input_head_stride) elements;
+ * strides 0 = dense [T][heads][head_dim].  norm_weight: device bf16[head_dim].  flat_token_indices: device
+ * u32[T], the rotary position of each token.  output: device, dense [T][heads][head_dim]; may alias a dense
+ * input.  Per row: x * rsqrt(mean(x^2) + eps) rounded to dtype, times the weight rounded to dtype (product in
+ * dtype), dims below rope_dim rotated in f32 as pairs (d, d + rope_dim / 2).  Rows of tokens >=
+ * num_active_tokens keep their bytes. */
+int psi_hip_rms_norm_rope(psi_hip_ctx* ctx, const psi_hip_rms_norm_rope_config* cfg, const void* input,
+                          uint64_t input_token_stride, uint64_t input_head_stride, const void* norm_weight,
+                          const uint32_t* flat_token_indices, void* output, uint32_t num_total_tokens,
+                          uint32_t num_active_tokens);
+
+/* `GQAQGKVSplitKernel::invoke_bucketed` (crates/inference-backend-metal/src/components/gqa_qgkv_split.rs; kernel
+ * metal/gqa_qgkv_split.metal:5-43).  qgkv: device [T][q_0|g_0|q_1|g_1|...|k|v]; q, g: device [T][Hq][D];
+ * k, v: device [T][Hkv][D]. */
+int psi_hip_qgkv_split(psi_hip_ctx* ctx, uint32_t num_q_heads, uint32_t num_kv_heads, uint32_t head_dim,
+                       uint32_t dtype, const void* qgkv, void* q, void* g, void* k, void* v,
+                       uint32_t num_total_tokens, uint32_t num_active_tokens);
+
+/* `GQAActivationGateKernel::invoke_bucketed` (gqa_split_kv_single_q.rs:453-543; kernel
+ * metal/gqa_activation_gate.metal:13-38): output = attention_output * sigmoid(gates), all [T][Hq][D] in dtype;
+ * the 2-byte variants round after every step of the sigmoid.  output may alias attention_output. */
+int psi_hip_activation_gate(psi_hip_ctx* ctx, uint32_t num_q_heads, uint32_t head_dim, uint32_t dtype,
+                            const void* attention_output, const void* gates, void* output,
+                            uint32_t num_total_tokens, uint32_t num_active_tokens);
+
 /* ------------------------------------------------------------------ KV append */
 
 /* `GQAKVPageWrite::invoke_bucketed(...)` recorded and submitted
@@ -212,6 +287,22 @@ int psi_hip_kv_page_write(psi_hip_ctx* ctx, const psi_hip_gqa_config* cfg, const
                           const uint32_t* req_slots, const uint32_t* flat_token_indices, const uint32_t* page_ids,
                           uint32_t num_total_token_writes, uint32_t num_active_token_writes,
                           uint32_t gqa_layer_index);
+
+/* The K-side RMSNorm + RoPE (psi_hip_rms_norm_rope with num_heads = num_kv_heads, positions =
+ * flat_token_indices) fused into the append: the raw K rows are normalised, rotated and written straight into
+ * their page lines; V rows are copied.  No counterpart as one kernel in the reference, which records
+ * RMSNormRope(k) then GQAKVPageWrite (backend.rs:470-560).  raw_k / flat_v: row (token, kv_head) at
+ * base + token * token_stride + kv_head * head_dim elements (token strides 0 = dense [T][Hkv][D]; the projection
+ * output in place: pointers qgkv + 2*Hq*D and qgkv + (2*Hq + Hkv)*D, strides 2*(Hq+Hkv)*D).
+ * norm_cfg->num_heads must equal cfg->num_kv_heads, head_dim and dtype must match cfg. */
+int psi_hip_kv_page_write_norm_rope(psi_hip_ctx* ctx, const psi_hip_gqa_config* cfg,
+                                    const psi_hip_page_table_layout* layout,
+                                    const psi_hip_rms_norm_rope_config* norm_cfg, void* pages, uint64_t pages_bytes,
+                                    const void* raw_k, uint64_t k_token_stride, const void* flat_v,
+                                    uint64_t v_token_stride, const void* norm_weight, const uint32_t* req_slots,
+                                    const uint32_t* flat_token_indices, const uint32_t* page_ids,
+                                    uint32_t num_total_token_writes, uint32_t num_active_token_writes,
+                                    uint32_t gqa_layer_index);
 
 /* ------------------------------------------------------------------ split-KV decode (SingleQ) */
 
@@ -249,11 +340,15 @@ int psi_hip_split_kv_single_q_map_balanced(psi_hip_ctx* ctx, const psi_hip_gqa_c
  * metal/gqa_split_kv_single_q_reduce.metal:10-49).  cu_kv_splits: device u32[num_total_tokens + 1];
  * output: device [num_total_tokens, Hq, D]; rows >= num_active_tokens keep their bytes. */
 /* partial_row_index: device u32[num_total_kv_splits] from psi_hip_split_kv_order_longest_first, or null
- * when the rows of a token are adjacent as planned. */
+ * when the rows of a token are adjacent as planned.
+ * gate: null, or the attention-output gate of a gated GQA layer (metal/gqa_activation_gate.metal:13-38) applied
+ * to each output element right after it is rounded to the IO dtype -- the result of the combine followed by
+ * psi_hip_activation_gate, without the round trip. */
 int psi_hip_split_kv_single_q_reduce(psi_hip_ctx* ctx, const psi_hip_gqa_config* cfg, const void* scratch,
                                      uint64_t scratch_bytes, const uint32_t* cu_kv_splits, void* output,
                                      uint32_t num_total_tokens, uint32_t num_total_kv_splits,
-                                     uint32_t num_active_tokens, const uint32_t* partial_row_index);
+                                     uint32_t num_active_tokens, const uint32_t* partial_row_index,
+                                     const psi_hip_output_gate* gate);
 
 /* ------------------------------------------------------------------ split-KV verify / prefill (TiledQ) */
 
@@ -318,7 +413,8 @@ int psi_hip_split_kv_tiled_q_reduce(psi_hip_ctx* ctx, const psi_hip_gqa_config* 
                                     const void* scratch, uint64_t scratch_bytes, const uint32_t* q_token_tiles,
                                     const uint32_t* cu_kv_splits, void* output, uint32_t num_total_tokens,
                                     uint32_t num_total_q_token_tiles, uint32_t num_total_kv_splits,
-                                    uint32_t num_active_q_token_tiles, const uint32_t* partial_row_index);
+                                    uint32_t num_active_q_token_tiles, const uint32_t* partial_row_index,
+                                    const psi_hip_output_gate* gate);
 
 /* ------------------------------------------------------------------ request page table */
 

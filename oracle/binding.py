@@ -54,6 +54,16 @@ def load():
     lib.psi_oracle_paged_gqa.argtypes = [c_uint32, c_uint32, c_uint32, c_float, c_uint32, c_uint32, c_uint32,
                                          c_uint32, c_uint32, c_uint32, c_uint32, c_uint32, c_void_p, c_void_p,
                                          c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int]
+    lib.psi_oracle_qgkv_split.restype = c_int
+    lib.psi_oracle_qgkv_split.argtypes = [c_void_p] * 5 + [c_uint32] * 5
+    lib.psi_oracle_rope_parameters.restype = c_int
+    lib.psi_oracle_rope_parameters.argtypes = [c_uint32, c_float, c_int, c_float, c_float, c_float, c_float, c_uint32,
+                                               c_int, c_void_p, POINTER(c_float), c_void_p]
+    lib.psi_oracle_rms_norm_rope.restype = c_int
+    lib.psi_oracle_rms_norm_rope.argtypes = [c_void_p, c_void_p, c_void_p, c_void_p, c_uint32, c_uint32, c_uint32,
+                                             c_uint32, c_float, c_void_p, c_float, c_uint32]
+    lib.psi_oracle_activation_gate.restype = c_int
+    lib.psi_oracle_activation_gate.argtypes = [c_void_p, c_void_p, c_void_p, c_uint64, c_uint32]
     _lib = lib
     return lib
 
@@ -154,4 +164,59 @@ def paged_gqa(num_q_heads, num_kv_heads, head_dim, scale, page_bytes, dtype, lay
                                      _p(pages), _p(pid), _p(out), num_threads)
     if rc != 0:
         raise ValueError("paged_gqa oracle rejected its input")
+    return out
+
+
+def _storage(dtype):
+    return np.float32 if dtype == F32 else np.uint16
+
+
+def qgkv_split(qgkv, num_tokens, num_q_heads, num_kv_heads, head_dim, dtype):
+    """Storage array [tokens][2*Hq*D + 2*Hkv*D] -> (q, g, k, v) storage arrays."""
+    qgkv = np.ascontiguousarray(qgkv, dtype=_storage(dtype))
+    q = np.zeros(num_tokens * num_q_heads * head_dim, _storage(dtype))
+    g = np.zeros_like(q)
+    k = np.zeros(num_tokens * num_kv_heads * head_dim, _storage(dtype))
+    v = np.zeros_like(k)
+    load().psi_oracle_qgkv_split(_p(qgkv), _p(q), _p(g), _p(k), _p(v), num_tokens, num_q_heads, num_kv_heads, head_dim,
+                                 dtype)
+    return q, g, k, v
+
+
+def rope_parameters(rope_dim, rope_theta, yarn=None):
+    """yarn: None or dict(factor, attention_factor, beta_fast, beta_slow, original_max_position_embeddings,
+    truncate).  Returns (inverse_frequencies f32[rope_dim / 2], attention_factor, (low, high) or None)."""
+    inv = np.zeros(rope_dim // 2, np.float32)
+    corr = np.zeros(2, np.float32)
+    factor = c_float()
+    y = yarn or {}
+    rc = load().psi_oracle_rope_parameters(
+        rope_dim, rope_theta, 1 if yarn else 0, y.get("factor", 1.0), y.get("attention_factor", 1.0),
+        y.get("beta_fast", 1.0), y.get("beta_slow", 1.0), y.get("original_max_position_embeddings", 1),
+        1 if y.get("truncate", False) else 0, _p(inv), ctypes.byref(factor), _p(corr))
+    if rc != 0:
+        raise ValueError("rope parameters rejected")
+    return inv, factor.value, (tuple(float(x) for x in corr) if yarn else None)
+
+
+def rms_norm_rope(x, norm_weight_bf16, positions, num_heads, head_dim, rope_dim, eps, inverse_frequencies,
+                  attention_factor, dtype):
+    """x: storage array [tokens][heads][head_dim]; norm_weight_bf16: uint16[head_dim]; returns a storage array."""
+    x = np.ascontiguousarray(x, dtype=_storage(dtype))
+    w = np.ascontiguousarray(norm_weight_bf16, dtype=np.uint16)
+    pos = _u32(positions)
+    inv = np.ascontiguousarray(inverse_frequencies, dtype=np.float32)
+    out = x.copy()
+    rc = load().psi_oracle_rms_norm_rope(_p(x), _p(w), _p(pos), _p(out), len(pos), num_heads, head_dim, rope_dim, eps,
+                                         _p(inv), attention_factor, dtype)
+    if rc != 0:
+        raise ValueError("rms_norm_rope oracle rejected its input")
+    return out
+
+
+def activation_gate(attention_output, gates, dtype):
+    a = np.ascontiguousarray(attention_output, dtype=_storage(dtype)).ravel()
+    g = np.ascontiguousarray(gates, dtype=_storage(dtype)).ravel()
+    out = np.zeros_like(a)
+    load().psi_oracle_activation_gate(_p(a), _p(g), _p(out), a.size, dtype)
     return out

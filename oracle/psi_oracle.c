@@ -315,3 +315,161 @@ int psi_oracle_paged_gqa(uint32_t num_q_heads, uint32_t num_kv_heads, uint32_t h
     free(qf);
     return status;
 }
+
+/* ---------------------------------------------------------------- projections around the attention
+ *
+ * Restated from the reference's pre / post kernels of a gated GQA layer:
+ *   psi_oracle_qgkv_split            crates/inference-backend-metal/src/components/metal/gqa_qgkv_split.metal:5-43
+ *   psi_oracle_rope_parameters       crates/inference-backend-metal/src/components/rms_norm_rope.rs:170-238
+ *   psi_oracle_rms_norm_rope         crates/inference-backend-metal/src/components/metal/rms_norm_rope.metal:7-82
+ *   psi_oracle_activation_gate       crates/inference-backend-metal/src/components/metal/gqa_activation_gate.metal:13-38
+ * What pins them (tests/test_oracle.py): the two-token split / norm_rope_2 / gate closed forms of
+ * crates/inference-executor-metal/src/attn/gqa/backend.rs:883-1027, the Yarn correction range 14 / 29 and the
+ * long-context Yarn closed form of rms_norm_rope.rs:395-470, and the bf16 rounding-order vector of
+ * rms_norm_rope.rs:472-517.  The reference's kernels call Metal's fast cos / sin / exp; this file uses libm, and
+ * the reference's own tests allow 1e-3 (long context) and 2e-5 (small positions) for that.
+ */
+
+/* One token row [q_0 | g_0 | q_1 | g_1 | ... | k | v] -> q, g [Hq][D] and k, v [Hkv][D]. */
+int psi_oracle_qgkv_split(const void* qgkv, void* q, void* g, void* k, void* v, uint32_t num_active_tokens,
+                          uint32_t num_q_heads, uint32_t num_kv_heads, uint32_t head_dim, uint32_t dtype) {
+    const size_t es = dtype_size(dtype);
+    const uint64_t q_slots = (uint64_t)num_q_heads * head_dim, kv_slots = (uint64_t)num_kv_heads * head_dim;
+    const uint64_t width = 2 * q_slots + 2 * kv_slots;
+    for (uint64_t gid = 0; gid < (uint64_t)num_active_tokens * width; ++gid) {
+        const uint64_t token = gid / width;
+        uint64_t slot = gid - token * width;
+        const char* src = (const char*)qgkv + gid * es;
+        if (slot < 2 * q_slots) {
+            const uint64_t pair = slot / (2 * head_dim), in_pair = slot - pair * 2 * head_dim;
+            const uint64_t dst = (token * num_q_heads + pair) * head_dim + in_pair % head_dim;
+            memcpy((char*)(in_pair < head_dim ? q : g) + dst * es, src, es);
+            continue;
+        }
+        slot -= 2 * q_slots;
+        if (slot < kv_slots) {
+            memcpy((char*)k + (token * kv_slots + slot) * es, src, es);
+            continue;
+        }
+        slot -= kv_slots;
+        memcpy((char*)v + (token * kv_slots + slot) * es, src, es);
+    }
+    return 0;
+}
+
+/* Inverse frequencies [rope_dim / 2] and the attention factor.  yarn == 0: plain RoPE.
+ * correction[2] receives the (low, high) Yarn correction range when yarn != 0. */
+int psi_oracle_rope_parameters(uint32_t rope_dim, float rope_theta, int yarn, float factor, float attention_factor,
+                               float beta_fast, float beta_slow, uint32_t original_max_position_embeddings,
+                               int truncate, float* inverse_frequencies, float* out_attention_factor,
+                               float* correction) {
+    if (rope_dim == 0 || rope_dim % 2 != 0 || !(rope_theta > 0.0f)) return -1;
+    float low = 0.0f, high = 0.0f;
+    if (yarn) {
+        const double dimension = (double)rope_dim, base = (double)rope_theta;
+        const double original_length = (double)original_max_position_embeddings;
+        const double tau = 6.283185307179586476925286766559;
+        low = (float)(dimension * log(original_length / ((double)beta_fast * tau)) / (2.0 * log(base)));
+        high = (float)(dimension * log(original_length / ((double)beta_slow * tau)) / (2.0 * log(base)));
+        if (low < 0.0f) low = 0.0f;
+        const float cap = (float)(rope_dim > 0 ? rope_dim - 1 : 0);
+        if (high > cap) high = cap;
+        if (truncate) {
+            low = floorf(low);
+            high = ceilf(high);
+        }
+        if (low > high) return -1;
+        if (low == high) high += 0.001f;
+        if (correction) {
+            correction[0] = low;
+            correction[1] = high;
+        }
+    }
+    const uint32_t half = rope_dim / 2;
+    for (uint32_t d = 0; d < half; ++d) {
+        float inv = powf(rope_theta, -((float)d / (float)half));
+        if (yarn) {
+            float ramp = ((float)d - low) / (high - low);
+            ramp = ramp < 0.0f ? 0.0f : (ramp > 1.0f ? 1.0f : ramp);
+            inv *= 1.0f + ramp * (1.0f / factor - 1.0f);
+        }
+        inverse_frequencies[d] = inv;
+    }
+    *out_attention_factor = yarn ? attention_factor : 1.0f;
+    return 0;
+}
+
+/* Rounds through the storage type: T(x) of the Metal source. */
+static float round_to(float v, uint32_t dtype) {
+    if (dtype == PSI_ORACLE_BF16) return psi_oracle_bf16_to_f32(psi_oracle_f32_to_bf16(v));
+    if (dtype == PSI_ORACLE_F16) return psi_oracle_f16_to_f32(psi_oracle_f32_to_f16(v));
+    return v;
+}
+static void store_elem(void* base, uint64_t index, uint32_t dtype, float v) {
+    if (dtype == PSI_ORACLE_F32) ((float*)base)[index] = v;
+    else if (dtype == PSI_ORACLE_BF16) ((uint16_t*)base)[index] = psi_oracle_f32_to_bf16(v);
+    else ((uint16_t*)base)[index] = psi_oracle_f32_to_f16(v);
+}
+
+/* rows = num_active_tokens * num_heads; input / output [tokens][heads][head_dim] in `dtype`; norm_weight is bf16
+ * bits.  Per row: inv = 1 / sqrt(mean(x^2) + eps) in f32 (sequential sum); normalised element
+ * T(T(w) * T(x * inv)); dims d < rope_dim / 2 rotate with their partner d + rope_dim / 2 in f32 at angle
+ * position * inverse_frequencies[d]; dims >= rope_dim are the normalised element.  The weight product is
+ * formed in the storage type: for bf16, a product of two bf16 values rounded once. */
+int psi_oracle_rms_norm_rope(const void* input, const uint16_t* norm_weight, const uint32_t* flat_token_indices,
+                             void* output, uint32_t num_active_tokens, uint32_t num_heads, uint32_t head_dim,
+                             uint32_t rope_dim, float eps, const float* inverse_frequencies, float attention_factor,
+                             uint32_t dtype) {
+    if (rope_dim > head_dim || rope_dim % 2 != 0) return -1;
+    const uint32_t half = rope_dim / 2;
+    for (uint64_t row = 0; row < (uint64_t)num_active_tokens * num_heads; ++row) {
+        const uint64_t base = row * head_dim;
+        float acc = 0.0f;
+        for (uint32_t d = 0; d < head_dim; ++d) {
+            const float x = load_elem(input, base + d, dtype);
+            acc += x * x;
+        }
+        const float inv = 1.0f / sqrtf(acc / (float)head_dim + eps);
+        const float position = (float)flat_token_indices[row / num_heads];
+        for (uint32_t d = 0; d < head_dim; ++d) {
+            if (d < half) {
+                const uint32_t d2 = d + half;
+                const float x1 = round_to(round_to(psi_oracle_bf16_to_f32(norm_weight[d]), dtype) *
+                                              round_to(load_elem(input, base + d, dtype) * inv, dtype), dtype);
+                const float x2 = round_to(round_to(psi_oracle_bf16_to_f32(norm_weight[d2]), dtype) *
+                                              round_to(load_elem(input, base + d2, dtype) * inv, dtype), dtype);
+                const float theta = position * inverse_frequencies[d];
+                const float c = cosf(theta), s = sinf(theta);
+                store_elem(output, base + d, dtype, attention_factor * (x1 * c - x2 * s));
+                store_elem(output, base + d2, dtype, attention_factor * (x1 * s + x2 * c));
+            } else if (d >= rope_dim) {
+                store_elem(output, base + d, dtype,
+                           round_to(psi_oracle_bf16_to_f32(norm_weight[d]), dtype) *
+                               round_to(load_elem(input, base + d, dtype) * inv, dtype));
+            }
+        }
+    }
+    return 0;
+}
+
+/* sigmoid(x) = y or 1 - y with y = 1 / (1 + exp(-|x|)); the bf16 variant rounds to bf16 after every step
+ * (gqa_activation_gate.metal:13-27).  output = T(attention_output * sigmoid(gate)). */
+int psi_oracle_activation_gate(const void* attention_output, const void* gates, void* output, uint64_t count,
+                               uint32_t dtype) {
+    for (uint64_t i = 0; i < count; ++i) {
+        const float a = load_elem(attention_output, i, dtype), x = load_elem(gates, i, dtype);
+        float s;
+        if (dtype == PSI_ORACLE_F32) {
+            const float y = 1.0f / (1.0f + expf(-fabsf(x)));
+            s = x < 0.0f ? 1.0f - y : y;
+        } else {
+            const float abs_x = round_to(fabsf(x), dtype);
+            const float exp_x = round_to(expf(-abs_x), dtype);
+            const float denom = round_to(1.0f + exp_x, dtype);
+            const float y = round_to(1.0f / denom, dtype);
+            s = x < 0.0f ? round_to(1.0f - y, dtype) : y;
+        }
+        store_elem(output, i, dtype, a * s);
+    }
+    return 0;
+}

@@ -16,12 +16,14 @@ from .gqa import *  # noqa: F401,F403
 from .gqa import (  # noqa: F401
     Device,
     Dtype,
+    GQAActivationGateKernel,
     GQAKVPageWrite,
     GQAKVPageWriteBuffers,
     GQAKVPageWriteConfig,
     GQAKVPageWriteShape,
     GQAMetadataBuffers,
     GQAPageTableLayout,
+    GQAQGKVSplitKernel,
     GQAReplayBucketPolicy,
     GQAReplayShape,
     GQARequestPageTable,
@@ -36,7 +38,11 @@ from .gqa import (  # noqa: F401
     GQASplitKVTiledQScratch,
     GQASplitKVTiledQShape,
     GQASplitKVVariant,
+    OutputGate,
     ReplayBucketPolicy,
+    RMSNormRopeConfig,
+    RMSNormRopeKernel,
+    RopeScaling,
     balanced_workers,
     select_split_kv_variant,
 )

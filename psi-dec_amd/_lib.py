@@ -65,6 +65,34 @@ class VariantStruct(ctypes.Structure):
     ]
 
 
+class RopeScalingStruct(ctypes.Structure):
+    _fields_ = [
+        ("kind", c_uint32),
+        ("factor", c_float),
+        ("attention_factor", c_float),
+        ("beta_fast", c_float),
+        ("beta_slow", c_float),
+        ("original_max_position_embeddings", c_uint32),
+        ("truncate", c_uint32),
+    ]
+
+
+class RMSNormRopeConfigStruct(ctypes.Structure):
+    _fields_ = [
+        ("num_heads", c_uint32),
+        ("head_dim", c_uint32),
+        ("rope_dim", c_uint32),
+        ("eps", c_float),
+        ("rope_theta", c_float),
+        ("scaling", RopeScalingStruct),
+        ("dtype", c_uint32),
+    ]
+
+
+class OutputGateStruct(ctypes.Structure):
+    _fields_ = [("gates", c_void_p), ("token_stride", c_uint64), ("head_stride", c_uint64)]
+
+
 class ReplayShapeStruct(ctypes.Structure):
     _fields_ = [
         ("num_tokens", c_uint32),
@@ -158,7 +186,23 @@ PROTOTYPES = {
          c_uint32, c_uint32, c_uint32, c_uint32, c_uint32],
     ),
     "psi_hip_split_kv_single_q_reduce": (
-        c_int, [c_void_p, _CFG, c_void_p, c_uint64, c_void_p, c_void_p, c_uint32, c_uint32, c_uint32, c_void_p]),
+        c_int, [c_void_p, _CFG, c_void_p, c_uint64, c_void_p, c_void_p, c_uint32, c_uint32, c_uint32, c_void_p,
+                POINTER(OutputGateStruct)]),
+    "psi_hip_rope_parameters": (c_int, [POINTER(RMSNormRopeConfigStruct), POINTER(c_float), POINTER(c_float),
+                                        POINTER(c_float)]),
+    "psi_hip_rms_norm_rope": (
+        c_int, [c_void_p, POINTER(RMSNormRopeConfigStruct), c_void_p, c_uint64, c_uint64, c_void_p, c_void_p, c_void_p,
+                c_uint32, c_uint32]),
+    "psi_hip_qgkv_split": (
+        c_int, [c_void_p, c_uint32, c_uint32, c_uint32, c_uint32, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p,
+                c_uint32, c_uint32]),
+    "psi_hip_activation_gate": (
+        c_int, [c_void_p, c_uint32, c_uint32, c_uint32, c_void_p, c_void_p, c_void_p, c_uint32, c_uint32]),
+    "psi_hip_kv_page_write_norm_rope": (
+        c_int,
+        [c_void_p, _CFG, _LAYOUT, POINTER(RMSNormRopeConfigStruct), c_void_p, c_uint64, c_void_p, c_uint64, c_void_p,
+         c_uint64, c_void_p, c_void_p, c_void_p, c_void_p, c_uint32, c_uint32, c_uint32],
+    ),
     "psi_hip_split_kv_order_longest_first": (c_int, [_U32P, c_uint32, _U32P]),
     "psi_hip_split_kv_tiled_q_scratch_bytes": (c_int, [_CFG, c_uint32, c_uint32, POINTER(c_uint64)]),
     "psi_hip_split_kv_tiled_q_map": (
@@ -178,7 +222,7 @@ PROTOTYPES = {
     "psi_hip_split_kv_tiled_q_reduce": (
         c_int,
         [c_void_p, _CFG, c_uint32, c_void_p, c_uint64, c_void_p, c_void_p, c_void_p, c_uint32, c_uint32, c_uint32,
-         c_uint32, c_void_p],
+         c_uint32, c_void_p, POINTER(OutputGateStruct)],
     ),
     "psi_hip_page_table_write_page_ids": (
         c_int, [c_void_p, _LAYOUT, c_void_p, c_uint32, c_uint32, c_uint32, _U32P, c_uint32, c_uint32]),

@@ -66,6 +66,34 @@ __device__ __forceinline__ void store_from_f32<F16Tag>(void* base, uint64_t inde
     reinterpret_cast<uint16_t*>(base)[index] = f32_to_f16_bits(v);
 }
 
+// T(v): v rounded through the storage type.
+template <typename Tag>
+__device__ __forceinline__ float round_through(float v);
+template <>
+__device__ __forceinline__ float round_through<F32Tag>(float v) { return v; }
+template <>
+__device__ __forceinline__ float round_through<BF16Tag>(float v) { return bf16_bits_to_f32(f32_to_bf16_bits(v)); }
+template <>
+__device__ __forceinline__ float round_through<F16Tag>(float v) { return f16_bits_to_f32(f32_to_f16_bits(v)); }
+
+// Element `index` of an array whose element type is only known at run time (0 f32, 1 bf16, 2 f16).
+__device__ __forceinline__ float load_any_as_f32(const void* base, uint64_t index, uint32_t dtype) {
+    if (dtype == F32Tag::id) return load_as_f32<F32Tag>(base, index);
+    if (dtype == BF16Tag::id) return load_as_f32<BF16Tag>(base, index);
+    return load_as_f32<F16Tag>(base, index);
+}
+
+// Gate of a gated GQA layer, crates/inference-backend-metal/src/components/metal/gqa_activation_gate.metal:13-27:
+// sigmoid(x) = y or 1 - y with y = 1 / (1 + exp(-|x|)); in a 2-byte type every step is rounded to that type.
+template <typename Tag>
+__device__ __forceinline__ float gate_sigmoid(float x) {
+    const float abs_x = round_through<Tag>(fabsf(x));
+    const float exp_x = round_through<Tag>(expf(-abs_x));
+    const float denom = round_through<Tag>(1.0f + exp_x);
+    const float y = round_through<Tag>(1.0f / denom);
+    return x < 0.0f ? round_through<Tag>(1.0f - y) : y;
+}
+
 // Page-table walk shared by every attention kernel; the expressions of
 // crates/inference-backend-metal/src/components/metal/gqa_split_kv_single_q_map.metal:96-111.
 struct PageWalk {

@@ -70,7 +70,36 @@ struct ReduceArgs {
     const uint32_t* q_token_tiles = nullptr;
     uint32_t rows_per_split_head = 1;
     uint32_t num_active_q_token_tiles = 0;
+    // Optional attention-output gate: element (token, q_head, d) at gates[token * gate_token_stride +
+    // q_head * gate_head_stride + d], in gate_dtype (the IO dtype of the layer).
+    const void* gates = nullptr;
+    uint64_t gate_token_stride = 0, gate_head_stride = 0;
+    uint32_t gate_dtype = PSI_HIP_F32;
 };
+
+// The combine's last step: the output element in f32 -> what is stored.  With a gate the element is
+// first rounded to the output type, as the separate attention output would have been, then
+// multiplied by sigmoid(gate) in that type (gqa_activation_gate.metal:29-38).
+template <typename Tag>
+__device__ __forceinline__ float finish_output(const ReduceArgs& a, float value, uint32_t token, uint32_t q_head,
+                                               uint32_t d) {
+    if (a.gates == nullptr) return value;
+    const float gate = load_any_as_f32(a.gates, token * a.gate_token_stride + q_head * a.gate_head_stride + d, a.gate_dtype);
+    return round_through<Tag>(value) * gate_sigmoid<Tag>(gate);
+}
+
+// Copies an optional psi_hip_output_gate into the kernel arguments; PSI_HIP_OK or an argument error.
+inline int set_output_gate(ReduceArgs* a, const psi_hip_output_gate* gate, const Geometry& g) {
+    if (gate == nullptr) return PSI_HIP_OK;
+    PSI_REQUIRE(gate->gates != nullptr, "GQA output gate pointer must not be null");
+    PSI_REQUIRE(gate->head_stride >= g.d && gate->token_stride >= (uint64_t)(g.hq - 1) * gate->head_stride + g.d,
+                "GQA output gate strides overlap rows");
+    a->gates = gate->gates;
+    a->gate_token_stride = gate->token_stride;
+    a->gate_head_stride = gate->head_stride;
+    a->gate_dtype = g.dtype;
+    return PSI_HIP_OK;
+}
 
 // Prefill-chunk map: a workgroup serves up to kChunkCols query columns (tokens of a row group x
 // heads).  The heads of one KV head are dealt to chunk_head_subsets() workgroups, and a row group

@@ -54,7 +54,8 @@ __global__ __launch_bounds__(256) void split_kv_reduce_fast(ReduceArgs a) {
     const float inv = weight_sum > 0.0f ? 1.0f / weight_sum : 0.0f;
     const uint64_t out_index = row_out * D + lane * kPerLane;
 #pragma unroll
-    for (int e = 0; e < kPerLane; ++e) store_from_f32<Tag>(a.output, out_index + e, value[e] * inv);
+    for (int e = 0; e < kPerLane; ++e)
+        store_from_f32<Tag>(a.output, out_index + e, finish_output<Tag>(a, value[e] * inv, token, q_head, lane * kPerLane + e));
 }
 
 // The combine for long split lists (long contexts, few tokens): one workgroup of eight waves per
@@ -123,7 +124,8 @@ __global__ __launch_bounds__(64 * kWideWaves) void split_kv_reduce_wide(ReduceAr
     const float inv = weight_sum > 0.0f ? 1.0f / weight_sum : 0.0f;
     const uint64_t out_index = row_out * D + lane * kPerLane;
 #pragma unroll
-    for (int e = 0; e < kPerLane; ++e) store_from_f32<Tag>(a.output, out_index + e, value[e] * inv);
+    for (int e = 0; e < kPerLane; ++e)
+        store_from_f32<Tag>(a.output, out_index + e, finish_output<Tag>(a, value[e] * inv, token, q_head, lane * kPerLane + e));
 }
 
 // The same combine for Q-token tiles: one wave per (tile, token in tile, q_head); the tile's partial
@@ -177,7 +179,8 @@ __global__ __launch_bounds__(256) void split_kv_reduce_tiled_fast(ReduceArgs a) 
     const float inv = weight_sum > 0.0f ? 1.0f / weight_sum : 0.0f;
     const uint64_t out_index = ((uint64_t)token * a.hq + q_head) * D + lane * kPerLane;
 #pragma unroll
-    for (int e = 0; e < kPerLane; ++e) store_from_f32<Tag>(a.output, out_index + e, value[e] * inv);
+    for (int e = 0; e < kPerLane; ++e)
+        store_from_f32<Tag>(a.output, out_index + e, finish_output<Tag>(a, value[e] * inv, token, q_head, lane * kPerLane + e));
 }
 
 int launch_decode_map_fast(psi_hip_ctx* ctx, const Geometry& g, const MapArgs& a) {

@@ -142,7 +142,7 @@ __global__ __launch_bounds__(256) void split_kv_reduce_generic(ReduceArgs a, uin
         value += w * a.part_acc[row * a.d + dim];
     }
     store_from_f32<Tag>(a.output, ((uint64_t)token * a.hq + q_head) * a.d + dim,
-                        weight_sum > 0.0f ? value / weight_sum : 0.0f);
+                        finish_output<Tag>(a, weight_sum > 0.0f ? value / weight_sum : 0.0f, token, q_head, dim));
 }
 
 void launch_map_generic(psi_hip_ctx* ctx, const Geometry& g, const MapArgs& a) {

@@ -133,7 +133,8 @@ extern "C" int psi_hip_split_kv_single_q_map_balanced(psi_hip_ctx* ctx, const ps
 extern "C" int psi_hip_split_kv_single_q_reduce(psi_hip_ctx* ctx, const psi_hip_gqa_config* cfg, const void* scratch,
                                                 uint64_t scratch_bytes, const uint32_t* cu_kv_splits, void* output,
                                                 uint32_t num_total_tokens, uint32_t num_total_kv_splits,
-                                                uint32_t num_active_tokens, const uint32_t* partial_row_index) {
+                                                uint32_t num_active_tokens, const uint32_t* partial_row_index,
+                                                const psi_hip_output_gate* gate) {
     PSI_REQUIRE(ctx != nullptr, "ctx must not be null");
     Geometry g;
     int rc = make_geometry(cfg, &g);
@@ -159,6 +160,8 @@ extern "C" int psi_hip_split_kv_single_q_reduce(psi_hip_ctx* ctx, const psi_hip_
     a.out_dtype = ctx->f32_output ? PSI_HIP_F32 : g.dtype;
     a.num_active_tokens = num_active_tokens;
     a.num_total_kv_splits = num_total_kv_splits;
+    rc = set_output_gate(&a, gate, g);
+    if (rc != PSI_HIP_OK) return rc;
 
     LaunchScope scope(ctx, "split_kv_reduce");
     rc = launch_reduce_fast(ctx, g, a);

@@ -152,7 +152,7 @@ extern "C" int psi_hip_split_kv_tiled_q_reduce(psi_hip_ctx* ctx, const psi_hip_g
                                                const uint32_t* cu_kv_splits, void* output, uint32_t num_total_tokens,
                                                uint32_t num_total_q_token_tiles, uint32_t num_total_kv_splits,
                                                uint32_t num_active_q_token_tiles,
-                                               const uint32_t* partial_row_index) {
+                                               const uint32_t* partial_row_index, const psi_hip_output_gate* gate) {
     PSI_REQUIRE(ctx != nullptr, "ctx must not be null");
     Geometry g;
     int rc = make_geometry(cfg, &g);
@@ -180,6 +180,8 @@ extern "C" int psi_hip_split_kv_tiled_q_reduce(psi_hip_ctx* ctx, const psi_hip_g
     a.q_token_tiles = q_token_tiles;
     a.rows_per_split_head = q_token_tile_size;
     a.num_active_q_token_tiles = num_active_q_token_tiles;
+    rc = set_output_gate(&a, gate, g);
+    if (rc != PSI_HIP_OK) return rc;
 
     LaunchScope scope(ctx, "tiled_q_reduce");
     if (launch_reduce_fast(ctx, g, a) == PSI_HIP_ERR_UNSUPPORTED) launch_reduce_generic(ctx, g, a, num_active_q_token_tiles);

@@ -222,6 +222,128 @@ class GQAKVPageWrite:
             _ptr(buffers.flat_k), _ptr(buffers.flat_v), _ptr(buffers.req_slots), _ptr(buffers.flat_token_indices),
             _ptr(buffers.page_ids), shape.num_total_token_writes, num_active_token_writes, page_table_index))
 
+    def invoke_norm_rope_bucketed(self, shape, buffers, norm: "RMSNormRopeConfig", norm_weight,
+                                  num_active_token_writes: int, page_table_index: int, k_token_stride: int = 0,
+                                  v_token_stride: int = 0):
+        """The append with the K-side RMSNorm + RoPE fused in: `buffers.flat_k` holds the raw K rows
+        (token strides in elements, 0 = dense), `norm` is the K norm config (num_heads = KV heads)."""
+        cfg, layout, ncfg = self.config.struct(), shape.page_table_layout.struct(), norm.struct()
+        L.check(self.device.lib.psi_hip_kv_page_write_norm_rope(
+            self.device.ctx, ctypes.byref(cfg), ctypes.byref(layout), ctypes.byref(ncfg), _ptr(buffers.pages),
+            _nbytes(buffers.pages), _ptr(buffers.flat_k), k_token_stride, _ptr(buffers.flat_v), v_token_stride,
+            _ptr(norm_weight), _ptr(buffers.req_slots), _ptr(buffers.flat_token_indices), _ptr(buffers.page_ids),
+            shape.num_total_token_writes, num_active_token_writes, page_table_index))
+
+
+# ------------------------------------------------------------------ projections around the attention
+
+
+@dataclass(frozen=True)
+class RopeScaling:
+    """`RopeScaling::{Default, Yarn}` (components/rms_norm_rope.rs:16-27)."""
+    kind: str = "Default"
+    factor: float = 1.0
+    attention_factor: float = 1.0
+    beta_fast: float = 1.0
+    beta_slow: float = 1.0
+    original_max_position_embeddings: int = 1
+    truncate: bool = False
+
+    @staticmethod
+    def Yarn(factor, attention_factor, beta_fast, beta_slow, original_max_position_embeddings, truncate):
+        return RopeScaling("Yarn", factor, attention_factor, beta_fast, beta_slow, original_max_position_embeddings,
+                           truncate)
+
+    def struct(self):
+        return L.RopeScalingStruct(1 if self.kind == "Yarn" else 0, self.factor, self.attention_factor, self.beta_fast,
+                                   self.beta_slow, self.original_max_position_embeddings, 1 if self.truncate else 0)
+
+
+@dataclass(frozen=True)
+class RMSNormRopeConfig:
+    """`RMSNormRopeConfig` (components/rms_norm_rope.rs:40-96)."""
+    num_heads: int
+    head_dim: int
+    rope_dim: int
+    eps: float
+    rope_theta: float
+    dtype: Dtype = Dtype.Bfloat16
+    rope_scaling: RopeScaling = RopeScaling()
+
+    def struct(self):
+        return L.RMSNormRopeConfigStruct(self.num_heads, self.head_dim, self.rope_dim, self.eps, self.rope_theta,
+                                         self.rope_scaling.struct(), int(self.dtype))
+
+    def kernel_parameters(self):
+        """(inverse_frequencies f32[rope_dim / 2], attention_factor, (low, high) or None): the host
+        values the kernels use (`RopeScaling::kernel_parameters`)."""
+        cfg = self.struct()
+        inv = np.zeros(max(self.rope_dim // 2, 1), np.float32)
+        factor, corr = ctypes.c_float(), (ctypes.c_float * 2)()
+        L.check(L.load().psi_hip_rope_parameters(ctypes.byref(cfg), inv.ctypes.data_as(ctypes.POINTER(ctypes.c_float)),
+                                                 ctypes.byref(factor), corr))
+        return inv, factor.value, ((corr[0], corr[1]) if self.rope_scaling.kind == "Yarn" else None)
+
+
+class RMSNormRopeKernel:
+    """`RMSNormRopeKernel::{invoke, invoke_bucketed}` (components/rms_norm_rope.rs:252-296)."""
+
+    def __init__(self, device: Device, config: RMSNormRopeConfig):
+        config.kernel_parameters()  # validates
+        self.device, self.config = device, config
+
+    def invoke(self, num_total_tokens: int, input, norm_weight, flat_token_indices, output):
+        self.invoke_bucketed(num_total_tokens, input, norm_weight, flat_token_indices, output, num_total_tokens)
+
+    def invoke_bucketed(self, num_total_tokens: int, input, norm_weight, flat_token_indices, output,
+                        num_active_tokens: int, input_token_stride: int = 0, input_head_stride: int = 0):
+        cfg = self.config.struct()
+        L.check(self.device.lib.psi_hip_rms_norm_rope(
+            self.device.ctx, ctypes.byref(cfg), _ptr(input), input_token_stride, input_head_stride, _ptr(norm_weight),
+            _ptr(flat_token_indices), _ptr(output), num_total_tokens, num_active_tokens))
+
+
+class GQAQGKVSplitKernel:
+    """`GQAQGKVSplitKernel::invoke_bucketed` (components/gqa_qgkv_split.rs)."""
+
+    def __init__(self, device: Device, num_q_heads: int, num_kv_heads: int, head_dim: int, dtype: Dtype):
+        self.device, self.shape, self.dtype = device, (num_q_heads, num_kv_heads, head_dim), dtype
+
+    def invoke_bucketed(self, num_total_tokens: int, qgkv, q, g, k, v, num_active_tokens: int):
+        hq, hkv, d = self.shape
+        L.check(self.device.lib.psi_hip_qgkv_split(self.device.ctx, hq, hkv, d, int(self.dtype), _ptr(qgkv), _ptr(q),
+                                                   _ptr(g), _ptr(k), _ptr(v), num_total_tokens, num_active_tokens))
+
+
+class GQAActivationGateKernel:
+    """`GQAActivationGateKernel::invoke_bucketed` (components/gqa_split_kv_single_q.rs:453-543)."""
+
+    def __init__(self, device: Device, num_q_heads: int, head_dim: int, dtype: Dtype):
+        self.device, self.shape, self.dtype = device, (num_q_heads, head_dim), dtype
+
+    def invoke_bucketed(self, num_total_tokens: int, attention_output, g, output, num_active_tokens: int):
+        hq, d = self.shape
+        L.check(self.device.lib.psi_hip_activation_gate(self.device.ctx, hq, d, int(self.dtype), _ptr(attention_output),
+                                                        _ptr(g), _ptr(output), num_total_tokens, num_active_tokens))
+
+
+@dataclass
+class OutputGate:
+    """Gate operand of the combine: a tensor (or a view into the projection output: pass `offset`
+    elements) with element strides per token and head."""
+    gates: object
+    token_stride: int
+    head_stride: int
+    offset: int = 0
+
+    def struct(self):
+        base = self.gates.data_ptr() + self.offset * self.gates.element_size()
+        return L.OutputGateStruct(ctypes.c_void_p(base), self.token_stride, self.head_stride)
+
+
+def _gate_ref(gate):
+    return ctypes.byref(gate.struct()) if gate is not None else None
+
 
 # ------------------------------------------------------------------ variant selection
 
@@ -680,12 +802,13 @@ class GQASplitKVSingleQKernels:
         self.invoke_reduce_bucketed(scratch, cu_sdpa_partial_outputs, output, self.shape.num_total_tokens)
 
     def invoke_reduce_bucketed(self, scratch, cu_sdpa_partial_outputs, output, num_active_tokens: int,
-                               partial_row_index=None):
+                               partial_row_index=None, gate: Optional["OutputGate"] = None):
+        """`gate`: fuses the sigmoid gate of a gated GQA layer into the combine."""
         cfg = self.config.struct()
         L.check(self.device.lib.psi_hip_split_kv_single_q_reduce(
             self.device.ctx, ctypes.byref(cfg), _ptr(scratch.buffer), scratch.bytes, _ptr(cu_sdpa_partial_outputs),
             _ptr(output), self.shape.num_total_tokens, self.shape.num_total_sdpa_map_task_templates,
-            num_active_tokens, _ptr(partial_row_index)))
+            num_active_tokens, _ptr(partial_row_index), _gate_ref(gate)))
 
 
 # ------------------------------------------------------------------ TiledQ verify / prefill
@@ -778,10 +901,11 @@ class GQASplitKVTiledQKernels:
                                     self.shape.num_total_q_token_tiles)
 
     def invoke_reduce_bucketed(self, scratch, q_token_tiles, cu_sdpa_partial_outputs, output,
-                               num_active_q_token_tiles: int, partial_row_index=None):
+                               num_active_q_token_tiles: int, partial_row_index=None,
+                               gate: Optional["OutputGate"] = None):
         cfg, s = self.config.struct(), self.shape
         L.check(self.device.lib.psi_hip_split_kv_tiled_q_reduce(
             self.device.ctx, ctypes.byref(cfg), self.config.q_token_tile_size, _ptr(scratch.buffer), scratch.bytes,
             _ptr(q_token_tiles), _ptr(cu_sdpa_partial_outputs), _ptr(output), s.num_total_tokens,
             s.num_total_q_token_tiles, s.num_total_sdpa_map_task_templates, num_active_q_token_tiles,
-            _ptr(partial_row_index)))
+            _ptr(partial_row_index), _gate_ref(gate)))
