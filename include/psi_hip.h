@@ -304,6 +304,19 @@ int psi_hip_kv_page_write_norm_rope(psi_hip_ctx* ctx, const psi_hip_gqa_config* 
                                     uint32_t num_total_token_writes, uint32_t num_active_token_writes,
                                     uint32_t gqa_layer_index);
 
+/* Everything a gated GQA layer does between its projection and the attention, in one launch: the Q-side
+ * RMSNorm + RoPE (psi_hip_rms_norm_rope on raw_q with its strides, into the dense q_output [T][Hq][D]) and the
+ * fused append above.  The two norm configs differ in num_heads (Hq / Hkv), eps and weights at most: rope_dim,
+ * rope_theta and scaling must be equal.  No single-kernel counterpart in the reference (backend.rs:470-560
+ * records four operators). */
+int psi_hip_qk_norm_rope_kv_page_write(
+    psi_hip_ctx* ctx, const psi_hip_gqa_config* cfg, const psi_hip_page_table_layout* layout,
+    const psi_hip_rms_norm_rope_config* q_norm_cfg, const psi_hip_rms_norm_rope_config* k_norm_cfg, const void* raw_q,
+    uint64_t q_token_stride, uint64_t q_head_stride, const void* q_norm_weight, void* q_output, void* pages,
+    uint64_t pages_bytes, const void* raw_k, uint64_t k_token_stride, const void* flat_v, uint64_t v_token_stride,
+    const void* k_norm_weight, const uint32_t* req_slots, const uint32_t* flat_token_indices, const uint32_t* page_ids,
+    uint32_t num_total_tokens, uint32_t num_active_tokens, uint32_t gqa_layer_index);
+
 /* ------------------------------------------------------------------ split-KV decode (SingleQ) */
 
 /* Scratch for the partial states of `num_total_kv_splits` splits: replaces `GQASplitKVSingleQScratch::new`

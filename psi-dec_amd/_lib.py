@@ -198,6 +198,12 @@ PROTOTYPES = {
                 c_uint32, c_uint32]),
     "psi_hip_activation_gate": (
         c_int, [c_void_p, c_uint32, c_uint32, c_uint32, c_void_p, c_void_p, c_void_p, c_uint32, c_uint32]),
+    "psi_hip_qk_norm_rope_kv_page_write": (
+        c_int,
+        [c_void_p, _CFG, _LAYOUT, POINTER(RMSNormRopeConfigStruct), POINTER(RMSNormRopeConfigStruct), c_void_p,
+         c_uint64, c_uint64, c_void_p, c_void_p, c_void_p, c_uint64, c_void_p, c_uint64, c_void_p, c_uint64, c_void_p,
+         c_void_p, c_void_p, c_void_p, c_uint32, c_uint32, c_uint32],
+    ),
     "psi_hip_kv_page_write_norm_rope": (
         c_int,
         [c_void_p, _CFG, _LAYOUT, POINTER(RMSNormRopeConfigStruct), c_void_p, c_uint64, c_void_p, c_uint64, c_void_p,

@@ -7,6 +7,7 @@
 // decode step: they are launch-latency bound, so the design goal is fewer launches and no extra
 // round trip through HBM, not bandwidth.  One wave handles one (token, head) row.
 #include <cmath>
+#include <cstring>
 
 #include "common.h"
 #include "device_types.h"
@@ -99,11 +100,8 @@ struct FusedAppendArgs {
 // One wave per (token write, kv_head): the K row is normalised and rotated on its way into its page
 // line, the V row is copied.  Page index contract of gqa_kv_page_write.metal:29-47.
 template <typename Tag>
-__global__ __launch_bounds__(256) void kv_page_write_norm_rope_kernel(FusedAppendArgs a, RopeTable table) {
+__device__ __forceinline__ void append_row(const FusedAppendArgs& a, const RopeTable& table, uint64_t item, uint32_t lane) {
     using Elem = typename Tag::storage;
-    const uint32_t lane = threadIdx.x & 63;
-    const uint64_t item = (uint64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
-    if (item >= (uint64_t)a.num_active * a.hkv) return;
     const uint32_t write = (uint32_t)(item / a.hkv), head = (uint32_t)(item % a.hkv);
     const uint32_t req_slot = a.req_slots[write];
     const uint32_t token = a.flat_token_indices[write];
@@ -121,6 +119,37 @@ __global__ __launch_bounds__(256) void kv_page_write_norm_rope_kernel(FusedAppen
                        [&](uint32_t d, float v) { store_from_f32<Tag>(a.pages, k_line + d, v); });
     Elem* v_dst = static_cast<Elem*>(a.pages) + v_line;
     for (uint32_t d = lane; d < a.d; d += 64) v_dst[d] = v_row[d];
+}
+
+template <typename Tag>
+__global__ __launch_bounds__(256) void kv_page_write_norm_rope_kernel(FusedAppendArgs a, RopeTable table) {
+    const uint32_t lane = threadIdx.x & 63;
+    const uint64_t item = (uint64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
+    if (item >= (uint64_t)a.num_active * a.hkv) return;
+    append_row<Tag>(a, table, item, lane);
+}
+
+// The whole pre-attention step of a gated GQA layer in one launch: waves [0, T * Hq) normalise and
+// rotate the query rows into the dense Q buffer, waves [T * Hq, T * (Hq + Hkv)) do the fused append.
+template <typename Tag>
+__global__ __launch_bounds__(256) void qk_norm_rope_append_kernel(NormRopeArgs q, FusedAppendArgs kv, RopeTable table) {
+    using Elem = typename Tag::storage;
+    const uint32_t lane = threadIdx.x & 63;
+    const uint64_t wave_id = (uint64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
+    const uint64_t q_rows = (uint64_t)q.num_active_tokens * q.num_heads;
+    if (wave_id < q_rows) {
+        const uint32_t token = (uint32_t)(wave_id / q.num_heads), head = (uint32_t)(wave_id % q.num_heads);
+        const char* in = static_cast<const char*>(q.input) +
+                         (token * q.in_token_stride + head * q.in_head_stride) * sizeof(Elem);
+        const uint64_t out_base = wave_id * q.head_dim;
+        norm_rope_row<Tag>(in, q.norm_weight, (float)q.positions[token], q.head_dim, q.rope_dim, q.eps,
+                           q.attention_factor, table, lane,
+                           [&](uint32_t d, float v) { store_from_f32<Tag>(q.output, out_base + d, v); });
+        return;
+    }
+    const uint64_t item = wave_id - q_rows;
+    if (item >= (uint64_t)kv.num_active * kv.hkv) return;
+    append_row<Tag>(kv, table, item, lane);
 }
 
 template <typename Elem>
@@ -240,13 +269,10 @@ extern "C" int psi_hip_rope_parameters(const psi_hip_rms_norm_rope_config* cfg, 
     return rope_parameters(cfg, out_inverse_frequencies, out_attention_factor, out_correction);
 }
 
-extern "C" int psi_hip_rms_norm_rope(psi_hip_ctx* ctx, const psi_hip_rms_norm_rope_config* cfg, const void* input,
-                                     uint64_t input_token_stride, uint64_t input_head_stride,
-                                     const void* norm_weight, const uint32_t* flat_token_indices, void* output,
-                                     uint32_t num_total_tokens, uint32_t num_active_tokens) {
-    PSI_REQUIRE(ctx != nullptr, "ctx must not be null");
-    int rc = check_norm_config(cfg);
-    if (rc != PSI_HIP_OK) return rc;
+// Validates one RMSNorm + RoPE operand set and fills the kernel arguments (everything but the table).
+static int make_norm_args(const psi_hip_rms_norm_rope_config* cfg, const void* input, uint64_t input_token_stride,
+                          uint64_t input_head_stride, const void* norm_weight, const uint32_t* flat_token_indices,
+                          void* output, uint32_t num_total_tokens, uint32_t num_active_tokens, NormRopeArgs* a) {
     PSI_REQUIRE(input && norm_weight && flat_token_indices && output, "RMSNorm/RoPE buffers must not be null");
     PSI_REQUIRE(num_total_tokens > 0, "RMSNorm/RoPE requires tokens");
     PSI_REQUIRE(num_active_tokens > 0 && num_active_tokens <= num_total_tokens,
@@ -255,20 +281,82 @@ extern "C" int psi_hip_rms_norm_rope(psi_hip_ctx* ctx, const psi_hip_rms_norm_ro
                 "RMSNorm/RoPE elements exceeds the shader u32 element-index domain");
     PSI_REQUIRE((input_token_stride == 0) == (input_head_stride == 0),
                 "RMSNorm/RoPE input strides must both be given or both be 0 (dense)");
-    NormRopeArgs a;
-    a.input = input;
-    a.norm_weight = static_cast<const uint16_t*>(norm_weight);
-    a.positions = flat_token_indices;
-    a.output = output;
-    a.in_head_stride = input_head_stride ? input_head_stride : cfg->head_dim;
-    a.in_token_stride = input_token_stride ? input_token_stride : (uint64_t)cfg->num_heads * cfg->head_dim;
-    PSI_REQUIRE(a.in_head_stride >= cfg->head_dim && a.in_token_stride >= cfg->num_heads * a.in_head_stride - (a.in_head_stride - cfg->head_dim),
+    a->input = input;
+    a->norm_weight = static_cast<const uint16_t*>(norm_weight);
+    a->positions = flat_token_indices;
+    a->output = output;
+    a->in_head_stride = input_head_stride ? input_head_stride : cfg->head_dim;
+    a->in_token_stride = input_token_stride ? input_token_stride : (uint64_t)cfg->num_heads * cfg->head_dim;
+    PSI_REQUIRE(a->in_head_stride >= cfg->head_dim &&
+                    a->in_token_stride >= (uint64_t)(cfg->num_heads - 1) * a->in_head_stride + cfg->head_dim,
                 "RMSNorm/RoPE input strides overlap rows");
-    a.num_active_tokens = num_active_tokens;
-    a.num_heads = cfg->num_heads;
-    a.head_dim = cfg->head_dim;
-    a.rope_dim = cfg->rope_dim;
-    a.eps = cfg->eps;
+    a->num_active_tokens = num_active_tokens;
+    a->num_heads = cfg->num_heads;
+    a->head_dim = cfg->head_dim;
+    a->rope_dim = cfg->rope_dim;
+    a->eps = cfg->eps;
+    return PSI_HIP_OK;
+}
+
+// Validates the operands of the fused append and fills its kernel arguments (everything but the table).
+static int make_append_args(const psi_hip_gqa_config* cfg, const psi_hip_page_table_layout* layout,
+                            const psi_hip_rms_norm_rope_config* norm_cfg, void* pages, uint64_t pages_bytes,
+                            const void* raw_k, uint64_t k_token_stride, const void* flat_v, uint64_t v_token_stride,
+                            const void* norm_weight, const uint32_t* req_slots, const uint32_t* flat_token_indices,
+                            const uint32_t* page_ids, uint32_t num_total_token_writes,
+                            uint32_t num_active_token_writes, uint32_t gqa_layer_index, Geometry* g,
+                            FusedAppendArgs* a) {
+    int rc = make_geometry(cfg, g);
+    if (rc != PSI_HIP_OK) return rc;
+    rc = check_layout(layout);
+    if (rc != PSI_HIP_OK) return rc;
+    PSI_REQUIRE(norm_cfg->num_heads == g->hkv && norm_cfg->head_dim == g->d && norm_cfg->dtype == g->dtype,
+                "fused append: the K norm config must match the page geometry (%u heads of %u, dtype %u)", g->hkv,
+                g->d, g->dtype);
+    PSI_REQUIRE(pages && raw_k && flat_v && norm_weight && req_slots && flat_token_indices && page_ids,
+                "GQA KV page write buffers must not be null");
+    PSI_REQUIRE(gqa_layer_index < layout->num_gqa_layers, "GQA page-table index exceeds layer count");
+    PSI_REQUIRE(num_total_token_writes > 0, "GQA KV page write requires tokens");
+    PSI_REQUIRE(num_active_token_writes > 0 && num_active_token_writes <= num_total_token_writes,
+                "GQA KV page write active token count must be in 1..capacity");
+    PSI_REQUIRE(pages_bytes == 0 || pages_bytes >= cfg->page_bytes, "GQA page arena is smaller than one page");
+    const uint64_t dense = (uint64_t)g->hkv * g->d;
+    PSI_REQUIRE((k_token_stride == 0 || k_token_stride >= dense) && (v_token_stride == 0 || v_token_stride >= dense),
+                "fused append: token strides must cover a token's K / V rows");
+    a->pages = pages;
+    a->raw_k = raw_k;
+    a->flat_v = flat_v;
+    a->norm_weight = static_cast<const uint16_t*>(norm_weight);
+    a->req_slots = req_slots;
+    a->flat_token_indices = flat_token_indices;
+    a->page_ids = page_ids;
+    a->k_token_stride = k_token_stride ? k_token_stride : dense;
+    a->v_token_stride = v_token_stride ? v_token_stride : dense;
+    a->num_active = num_active_token_writes;
+    a->layer = gqa_layer_index;
+    a->num_layers = layout->num_gqa_layers;
+    a->num_blocks = layout->num_blocks;
+    a->ids_per_block = layout->num_page_ids_per_block;
+    a->hkv = g->hkv;
+    a->d = g->d;
+    a->tokens_per_page = g->tokens_per_page;
+    a->rope_dim = norm_cfg->rope_dim;
+    a->page_elems = g->page_elems;
+    a->eps = norm_cfg->eps;
+    return PSI_HIP_OK;
+}
+
+extern "C" int psi_hip_rms_norm_rope(psi_hip_ctx* ctx, const psi_hip_rms_norm_rope_config* cfg, const void* input,
+                                     uint64_t input_token_stride, uint64_t input_head_stride,
+                                     const void* norm_weight, const uint32_t* flat_token_indices, void* output,
+                                     uint32_t num_total_tokens, uint32_t num_active_tokens) {
+    PSI_REQUIRE(ctx != nullptr, "ctx must not be null");
+    int rc = check_norm_config(cfg);
+    if (rc != PSI_HIP_OK) return rc;
+    NormRopeArgs a;
+    rc = make_norm_args(cfg, input, input_token_stride, input_head_stride, norm_weight, flat_token_indices, output,
+                        num_total_tokens, num_active_tokens, &a);
+    if (rc != PSI_HIP_OK) return rc;
     RopeTable table;
     rc = fill_table(cfg, &table, &a.attention_factor);
     if (rc != PSI_HIP_OK) return rc;
@@ -291,47 +379,14 @@ extern "C" int psi_hip_kv_page_write_norm_rope(psi_hip_ctx* ctx, const psi_hip_g
                                                const uint32_t* page_ids, uint32_t num_total_token_writes,
                                                uint32_t num_active_token_writes, uint32_t gqa_layer_index) {
     PSI_REQUIRE(ctx != nullptr, "ctx must not be null");
+    int rc = check_norm_config(norm_cfg);
+    if (rc != PSI_HIP_OK) return rc;
     Geometry g;
-    int rc = make_geometry(cfg, &g);
-    if (rc != PSI_HIP_OK) return rc;
-    rc = check_layout(layout);
-    if (rc != PSI_HIP_OK) return rc;
-    rc = check_norm_config(norm_cfg);
-    if (rc != PSI_HIP_OK) return rc;
-    PSI_REQUIRE(norm_cfg->num_heads == g.hkv && norm_cfg->head_dim == g.d && norm_cfg->dtype == g.dtype,
-                "fused append: the K norm config must match the page geometry (%u heads of %u, dtype %u)", g.hkv, g.d,
-                g.dtype);
-    PSI_REQUIRE(pages && raw_k && flat_v && norm_weight && req_slots && flat_token_indices && page_ids,
-                "GQA KV page write buffers must not be null");
-    PSI_REQUIRE(gqa_layer_index < layout->num_gqa_layers, "GQA page-table index exceeds layer count");
-    PSI_REQUIRE(num_total_token_writes > 0, "GQA KV page write requires tokens");
-    PSI_REQUIRE(num_active_token_writes > 0 && num_active_token_writes <= num_total_token_writes,
-                "GQA KV page write active token count must be in 1..capacity");
-    PSI_REQUIRE(pages_bytes == 0 || pages_bytes >= cfg->page_bytes, "GQA page arena is smaller than one page");
-    const uint64_t dense = (uint64_t)g.hkv * g.d;
-    PSI_REQUIRE((k_token_stride == 0 || k_token_stride >= dense) && (v_token_stride == 0 || v_token_stride >= dense),
-                "fused append: token strides must cover a token's K / V rows");
     FusedAppendArgs a;
-    a.pages = pages;
-    a.raw_k = raw_k;
-    a.flat_v = flat_v;
-    a.norm_weight = static_cast<const uint16_t*>(norm_weight);
-    a.req_slots = req_slots;
-    a.flat_token_indices = flat_token_indices;
-    a.page_ids = page_ids;
-    a.k_token_stride = k_token_stride ? k_token_stride : dense;
-    a.v_token_stride = v_token_stride ? v_token_stride : dense;
-    a.num_active = num_active_token_writes;
-    a.layer = gqa_layer_index;
-    a.num_layers = layout->num_gqa_layers;
-    a.num_blocks = layout->num_blocks;
-    a.ids_per_block = layout->num_page_ids_per_block;
-    a.hkv = g.hkv;
-    a.d = g.d;
-    a.tokens_per_page = g.tokens_per_page;
-    a.rope_dim = norm_cfg->rope_dim;
-    a.page_elems = g.page_elems;
-    a.eps = norm_cfg->eps;
+    rc = make_append_args(cfg, layout, norm_cfg, pages, pages_bytes, raw_k, k_token_stride, flat_v, v_token_stride,
+                          norm_weight, req_slots, flat_token_indices, page_ids, num_total_token_writes,
+                          num_active_token_writes, gqa_layer_index, &g, &a);
+    if (rc != PSI_HIP_OK) return rc;
     RopeTable table;
     rc = fill_table(norm_cfg, &table, &a.attention_factor);
     if (rc != PSI_HIP_OK) return rc;
@@ -342,6 +397,49 @@ extern "C" int psi_hip_kv_page_write_norm_rope(psi_hip_ctx* ctx, const psi_hip_g
     if (g.dtype == PSI_HIP_F32) hipLaunchKernelGGL(kv_page_write_norm_rope_kernel<F32Tag>, grid, block, 0, ctx->stream, a, table);
     else if (g.dtype == PSI_HIP_BF16) hipLaunchKernelGGL(kv_page_write_norm_rope_kernel<BF16Tag>, grid, block, 0, ctx->stream, a, table);
     else hipLaunchKernelGGL(kv_page_write_norm_rope_kernel<F16Tag>, grid, block, 0, ctx->stream, a, table);
+    PSI_HIP_CHECK(hipGetLastError());
+    return PSI_HIP_OK;
+}
+
+extern "C" int psi_hip_qk_norm_rope_kv_page_write(
+    psi_hip_ctx* ctx, const psi_hip_gqa_config* cfg, const psi_hip_page_table_layout* layout,
+    const psi_hip_rms_norm_rope_config* q_norm_cfg, const psi_hip_rms_norm_rope_config* k_norm_cfg, const void* raw_q,
+    uint64_t q_token_stride, uint64_t q_head_stride, const void* q_norm_weight, void* q_output, void* pages,
+    uint64_t pages_bytes, const void* raw_k, uint64_t k_token_stride, const void* flat_v, uint64_t v_token_stride,
+    const void* k_norm_weight, const uint32_t* req_slots, const uint32_t* flat_token_indices, const uint32_t* page_ids,
+    uint32_t num_total_tokens, uint32_t num_active_tokens, uint32_t gqa_layer_index) {
+    PSI_REQUIRE(ctx != nullptr, "ctx must not be null");
+    int rc = check_norm_config(q_norm_cfg);
+    if (rc != PSI_HIP_OK) return rc;
+    rc = check_norm_config(k_norm_cfg);
+    if (rc != PSI_HIP_OK) return rc;
+    Geometry g;
+    FusedAppendArgs kv;
+    rc = make_append_args(cfg, layout, k_norm_cfg, pages, pages_bytes, raw_k, k_token_stride, flat_v, v_token_stride,
+                          k_norm_weight, req_slots, flat_token_indices, page_ids, num_total_tokens, num_active_tokens,
+                          gqa_layer_index, &g, &kv);
+    if (rc != PSI_HIP_OK) return rc;
+    PSI_REQUIRE(q_norm_cfg->num_heads == g.hq && q_norm_cfg->head_dim == g.d && q_norm_cfg->dtype == g.dtype,
+                "the Q norm config must match the attention geometry (%u heads of %u, dtype %u)", g.hq, g.d, g.dtype);
+    // one rotation table serves both operands
+    PSI_REQUIRE(q_norm_cfg->rope_dim == k_norm_cfg->rope_dim && q_norm_cfg->rope_theta == k_norm_cfg->rope_theta &&
+                    std::memcmp(&q_norm_cfg->scaling, &k_norm_cfg->scaling, sizeof(psi_hip_rope_scaling)) == 0,
+                "the Q and K norm configs must share rope_dim, rope_theta and scaling");
+    NormRopeArgs qa;
+    rc = make_norm_args(q_norm_cfg, raw_q, q_token_stride, q_head_stride, q_norm_weight, flat_token_indices, q_output,
+                        num_total_tokens, num_active_tokens, &qa);
+    if (rc != PSI_HIP_OK) return rc;
+    RopeTable table;
+    rc = fill_table(k_norm_cfg, &table, &kv.attention_factor);
+    if (rc != PSI_HIP_OK) return rc;
+    qa.attention_factor = kv.attention_factor;
+    const uint64_t waves = (uint64_t)num_active_tokens * (g.hq + g.hkv);
+    PSI_REQUIRE((waves + 3) / 4 <= 0x7fffffffull, "GQA prepare grid exceeds the launch domain");
+    const dim3 grid((uint32_t)((waves + 3) / 4)), block(256);
+    LaunchScope scope(ctx, "qk_norm_rope_kv_page_write");
+    if (g.dtype == PSI_HIP_F32) hipLaunchKernelGGL(qk_norm_rope_append_kernel<F32Tag>, grid, block, 0, ctx->stream, qa, kv, table);
+    else if (g.dtype == PSI_HIP_BF16) hipLaunchKernelGGL(qk_norm_rope_append_kernel<BF16Tag>, grid, block, 0, ctx->stream, qa, kv, table);
+    else hipLaunchKernelGGL(qk_norm_rope_append_kernel<F16Tag>, grid, block, 0, ctx->stream, qa, kv, table);
     PSI_HIP_CHECK(hipGetLastError());
     return PSI_HIP_OK;
 }

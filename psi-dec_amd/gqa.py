@@ -234,6 +234,21 @@ class GQAKVPageWrite:
             _ptr(norm_weight), _ptr(buffers.req_slots), _ptr(buffers.flat_token_indices), _ptr(buffers.page_ids),
             shape.num_total_token_writes, num_active_token_writes, page_table_index))
 
+    def invoke_prepare_bucketed(self, shape, buffers, attention_config, q_norm: "RMSNormRopeConfig",
+                                k_norm: "RMSNormRopeConfig", raw_q, q_norm_weight, q_output, k_norm_weight,
+                                num_active_tokens: int, page_table_index: int, q_token_stride: int = 0,
+                                q_head_stride: int = 0, k_token_stride: int = 0, v_token_stride: int = 0):
+        """Q norm + rope and the fused append in one launch (psi_hip_qk_norm_rope_kv_page_write);
+        `attention_config` is the attention's config (it carries the Q head count)."""
+        cfg, layout = attention_config.struct(), shape.page_table_layout.struct()
+        qc, kc = q_norm.struct(), k_norm.struct()
+        L.check(self.device.lib.psi_hip_qk_norm_rope_kv_page_write(
+            self.device.ctx, ctypes.byref(cfg), ctypes.byref(layout), ctypes.byref(qc), ctypes.byref(kc), _ptr(raw_q),
+            q_token_stride, q_head_stride, _ptr(q_norm_weight), _ptr(q_output), _ptr(buffers.pages),
+            _nbytes(buffers.pages), _ptr(buffers.flat_k), k_token_stride, _ptr(buffers.flat_v), v_token_stride,
+            _ptr(k_norm_weight), _ptr(buffers.req_slots), _ptr(buffers.flat_token_indices), _ptr(buffers.page_ids),
+            shape.num_total_token_writes, num_active_tokens, page_table_index))
+
 
 # ------------------------------------------------------------------ projections around the attention
 

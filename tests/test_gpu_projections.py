@@ -288,3 +288,47 @@ def test_gate_fused_into_the_combine(psi, oracle, device, q_len, in_place):
     exp = oracle.activation_gate(oracle.from_f32(attn.reshape(-1), oracle.BF16), gates, oracle.BF16)
     got_f, exp_f = oracle.to_f32(fused, oracle.BF16), oracle.to_f32(exp, oracle.BF16)
     assert np.abs(got_f - exp_f).max() <= 2e-3 and np.sqrt(((got_f - exp_f) ** 2).sum() / (exp_f ** 2).sum()) <= 6e-3
+
+
+def test_single_launch_prepare_equals_the_separate_kernels(psi, oracle, device):
+    """Q norm + rope and the fused append as one launch, reading the projection output in place:
+    the Q buffer and the page arena equal, bit for bit, what the two separate entry points write."""
+    import torch
+
+    wl = importlib_workloads(psi)
+    hq, hkv, d = 12, 2, 256
+    w = wl.make_workload(51, [130, 17, 700], hq, hkv, d, psi.Dtype.Bfloat16, 16, q_lens=[2, 1, 4])
+    rng = np.random.default_rng(52)
+    tokens, width = w.num_tokens, 2 * (hq + hkv) * d
+    qgkv = device.from_numpy(oracle.from_f32(rng.normal(0, 1, tokens * width).astype(np.float32), oracle.BF16))
+    wq = device.from_numpy(oracle.from_f32(rng.uniform(0.5, 1.5, d).astype(np.float32), oracle.BF16))
+    wk = device.from_numpy(oracle.from_f32(rng.uniform(0.5, 1.5, d).astype(np.float32), oracle.BF16))
+    q_norm = psi.RMSNormRopeConfig(hq, d, 64, 1e-6, 1e7, psi.Dtype.Bfloat16)
+    k_norm = psi.RMSNormRopeConfig(hkv, d, 64, 2e-6, 1e7, psi.Dtype.Bfloat16)
+    results = []
+    for single_launch in (False, True):
+        dw = wl.DeviceWorkload(device, w)
+        m = dw.meta
+        q_out = torch.zeros(tokens * hq * d, dtype=torch.int16, device=device.torch_device)
+        buffers = psi.GQAKVPageWriteBuffers(dw.pages, qgkv[2 * hq * d:], qgkv[(2 * hq + hkv) * d:], m.d_req_slots,
+                                            m.d_flat_token_indices, dw.page_ids)
+        if single_launch:
+            dw.write.invoke_prepare_bucketed(dw.write_shape, buffers, dw.cfg, q_norm, k_norm, qgkv, wq, q_out, wk,
+                                             tokens, w.layer, q_token_stride=width, q_head_stride=2 * d,
+                                             k_token_stride=width, v_token_stride=width)
+        else:
+            psi.RMSNormRopeKernel(device, q_norm).invoke_bucketed(tokens, qgkv, wq, m.d_flat_token_indices, q_out,
+                                                                  tokens, input_token_stride=width,
+                                                                  input_head_stride=2 * d)
+            dw.write.invoke_norm_rope_bucketed(dw.write_shape, buffers, k_norm, wk, tokens, w.layer,
+                                               k_token_stride=width, v_token_stride=width)
+        device.sync()
+        results.append((q_out.cpu().numpy().copy(), dw.pages_host().copy()))
+    assert np.array_equal(results[0][0], results[1][0]) and results[0][0].any()
+    assert np.array_equal(results[0][1].view(np.uint8), results[1][1].view(np.uint8))
+    mismatch = psi.RMSNormRopeConfig(hkv, d, 128, 2e-6, 1e7, psi.Dtype.Bfloat16)
+    with pytest.raises(psi.PsiHipError) as err:
+        dw.write.invoke_prepare_bucketed(dw.write_shape, buffers, dw.cfg, q_norm, mismatch, qgkv, wq, q_out, wk, tokens,
+                                         w.layer, q_token_stride=width, q_head_stride=2 * d, k_token_stride=width,
+                                         v_token_stride=width)
+    assert "must share rope_dim" in str(err.value)
