@@ -122,6 +122,17 @@ int psi_hip_ctx_reset_timing(psi_hip_ctx* ctx);
 #define PSI_HIP_FLAG_DECODE_WAVES 4u
 int psi_hip_ctx_set_flag(psi_hip_ctx* ctx, uint32_t flag, uint32_t value);
 
+/* Device-side active counts for captured launches: the counterpart of `ReplayU32::Parameter`
+ * (crates/inference-backend-metal/src/metal/replay.rs; bound at submit by `ReplayArguments::with_u32`).
+ * device_counts: device u32[4] = {num_active_tokens (= token writes), num_active_q_token_tiles,
+ * num_active_kv_splits, reserved}, or null to unbind.  While bound, every kernel launched through this
+ * context reads its active counts from the block when it RUNS; the num_active_* arguments of the entry
+ * points then are upper bounds (pass the capacities): grids are cut for them and the device values are
+ * clamped to them.  A HIP graph captured with the block bound therefore serves every batch of its
+ * capacity bucket: refresh the metadata arrays and the block, replay.  Lanes beyond the device counts
+ * touch nothing, as with the by-value counts. */
+int psi_hip_ctx_bind_replay_counts(psi_hip_ctx* ctx, const uint32_t* device_counts);
+
 /* ------------------------------------------------------------------ geometry (host only) */
 
 /* `GQAKVPageWriteConfig::num_tokens_per_page` (gqa_kv_page_write.rs:57-70). */

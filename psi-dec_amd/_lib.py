@@ -154,6 +154,7 @@ PROTOTYPES = {
     "psi_hip_ctx_set_timing": (c_int, [c_void_p, c_int]),
     "psi_hip_ctx_kernel_time_ms": (c_int, [c_void_p, c_char_p, POINTER(c_double), POINTER(c_uint64)]),
     "psi_hip_ctx_reset_timing": (c_int, [c_void_p]),
+    "psi_hip_ctx_bind_replay_counts": (c_int, [c_void_p, c_void_p]),
     "psi_hip_ctx_set_flag": (c_int, [c_void_p, c_uint32, c_uint32]),
     "psi_hip_gqa_tokens_per_page": (c_int, [_CFG, _U32P]),
     "psi_hip_split_kv_select": (c_int, [_CFG, c_int, c_uint32, c_uint32, _VARIANT]),

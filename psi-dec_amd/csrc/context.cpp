@@ -129,6 +129,12 @@ int psi_hip_sync(psi_hip_ctx* ctx) {
     return PSI_HIP_OK;
 }
 
+int psi_hip_ctx_bind_replay_counts(psi_hip_ctx* ctx, const uint32_t* device_counts) {
+    PSI_REQUIRE(ctx != nullptr, "ctx must not be null");
+    ctx->replay_counts = device_counts;
+    return PSI_HIP_OK;
+}
+
 int psi_hip_ctx_set_flag(psi_hip_ctx* ctx, uint32_t flag, uint32_t value) {
     PSI_REQUIRE(ctx != nullptr, "ctx must not be null");
     switch (flag) {

@@ -94,6 +94,14 @@ __device__ __forceinline__ float gate_sigmoid(float x) {
     return x < 0.0f ? round_through<Tag>(1.0f - y) : y;
 }
 
+// Active counts at kernel run time.  `replay_counts` (null or device u32[4] = {tokens, Q-token tiles, KV
+// splits, reserved}) lets a captured launch serve any batch of its capacity bucket: the value passed
+// with the launch is then only an upper bound.  Index constants below.
+constexpr int kReplayTokens = 0, kReplayTiles = 1, kReplaySplits = 2;
+__device__ __forceinline__ uint32_t active_count(const uint32_t* replay_counts, int which, uint32_t by_value) {
+    return replay_counts != nullptr ? min(replay_counts[which], by_value) : by_value;
+}
+
 // Page-table walk shared by every attention kernel; the expressions of
 // crates/inference-backend-metal/src/components/metal/gqa_split_kv_single_q_map.metal:96-111.
 struct PageWalk {

@@ -4,6 +4,7 @@
 // (token, K|V, kv_head) line, so a 512-byte line is written by 32 adjacent lanes with 128-bit
 // stores.  Pure bit copy: the destination bytes equal the source bytes.
 #include "common.h"
+#include "device_types.h"
 
 namespace psi {
 
@@ -20,6 +21,7 @@ struct PageWriteArgs {
     uint32_t hkv, d, tokens_per_page;
     uint64_t page_elems;
     uint32_t units_per_line;  // chunks (vector path) or elements (scalar path) per (token, head) line
+    const uint32_t* replay_counts;  // see active_count()
 };
 
 // Element offset of (kind, head, token, 0) -- the index contract shared with the attention
@@ -40,7 +42,7 @@ template <typename Unit, int kUnitsAreChunks>
 __global__ __launch_bounds__(256) void kv_page_write_kernel(PageWriteArgs a, uint32_t elems_per_unit) {
     const uint32_t per_write = 2u * a.hkv * a.units_per_line;
     const uint64_t gid = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x;
-    if (gid >= (uint64_t)a.num_active * per_write) return;
+    if (gid >= (uint64_t)active_count(a.replay_counts, kReplayTokens, a.num_active) * per_write) return;
     const uint32_t write = (uint32_t)(gid / per_write);
     uint32_t rest = (uint32_t)(gid - (uint64_t)write * per_write);
     const uint32_t kind = rest / (a.hkv * a.units_per_line);
@@ -90,6 +92,7 @@ extern "C" int psi_hip_kv_page_write(psi_hip_ctx* ctx, const psi_hip_gqa_config*
     a.flat_token_indices = flat_token_indices;
     a.page_ids = page_ids;
     a.num_active = num_active_token_writes;
+    a.replay_counts = ctx->replay_counts;
     a.layer = gqa_layer_index;
     a.num_layers = layout->num_gqa_layers;
     a.num_blocks = layout->num_blocks;

@@ -28,6 +28,7 @@ struct NormRopeArgs {
     uint64_t in_token_stride, in_head_stride;
     uint32_t num_active_tokens, num_heads, head_dim, rope_dim;
     float eps, attention_factor;
+    const uint32_t* replay_counts = nullptr;  // see active_count()
 };
 
 __device__ __forceinline__ float wave_sum(float v) {
@@ -71,7 +72,7 @@ template <typename Tag>
 __global__ __launch_bounds__(256) void rms_norm_rope_kernel(NormRopeArgs a, RopeTable table) {
     const uint32_t lane = threadIdx.x & 63;
     const uint64_t row = (uint64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
-    if (row >= (uint64_t)a.num_active_tokens * a.num_heads) return;
+    if (row >= (uint64_t)active_count(a.replay_counts, kReplayTokens, a.num_active_tokens) * a.num_heads) return;
     const uint32_t token = (uint32_t)(row / a.num_heads), head = (uint32_t)(row % a.num_heads);
     const char* in = static_cast<const char*>(a.input) +
                      (token * a.in_token_stride + head * a.in_head_stride) * sizeof(typename Tag::storage);
@@ -95,6 +96,7 @@ struct FusedAppendArgs {
     uint32_t hkv, d, tokens_per_page, rope_dim;
     uint64_t page_elems;
     float eps, attention_factor;
+    const uint32_t* replay_counts = nullptr;  // see active_count()
 };
 
 // One wave per (token write, kv_head): the K row is normalised and rotated on its way into its page
@@ -125,7 +127,7 @@ template <typename Tag>
 __global__ __launch_bounds__(256) void kv_page_write_norm_rope_kernel(FusedAppendArgs a, RopeTable table) {
     const uint32_t lane = threadIdx.x & 63;
     const uint64_t item = (uint64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
-    if (item >= (uint64_t)a.num_active * a.hkv) return;
+    if (item >= (uint64_t)active_count(a.replay_counts, kReplayTokens, a.num_active) * a.hkv) return;
     append_row<Tag>(a, table, item, lane);
 }
 
@@ -136,8 +138,11 @@ __global__ __launch_bounds__(256) void qk_norm_rope_append_kernel(NormRopeArgs q
     using Elem = typename Tag::storage;
     const uint32_t lane = threadIdx.x & 63;
     const uint64_t wave_id = (uint64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
+    // the grid is cut for the capacity: Q rows first, then the K / V rows
     const uint64_t q_rows = (uint64_t)q.num_active_tokens * q.num_heads;
+    const uint32_t active = active_count(q.replay_counts, kReplayTokens, q.num_active_tokens);
     if (wave_id < q_rows) {
+        if (wave_id >= (uint64_t)active * q.num_heads) return;
         const uint32_t token = (uint32_t)(wave_id / q.num_heads), head = (uint32_t)(wave_id % q.num_heads);
         const char* in = static_cast<const char*>(q.input) +
                          (token * q.in_token_stride + head * q.in_head_stride) * sizeof(Elem);
@@ -148,18 +153,18 @@ __global__ __launch_bounds__(256) void qk_norm_rope_append_kernel(NormRopeArgs q
         return;
     }
     const uint64_t item = wave_id - q_rows;
-    if (item >= (uint64_t)kv.num_active * kv.hkv) return;
+    if (item >= (uint64_t)active * kv.hkv) return;
     append_row<Tag>(kv, table, item, lane);
 }
 
 template <typename Elem>
 __global__ __launch_bounds__(256) void qgkv_split_kernel(const Elem* qgkv, Elem* q, Elem* g, Elem* k, Elem* v,
                                                          uint32_t num_active_tokens, uint32_t hq, uint32_t hkv,
-                                                         uint32_t d) {
+                                                         uint32_t d, const uint32_t* replay_counts) {
     const uint64_t q_slots = (uint64_t)hq * d, kv_slots = (uint64_t)hkv * d;
     const uint64_t width = 2 * q_slots + 2 * kv_slots;
     const uint64_t gid = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x;
-    if (gid >= (uint64_t)num_active_tokens * width) return;
+    if (gid >= (uint64_t)active_count(replay_counts, kReplayTokens, num_active_tokens) * width) return;
     const uint64_t token = gid / width;
     uint64_t slot = gid - token * width;
     const Elem value = qgkv[gid];
@@ -179,9 +184,10 @@ __global__ __launch_bounds__(256) void qgkv_split_kernel(const Elem* qgkv, Elem*
 
 template <typename Tag>
 __global__ __launch_bounds__(256) void activation_gate_kernel(const void* attention_output, const void* gates,
-                                                              void* output, uint64_t count) {
+                                                              void* output, uint32_t num_active_tokens,
+                                                              uint64_t per_token, const uint32_t* replay_counts) {
     const uint64_t gid = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x;
-    if (gid >= count) return;
+    if (gid >= active_count(replay_counts, kReplayTokens, num_active_tokens) * per_token) return;
     store_from_f32<Tag>(output, gid,
                         load_as_f32<Tag>(attention_output, gid) * gate_sigmoid<Tag>(load_as_f32<Tag>(gates, gid)));
 }
@@ -357,6 +363,7 @@ extern "C" int psi_hip_rms_norm_rope(psi_hip_ctx* ctx, const psi_hip_rms_norm_ro
     rc = make_norm_args(cfg, input, input_token_stride, input_head_stride, norm_weight, flat_token_indices, output,
                         num_total_tokens, num_active_tokens, &a);
     if (rc != PSI_HIP_OK) return rc;
+    a.replay_counts = ctx->replay_counts;
     RopeTable table;
     rc = fill_table(cfg, &table, &a.attention_factor);
     if (rc != PSI_HIP_OK) return rc;
@@ -387,6 +394,7 @@ extern "C" int psi_hip_kv_page_write_norm_rope(psi_hip_ctx* ctx, const psi_hip_g
                           norm_weight, req_slots, flat_token_indices, page_ids, num_total_token_writes,
                           num_active_token_writes, gqa_layer_index, &g, &a);
     if (rc != PSI_HIP_OK) return rc;
+    a.replay_counts = ctx->replay_counts;
     RopeTable table;
     rc = fill_table(norm_cfg, &table, &a.attention_factor);
     if (rc != PSI_HIP_OK) return rc;
@@ -429,6 +437,7 @@ extern "C" int psi_hip_qk_norm_rope_kv_page_write(
     rc = make_norm_args(q_norm_cfg, raw_q, q_token_stride, q_head_stride, q_norm_weight, flat_token_indices, q_output,
                         num_total_tokens, num_active_tokens, &qa);
     if (rc != PSI_HIP_OK) return rc;
+    qa.replay_counts = ctx->replay_counts;
     RopeTable table;
     rc = fill_table(k_norm_cfg, &table, &kv.attention_factor);
     if (rc != PSI_HIP_OK) return rc;
@@ -463,11 +472,12 @@ extern "C" int psi_hip_qgkv_split(psi_hip_ctx* ctx, uint32_t num_q_heads, uint32
     if (dtype == PSI_HIP_F32)
         hipLaunchKernelGGL(qgkv_split_kernel<float>, grid, block, 0, ctx->stream, static_cast<const float*>(qgkv),
                            static_cast<float*>(q), static_cast<float*>(g), static_cast<float*>(k), static_cast<float*>(v),
-                           num_active_tokens, num_q_heads, num_kv_heads, head_dim);
+                           num_active_tokens, num_q_heads, num_kv_heads, head_dim, ctx->replay_counts);
     else
         hipLaunchKernelGGL(qgkv_split_kernel<uint16_t>, grid, block, 0, ctx->stream, static_cast<const uint16_t*>(qgkv),
                            static_cast<uint16_t*>(q), static_cast<uint16_t*>(g), static_cast<uint16_t*>(k),
-                           static_cast<uint16_t*>(v), num_active_tokens, num_q_heads, num_kv_heads, head_dim);
+                           static_cast<uint16_t*>(v), num_active_tokens, num_q_heads, num_kv_heads, head_dim,
+                           ctx->replay_counts);
     PSI_HIP_CHECK(hipGetLastError());
     return PSI_HIP_OK;
 }
@@ -488,9 +498,10 @@ extern "C" int psi_hip_activation_gate(psi_hip_ctx* ctx, uint32_t num_q_heads, u
     const uint64_t count = (uint64_t)num_active_tokens * num_q_heads * head_dim;
     const dim3 grid((uint32_t)((count + 255) / 256)), block(256);
     LaunchScope scope(ctx, "activation_gate");
-    if (dtype == PSI_HIP_F32) hipLaunchKernelGGL(activation_gate_kernel<F32Tag>, grid, block, 0, ctx->stream, attention_output, gates, output, count);
-    else if (dtype == PSI_HIP_BF16) hipLaunchKernelGGL(activation_gate_kernel<BF16Tag>, grid, block, 0, ctx->stream, attention_output, gates, output, count);
-    else hipLaunchKernelGGL(activation_gate_kernel<F16Tag>, grid, block, 0, ctx->stream, attention_output, gates, output, count);
+    const uint64_t per_token = (uint64_t)num_q_heads * head_dim;
+    if (dtype == PSI_HIP_F32) hipLaunchKernelGGL(activation_gate_kernel<F32Tag>, grid, block, 0, ctx->stream, attention_output, gates, output, num_active_tokens, per_token, ctx->replay_counts);
+    else if (dtype == PSI_HIP_BF16) hipLaunchKernelGGL(activation_gate_kernel<BF16Tag>, grid, block, 0, ctx->stream, attention_output, gates, output, num_active_tokens, per_token, ctx->replay_counts);
+    else hipLaunchKernelGGL(activation_gate_kernel<F16Tag>, grid, block, 0, ctx->stream, attention_output, gates, output, num_active_tokens, per_token, ctx->replay_counts);
     PSI_HIP_CHECK(hipGetLastError());
     return PSI_HIP_OK;
 }

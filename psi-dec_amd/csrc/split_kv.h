@@ -51,7 +51,15 @@ struct MapArgs {
     // [worker_cu[w], worker_cu[w + 1]).
     const uint32_t* worker_cu = nullptr;
     uint32_t num_workers = 0;
+    const uint32_t* replay_counts = nullptr;  // see active_count()
 };
+
+// First statement of every map kernel.
+__device__ __forceinline__ void resolve_active(MapArgs& a) {
+    a.num_active_tokens = active_count(a.replay_counts, kReplayTokens, a.num_active_tokens);
+    a.num_active_q_token_tiles = active_count(a.replay_counts, kReplayTiles, a.num_active_q_token_tiles);
+    a.num_active_kv_splits = active_count(a.replay_counts, kReplaySplits, a.num_active_kv_splits);
+}
 
 struct ReduceArgs {
     const float* part_max;
@@ -75,7 +83,14 @@ struct ReduceArgs {
     const void* gates = nullptr;
     uint64_t gate_token_stride = 0, gate_head_stride = 0;
     uint32_t gate_dtype = PSI_HIP_F32;
+    const uint32_t* replay_counts = nullptr;  // see active_count()
 };
+
+// First statement of every combine kernel.
+__device__ __forceinline__ void resolve_active(ReduceArgs& a) {
+    a.num_active_tokens = active_count(a.replay_counts, kReplayTokens, a.num_active_tokens);
+    a.num_active_q_token_tiles = active_count(a.replay_counts, kReplayTiles, a.num_active_q_token_tiles);
+}
 
 // The combine's last step: the output element in f32 -> what is stored.  With a gate the element is
 // first rounded to the output type, as the separate attention output would have been, then

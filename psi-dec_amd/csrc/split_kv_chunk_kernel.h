@@ -111,6 +111,7 @@ __global__ __launch_bounds__(64 * kChunkWaves, 2) void split_kv_chunk_map(
     const uint32_t* __restrict__ req_slots, const uint16_t* __restrict__ q, const uint16_t* __restrict__ pages,
     const uint32_t* __restrict__ q_token_tiles, const uint32_t* __restrict__ flat_token_indices,
     const uint32_t* __restrict__ row_groups, uint32_t group_tiles, uint32_t num_groups, uint32_t head_subsets) {
+    resolve_active(a);
     static_assert(D == 256, "the tile loaders are laid out for head_dim 256");
     constexpr int kKSteps = D / 32;              // MFMA k-steps of QK^T
     constexpr int kDimBlocks = D / 16;           // 16-dim output blocks of PV

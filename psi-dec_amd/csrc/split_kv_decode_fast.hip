@@ -14,6 +14,7 @@ int launch_decode_map_f16_d128(psi_hip_ctx* ctx, const Geometry& g, const MapArg
 // keeps several 1 KiB reads in flight instead of one.
 template <typename Tag, int D, bool kIndexed>
 __global__ __launch_bounds__(256) void split_kv_reduce_fast(ReduceArgs a) {
+    resolve_active(a);
     constexpr int kPerLane = D / 64;  // 4 or 2
     constexpr int kUnroll = 4;
     const uint32_t lane = threadIdx.x & 63;
@@ -64,6 +65,7 @@ __global__ __launch_bounds__(256) void split_kv_reduce_fast(ReduceArgs a) {
 constexpr int kWideWaves = 8;
 template <typename Tag, int D, bool kIndexed>
 __global__ __launch_bounds__(64 * kWideWaves) void split_kv_reduce_wide(ReduceArgs a) {
+    resolve_active(a);
     constexpr int kPerLane = D / 64;
     constexpr int kUnroll = 4;
     __shared__ float wave_max[kWideWaves];
@@ -132,6 +134,7 @@ __global__ __launch_bounds__(64 * kWideWaves) void split_kv_reduce_wide(ReduceAr
 // rows are cu_kv_splits[tile] .. cu_kv_splits[tile + 1].
 template <typename Tag, int D, bool kIndexed>
 __global__ __launch_bounds__(256) void split_kv_reduce_tiled_fast(ReduceArgs a) {
+    resolve_active(a);
     constexpr int kPerLane = D / 64;
     const uint32_t lane = threadIdx.x & 63;
     const uint64_t id = (uint64_t)blockIdx.x * 4 + (threadIdx.x >> 6);

@@ -84,6 +84,7 @@ __global__ __launch_bounds__(64 * kWaves, PSI_DECODE_WAVES_PER_SIMD) void split_
     MapArgs a, const uint32_t* __restrict__ page_ids, const uint32_t* __restrict__ kv_splits,
     const uint32_t* __restrict__ req_slots, const uint16_t* __restrict__ q, const uint16_t* __restrict__ pages,
     const uint32_t* __restrict__ worker_cu) {
+    resolve_active(a);
     constexpr int kVLanesPerToken = D / 8;                  // 32 (D=256) or 16 (D=128)
     constexpr int kVTokensPerLoad = 64 / kVLanesPerToken;   // 2 or 4
     constexpr int kVLoads = kTileTokens / kVTokensPerLoad;  // 8 or 4

@@ -79,6 +79,7 @@ struct TileRegs {
 
 template <typename Tag, int D, int G>
 __global__ __launch_bounds__(256, 2) void split_kv_decode_map_valu(MapArgs a) {
+    resolve_active(a);
     constexpr int kVLanesPerToken = D / 8;                  // 32 (D=256) or 16 (D=128)
     constexpr int kVTokensPerLoad = 64 / kVLanesPerToken;   // 2 or 4
     constexpr int kVLoads = kTileTokens / kVTokensPerLoad;  // 8 or 4

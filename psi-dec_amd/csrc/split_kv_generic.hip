@@ -26,6 +26,7 @@ __device__ __forceinline__ float wave_sum(float v) {
 // tile for QK, lane = dim for PV.
 template <typename Tag>
 __global__ __launch_bounds__(64) void split_kv_map_generic(MapArgs a) {
+    resolve_active(a);
     const uint32_t d = a.walk.d;
     const uint32_t dim_slices = (d + 63) / 64;
     uint32_t b = blockIdx.x;
@@ -104,6 +105,7 @@ __global__ __launch_bounds__(64) void split_kv_map_generic(MapArgs a) {
 // token's offset inside the tile.
 template <typename Tag>
 __global__ __launch_bounds__(256) void split_kv_reduce_generic(ReduceArgs a, uint32_t num_tile_slots) {
+    resolve_active(a);
     const uint64_t gid = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x;
     uint32_t token, q_head, dim, begin, end, tile_row = 0;
     if (a.q_token_tiles == nullptr) {

@@ -84,6 +84,7 @@ static int single_q_map_impl(psi_hip_ctx* ctx, const psi_hip_gqa_config* cfg, co
     a.num_total_kv_splits = num_total_kv_splits;
     a.num_active_tokens = num_active_tokens;
     a.num_active_kv_splits = num_active_kv_splits;
+    a.replay_counts = ctx->replay_counts;
     a.scale_log2 = g.scale * kLog2e;
     a.worker_cu = worker_cu;
     a.num_workers = num_workers;
@@ -154,6 +155,7 @@ extern "C" int psi_hip_split_kv_single_q_reduce(psi_hip_ctx* ctx, const psi_hip_
     a.part_acc = reinterpret_cast<const float*>(static_cast<const char*>(scratch) + pl.acc_offset);
     a.cu_kv_splits = cu_kv_splits;
     a.row_index = partial_row_index;
+    a.replay_counts = ctx->replay_counts;
     a.output = output;
     a.hq = g.hq;
     a.d = g.d;

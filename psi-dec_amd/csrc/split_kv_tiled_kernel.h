@@ -94,6 +94,7 @@ __global__ __launch_bounds__(64 * kTiledTileWaves * CG, (TiledOccupancy<NB, CG>:
     MapArgs a, const uint32_t* __restrict__ page_ids, const uint32_t* __restrict__ kv_splits,
     const uint32_t* __restrict__ req_slots, const uint16_t* __restrict__ q, const uint16_t* __restrict__ pages,
     const uint32_t* __restrict__ q_token_tiles, const uint32_t* __restrict__ flat_token_indices) {
+    resolve_active(a);
     constexpr int kTileWaves = kTiledTileWaves;
     constexpr int kWaves = kTileWaves * CG;
     constexpr int kVLanesPerToken = D / 8;                  // 32 (D=256) or 16 (D=128)

@@ -87,6 +87,7 @@ static int tiled_q_map(psi_hip_ctx* ctx, const psi_hip_gqa_config* cfg, const ps
     a.num_total_kv_splits = num_total_kv_splits;
     a.num_active_tokens = num_active_tokens;
     a.num_active_kv_splits = num_active_kv_splits;
+    a.replay_counts = ctx->replay_counts;
     a.scale_log2 = g.scale * kLog2eTiled;
     a.q_token_tiles = q_token_tiles;
     a.flat_token_indices = flat_token_indices;
@@ -172,6 +173,7 @@ extern "C" int psi_hip_split_kv_tiled_q_reduce(psi_hip_ctx* ctx, const psi_hip_g
     a.part_acc = reinterpret_cast<const float*>(static_cast<const char*>(scratch) + pl.acc_offset);
     a.cu_kv_splits = cu_kv_splits;
     a.row_index = partial_row_index;
+    a.replay_counts = ctx->replay_counts;
     a.output = output;
     a.hq = g.hq;
     a.d = g.d;

@@ -80,6 +80,12 @@ class Device:
         self.stream = stream
         L.check(self.lib.psi_hip_ctx_set_stream(self.ctx, ctypes.c_void_p(stream.cuda_stream)))
 
+    def bind_replay_counts(self, counts=None):
+        """Device int32[4] = {active tokens, active Q-token tiles, active KV splits, 0} that every
+        kernel reads when it runs (graph replay); None restores the by-value counts."""
+        self._replay_counts = counts  # keep the tensor alive while it is bound
+        L.check(self.lib.psi_hip_ctx_bind_replay_counts(self.ctx, _ptr(counts)))
+
     def set_timing(self, enabled: bool):
         L.check(self.lib.psi_hip_ctx_set_timing(self.ctx, int(enabled)))
 

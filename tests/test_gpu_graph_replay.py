@@ -61,3 +61,92 @@ def test_captured_layer_step_replays(psi, device, q_len):
             assert torch.equal(dw.output.view(torch.int16), base.view(torch.int16))
         # eager work of the program between replays
         _ = (dw.output.float() * 2).sum().item()
+
+
+def test_one_captured_step_serves_every_batch_of_its_bucket(psi, device):
+    """Device-side active counts (`ReplayU32::Parameter` of the reference): a decode step captured once at the
+    capacity of its bucket (5 tokens, 16 splits) with the counts bound, then replayed for batches of 5, 3, 1 and
+    4 requests after refreshing only the metadata arrays, the inputs and the 16-byte count block.  Each replay
+    equals the eager step with by-value counts, bit for bit, in the output rows and in the page arena; rows
+    beyond the active count keep a canary."""
+    import torch
+
+    wl = importlib_workloads(psi)
+    ctx_lens = [700, 33, 1500, 512, 64]
+    w = wl.make_workload(111, ctx_lens, 24, 4, 256, psi.Dtype.Bfloat16, 16)
+    cap_tokens, cap_splits = 5, 16
+    dw = wl.DeviceWorkload(device, w, partition_tokens=512)  # owns pages, page table, q, flat_k, flat_v
+    pristine = dw.pages.clone()
+    variant = dw.variant
+    cfg = dw.cfg
+    kernels = psi.GQASplitKVSingleQKernels(device, cfg, psi.GQASplitKVSingleQShape(cap_tokens, cap_splits))
+    scratch = psi.GQASplitKVSingleQScratch(device, cfg, psi.GQASplitKVSingleQShape(cap_tokens, cap_splits))
+    write_shape = psi.GQAKVPageWriteShape(cap_tokens, w.layout)
+    row = w.num_q_heads * w.head_dim
+    kv_row = w.num_kv_heads * w.head_dim
+    i32 = dict(dtype=torch.int32, device=device.torch_device)
+    d_slots, d_pos = torch.zeros(cap_tokens, **i32), torch.zeros(cap_tokens, **i32)
+    d_splits, d_cu = torch.zeros(cap_splits * 3, **i32), torch.zeros(cap_tokens + 1, **i32)
+    d_counts = torch.zeros(4, **i32)
+    q, fk, fv = torch.zeros_like(dw.q), torch.zeros_like(dw.flat_k), torch.zeros_like(dw.flat_v)
+    out = torch.zeros(cap_tokens * row, dtype=torch.bfloat16, device=device.torch_device)
+    host_meta = psi.GQAMetadataBuffers(None, cap_tokens, max_kv_splits=cap_splits)
+
+    def load_batch(picks):
+        n = len(picks)
+        shape = host_meta.update_fixed_partition(w.req_slots[picks], w.token_indices[picks], list(range(n + 1)), variant,
+                                                 512)
+        for dst, src in ((d_slots, host_meta.h_req_slots), (d_pos, host_meta.h_flat_token_indices),
+                         (d_splits, host_meta.h_kv_splits), (d_cu, host_meta.h_cu_kv_splits)):
+            dst.copy_(device.from_numpy(src))
+        for dst, src, width in ((q, dw.q, row), (fk, dw.flat_k, kv_row), (fv, dw.flat_v, kv_row)):
+            dst.zero_()
+            for i, r in enumerate(picks):
+                dst[i * width:(i + 1) * width] = src[r * width:(r + 1) * width]
+        d_counts.copy_(torch.tensor([shape.num_tokens, shape.num_q_token_tiles, shape.num_sdpa_map_task_templates, 0],
+                                    dtype=torch.int32))
+        return shape
+
+    def step(active_tokens, active_splits):
+        bufs = psi.GQAKVPageWriteBuffers(dw.pages, fk, fv, d_slots, d_pos, dw.page_ids)
+        dw.write.invoke_bucketed(write_shape, bufs, active_tokens, w.layer)
+        kernels.invoke_map_bucketed(q, dw.pages, d_slots, dw.page_ids, d_splits, scratch, w.layer, active_tokens,
+                                    active_splits)
+        kernels.invoke_reduce_bucketed(scratch, d_cu, out, active_tokens)
+
+    # capture at capacity with the count block bound
+    load_batch([0, 1, 2, 3, 4])
+    side, main = torch.cuda.Stream(), device.stream
+    graph = torch.cuda.CUDAGraph()
+    try:
+        side.wait_stream(torch.cuda.current_stream())
+        with torch.cuda.stream(side):
+            device.use_stream(side)
+            device.bind_replay_counts(d_counts)
+            step(cap_tokens, cap_splits)  # warm-up on the capture stream
+            side.synchronize()
+            with torch.cuda.graph(graph, stream=side):
+                step(cap_tokens, cap_splits)
+    finally:
+        device.bind_replay_counts(None)
+        device.use_stream(main)
+    torch.cuda.synchronize()
+
+    for picks in ([0, 1, 2, 3, 4], [2, 0, 4], [3], [4, 3, 1, 0]):
+        shape = load_batch(picks)
+        n = shape.num_tokens
+        dw.pages.copy_(pristine)
+        out.fill_(-768.0)
+        step(shape.num_tokens, shape.num_sdpa_map_task_templates)  # eager, counts by value
+        device.sync()
+        eager_out, eager_pages = out.clone(), dw.pages.clone()
+        dw.pages.copy_(pristine)
+        out.fill_(-768.0)
+        scratch.buffer.zero_()
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(out.view(torch.int16), eager_out.view(torch.int16)), picks
+        assert torch.equal(dw.pages.view(torch.int16), eager_pages.view(torch.int16)), picks
+        assert (out[n * row:].float() == -768.0).all() and (out[:n * row].float() != -768.0).any()
+        _ = out.float().sum().item()  # eager work between replays
