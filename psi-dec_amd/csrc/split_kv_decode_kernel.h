@@ -71,6 +71,11 @@ __device__ __forceinline__ void wave_lds_fence() { asm volatile("s_waitcnt lgkmc
 #define PSI_DECODE_WAVES_PER_SIMD 3
 #endif
 
+// Workgroups per SIMD the register allocator is held to.  Three (168 registers) fits up to six query heads per
+// KV head; seven and eight need 181 and 190 registers and would spill, and a kernel with a private segment
+// starts far slower than one resident wave less costs, so those are held to two.
+constexpr int decode_waves_per_simd(int group) { return group > 6 ? 2 : PSI_DECODE_WAVES_PER_SIMD; }
+
 constexpr int kTileTokens = 16;
 
 // Page IDs behind one 16-token tile: one page when a page holds at least 16 tokens, two when it
@@ -80,7 +85,7 @@ struct TilePages {
 };
 
 template <typename Tag, int D, int G, int kWaves, bool kHalfPage>
-__global__ __launch_bounds__(64 * kWaves, PSI_DECODE_WAVES_PER_SIMD) void split_kv_decode_map(
+__global__ __launch_bounds__(64 * kWaves, decode_waves_per_simd(G)) void split_kv_decode_map(
     MapArgs a, const uint32_t* __restrict__ page_ids, const uint32_t* __restrict__ kv_splits,
     const uint32_t* __restrict__ req_slots, const uint16_t* __restrict__ q, const uint16_t* __restrict__ pages,
     const uint32_t* __restrict__ worker_cu) {
