@@ -374,6 +374,25 @@ int psi_hip_split_kv_single_q_reduce(psi_hip_ctx* ctx, const psi_hip_gqa_config*
                                      uint32_t num_active_tokens, const uint32_t* partial_row_index,
                                      const psi_hip_output_gate* gate);
 
+/* A partial result another attention task produced for each token, entered into the split row the map leaves
+ * alone for it.  Replaces the direct writes of a second producer into the SingleQ partial arrays
+ * (metal/gqa_block_sdpa.metal:47-76, the block attention of the second speculator) under the rule of
+ * metal/gqa_split_kv_single_q_map.metal:49-53: a kv_splits row whose first field is >= num_active_tokens is
+ * skipped by the map and may be filled by someone else before the combine, which merges every row of
+ * [cu_kv_splits[t], cu_kv_splits[t + 1]).  Call between the map and the reduce, on the same stream.
+ * slot_rows: device u32[num_total_tokens], the kv_splits row reserved for token t
+ * (`block_sdpa_map_task_template_indices`, crates/inference-executor-metal/src/attn/dspark/metadata.rs:207-212);
+ * a value >= num_total_kv_splits means the token has none.  partial_exp_sums / partial_max_logits: device
+ * f32[num_total_tokens, Hq] in the reference's form (sum of exp(logit - max); max of the scaled natural-log
+ * logits).  partial_output: device [num_total_tokens, Hq, D] in the IO dtype, already divided by the exp sum.
+ * partial_row_index: as for the reduce. */
+int psi_hip_split_kv_single_q_store_partials(psi_hip_ctx* ctx, const psi_hip_gqa_config* cfg, void* scratch,
+                                             uint64_t scratch_bytes, const uint32_t* slot_rows,
+                                             const float* partial_exp_sums, const float* partial_max_logits,
+                                             const void* partial_output, uint32_t num_total_tokens,
+                                             uint32_t num_total_kv_splits, uint32_t num_active_tokens,
+                                             const uint32_t* partial_row_index);
+
 /* ------------------------------------------------------------------ split-KV verify / prefill (TiledQ) */
 
 /* `GQASplitKVTiledQConfig::partial_output_bytes + 2 * partial_output_stats_bytes`
@@ -582,6 +601,35 @@ int psi_hip_decoder_blocks_counts(const psi_hip_decoder_blocks* blocks, size_t* 
  * (blocks/trie/token.rs:10-181); out may be null to count only. */
 int psi_hip_decoder_blocks_tokens(const psi_hip_decoder_blocks* blocks, uint32_t which, uint32_t* out,
                                   size_t capacity, size_t* count);
+
+/* ------------------------------------------------------------------ state snapshot of selected entries
+ * A snapshot of selected state stores, for a buffer of fixed-size entries, the bytes of the selected entry
+ * ranges concatenated in order (`StateSnapshotWriter::write_selected_buffer` /
+ * `StateSnapshotReader::read_selected_buffer`, crates/inference-executor-metal/src/model/state_snapshot.rs:249-304,
+ * :533-591, ranges from :743-772).  The page arena is selected by page-ID ranges with entry_bytes = page_bytes
+ * (model/page_arena/file_io.rs:28-49), the GQA page table by request-slot ranges with entry_bytes =
+ * page IDs per request * 4 (attn/gqa/request_page_table/file_io.rs:28-59).  The reference streams each range
+ * between unified memory and the file; here the ranges are gathered into (scattered from) one payload in device
+ * memory, which then crosses the host link in a single transfer.  File layout, manifest and publishing stay with
+ * the caller.
+ * entry_ranges: host u32[num_ranges][2] = [begin, end) entry indices, in the reference's canonical form (every
+ * range non-empty; sorted, disjoint and not adjacent; state_snapshot.rs:774-776) and inside the buffer, else
+ * PSI_HIP_ERR_INVALID_ARGUMENT with the reference's message. */
+
+/* Bytes of the payload of a selection (also validates it). */
+int psi_hip_selected_ranges_payload_bytes(const uint32_t* entry_ranges, uint32_t num_ranges, uint64_t entry_bytes,
+                                          uint64_t buffer_bytes, uint64_t* out_payload_bytes);
+
+/* buffer (device) -> payload (device, payload_bytes must equal the selection's size), on the context's stream. */
+int psi_hip_buffer_pack_selected(psi_hip_ctx* ctx, const void* buffer, uint64_t buffer_bytes,
+                                 const uint32_t* entry_ranges, uint32_t num_ranges, uint64_t entry_bytes,
+                                 void* payload, uint64_t payload_bytes);
+
+/* payload -> buffer; bytes of the buffer outside the selection are left as they are.  A payload whose size is not
+ * the selection's is the reference's "file length mismatch" (state_snapshot.rs:549-559). */
+int psi_hip_buffer_unpack_selected(psi_hip_ctx* ctx, void* buffer, uint64_t buffer_bytes,
+                                   const uint32_t* entry_ranges, uint32_t num_ranges, uint64_t entry_bytes,
+                                   const void* payload, uint64_t payload_bytes);
 
 #ifdef __cplusplus
 }

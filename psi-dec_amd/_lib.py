@@ -189,6 +189,15 @@ PROTOTYPES = {
     "psi_hip_split_kv_single_q_reduce": (
         c_int, [c_void_p, _CFG, c_void_p, c_uint64, c_void_p, c_void_p, c_uint32, c_uint32, c_uint32, c_void_p,
                 POINTER(OutputGateStruct)]),
+    "psi_hip_split_kv_single_q_store_partials": (
+        c_int, [c_void_p, _CFG, c_void_p, c_uint64, c_void_p, c_void_p, c_void_p, c_void_p, c_uint32, c_uint32,
+                c_uint32, c_void_p]),
+    "psi_hip_selected_ranges_payload_bytes": (c_int, [POINTER(c_uint32), c_uint32, c_uint64, c_uint64,
+                                                      POINTER(c_uint64)]),
+    "psi_hip_buffer_pack_selected": (c_int, [c_void_p, c_void_p, c_uint64, POINTER(c_uint32), c_uint32, c_uint64,
+                                             c_void_p, c_uint64]),
+    "psi_hip_buffer_unpack_selected": (c_int, [c_void_p, c_void_p, c_uint64, POINTER(c_uint32), c_uint32, c_uint64,
+                                               c_void_p, c_uint64]),
     "psi_hip_rope_parameters": (c_int, [POINTER(RMSNormRopeConfigStruct), POINTER(c_float), POINTER(c_float),
                                         POINTER(c_float)]),
     "psi_hip_rms_norm_rope": (

@@ -26,6 +26,42 @@ static int check_single_q_shape(const Geometry& g, uint32_t num_total_tokens, ui
     return PSI_HIP_OK;
 }
 
+struct StorePartialsArgs {
+    const uint32_t* slot_rows;
+    const uint32_t* row_index;
+    const uint32_t* replay_counts;
+    const float* exp_sums;
+    const float* max_logits;
+    const void* partial_output;
+    float* part_max;
+    float* part_sum;
+    float* part_acc;
+    uint32_t hq, d, dtype, num_active_tokens, num_total_kv_splits;
+};
+
+// One wave per (token, query head): the partial result another attention task produced for the token, in the
+// form crates/inference-backend-metal/src/components/metal/gqa_block_sdpa.metal:47-76 writes it (maximum of
+// the scaled natural-log logits, sum of exponentials, output already divided by that sum), entered into the
+// split row reserved for it in the form the combine merges (base-2 maximum, sum, undivided output).
+__global__ __launch_bounds__(256) void store_partials_kernel(StorePartialsArgs a) {
+    const uint32_t active = active_count(a.replay_counts, kReplayTokens, a.num_active_tokens);
+    const uint32_t item = (blockIdx.x * 256 + threadIdx.x) / 64, lane = threadIdx.x % 64;
+    if (item >= active * a.hq) return;
+    const uint32_t token = item / a.hq, head = item % a.hq;
+    uint32_t row = a.slot_rows[token];
+    if (row >= a.num_total_kv_splits) return;  // a token without a reserved row
+    if (a.row_index != nullptr) row = a.row_index[row];
+    const uint64_t src = (uint64_t)token * a.hq + head, dst = (uint64_t)row * a.hq + head;
+    const float max_logit = a.max_logits[src], exp_sum = a.exp_sums[src];
+    const bool live = isfinite(max_logit) && exp_sum > 0.0f;
+    for (uint32_t dim = lane; dim < a.d; dim += 64)
+        a.part_acc[dst * a.d + dim] = live ? load_any_as_f32(a.partial_output, src * a.d + dim, a.dtype) * exp_sum : 0.0f;
+    if (lane == 0) {
+        a.part_max[dst] = live ? max_logit * kLog2e : -INFINITY;
+        a.part_sum[dst] = live ? exp_sum : 0.0f;
+    }
+}
+
 }  // namespace psi
 
 using namespace psi;
@@ -172,6 +208,49 @@ extern "C" int psi_hip_split_kv_single_q_reduce(psi_hip_ctx* ctx, const psi_hip_
         rc = PSI_HIP_OK;
     }
     if (rc != PSI_HIP_OK) return rc;
+    PSI_HIP_CHECK(hipGetLastError());
+    return PSI_HIP_OK;
+}
+
+extern "C" int psi_hip_split_kv_single_q_store_partials(psi_hip_ctx* ctx, const psi_hip_gqa_config* cfg, void* scratch,
+                                                        uint64_t scratch_bytes, const uint32_t* slot_rows,
+                                                        const float* partial_exp_sums, const float* partial_max_logits,
+                                                        const void* partial_output, uint32_t num_total_tokens,
+                                                        uint32_t num_total_kv_splits, uint32_t num_active_tokens,
+                                                        const uint32_t* partial_row_index) {
+    PSI_REQUIRE(ctx != nullptr, "ctx must not be null");
+    Geometry g;
+    int rc = make_geometry(cfg, &g);
+    if (rc != PSI_HIP_OK) return rc;
+    rc = check_single_q_shape(g, num_total_tokens, num_total_kv_splits);
+    if (rc != PSI_HIP_OK) return rc;
+    PSI_REQUIRE(scratch && slot_rows && partial_exp_sums && partial_max_logits && partial_output,
+                "GQA SplitKV SingleQ partial-output buffers must not be null");
+    PSI_REQUIRE(num_active_tokens > 0, "GQA SplitKV SingleQ active token count must be positive");
+    PSI_REQUIRE(num_active_tokens <= num_total_tokens,
+                "GQA SplitKV SingleQ active token count exceeds recorded capacity");
+    const PartialLayout pl = partial_layout(num_total_kv_splits, g.hq, g.d, 1);
+    PSI_REQUIRE(scratch_bytes >= pl.total_bytes, "GQA SplitKV SingleQ scratch too small: %llu < %llu",
+                (unsigned long long)scratch_bytes, (unsigned long long)pl.total_bytes);
+    StorePartialsArgs a;
+    a.slot_rows = slot_rows;
+    a.row_index = partial_row_index;
+    a.replay_counts = ctx->replay_counts;
+    a.exp_sums = partial_exp_sums;
+    a.max_logits = partial_max_logits;
+    a.partial_output = partial_output;
+    a.part_max = reinterpret_cast<float*>(static_cast<char*>(scratch) + pl.max_offset);
+    a.part_sum = reinterpret_cast<float*>(static_cast<char*>(scratch) + pl.sum_offset);
+    a.part_acc = reinterpret_cast<float*>(static_cast<char*>(scratch) + pl.acc_offset);
+    a.hq = g.hq;
+    a.d = g.d;
+    a.dtype = g.dtype;
+    a.num_active_tokens = num_active_tokens;
+    a.num_total_kv_splits = num_total_kv_splits;
+
+    LaunchScope scope(ctx, "split_kv_store_partials");
+    const uint64_t waves = (uint64_t)num_active_tokens * g.hq;
+    hipLaunchKernelGGL(store_partials_kernel, dim3((uint32_t)((waves + 3) / 4)), dim3(256), 0, ctx->stream, a);
     PSI_HIP_CHECK(hipGetLastError());
     return PSI_HIP_OK;
 }

@@ -819,6 +819,17 @@ class GQASplitKVSingleQKernels:
             _ptr(scratch.buffer), scratch.bytes, page_table_index, self.shape.num_total_tokens,
             self.shape.num_total_sdpa_map_task_templates, num_active_tokens, num_active_kv_splits))
 
+    def invoke_store_partials(self, scratch, slot_rows, partial_exp_sums, partial_max_logits, partial_output,
+                              num_active_tokens: int, partial_row_index=None):
+        """Enters another attention task's partial results (one per token and query head, in the form
+        `gqa_block_sdpa.metal` writes them) into the split rows the map skips for them; call between the map
+        and the reduce.  `slot_rows[t]`: the split row reserved for token t."""
+        cfg = self.config.struct()
+        L.check(self.device.lib.psi_hip_split_kv_single_q_store_partials(
+            self.device.ctx, ctypes.byref(cfg), _ptr(scratch.buffer), scratch.bytes, _ptr(slot_rows),
+            _ptr(partial_exp_sums), _ptr(partial_max_logits), _ptr(partial_output), self.shape.num_total_tokens,
+            self.shape.num_total_sdpa_map_task_templates, num_active_tokens, _ptr(partial_row_index)))
+
     def invoke_reduce(self, scratch, cu_sdpa_partial_outputs, output):
         self.invoke_reduce_bucketed(scratch, cu_sdpa_partial_outputs, output, self.shape.num_total_tokens)
 
