@@ -125,7 +125,10 @@ int psi_hip_ctx_set_flag(psi_hip_ctx* ctx, uint32_t flag, uint32_t value);
 /* Device-side active counts for captured launches: the counterpart of `ReplayU32::Parameter`
  * (crates/inference-backend-metal/src/metal/replay.rs; bound at submit by `ReplayArguments::with_u32`).
  * device_counts: device u32[4] = {num_active_tokens (= token writes), num_active_q_token_tiles,
- * num_active_kv_splits, reserved}, or null to unbind.  While bound, every kernel launched through this
+ * num_active_kv_splits, gqa_layer_index + 1}, or null to unbind.  The last word binds the page-table layer the
+ * same way (`qwen3.5.mtp.gqa_layer_index`, crates/inference-executor-metal/src/model/qwen/v3_5/mtp/layer.rs:88,
+ * mtp/mod.rs:335-339: one recorded program serves every MTP step): 0 keeps the gqa_layer_index argument of the
+ * entry point, n > 0 selects layer n - 1 (clamped to the table's layers) for the append and the maps.  While bound, every kernel launched through this
  * context reads its active counts from the block when it RUNS; the num_active_* arguments of the entry
  * points then are upper bounds (pass the capacities): grids are cut for them and the device values are
  * clamped to them.  A HIP graph captured with the block bound therefore serves every batch of its

@@ -97,9 +97,18 @@ __device__ __forceinline__ float gate_sigmoid(float x) {
 // Active counts at kernel run time.  `replay_counts` (null or device u32[4] = {tokens, Q-token tiles, KV
 // splits, reserved}) lets a captured launch serve any batch of its capacity bucket: the value passed
 // with the launch is then only an upper bound.  Index constants below.
-constexpr int kReplayTokens = 0, kReplayTiles = 1, kReplaySplits = 2;
+constexpr int kReplayTokens = 0, kReplayTiles = 1, kReplaySplits = 2, kReplayLayer = 3;
 __device__ __forceinline__ uint32_t active_count(const uint32_t* replay_counts, int which, uint32_t by_value) {
     return replay_counts != nullptr ? min(replay_counts[which], by_value) : by_value;
+}
+
+// Word 3 of the block carries the page-table layer of the launch, plus one (`gqa_layer_index` bound as a
+// parameter, crates/inference-executor-metal/src/model/qwen/v3_5/mtp/layer.rs:88); zero leaves the by-value layer
+// in force.  Clamped to the table's layers, so that a stale block cannot index outside it.
+__device__ __forceinline__ uint32_t active_layer(const uint32_t* replay_counts, uint32_t by_value, uint32_t num_layers) {
+    if (replay_counts == nullptr) return by_value;
+    const uint32_t bound = replay_counts[kReplayLayer];
+    return bound == 0 ? by_value : min(bound - 1, num_layers - 1);
 }
 
 // Page-table walk shared by every attention kernel; the expressions of

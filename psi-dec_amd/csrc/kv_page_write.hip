@@ -33,7 +33,9 @@ __device__ __forceinline__ uint64_t line_offset(const PageWriteArgs& a, uint32_t
     const uint32_t id_index = (token / a.tokens_per_page) % a.ids_per_block;
     const uint32_t page_token = token % a.tokens_per_page;
     const uint64_t table_index =
-        (((uint64_t)req_slot * a.num_layers + a.layer) * a.num_blocks + block) * a.ids_per_block + id_index;
+        (((uint64_t)req_slot * a.num_layers + active_layer(a.replay_counts, a.layer, a.num_layers)) * a.num_blocks + block) *
+            a.ids_per_block +
+        id_index;
     const uint64_t page_id = a.page_ids[table_index];
     return page_id * a.page_elems + (((uint64_t)kind * a.hkv + head) * a.tokens_per_page + page_token) * a.d;
 }

@@ -111,7 +111,9 @@ __device__ __forceinline__ void append_row(const FusedAppendArgs& a, const RopeT
     const uint32_t id_index = (token / a.tokens_per_page) % a.ids_per_block;
     const uint32_t page_token = token % a.tokens_per_page;
     const uint64_t table_index =
-        (((uint64_t)req_slot * a.num_layers + a.layer) * a.num_blocks + block) * a.ids_per_block + id_index;
+        (((uint64_t)req_slot * a.num_layers + active_layer(a.replay_counts, a.layer, a.num_layers)) * a.num_blocks + block) *
+            a.ids_per_block +
+        id_index;
     const uint64_t page_base = (uint64_t)a.page_ids[table_index] * a.page_elems;
     const uint64_t k_line = page_base + ((uint64_t)head * a.tokens_per_page + page_token) * a.d;
     const uint64_t v_line = page_base + ((uint64_t)(a.hkv + head) * a.tokens_per_page + page_token) * a.d;

@@ -59,6 +59,7 @@ __device__ __forceinline__ void resolve_active(MapArgs& a) {
     a.num_active_tokens = active_count(a.replay_counts, kReplayTokens, a.num_active_tokens);
     a.num_active_q_token_tiles = active_count(a.replay_counts, kReplayTiles, a.num_active_q_token_tiles);
     a.num_active_kv_splits = active_count(a.replay_counts, kReplaySplits, a.num_active_kv_splits);
+    a.layer = active_layer(a.replay_counts, a.layer, a.walk.num_layers);
 }
 
 struct ReduceArgs {

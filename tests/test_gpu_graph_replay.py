@@ -150,3 +150,69 @@ def test_one_captured_step_serves_every_batch_of_its_bucket(psi, device):
         assert torch.equal(dw.pages.view(torch.int16), eager_pages.view(torch.int16)), picks
         assert (out[n * row:].float() == -768.0).all() and (out[:n * row].float() != -768.0).any()
         _ = out.float().sum().item()  # eager work between replays
+
+
+def test_one_captured_step_serves_every_layer_of_the_table(psi, device):
+    """The page-table layer as a device-side parameter (`qwen3.5.mtp.gqa_layer_index` of the reference: one
+    recorded program serves every MTP step).  A step captured once against a 3-layer table with the count
+    block bound is replayed with word 3 = 1, 2, 3; each replay equals the eager step of that layer with the
+    layer passed by value, bit for bit, and only that layer's pages change.  Word 3 = 0 keeps the by-value
+    layer of the capture."""
+    import torch
+
+    wl = importlib_workloads(psi)
+    import dataclasses
+
+    ctx_lens = [300, 33, 700]
+    layers = 3
+    needed = sum(-(-c // 16) for c in ctx_lens)
+    w0 = wl.make_workload(121, ctx_lens, 24, 4, 256, psi.Dtype.Bfloat16, 16, num_gqa_layers=layers, layer=0,
+                          spare_pages=2 * needed + 3)
+    # layers 1 and 2 get pages of their own from the spare part of the pool
+    lay = w0.layout
+    table = w0.page_ids.reshape(lay.num_req_slots, layers, lay.num_blocks * lay.num_page_ids_per_block).copy()
+    free = [p for p in range(w0.num_pages) if p not in set(table[:, 0].ravel().tolist())]
+    for layer in (1, 2):
+        for r, c in enumerate(ctx_lens):
+            n = -(-c // 16)
+            table[int(w0.req_slots[r]), layer, :n] = [free.pop() for _ in range(n)]
+    ws = [dataclasses.replace(w0, page_ids=table.reshape(-1), layer=l) for l in range(layers)]
+    dws = [wl.DeviceWorkload(device, w, partition_tokens=256) for w in ws]
+    pristine = dws[0].pages.clone()
+    eager = []
+    for dw in dws:  # same inputs, same arena contents, layer by value
+        dw.pages.copy_(pristine)
+        dw.step()
+        device.sync()
+        eager.append((dw.output.clone(), dw.pages.clone()))
+    assert not torch.equal(eager[0][0], eager[1][0]) and not torch.equal(eager[0][1], eager[2][1])
+
+    dw = dws[1]  # captured with layer 1 by value
+    counts = torch.tensor([dw.shape.num_tokens, dw.shape.num_q_token_tiles, dw.shape.num_sdpa_map_task_templates, 0],
+                          dtype=torch.int32, device=device.torch_device)
+    side, main = torch.cuda.Stream(), device.stream
+    graph = torch.cuda.CUDAGraph()
+    try:
+        side.wait_stream(torch.cuda.current_stream())
+        with torch.cuda.stream(side):
+            device.use_stream(side)
+            device.bind_replay_counts(counts)
+            dw.step()  # warm-up on the capture stream
+            side.synchronize()
+            with torch.cuda.graph(graph, stream=side):
+                dw.step()
+    finally:
+        device.bind_replay_counts(None)
+        device.use_stream(main)
+    torch.cuda.synchronize()
+
+    for word, layer in ((1, 0), (3, 2), (0, 1), (2, 1), (1, 0)):
+        counts[3] = word
+        dw.pages.copy_(pristine)
+        dw.output.fill_(-768.0)
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(dw.output.view(torch.int16), eager[layer][0].view(torch.int16)), (word, layer)
+        assert torch.equal(dw.pages.view(torch.int16), eager[layer][1].view(torch.int16)), (word, layer)
+        _ = dw.output.float().sum().item()  # eager work between replays
