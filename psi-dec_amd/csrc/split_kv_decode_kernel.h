@@ -192,7 +192,7 @@ __global__ __launch_bounds__(64 * kWaves, decode_waves_per_simd(G)) void split_k
         else
             k_lane = head_base(p.a) + (((tile * kTileTokens) & page_mask) + mt) * D + mc * 8;
 #pragma unroll
-        for (int i = 0; i < kKSteps; ++i) kreg[i] = *reinterpret_cast<const uint4*>(k_lane + i * 32);
+        for (int i = 0; i < kKSteps; ++i) kreg[i] = stream_load_b128(k_lane + i * 32);
     };
     auto issue_v = [&](uint32_t tile, TilePages p) {
 #pragma unroll
@@ -204,7 +204,7 @@ __global__ __launch_bounds__(64 * kWaves, decode_waves_per_simd(G)) void split_k
             else
                 v_lane = head_base(p.a) + v_region +
                          (((tile * kTileTokens) & page_mask) + j * kVTokensPerLoad + vsub) * D + vdl * 8;
-            vreg[j] = *reinterpret_cast<const uint4*>(v_lane);
+            vreg[j] = stream_load_b128(v_lane);
         }
     };
 

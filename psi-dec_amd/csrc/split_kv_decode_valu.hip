@@ -146,10 +146,10 @@ __global__ __launch_bounds__(256, 2) void split_kv_decode_map_valu(MapArgs a) {
         const uint16_t* v_base = k_base + v_region;
         const uint16_t* k_lane = k_base + kt * D + kc * 8;
 #pragma unroll
-        for (int i = 0; i < kKLoads; ++i) r.k[i] = *reinterpret_cast<const uint4*>(k_lane + i * 32);
+        for (int i = 0; i < kKLoads; ++i) r.k[i] = stream_load_b128(k_lane + i * 32);
         const uint16_t* v_lane = v_base + vsub * D + vdl * 8;
 #pragma unroll
-        for (int j = 0; j < kVLoads; ++j) r.v[j] = *reinterpret_cast<const uint4*>(v_lane + j * kVTokensPerLoad * D);
+        for (int j = 0; j < kVLoads; ++j) r.v[j] = stream_load_b128(v_lane + j * kVTokensPerLoad * D);
     };
 
     uint32_t tile = tile_begin + wave;
