@@ -44,6 +44,8 @@ def parse_args():
     p.add_argument("--decode-waves", type=int, default=0, help="waves per decode workgroup (0 = automatic)")
     p.add_argument("--plan-order", action="store_true",
                    help="dispatch the split rows in plan order instead of longest first")
+    p.add_argument("--separate-append", action="store_true",
+                   help="decode workload: launch the append as its own kernel instead of folding it into the map")
     p.add_argument("--balance", action="store_true", help="equal-tile worker plan instead of one workgroup per partition")
     p.add_argument("--kernel-only", action="store_true", help="time only the map kernel (for profiling runs)")
     p.add_argument("--graph", action="store_true",
@@ -193,7 +195,8 @@ def main():
         w.seed = args.seed + 1000 * i  # same geometry, different page contents
         arenas.append(wl.DeviceWorkload(device, w, partition_tokens=args.partition, balanced=args.balance,
                                         longest_first=not args.plan_order,
-                                        grouped=prefill and not args.no_row_groups))
+                                        grouped=prefill and not args.no_row_groups,
+                                        fused_append=not args.separate_append))
     w = arenas[0].w
     shape = arenas[0].shape
     step_bytes = w.algorithmic_bytes()
@@ -289,6 +292,7 @@ def main():
             "arenas_rotated": len(arenas),
             "kernel_us_in_step": kernels_us,
             "dispatch_order": "plan order" if args.plan_order or args.balance else "longest split first",
+            "append": "folded into the map launch" if arenas[0].fused_append else "separate kernel",
         },
         "roofline": {
             "bound": "hbm",

@@ -350,6 +350,22 @@ int psi_hip_split_kv_single_q_map(psi_hip_ctx* ctx, const psi_hip_gqa_config* cf
                                   uint32_t num_total_kv_splits, uint32_t num_active_tokens,
                                   uint32_t num_active_kv_splits);
 
+/* The append and the map of a decode step in one launch (no counterpart as one kernel in the reference, which
+ * records gqa_kv_page_write and then gqa_split_kv_single_q_map, attn/gqa/backend.rs:394-658): the page arena ends
+ * up as after psi_hip_kv_page_write, bit for bit, and the partial states as after psi_hip_split_kv_single_q_map up
+ * to the order of summation.  The workgroup whose kv_splits row ends at a token's own position
+ * (flat_token_indices[t] + 1) writes that token's K/V lines; every position appended in this step is read from
+ * flat_k / flat_v instead of its page, after the paged positions of the row.
+ * Requires what the two calls require plus: each active token owns a row that ends at its position + 1 (true of
+ * every plan of psi_hip_gqa_metadata_update), and the tokens of a request are adjacent and in position order.
+ * Shapes outside the gfx950 decode kernel run the two launches. */
+int psi_hip_kv_page_write_split_kv_single_q_map(
+    psi_hip_ctx* ctx, const psi_hip_gqa_config* cfg, const psi_hip_page_table_layout* layout, const void* q,
+    void* kv_pages, uint64_t kv_pages_bytes, const void* flat_k, const void* flat_v, const uint32_t* req_slots,
+    const uint32_t* flat_token_indices, const uint32_t* page_ids, const uint32_t* kv_splits, void* scratch,
+    uint64_t scratch_bytes, uint32_t gqa_layer_index, uint32_t num_total_tokens, uint32_t num_total_kv_splits,
+    uint32_t num_active_tokens, uint32_t num_active_kv_splits);
+
 /* The same map launched over a balanced plan: workgroup w of each KV head serves kv_splits rows
  * [worker_cu[w], worker_cu[w + 1]) (device u32[num_workers + 1], from psi_hip_split_kv_balance_plan).
  * Falls back to the row-per-workgroup launch for shapes outside the gfx950 kernels' domain. */

@@ -52,6 +52,11 @@ struct MapArgs {
     const uint32_t* worker_cu = nullptr;
     uint32_t num_workers = 0;
     const uint32_t* replay_counts = nullptr;  // see active_count()
+    // Decode map with the append folded in (null otherwise): the step's new K/V rows [token][Hkv][D].  The
+    // workgroup whose row ends at a token's own position writes that token's lines into its page, and every
+    // position appended in this step is read from these rows instead of the page.
+    const void* flat_k = nullptr;
+    const void* flat_v = nullptr;
 };
 
 // First statement of every map kernel.
@@ -143,6 +148,7 @@ void fill_walk(PageWalk* walk, const Geometry& g, const psi_hip_page_table_layou
 // Fast decode map for head_dim 256 / 128, 2-byte elements, power-of-two pages; returns
 // PSI_HIP_ERR_UNSUPPORTED when the shape is outside its domain (caller falls back).
 int launch_decode_map_fast(psi_hip_ctx* ctx, const Geometry& g, const MapArgs& a);
+bool decode_map_takes_append(const psi_hip_ctx* ctx, const Geometry& g, const MapArgs& a);
 int launch_reduce_fast(psi_hip_ctx* ctx, const Geometry& g, const ReduceArgs& a);
 // The same decode map with the QK^T contraction on the vector ALU (comparison variant).
 int launch_decode_map_valu(psi_hip_ctx* ctx, const Geometry& g, const MapArgs& a);

@@ -186,6 +186,17 @@ __global__ __launch_bounds__(256) void split_kv_reduce_tiled_fast(ReduceArgs a) 
         store_from_f32<Tag>(a.output, out_index + e, finish_output<Tag>(a, value[e] * inv, token, q_head, lane * kPerLane + e));
 }
 
+// Shapes and pointers for which the MFMA decode map runs, i.e. for which the append can be folded into it.
+bool decode_map_takes_append(const psi_hip_ctx* ctx, const Geometry& g, const MapArgs& a) {
+    if (ctx->force_generic || ctx->decode_valu_qk) return false;
+    const bool two_byte = g.dtype == PSI_HIP_BF16 || g.dtype == PSI_HIP_F16;
+    const uint32_t p = g.tokens_per_page;
+    const bool page_ok = p >= 8 && (p & (p - 1)) == 0;
+    auto aligned = [](const void* ptr) { return reinterpret_cast<uintptr_t>(ptr) % 16 == 0; };
+    return two_byte && page_ok && g.group <= 8 && (g.d == 256 || g.d == 128) && aligned(a.q) && aligned(a.kv_pages) &&
+           aligned(a.flat_k) && aligned(a.flat_v) && (uint64_t)a.num_total_kv_splits * g.hkv <= 0x7fffffffull;
+}
+
 int launch_decode_map_fast(psi_hip_ctx* ctx, const Geometry& g, const MapArgs& a) {
     if (ctx->force_generic) return PSI_HIP_ERR_UNSUPPORTED;
     if (ctx->decode_valu_qk) {

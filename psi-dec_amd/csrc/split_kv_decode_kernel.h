@@ -71,10 +71,11 @@ __device__ __forceinline__ void wave_lds_fence() { asm volatile("s_waitcnt lgkmc
 #define PSI_DECODE_WAVES_PER_SIMD 3
 #endif
 
-// Workgroups per SIMD the register allocator is held to.  Three (168 registers) fits up to six query heads per
-// KV head; seven and eight need 181 and 190 registers and would spill, and a kernel with a private segment
-// starts far slower than one resident wave less costs, so those are held to two.
-constexpr int decode_waves_per_simd(int group) { return group > 6 ? 2 : PSI_DECODE_WAVES_PER_SIMD; }
+// Workgroups per SIMD the register allocator is held to.  Three (168 registers) fits up to five query heads per
+// KV head; six to eight need 172 to 198 registers and would spill, and a kernel with a private segment starts far
+// slower than one resident wave less costs (two and three workgroups per SIMD stream equally fast), so those
+// are held to two.
+constexpr int decode_waves_per_simd(int group) { return group > 5 ? 2 : PSI_DECODE_WAVES_PER_SIMD; }
 
 constexpr int kTileTokens = 16;
 
@@ -155,8 +156,38 @@ __global__ __launch_bounds__(64 * kWaves, decode_waves_per_simd(G)) void split_k
                                                       a.walk.num_blocks * a.walk.ids_per_block;
     const uint64_t v_region = (uint64_t)a.walk.hkv * a.walk.tokens_per_page * D;
 
+    // Append folded into the map (a.flat_k set): positions [new_begin, own] of this request are this step's
+    // new tokens.  They are read from the flat rows after the paged tiles, never from the page, which another
+    // workgroup may be writing right now; the paged part of the row ends at page_end.
+    uint32_t page_end = kv_end, new_begin = kv_end;
+    if (a.flat_k != nullptr) {
+        const uint32_t own = a.flat_token_indices[q_token];  // this token's position
+        if (kv_end + q_token > own) {  // the row can reach a token of this step (at most q_token of them precede)
+            uint32_t before = 0;
+            while (before < q_token && req_slots[q_token - before - 1] == req_slot &&
+                   a.flat_token_indices[q_token - before - 1] + before + 1 == own)
+                ++before;
+            new_begin = max(own - before, kv_begin);
+            page_end = min(kv_end, new_begin);
+        }
+        if (kv_end == own + 1 && wave == 0) {
+            // this workgroup owns the token's append for its KV head: one 16-byte chunk per lane, K line then V line
+            const uint32_t page_id = table_row[own >> log2p];
+            constexpr uint32_t kChunks = D / 8;
+            const uint16_t* flat[2] = {reinterpret_cast<const uint16_t*>(a.flat_k),
+                                       reinterpret_cast<const uint16_t*>(a.flat_v)};
+            for (uint32_t c = lane; c < 2 * kChunks; c += 64) {
+                const uint32_t kind = c / kChunks, chunk = c % kChunks;
+                const uint16_t* src = flat[kind] + ((uint64_t)q_token * a.walk.hkv + kv_head) * D + chunk * 8;
+                uint16_t* dst = const_cast<uint16_t*>(pages) + (uint64_t)page_id * a.walk.page_elems + kind * v_region +
+                                ((uint64_t)kv_head * a.walk.tokens_per_page + (own & page_mask)) * D + chunk * 8;
+                *reinterpret_cast<uint4*>(dst) = *reinterpret_cast<const uint4*>(src);
+            }
+        }
+    }
+
     const uint32_t tile_begin = kv_begin / kTileTokens;
-    const uint32_t tile_end = (kv_end + kTileTokens - 1) / kTileTokens;
+    const uint32_t tile_end = page_end > kv_begin ? (page_end + kTileTokens - 1) / kTileTokens : tile_begin;
 
     float run_max = -INFINITY, lane_sum = 0.0f;  // of query row mt, over this lane's tokens
     float acc[G][8];
@@ -165,7 +196,7 @@ __global__ __launch_bounds__(64 * kWaves, decode_waves_per_simd(G)) void split_k
 #pragma unroll
         for (int e = 0; e < 8; ++e) acc[h][e] = 0.0f;
 
-    const uint32_t last_page = (kv_end - 1) >> log2p;
+    const uint32_t last_page = (max(page_end, 1u) - 1) >> log2p;
     auto load_page_id = [&](uint32_t tile) -> TilePages {
         TilePages p{0u, 0u};
         if (tile < tile_end) {
@@ -214,8 +245,9 @@ __global__ __launch_bounds__(64 * kWaves, decode_waves_per_simd(G)) void split_k
     // One 16-token tile.  `partial`: the tile holds tokens outside [kv_begin, kv_end).
     // `has_next`: another tile of this wave follows; its K and V are requested on the way, each
     // into the registers the current tile has just finished with.  Both flags are wave-uniform.
-    auto process_tile = [&](uint32_t tile, bool partial, auto has_next_tag, uint32_t next, TilePages next_pid)
-                            __attribute__((always_inline)) {
+    // `base`: position of the tile's first token; positions outside [lo, hi) are masked.
+    auto process_tile = [&](uint32_t base, uint32_t lo, uint32_t hi, bool partial, auto has_next_tag, uint32_t next,
+                            TilePages next_pid) __attribute__((always_inline)) {
         // compile-time flag: the steady-state copy issues its refill loads unconditionally, which
         // keeps the hardware load counter's order exact for the waits that follow
         constexpr bool has_next = decltype(has_next_tag)::value;
@@ -234,8 +266,8 @@ __global__ __launch_bounds__(64 * kWaves, decode_waves_per_simd(G)) void split_k
         float m = -INFINITY;
 #pragma unroll
         for (int r = 0; r < 4; ++r) {
-            const uint32_t token = tile * kTileTokens + mc * 4 + r;
-            const bool valid = token >= kv_begin && token < kv_end;
+            const uint32_t token = base + mc * 4 + r;
+            const bool valid = token >= lo && token < hi;
             v[r] = valid ? (s0[r] + s1[r]) * a.scale_log2 : -INFINITY;
             m = fmaxf(m, v[r]);
         }
@@ -278,8 +310,8 @@ __global__ __launch_bounds__(64 * kWaves, decode_waves_per_simd(G)) void split_k
             // tokens outside the split carry probability 0, but their V bytes may be NaN/Inf
 #pragma unroll
             for (int j = 0; j < kVLoads; ++j) {
-                const uint32_t vtoken = tile * kTileTokens + j * kVTokensPerLoad + vsub;
-                if (vtoken < kv_begin || vtoken >= kv_end) vreg[j] = make_uint4(0, 0, 0, 0);
+                const uint32_t vtoken = base + j * kVTokensPerLoad + vsub;
+                if (vtoken < lo || vtoken >= hi) vreg[j] = make_uint4(0, 0, 0, 0);
             }
         }
         __builtin_amdgcn_sched_barrier(0);
@@ -319,15 +351,36 @@ __global__ __launch_bounds__(64 * kWaves, decode_waves_per_simd(G)) void split_k
             issue_v(tile, pid);
         }
         TilePages pid_next = load_page_id(tile + kWaves);
-        auto is_partial = [&](uint32_t t) { return t * kTileTokens < kv_begin || (t + 1) * kTileTokens > kv_end; };
+        auto is_partial = [&](uint32_t t) { return t * kTileTokens < kv_begin || (t + 1) * kTileTokens > page_end; };
         while (tile + kWaves < tile_end) {
             const uint32_t next = tile + kWaves;
             const TilePages pid_after = load_page_id(next + kWaves);
-            process_tile(tile, is_partial(tile), std::true_type(), next, pid_next);
+            process_tile(tile * kTileTokens, kv_begin, page_end, is_partial(tile), std::true_type(), next, pid_next);
             pid_next = pid_after;
             tile = next;
         }
-        process_tile(tile, is_partial(tile), std::false_type(), 0u, TilePages{0u, 0u});  // the wave's last tile
+        // the wave's last tile
+        process_tile(tile * kTileTokens, kv_begin, page_end, is_partial(tile), std::false_type(), 0u, TilePages{0u, 0u});
+    }
+    if (new_begin < kv_end && wave == kWaves - 1) {
+        // this step's tokens inside the row, sixteen at a time from the flat rows (one, in a decode batch)
+        const uint16_t* flat_k = reinterpret_cast<const uint16_t*>(a.flat_k);
+        const uint16_t* flat_v = reinterpret_cast<const uint16_t*>(a.flat_v);
+        const uint32_t new_end = min(kv_end, a.flat_token_indices[q_token] + 1);
+        const int64_t row0 = (int64_t)q_token - a.flat_token_indices[q_token];  // flat row of position p = row0 + p
+        for (uint32_t base = new_begin; base < new_end; base += kTileTokens) {
+            const uint32_t k_pos = min(base + mt, new_end - 1);
+            const uint16_t* k_lane = flat_k + ((uint64_t)(row0 + k_pos) * a.walk.hkv + kv_head) * D + mc * 8;
+#pragma unroll
+            for (int i = 0; i < kKSteps; ++i) kreg[i] = *reinterpret_cast<const uint4*>(k_lane + i * 32);
+#pragma unroll
+            for (int j = 0; j < kVLoads; ++j) {
+                const uint32_t v_pos = min(base + j * kVTokensPerLoad + vsub, new_end - 1);
+                vreg[j] = *reinterpret_cast<const uint4*>(flat_v + ((uint64_t)(row0 + v_pos) * a.walk.hkv + kv_head) * D +
+                                                          vdl * 8);
+            }
+            process_tile(base, base, new_end, true, std::false_type(), 0u, TilePages{0u, 0u});
+        }
     }
 
 #ifdef PSI_DECODE_TIMESTAMPS

@@ -82,7 +82,8 @@ static int single_q_map_impl(psi_hip_ctx* ctx, const psi_hip_gqa_config* cfg, co
                              const uint32_t* page_ids, const uint32_t* kv_splits, const uint32_t* worker_cu,
                              uint32_t num_workers, void* scratch, uint64_t scratch_bytes, uint32_t gqa_layer_index,
                              uint32_t num_total_tokens, uint32_t num_total_kv_splits, uint32_t num_active_tokens,
-                             uint32_t num_active_kv_splits) {
+                             uint32_t num_active_kv_splits, const void* flat_k = nullptr, const void* flat_v = nullptr,
+                             const uint32_t* flat_token_indices = nullptr) {
     PSI_REQUIRE(ctx != nullptr, "ctx must not be null");
     Geometry g;
     int rc = make_geometry(cfg, &g);
@@ -124,6 +125,20 @@ static int single_q_map_impl(psi_hip_ctx* ctx, const psi_hip_gqa_config* cfg, co
     a.scale_log2 = g.scale * kLog2e;
     a.worker_cu = worker_cu;
     a.num_workers = num_workers;
+    if (flat_k != nullptr) {
+        // the append travels with the map when the MFMA kernel serves the shape, else it is a launch of its own
+        a.flat_k = flat_k;
+        a.flat_v = flat_v;
+        a.flat_token_indices = flat_token_indices;
+        if (!decode_map_takes_append(ctx, g, a)) {
+            rc = psi_hip_kv_page_write(ctx, cfg, layout, const_cast<void*>(kv_pages), kv_pages_bytes, flat_k, flat_v,
+                                       req_slots, flat_token_indices, page_ids, num_total_tokens, num_active_tokens,
+                                       gqa_layer_index);
+            if (rc != PSI_HIP_OK) return rc;
+            a.flat_k = a.flat_v = nullptr;
+            a.flat_token_indices = nullptr;
+        }
+    }
 
     LaunchScope scope(ctx, "split_kv_map");
     rc = launch_decode_map_fast(ctx, g, a);
@@ -253,4 +268,16 @@ extern "C" int psi_hip_split_kv_single_q_store_partials(psi_hip_ctx* ctx, const 
     hipLaunchKernelGGL(store_partials_kernel, dim3((uint32_t)((waves + 3) / 4)), dim3(256), 0, ctx->stream, a);
     PSI_HIP_CHECK(hipGetLastError());
     return PSI_HIP_OK;
+}
+
+extern "C" int psi_hip_kv_page_write_split_kv_single_q_map(
+    psi_hip_ctx* ctx, const psi_hip_gqa_config* cfg, const psi_hip_page_table_layout* layout, const void* q,
+    void* kv_pages, uint64_t kv_pages_bytes, const void* flat_k, const void* flat_v, const uint32_t* req_slots,
+    const uint32_t* flat_token_indices, const uint32_t* page_ids, const uint32_t* kv_splits, void* scratch,
+    uint64_t scratch_bytes, uint32_t gqa_layer_index, uint32_t num_total_tokens, uint32_t num_total_kv_splits,
+    uint32_t num_active_tokens, uint32_t num_active_kv_splits) {
+    PSI_REQUIRE(flat_k && flat_v && flat_token_indices, "GQA KV page write buffers must not be null");
+    return single_q_map_impl(ctx, cfg, layout, q, kv_pages, kv_pages_bytes, req_slots, page_ids, kv_splits, nullptr, 0,
+                             scratch, scratch_bytes, gqa_layer_index, num_total_tokens, num_total_kv_splits,
+                             num_active_tokens, num_active_kv_splits, flat_k, flat_v, flat_token_indices);
 }

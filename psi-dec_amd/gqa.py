@@ -808,6 +808,20 @@ class GQASplitKVSingleQKernels:
             page_table_index, self.shape.num_total_tokens, self.shape.num_total_sdpa_map_task_templates,
             num_active_tokens, num_active_kv_splits))
 
+    def invoke_append_map_bucketed(self, q, kv_pages, flat_k, flat_v, req_slots, flat_token_indices, page_ids,
+                                   sdpa_map_task_templates, scratch, page_table_index: int, num_active_tokens: int,
+                                   num_active_kv_splits: int):
+        """`GQAKVPageWrite.invoke_bucketed` and `invoke_map_bucketed` in one launch: the workgroup whose split row
+        ends at a token's position writes the token's K/V lines, and the step's new positions are read from
+        `flat_k` / `flat_v`.  Same arena as the two calls bit for bit; partial states equal up to summation order."""
+        cfg, layout = self.config.struct(), self.config.page_table_layout.struct()
+        L.check(self.device.lib.psi_hip_kv_page_write_split_kv_single_q_map(
+            self.device.ctx, ctypes.byref(cfg), ctypes.byref(layout), _ptr(q), _ptr(kv_pages), _nbytes(kv_pages),
+            _ptr(flat_k), _ptr(flat_v), _ptr(req_slots), _ptr(flat_token_indices), _ptr(page_ids),
+            _ptr(sdpa_map_task_templates), _ptr(scratch.buffer), scratch.bytes, page_table_index,
+            self.shape.num_total_tokens, self.shape.num_total_sdpa_map_task_templates, num_active_tokens,
+            num_active_kv_splits))
+
     def invoke_map_balanced(self, q, kv_pages, req_slots, page_ids, sdpa_map_task_templates, worker_cu,
                             num_workers: int, scratch, page_table_index: int, num_active_tokens: int,
                             num_active_kv_splits: int):

@@ -146,7 +146,7 @@ class DeviceWorkload:
     def __init__(self, device: G.Device, w: Workload, partition_tokens: Optional[int] = None,
                  max_tokens: Optional[int] = None, variant: Optional[G.GQASplitKVVariant] = None,
                  f32_output: bool = False, balanced: bool = False, longest_first: bool = False,
-                 grouped: bool = False):
+                 grouped: bool = False, fused_append: bool = False):
         import torch
 
         self.device, self.w = device, w
@@ -220,6 +220,8 @@ class DeviceWorkload:
             self.kernels = G.GQASplitKVSingleQKernels(device, self.cfg, self.kshape)
             self.scratch = G.GQASplitKVSingleQScratch(device, self.cfg, self.kshape)
         self._rows = rows
+        # decode only: the append rides in the map launch (one launch fewer per step)
+        self.fused_append = bool(fused_append) and not variant.is_tiled() and not self.balanced
         self.grouped = bool(grouped) and variant.is_tiled()
         if self.grouped:
             self.meta.group_rows(self.cfg)
@@ -269,10 +271,19 @@ class DeviceWorkload:
                                                 partial_row_index=m.d_partial_row_index)
         self.device.f32_output(False)
 
+    def append_map(self):
+        m, s = self.meta, self.shape
+        self.kernels.invoke_append_map_bucketed(self.q, self.pages, self.flat_k, self.flat_v, m.d_req_slots,
+                                                m.d_flat_token_indices, self.page_ids, m.d_kv_splits, self.scratch,
+                                                self.w.layer, s.num_tokens, s.num_sdpa_map_task_templates)
+
     def step(self):
         """One layer-step: append the new tokens, then attend (the new tokens see themselves)."""
-        self.append()
-        self.map()
+        if self.fused_append:
+            self.append_map()
+        else:
+            self.append()
+            self.map()
         self.reduce()
 
     def output_f32(self) -> np.ndarray:

@@ -136,3 +136,42 @@ def test_long_split_lists_use_the_wide_combine(psi, oracle, device, longest_firs
     assert dw.shape.num_sdpa_map_task_templates == 375 + 188
     _, dw2 = run_and_check(psi, oracle, device, w, "narrow combine", partition_tokens=1024, variant=variant)
     assert np.abs(dw.output_f32() - dw2.output_f32()).max() < 2e-5
+
+
+@pytest.mark.parametrize("dtype_name,hq,hkv,d,p,q_lens,partition", [
+    ("Bfloat16", 24, 4, 256, 16, 1, 512),                       # the decode batch of the headline configuration
+    ("Bfloat16", 24, 4, 256, 16, 1, None),                      # the reference's greedy plan
+    ("Float16", 16, 2, 256, 16, 1, 256),
+    ("Bfloat16", 32, 8, 128, 16, 1, 512),
+    ("Bfloat16", 24, 4, 256, 8, 1, 512),                        # 8-token pages
+    ("Bfloat16", 24, 4, 256, 16, [3, 1, 2, 1, 4, 1, 2], 512),   # several new tokens per request, each its own row set
+    ("Bfloat16", 16, 2, 256, 16, [20, 1, 17, 1, 1, 1, 1], 256),  # more than one tile of new tokens in a row
+    ("Float32", 6, 2, 64, 8, 1, None),                          # outside the MFMA kernel: two launches inside
+])
+def test_append_folded_into_the_map(psi, oracle, device, dtype_name, hq, hkv, d, p, q_lens, partition):
+    """The append and the map in one launch: the page arena equals the oracle's (and the append-then-map step's)
+    bit for bit; outputs are within tolerance of the oracle and differ from the two-launch step only by the order
+    of summation (the new tokens are folded in after the paged ones).  Contexts put new tokens at
+    the start of a page, at its end, across a partition boundary (513 = 512 + 1) and in a one-token context."""
+    wl = importlib_workloads(psi)
+    dtype = getattr(psi.Dtype, dtype_name)
+    ctx = [3000, 17, 1025, 2048, 700, 32, 513] if partition else [300, 17, 129, 256, 70, 32, 65]
+    if not np.isscalar(q_lens):
+        ctx = [max(c, q) for c, q in zip(ctx, q_lens)]
+    w = wl.make_workload(41, ctx, hq, hkv, d, dtype, p, q_lens=q_lens)
+    variant = psi.GQASplitKVVariant.SingleQ(256, 256, min(hq // hkv, 8))
+    what = f"append in map {dtype_name} {hq}/{hkv}/{d} P={p} q={q_lens}"
+    stats, dw = run_and_check(psi, oracle, device, w, what, partition_tokens=partition, variant=variant,
+                              fused_append=True, max_tokens=64)
+    assert dw.fused_append
+    plain = wl.DeviceWorkload(device, w, partition_tokens=partition, variant=variant, f32_output=True, max_tokens=64)
+    plain.step()
+    assert np.abs(plain.output_f32() - dw.output_f32()).max() < 2e-5
+    assert np.array_equal(plain.pages_host(), dw.pages_host())
+
+
+def test_append_folded_into_the_map_single_token_context(psi, oracle, device):
+    """A request whose whole context is the token being appended: the row has no paged part at all."""
+    wl = importlib_workloads(psi)
+    w = wl.make_workload(43, [1, 1, 2, 16, 17], 24, 4, 256, psi.Dtype.Bfloat16, 16)
+    run_and_check(psi, oracle, device, w, "append in map, one-token contexts", partition_tokens=512, fused_append=True)
