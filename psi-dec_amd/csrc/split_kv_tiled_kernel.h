@@ -222,7 +222,7 @@ __global__ __launch_bounds__(64 * kTiledTileWaves * CG, (TiledOccupancy<NB, CG>:
             else
                 v_lane = head_base(p.a) + v_region +
                          (((tile * kTileTokens) & page_mask) + j * kVTokensPerLoad + vsub) * D + vdl * 8;
-            vreg[j] = *reinterpret_cast<const uint4*>(v_lane);
+            vreg[j] = stream_load_b128(v_lane);  // V rows are whole lines read once; K keeps ordinary loads (two loads share each line)
         }
     };
 
