@@ -10,13 +10,15 @@ from parity_util import importlib_workloads
 pytestmark = pytest.mark.gpu
 
 
-@pytest.mark.parametrize("q_len", [1, 2])
-def test_captured_layer_step_replays(psi, device, q_len):
+@pytest.mark.parametrize("q_len,fused_append", [(1, False), (2, False), (1, True)])
+def test_captured_layer_step_replays(psi, device, q_len, fused_append):
+    """`fused_append`: the append rides in the decode map launch (two nodes in the graph instead of three)."""
     import torch
 
     wl = importlib_workloads(psi)
     w = wl.make_workload(101 + q_len, [700, 33, 1500, 512, 64], 24, 4, 256, psi.Dtype.Bfloat16, 16, q_lens=q_len)
-    dw = wl.DeviceWorkload(device, w, partition_tokens=512)
+    dw = wl.DeviceWorkload(device, w, partition_tokens=512, fused_append=fused_append)
+    assert dw.fused_append == fused_append
     pristine = dw.pages.clone()
 
     def eager():
