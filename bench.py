@@ -48,7 +48,8 @@ def parse_args():
                    help="dispatch the split rows in plan order instead of longest first")
     p.add_argument("--separate-append", action="store_true",
                    help="decode workload: launch the append as its own kernel instead of folding it into the map")
-    p.add_argument("--balance", action="store_true", help="equal-tile worker plan instead of one workgroup per partition")
+    p.add_argument("--row-per-workgroup", action="store_true",
+                   help="decode workload: one workgroup per partition row instead of the balanced worker plan")
     p.add_argument("--kernel-only", action="store_true", help="time only the map kernel (for profiling runs)")
     p.add_argument("--graph", action="store_true",
                    help="replay a captured HIP graph per step instead of launching its three kernels one by one "
@@ -195,7 +196,7 @@ def main():
             w = wl.make_workload(args.seed, ctx, args.q_heads, args.kv_heads, 256, psi.Dtype.Bfloat16, 16,
                                  host_pages=False, shuffle_pages=not args.identity_pages)
         w.seed = args.seed + 1000 * i  # same geometry, different page contents
-        arenas.append(wl.DeviceWorkload(device, w, partition_tokens=args.partition, balanced=args.balance,
+        arenas.append(wl.DeviceWorkload(device, w, partition_tokens=args.partition, balanced=not args.row_per_workgroup,
                                         longest_first=not args.plan_order,
                                         grouped=prefill and not args.no_row_groups,
                                         fused_append=not args.separate_append))
@@ -315,7 +316,9 @@ def main():
             "algorithmic_bytes_per_step": step_bytes,
             "arenas_rotated": len(arenas),
             "kernel_us_in_step": kernels_us,
-            "dispatch_order": "plan order" if args.plan_order or args.balance else "longest split first",
+            "dispatch": ("one workgroup per compute unit and KV head over equal shares of the tiles of the "
+                         "512-token plan" if arenas[0].balanced else
+                         "one workgroup per plan row, " + ("plan order" if args.plan_order else "longest first")),
             "append": "folded into the map launch" if arenas[0].fused_append else "separate kernel",
         },
         "roofline": {

@@ -198,12 +198,15 @@ int psi_hip_gqa_metadata_update(uint32_t max_tokens, const uint32_t* req_slots, 
 int psi_hip_split_kv_order_longest_first(uint32_t* kv_splits, uint32_t num_kv_splits, uint32_t* partial_row_index);
 
 /* Balanced decode plan (no counterpart in the reference, whose planner budgets partial states, not
- * device occupancy).  Cuts the rows of an existing SingleQ plan at tile boundaries so that
- * `num_workers` consecutive groups of rows hold equal numbers of 16-token tiles; a decode-map
- * workgroup then serves one group per KV head and all workgroups finish together.
- * kv_splits_in[num_rows_in][3] / cu_in[num_tokens + 1] -> kv_splits_out (capacity rows_capacity
- * rows, at most num_rows_in + num_workers are produced), cu_out[num_tokens + 1],
- * worker_cu_out[num_workers + 1].  Every output row lies inside one input row. */
+ * device occupancy).  Re-cuts the rows of an existing SingleQ plan at 16-token tile boundaries into
+ * `num_workers` consecutive groups that hold equal numbers of tiles; a decode-map workgroup then serves one
+ * group per KV head and all workgroups finish together.  Inside a group, adjacent pieces of one token
+ * are one row -- one pass through the keys, one partial state -- whatever the partition of the input plan,
+ * so the output has at most num_workers + num_tokens rows (fewer row starts and partial states than a
+ * workgroup per input row: the launch streams faster and the combine reads less).
+ * kv_splits_in[num_rows_in][3] / cu_in[num_tokens + 1] -> kv_splits_out (capacity rows_capacity rows),
+ * cu_out[num_tokens + 1], worker_cu_out[num_workers + 1].  The rows of a token still tile [0, context)
+ * in order. */
 int psi_hip_split_kv_balance_plan(const uint32_t* kv_splits_in, uint32_t num_rows_in, const uint32_t* cu_in,
                                   uint32_t num_tokens, uint32_t num_workers, uint32_t* kv_splits_out,
                                   uint32_t rows_capacity, uint32_t* cu_out, uint32_t* worker_cu_out,
@@ -358,13 +361,15 @@ int psi_hip_split_kv_single_q_map(psi_hip_ctx* ctx, const psi_hip_gqa_config* cf
  * flat_k / flat_v instead of its page, after the paged positions of the row.
  * Requires what the two calls require plus: each active token owns a row that ends at its position + 1 (true of
  * every plan of psi_hip_gqa_metadata_update), and the tokens of a request are adjacent and in position order.
- * Shapes outside the gfx950 decode kernel run the two launches. */
+ * worker_cu / num_workers: null / 0 for a workgroup per row, or the worker table of a balanced plan as for
+ * psi_hip_split_kv_single_q_map_balanced.  Shapes outside the gfx950 decode kernel run the two launches. */
 int psi_hip_kv_page_write_split_kv_single_q_map(
     psi_hip_ctx* ctx, const psi_hip_gqa_config* cfg, const psi_hip_page_table_layout* layout, const void* q,
     void* kv_pages, uint64_t kv_pages_bytes, const void* flat_k, const void* flat_v, const uint32_t* req_slots,
-    const uint32_t* flat_token_indices, const uint32_t* page_ids, const uint32_t* kv_splits, void* scratch,
-    uint64_t scratch_bytes, uint32_t gqa_layer_index, uint32_t num_total_tokens, uint32_t num_total_kv_splits,
-    uint32_t num_active_tokens, uint32_t num_active_kv_splits);
+    const uint32_t* flat_token_indices, const uint32_t* page_ids, const uint32_t* kv_splits,
+    const uint32_t* worker_cu, uint32_t num_workers, void* scratch, uint64_t scratch_bytes, uint32_t gqa_layer_index,
+    uint32_t num_total_tokens, uint32_t num_total_kv_splits, uint32_t num_active_tokens,
+    uint32_t num_active_kv_splits);
 
 /* The same map launched over a balanced plan: workgroup w of each KV head serves kv_splits rows
  * [worker_cu[w], worker_cu[w + 1]) (device u32[num_workers + 1], from psi_hip_split_kv_balance_plan).

@@ -191,7 +191,7 @@ PROTOTYPES = {
                 POINTER(OutputGateStruct)]),
     "psi_hip_kv_page_write_split_kv_single_q_map": (
         c_int, [c_void_p, _CFG, _LAYOUT, c_void_p, c_void_p, c_uint64, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p,
-                c_void_p, c_void_p, c_uint64, c_uint32, c_uint32, c_uint32, c_uint32, c_uint32]),
+                c_void_p, c_void_p, c_uint32, c_void_p, c_uint64, c_uint32, c_uint32, c_uint32, c_uint32, c_uint32]),
     "psi_hip_split_kv_single_q_store_partials": (
         c_int, [c_void_p, _CFG, c_void_p, c_uint64, c_void_p, c_void_p, c_void_p, c_void_p, c_uint32, c_uint32,
                 c_uint32, c_void_p]),

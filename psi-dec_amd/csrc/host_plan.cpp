@@ -508,8 +508,10 @@ extern "C" int psi_hip_split_kv_balanced_workers(const psi_hip_gqa_config* cfg, 
     int rc = make_geometry(cfg, &g);
     if (rc != PSI_HIP_OK) return rc;
     PSI_REQUIRE(out_num_workers != nullptr, "out pointer must not be null");
-    // 256 compute units, three 4-wave workgroups resident on each
-    *out_num_workers = std::max(1u, (256u * 3u) / g.hkv);
+    // One 4-wave workgroup per compute unit (256 of them): equal shares of the tiles with as few rows, i.e.
+    // partial states and row starts, as the batch allows.  Measured on B=32, ctx 1k-8k, 24/4 heads: 256
+    // workgroups 93.7 us, 512 97.7 us, 768 101.6 us, against 104.0 us for a workgroup per 512-token row.
+    *out_num_workers = std::max(1u, 256u / g.hkv);
     return PSI_HIP_OK;
 }
 
@@ -554,11 +556,18 @@ extern "C" int psi_hip_split_kv_balance_plan(const uint32_t* kv_splits_in, uint3
             while (worker + 1 < num_workers && linear >= worker_end(worker)) worker_cu_out[++worker] = out_rows;
             const uint64_t room = worker + 1 < num_workers ? worker_end(worker) - linear : remaining;
             const uint64_t take = std::min<uint64_t>(remaining, std::max<uint64_t>(room, 1));
-            PSI_REQUIRE(out_rows < rows_capacity, "balanced plan exceeds the row capacity");
-            kv_splits_out[3 * out_rows] = kv_splits_in[3 * r];
-            kv_splits_out[3 * out_rows + 1] = std::max<uint32_t>(b, tile_cursor * kTile);
-            kv_splits_out[3 * out_rows + 2] = (uint32_t)std::min<uint64_t>(e, (uint64_t)(tile_cursor + take) * kTile);
-            ++out_rows;
+            const uint32_t piece_begin = std::max<uint32_t>(b, tile_cursor * kTile);
+            const uint32_t piece_end = (uint32_t)std::min<uint64_t>(e, (uint64_t)(tile_cursor + take) * kTile);
+            uint32_t* last = out_rows > worker_cu_out[worker] ? kv_splits_out + 3 * (out_rows - 1) : nullptr;
+            if (last != nullptr && last[0] == kv_splits_in[3 * r] && last[2] == piece_begin) {
+                last[2] = piece_end;  // same worker, same token, adjacent keys: one row, one partial state
+            } else {
+                PSI_REQUIRE(out_rows < rows_capacity, "balanced plan exceeds the row capacity");
+                kv_splits_out[3 * out_rows] = kv_splits_in[3 * r];
+                kv_splits_out[3 * out_rows + 1] = piece_begin;
+                kv_splits_out[3 * out_rows + 2] = piece_end;
+                ++out_rows;
+            }
             tile_cursor += (uint32_t)take;
             remaining -= take;
             linear += take;

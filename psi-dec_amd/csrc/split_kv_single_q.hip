@@ -273,11 +273,14 @@ extern "C" int psi_hip_split_kv_single_q_store_partials(psi_hip_ctx* ctx, const 
 extern "C" int psi_hip_kv_page_write_split_kv_single_q_map(
     psi_hip_ctx* ctx, const psi_hip_gqa_config* cfg, const psi_hip_page_table_layout* layout, const void* q,
     void* kv_pages, uint64_t kv_pages_bytes, const void* flat_k, const void* flat_v, const uint32_t* req_slots,
-    const uint32_t* flat_token_indices, const uint32_t* page_ids, const uint32_t* kv_splits, void* scratch,
-    uint64_t scratch_bytes, uint32_t gqa_layer_index, uint32_t num_total_tokens, uint32_t num_total_kv_splits,
-    uint32_t num_active_tokens, uint32_t num_active_kv_splits) {
+    const uint32_t* flat_token_indices, const uint32_t* page_ids, const uint32_t* kv_splits,
+    const uint32_t* worker_cu, uint32_t num_workers, void* scratch, uint64_t scratch_bytes, uint32_t gqa_layer_index,
+    uint32_t num_total_tokens, uint32_t num_total_kv_splits, uint32_t num_active_tokens,
+    uint32_t num_active_kv_splits) {
     PSI_REQUIRE(flat_k && flat_v && flat_token_indices, "GQA KV page write buffers must not be null");
-    return single_q_map_impl(ctx, cfg, layout, q, kv_pages, kv_pages_bytes, req_slots, page_ids, kv_splits, nullptr, 0,
-                             scratch, scratch_bytes, gqa_layer_index, num_total_tokens, num_total_kv_splits,
-                             num_active_tokens, num_active_kv_splits, flat_k, flat_v, flat_token_indices);
+    PSI_REQUIRE((worker_cu == nullptr) == (num_workers == 0), "a worker table needs its worker count and vice versa");
+    return single_q_map_impl(ctx, cfg, layout, q, kv_pages, kv_pages_bytes, req_slots, page_ids, kv_splits, worker_cu,
+                             num_workers, scratch, scratch_bytes, gqa_layer_index, num_total_tokens,
+                             num_total_kv_splits, num_active_tokens, num_active_kv_splits, flat_k, flat_v,
+                             flat_token_indices);
 }

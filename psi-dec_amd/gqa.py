@@ -496,7 +496,7 @@ class GQAReplayBucketPolicy:
 
 
 def balanced_workers(config: "GQASplitKVConfig") -> int:
-    """Decode-map workers per KV head that fill the device exactly once."""
+    """Decode-map workers per KV head: one workgroup per compute unit over all KV heads."""
     out, cfg = ctypes.c_uint32(), config.struct()
     L.check(L.load().psi_hip_split_kv_balanced_workers(ctypes.byref(cfg), ctypes.byref(out)))
     return out.value
@@ -647,7 +647,8 @@ class GQAMetadataBuffers:
 
     def balance(self, num_workers: int):
         """Re-cuts the current SingleQ plan into rows grouped for `num_workers` equal-work decode
-        workgroups per KV head (psi_hip_split_kv_balance_plan); returns the new replay shape."""
+        workgroups per KV head (psi_hip_split_kv_balance_plan); adjacent pieces of one token inside a group
+        become one row.  Returns the new replay shape."""
         s = self._shape
         assert s is not None and not self._variant.is_tiled()
         rows_in = s.num_sdpa_map_task_templates
@@ -810,7 +811,7 @@ class GQASplitKVSingleQKernels:
 
     def invoke_append_map_bucketed(self, q, kv_pages, flat_k, flat_v, req_slots, flat_token_indices, page_ids,
                                    sdpa_map_task_templates, scratch, page_table_index: int, num_active_tokens: int,
-                                   num_active_kv_splits: int):
+                                   num_active_kv_splits: int, worker_cu=None, num_workers: int = 0):
         """`GQAKVPageWrite.invoke_bucketed` and `invoke_map_bucketed` in one launch: the workgroup whose split row
         ends at a token's position writes the token's K/V lines, and the step's new positions are read from
         `flat_k` / `flat_v`.  Same arena as the two calls bit for bit; partial states equal up to summation order."""
@@ -818,9 +819,9 @@ class GQASplitKVSingleQKernels:
         L.check(self.device.lib.psi_hip_kv_page_write_split_kv_single_q_map(
             self.device.ctx, ctypes.byref(cfg), ctypes.byref(layout), _ptr(q), _ptr(kv_pages), _nbytes(kv_pages),
             _ptr(flat_k), _ptr(flat_v), _ptr(req_slots), _ptr(flat_token_indices), _ptr(page_ids),
-            _ptr(sdpa_map_task_templates), _ptr(scratch.buffer), scratch.bytes, page_table_index,
-            self.shape.num_total_tokens, self.shape.num_total_sdpa_map_task_templates, num_active_tokens,
-            num_active_kv_splits))
+            _ptr(sdpa_map_task_templates), _ptr(worker_cu), num_workers, _ptr(scratch.buffer), scratch.bytes,
+            page_table_index, self.shape.num_total_tokens, self.shape.num_total_sdpa_map_task_templates,
+            num_active_tokens, num_active_kv_splits))
 
     def invoke_map_balanced(self, q, kv_pages, req_slots, page_ids, sdpa_map_task_templates, worker_cu,
                             num_workers: int, scratch, page_table_index: int, num_active_tokens: int,

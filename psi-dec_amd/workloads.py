@@ -221,7 +221,7 @@ class DeviceWorkload:
             self.scratch = G.GQASplitKVSingleQScratch(device, self.cfg, self.kshape)
         self._rows = rows
         # decode only: the append rides in the map launch (one launch fewer per step)
-        self.fused_append = bool(fused_append) and not variant.is_tiled() and not self.balanced
+        self.fused_append = bool(fused_append) and not variant.is_tiled()
         self.grouped = bool(grouped) and variant.is_tiled()
         if self.grouped:
             self.meta.group_rows(self.cfg)
@@ -275,7 +275,9 @@ class DeviceWorkload:
         m, s = self.meta, self.shape
         self.kernels.invoke_append_map_bucketed(self.q, self.pages, self.flat_k, self.flat_v, m.d_req_slots,
                                                 m.d_flat_token_indices, self.page_ids, m.d_kv_splits, self.scratch,
-                                                self.w.layer, s.num_tokens, s.num_sdpa_map_task_templates)
+                                                self.w.layer, s.num_tokens, s.num_sdpa_map_task_templates,
+                                                worker_cu=m.d_worker_cu if self.balanced else None,
+                                                num_workers=m.num_workers if self.balanced else 0)
 
     def step(self):
         """One layer-step: append the new tokens, then attend (the new tokens see themselves)."""

@@ -175,3 +175,35 @@ def test_append_folded_into_the_map_single_token_context(psi, oracle, device):
     wl = importlib_workloads(psi)
     w = wl.make_workload(43, [1, 1, 2, 16, 17], 24, 4, 256, psi.Dtype.Bfloat16, 16)
     run_and_check(psi, oracle, device, w, "append in map, one-token contexts", partition_tokens=512, fused_append=True)
+
+
+@pytest.mark.parametrize("dtype_name,hq,hkv,d,p,q_lens,fused_append", [
+    ("Bfloat16", 24, 4, 256, 16, 1, False),
+    ("Bfloat16", 24, 4, 256, 16, 1, True),                      # the default decode step of the bench
+    ("Float16", 16, 2, 256, 16, 1, True),
+    ("Bfloat16", 32, 8, 128, 8, 1, True),                       # 8-token pages
+    ("Bfloat16", 24, 4, 256, 16, [3, 1, 2, 1, 4, 1, 2], True),  # several new tokens per request
+    ("Float32", 6, 2, 64, 8, 1, True),                          # generic kernels: row per workgroup, two launches
+])
+def test_balanced_plan_with_merged_rows(psi, oracle, device, dtype_name, hq, hkv, d, p, q_lens, fused_append):
+    """One workgroup per compute unit over equal shares of the tiles, a token's adjacent pieces inside a share
+    merged into one row; with and without the append folded into the launch.  Contexts from one token to several
+    shares long."""
+    wl = importlib_workloads(psi)
+    dtype = getattr(psi.Dtype, dtype_name)
+    ctx = [30000, 17, 1025, 9000, 700, 1, 513]
+    if not np.isscalar(q_lens):
+        ctx = [max(c, q) for c, q in zip(ctx, q_lens)]
+    w = wl.make_workload(47, ctx, hq, hkv, d, dtype, p, q_lens=q_lens)
+    variant = psi.GQASplitKVVariant.SingleQ(256, 256, min(hq // hkv, 8))
+    what = f"balanced {dtype_name} {hq}/{hkv}/{d} P={p} q={q_lens} fused={fused_append}"
+    stats, dw = run_and_check(psi, oracle, device, w, what, partition_tokens=512, variant=variant, balanced=True,
+                              fused_append=fused_append, max_tokens=64)
+    assert dw.balanced and dw.fused_append == fused_append
+    m = dw.meta
+    n = dw.shape.num_sdpa_map_task_templates
+    assert n <= m.num_workers + w.num_tokens
+    plain = wl.DeviceWorkload(device, w, partition_tokens=512, variant=variant, f32_output=True, max_tokens=64)
+    plain.step()
+    assert np.abs(plain.output_f32() - dw.output_f32()).max() < 2e-5
+    assert np.array_equal(plain.pages_host(), dw.pages_host())

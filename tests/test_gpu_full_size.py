@@ -12,10 +12,10 @@ from parity_util import assert_outputs_close, importlib_workloads, layout_tuple,
 pytestmark = pytest.mark.gpu
 
 
-def _full_c2(psi, device, partition, f32_output=True, seed=2):
+def _full_c2(psi, device, partition, f32_output=True, seed=2, **how):
     wl = importlib_workloads(psi)
     w = wl.config_c2(seed=seed, batch=32, host_pages=False)
-    return wl, w, wl.DeviceWorkload(device, w, partition_tokens=partition, f32_output=f32_output)
+    return wl, w, wl.DeviceWorkload(device, w, partition_tokens=partition, f32_output=f32_output, **how)
 
 
 def test_c2_full_batch_split_count_invariance(psi, device):
@@ -55,11 +55,20 @@ def test_c2_full_batch_page_placement_invariance(psi, device):
     assert torch.equal(dw.output.view(torch.int16), base.view(torch.int16))
 
 
-def test_c2_full_batch_sampled_against_oracle(psi, oracle, device):
+@pytest.mark.parametrize("how", [{}, {"balanced": True, "fused_append": True}], ids=["row per workgroup", "bench default"])
+def test_c2_full_batch_sampled_against_oracle(psi, oracle, device, how):
     """Three of the 32 requests (shortest, median, longest context) recomputed by the scalar oracle
-    from the device's own pages."""
-    wl, w, dw = _full_c2(psi, device, 512)
+    from the device's own pages.  `bench default`: the balanced worker plan with the append folded into the
+    map launch, as `bench.py` runs the step."""
+    wl, w, dw = _full_c2(psi, device, 512, **how)
     dw.step()
+    if how:
+        plain = _full_c2(psi, device, 512)[2]
+        plain.step()
+        assert np.abs(plain.output_f32() - dw.output_f32()).max() < 2e-5
+        assert np.array_equal(plain.pages_host(), dw.pages_host())
+        assert dw.shape.num_sdpa_map_task_templates <= dw.meta.num_workers + 32
+        del plain
     got = dw.output_f32().reshape(32, w.num_q_heads * w.head_dim)
     pages = dw.pages_host()
     order = np.argsort(w.context_lens)

@@ -439,6 +439,31 @@ def test_balance_plan_covers_the_same_ranges(psi):
         assert (part[:, 0] == row).all()
     w = md.h_worker_cu
     assert w[0] == 0 and w[-1] == s.num_sdpa_map_task_templates and (np.diff(w.astype(np.int64)) >= 0).all()
+    # equal shares of the 16-token tiles, and inside a worker one row per token: at most workers + tokens rows
+    tiles = (-(-ks[:, 2].astype(np.int64) // 16)) - ks[:, 1].astype(np.int64) // 16
+    per_worker = [int(tiles[w[i]:w[i + 1]].sum()) for i in range(24)]
+    assert max(per_worker) - min(per_worker) <= 1 and sum(per_worker) == sum(-(-c // 16) for c in ctx)
+    assert s.num_sdpa_map_task_templates <= 24 + len(ctx)
+    for i in range(24):
+        tokens = ks[w[i]:w[i + 1], 0].tolist()
+        assert len(set(tokens)) == len(tokens), "adjacent pieces of a token inside a worker must be one row"
+
+
+def test_balance_plan_with_more_workers_than_tiles(psi):
+    """Tiny batches: workers without work get empty row ranges, nothing is lost."""
+    md = psi.GQAMetadataBuffers(None, 4, max_kv_splits=16)
+    single = psi.GQASplitKVVariant.SingleQ(256, 256, 6)
+    ctx = [40, 1, 17]
+    md.update_fixed_partition(list(range(3)), [c - 1 for c in ctx], list(range(4)), single, 512)
+    s = md.balance(64)
+    ks = md.h_kv_splits[:3 * s.num_sdpa_map_task_templates].reshape(-1, 3)
+    cu = md.h_cu_kv_splits[:4]
+    for row, c in enumerate(ctx):
+        part = ks[cu[row]:cu[row + 1]]
+        assert part[0, 1] == 0 and part[-1, 2] == c and (part[1:, 1] == part[:-1, 2]).all()
+    w = md.h_worker_cu.astype(np.int64)
+    assert w[0] == 0 and w[-1] == s.num_sdpa_map_task_templates and (np.diff(w) >= 0).all()
+    assert (np.diff(w) == 0).sum() >= 64 - 6  # 6 tiles in all
 
 
 def test_longest_first_order(psi):
