@@ -533,45 +533,72 @@ extern "C" int psi_hip_split_kv_balance_plan(const uint32_t* kv_splits_in, uint3
         PSI_REQUIRE(kv_splits_in[3 * r] < num_tokens, "balanced plan input must not hold padding rows");
         total += tiles_of(r);
     }
+    // A worker's cost is its tiles plus kRowStartTiles per row it starts (split record -> slot -> page ID ->
+    // first keys, and the partial state written at the end: about 3.4 us against 0.62 us per tile on MI355X).
+    // Workers are filled in order up to a common budget; the budget is the smallest one that leaves the last
+    // worker no more than the others.
+    constexpr uint64_t kRowStartTiles = 5;
+    struct Piece {
+        uint32_t token, begin, end, worker;
+    };
+    std::vector<Piece> pieces;
+    auto fill = [&](uint64_t budget) -> uint64_t {  // returns the cost that lands on the last worker
+        pieces.clear();
+        uint32_t w = 0;
+        uint64_t used = 0;
+        bool open_row = false;  // the worker's last piece can still be extended (same token, adjacent keys)
+        for (uint32_t r = 0; r < num_rows_in; ++r) {
+            const uint32_t b = kv_splits_in[3 * r + 1], e = kv_splits_in[3 * r + 2];
+            uint64_t remaining = tiles_of(r);
+            uint32_t tile_cursor = b / kTile;
+            if (remaining == 0) {  // degenerate row: keep it so that row counts per token stay positive
+                pieces.push_back({kv_splits_in[3 * r], b, e, w});
+                open_row = false;
+                continue;
+            }
+            while (remaining > 0) {
+                const bool extends = open_row && !pieces.empty() && pieces.back().worker == w &&
+                                     pieces.back().token == kv_splits_in[3 * r] &&
+                                     pieces.back().end == std::max<uint32_t>(b, tile_cursor * kTile);
+                const uint64_t start_cost = extends ? 0 : kRowStartTiles;
+                if (w + 1 < num_workers && used + start_cost >= budget) {  // no room for even one tile: next worker
+                    ++w;
+                    used = 0;
+                    open_row = false;
+                    continue;
+                }
+                const uint64_t room = w + 1 < num_workers ? budget - used - start_cost : remaining;
+                const uint64_t take = std::min<uint64_t>(remaining, std::max<uint64_t>(room, 1));
+                const uint32_t piece_begin = std::max<uint32_t>(b, tile_cursor * kTile);
+                const uint32_t piece_end = (uint32_t)std::min<uint64_t>(e, (uint64_t)(tile_cursor + take) * kTile);
+                if (extends)
+                    pieces.back().end = piece_end;  // same worker, same token, adjacent keys: one row, one partial state
+                else
+                    pieces.push_back({kv_splits_in[3 * r], piece_begin, piece_end, w});
+                open_row = true;
+                tile_cursor += (uint32_t)take;
+                remaining -= take;
+                used += start_cost + take;
+            }
+        }
+        return w + 1 == num_workers ? used : 0;
+    };
+    uint64_t budget = std::max<uint64_t>((total + kRowStartTiles * ((uint64_t)num_tokens + num_workers)) / num_workers,
+                                        kRowStartTiles + 1);  // room for at least one tile
+    while (fill(budget) > budget) budget += std::max<uint64_t>(budget / 64, 1);
+
     uint32_t out_rows = 0, worker = 0;
-    uint64_t linear = 0;  // tiles emitted so far
-    auto worker_end = [&](uint32_t w) { return total * (w + 1) / num_workers; };
     worker_cu_out[0] = 0;
     uint32_t token = 0;
     cu_out[0] = 0;
-    for (uint32_t r = 0; r < num_rows_in; ++r) {
-        while (token < num_tokens && r >= cu_in[token + 1]) cu_out[++token] = out_rows;
-        const uint32_t b = kv_splits_in[3 * r + 1], e = kv_splits_in[3 * r + 2];
-        uint64_t remaining = tiles_of(r);
-        uint32_t tile_cursor = b / kTile;
-        if (remaining == 0) {  // degenerate row: keep it so that row counts per token stay positive
-            PSI_REQUIRE(out_rows < rows_capacity, "balanced plan exceeds the row capacity");
-            kv_splits_out[3 * out_rows] = kv_splits_in[3 * r];
-            kv_splits_out[3 * out_rows + 1] = b;
-            kv_splits_out[3 * out_rows + 2] = e;
-            ++out_rows;
-            continue;
-        }
-        while (remaining > 0) {
-            while (worker + 1 < num_workers && linear >= worker_end(worker)) worker_cu_out[++worker] = out_rows;
-            const uint64_t room = worker + 1 < num_workers ? worker_end(worker) - linear : remaining;
-            const uint64_t take = std::min<uint64_t>(remaining, std::max<uint64_t>(room, 1));
-            const uint32_t piece_begin = std::max<uint32_t>(b, tile_cursor * kTile);
-            const uint32_t piece_end = (uint32_t)std::min<uint64_t>(e, (uint64_t)(tile_cursor + take) * kTile);
-            uint32_t* last = out_rows > worker_cu_out[worker] ? kv_splits_out + 3 * (out_rows - 1) : nullptr;
-            if (last != nullptr && last[0] == kv_splits_in[3 * r] && last[2] == piece_begin) {
-                last[2] = piece_end;  // same worker, same token, adjacent keys: one row, one partial state
-            } else {
-                PSI_REQUIRE(out_rows < rows_capacity, "balanced plan exceeds the row capacity");
-                kv_splits_out[3 * out_rows] = kv_splits_in[3 * r];
-                kv_splits_out[3 * out_rows + 1] = piece_begin;
-                kv_splits_out[3 * out_rows + 2] = piece_end;
-                ++out_rows;
-            }
-            tile_cursor += (uint32_t)take;
-            remaining -= take;
-            linear += take;
-        }
+    PSI_REQUIRE(pieces.size() <= rows_capacity, "balanced plan exceeds the row capacity");
+    for (const Piece& piece : pieces) {
+        while (token < piece.token) cu_out[++token] = out_rows;
+        while (worker < piece.worker) worker_cu_out[++worker] = out_rows;
+        kv_splits_out[3 * out_rows] = piece.token;
+        kv_splits_out[3 * out_rows + 1] = piece.begin;
+        kv_splits_out[3 * out_rows + 2] = piece.end;
+        ++out_rows;
     }
     while (token < num_tokens) cu_out[++token] = out_rows;
     while (worker < num_workers) worker_cu_out[++worker] = out_rows;
