@@ -652,7 +652,7 @@ class GQAMetadataBuffers:
         s = self._shape
         assert s is not None and not self._variant.is_tiled()
         rows_in = s.num_sdpa_map_task_templates
-        cap = rows_in + num_workers
+        cap = max(rows_in + num_workers, self._max_kv_splits)  # the arrays are reused by the next update
         out_splits = np.full(cap * 3, L.SENTINEL, np.uint32)
         out_cu = np.zeros(self._max_tokens + 1, np.uint32)
         worker_cu = np.zeros(num_workers + 1, np.uint32)

@@ -65,18 +65,21 @@ def test_captured_layer_step_replays(psi, device, q_len, fused_append):
         _ = (dw.output.float() * 2).sum().item()
 
 
-def test_one_captured_step_serves_every_batch_of_its_bucket(psi, device):
+@pytest.mark.parametrize("balanced", [False, True])
+def test_one_captured_step_serves_every_batch_of_its_bucket(psi, device, balanced):
     """Device-side active counts (`ReplayU32::Parameter` of the reference): a decode step captured once at the
     capacity of its bucket (5 tokens, 16 splits) with the counts bound, then replayed for batches of 5, 3, 1 and
     4 requests after refreshing only the metadata arrays, the inputs and the 16-byte count block.  Each replay
     equals the eager step with by-value counts, bit for bit, in the output rows and in the page arena; rows
-    beyond the active count keep a canary."""
+    beyond the active count keep a canary.  `balanced`: the plan is re-cut into equal worker shares on the host
+    for every batch and the append rides in the map launch; the grid (workers x KV heads) is the same for all."""
     import torch
 
     wl = importlib_workloads(psi)
     ctx_lens = [700, 33, 1500, 512, 64]
     w = wl.make_workload(111, ctx_lens, 24, 4, 256, psi.Dtype.Bfloat16, 16)
-    cap_tokens, cap_splits = 5, 16
+    workers = 8
+    cap_tokens, cap_splits = 5, 16 + (workers if balanced else 0)
     dw = wl.DeviceWorkload(device, w, partition_tokens=512)  # owns pages, page table, q, flat_k, flat_v
     pristine = dw.pages.clone()
     variant = dw.variant
@@ -90,6 +93,7 @@ def test_one_captured_step_serves_every_batch_of_its_bucket(psi, device):
     d_slots, d_pos = torch.zeros(cap_tokens, **i32), torch.zeros(cap_tokens, **i32)
     d_splits, d_cu = torch.zeros(cap_splits * 3, **i32), torch.zeros(cap_tokens + 1, **i32)
     d_counts = torch.zeros(4, **i32)
+    d_workers = torch.zeros(workers + 1, **i32)
     q, fk, fv = torch.zeros_like(dw.q), torch.zeros_like(dw.flat_k), torch.zeros_like(dw.flat_v)
     out = torch.zeros(cap_tokens * row, dtype=torch.bfloat16, device=device.torch_device)
     host_meta = psi.GQAMetadataBuffers(None, cap_tokens, max_kv_splits=cap_splits)
@@ -98,9 +102,18 @@ def test_one_captured_step_serves_every_batch_of_its_bucket(psi, device):
         n = len(picks)
         shape = host_meta.update_fixed_partition(w.req_slots[picks], w.token_indices[picks], list(range(n + 1)), variant,
                                                  512)
-        for dst, src in ((d_slots, host_meta.h_req_slots), (d_pos, host_meta.h_flat_token_indices),
-                         (d_splits, host_meta.h_kv_splits), (d_cu, host_meta.h_cu_kv_splits)):
-            dst.copy_(device.from_numpy(src))
+        if balanced:
+            shape = host_meta.balance(workers)
+            d_workers.copy_(device.from_numpy(host_meta.h_worker_cu))
+            d_splits.fill_(-1)
+            d_splits[:len(host_meta.h_kv_splits)].copy_(device.from_numpy(host_meta.h_kv_splits))
+            d_slots.copy_(device.from_numpy(host_meta.h_req_slots))
+            d_pos.copy_(device.from_numpy(host_meta.h_flat_token_indices))
+            d_cu.copy_(device.from_numpy(host_meta.h_cu_kv_splits))
+        if not balanced:
+            for dst, src in ((d_slots, host_meta.h_req_slots), (d_pos, host_meta.h_flat_token_indices),
+                             (d_splits, host_meta.h_kv_splits), (d_cu, host_meta.h_cu_kv_splits)):
+                dst.copy_(device.from_numpy(src))
         for dst, src, width in ((q, dw.q, row), (fk, dw.flat_k, kv_row), (fv, dw.flat_v, kv_row)):
             dst.zero_()
             for i, r in enumerate(picks):
@@ -110,10 +123,15 @@ def test_one_captured_step_serves_every_batch_of_its_bucket(psi, device):
         return shape
 
     def step(active_tokens, active_splits):
-        bufs = psi.GQAKVPageWriteBuffers(dw.pages, fk, fv, d_slots, d_pos, dw.page_ids)
-        dw.write.invoke_bucketed(write_shape, bufs, active_tokens, w.layer)
-        kernels.invoke_map_bucketed(q, dw.pages, d_slots, dw.page_ids, d_splits, scratch, w.layer, active_tokens,
-                                    active_splits)
+        if balanced:
+            kernels.invoke_append_map_bucketed(q, dw.pages, fk, fv, d_slots, d_pos, dw.page_ids, d_splits, scratch,
+                                               w.layer, active_tokens, active_splits, worker_cu=d_workers,
+                                               num_workers=workers)
+        else:
+            bufs = psi.GQAKVPageWriteBuffers(dw.pages, fk, fv, d_slots, d_pos, dw.page_ids)
+            dw.write.invoke_bucketed(write_shape, bufs, active_tokens, w.layer)
+            kernels.invoke_map_bucketed(q, dw.pages, d_slots, dw.page_ids, d_splits, scratch, w.layer, active_tokens,
+                                        active_splits)
         kernels.invoke_reduce_bucketed(scratch, d_cu, out, active_tokens)
 
     # capture at capacity with the count block bound
