@@ -456,6 +456,19 @@ int psi_hip_split_kv_tiled_q_group_rows(const psi_hip_gqa_config* cfg, uint32_t 
                                         uint64_t row_groups_capacity, uint32_t* out_group_tiles,
                                         uint32_t* out_num_groups);
 
+/* The multi-query map launched over a balanced plan (psi_hip_split_kv_balance_plan on the TiledQ tables: its
+ * `num_tokens` is then the number of Q-token tiles and cu_in the per-tile cu_kv_splits): workgroup w of each KV head
+ * serves kv_splits rows [worker_cu[w], worker_cu[w + 1]).  Same results as psi_hip_split_kv_tiled_q_map up to the
+ * order of summation; shapes outside the gfx950 kernels run one workgroup per row. */
+int psi_hip_split_kv_tiled_q_map_balanced(
+    psi_hip_ctx* ctx, const psi_hip_gqa_config* cfg, const psi_hip_page_table_layout* layout,
+    uint32_t q_token_tile_size, const void* q, const void* kv_pages, uint64_t kv_pages_bytes,
+    const uint32_t* req_slots, const uint32_t* page_ids, const uint32_t* flat_token_indices,
+    const uint32_t* q_token_tiles, const uint32_t* kv_splits, const uint32_t* worker_cu, uint32_t num_workers,
+    void* scratch, uint64_t scratch_bytes, uint32_t gqa_layer_index, uint32_t num_total_tokens,
+    uint32_t num_total_q_token_tiles, uint32_t num_total_kv_splits, uint32_t num_active_tokens,
+    uint32_t num_active_q_token_tiles, uint32_t num_active_kv_splits, uint32_t max_active_q_tile_tokens);
+
 /* psi_hip_split_kv_tiled_q_map with one workgroup per (row group, KV head [, half of the Q heads]):
  * the group's K/V tiles are staged once in LDS for up to 128 query columns and both contractions run
  * on the matrix cores.  Same arguments, scratch layout and results (within rounding) as the plain map;

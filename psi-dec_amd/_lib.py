@@ -230,6 +230,12 @@ PROTOTYPES = {
          c_void_p, c_void_p, c_uint64, c_uint32, c_uint32, c_uint32, c_uint32, c_uint32, c_uint32, c_uint32,
          c_uint32],
     ),
+    "psi_hip_split_kv_tiled_q_map_balanced": (
+        c_int,
+        [c_void_p, _CFG, _LAYOUT, c_uint32, c_void_p, c_void_p, c_uint64, c_void_p, c_void_p, c_void_p, c_void_p,
+         c_void_p, c_void_p, c_uint32, c_void_p, c_uint64, c_uint32, c_uint32, c_uint32, c_uint32, c_uint32, c_uint32,
+         c_uint32, c_uint32],
+    ),
     "psi_hip_split_kv_tiled_q_map_grouped": (
         c_int,
         [c_void_p, _CFG, _LAYOUT, c_uint32, c_void_p, c_void_p, c_uint64, c_void_p, c_void_p, c_void_p, c_void_p,

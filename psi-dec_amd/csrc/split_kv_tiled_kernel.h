@@ -83,9 +83,13 @@ struct ProbOperand<F16Tag> {
 
 constexpr int kTiledTileWaves = 4;  // waves that share the KV tiles of a split among them
 
+// Two workgroups per SIMD for every shape.  Three would hold the one-column-block variant to 168 registers, which
+// it overflows into a private segment since it walks a range of rows (at a great loss, and the balanced launch
+// keeps one workgroup per compute unit anyway); one would let the wider variants move their accumulators into
+// AGPRs, which measures slower than their 0-48 bytes of private segment (verify q_len 4: 521 vs 455 us).
 template <int NB, int CG>
 struct TiledOccupancy {
-    static constexpr int value = CG == 2 ? 2 : (NB == 1 ? 3 : 2);
+    static constexpr int value = 2;
 };
 
 // NB: column blocks per wave (1 or 2); CG: column groups (1 or 2), each a set of four waves.
@@ -93,7 +97,8 @@ template <typename Tag, int D, int NB, int CG, bool kHalfPage>
 __global__ __launch_bounds__(64 * kTiledTileWaves * CG, (TiledOccupancy<NB, CG>::value)) void split_kv_tiled_map(
     MapArgs a, const uint32_t* __restrict__ page_ids, const uint32_t* __restrict__ kv_splits,
     const uint32_t* __restrict__ req_slots, const uint16_t* __restrict__ q, const uint16_t* __restrict__ pages,
-    const uint32_t* __restrict__ q_token_tiles, const uint32_t* __restrict__ flat_token_indices) {
+    const uint32_t* __restrict__ q_token_tiles, const uint32_t* __restrict__ flat_token_indices,
+    const uint32_t* __restrict__ worker_cu) {
     resolve_active(a);
     constexpr int kTileWaves = kTiledTileWaves;
     constexpr int kWaves = kTileWaves * CG;
@@ -121,25 +126,39 @@ __global__ __launch_bounds__(64 * kTiledTileWaves * CG, (TiledOccupancy<NB, CG>:
 
     const uint32_t G = a.group;
     const uint32_t kv_head = blockIdx.x % a.walk.hkv;
-    const uint32_t split = blockIdx.x / a.walk.hkv;
-    const uint32_t tid = threadIdx.x;
-    const uint32_t lane = tid & 63;
-    const uint32_t wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const uint32_t wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const uint32_t tile_wave = wave % kTileWaves;       // which KV tiles this wave takes
     const uint32_t col_base = (wave / kTileWaves) * NB;  // first column block of this wave
-    const uint32_t mt = lane & 15, mc = lane >> 4;
-    const uint32_t vsub = lane / kVLanesPerToken, vdl = lane % kVLanesPerToken;
 
-    if (split >= a.num_active_kv_splits) return;
+    // Rows of kv_splits this workgroup serves: one row (blockIdx / Hkv) in the plain launch, or the worker's row
+    // range when a balanced plan hands each workgroup an equal share of tiles.  Every skip below is uniform over
+    // the workgroup.
+    uint32_t row_begin = blockIdx.x / a.walk.hkv, row_end = row_begin + 1;
+    if (worker_cu != nullptr) {
+        row_begin = worker_cu[blockIdx.x / a.walk.hkv];
+        row_end = worker_cu[blockIdx.x / a.walk.hkv + 1];
+    }
+    bool lds_in_use = false;
+    for (uint32_t split = row_begin; split < row_end; ++split) {
+    if (split >= a.num_active_kv_splits) break;
     const uint32_t q_tile = kv_splits[split * 3];
-    if (q_tile >= a.num_active_q_token_tiles) return;  // sentinel padding
+    if (q_tile >= a.num_active_q_token_tiles) continue;  // sentinel padding
     const uint32_t kv_begin = kv_splits[split * 3 + 1];
     const uint32_t kv_end = kv_splits[split * 3 + 2];
     const uint32_t flat_begin = q_token_tiles[q_tile * 2], flat_end = q_token_tiles[q_tile * 2 + 1];
-    if (flat_begin >= a.num_active_tokens || flat_end > a.num_active_tokens || flat_end <= flat_begin) return;
+    if (flat_begin >= a.num_active_tokens || flat_end > a.num_active_tokens || flat_end <= flat_begin) continue;
     const uint32_t tile_tokens = flat_end - flat_begin;
     const uint32_t ncols = tile_tokens * G;
-    if (ncols > (uint32_t)kCols) return;  // the launcher sizes NB from the largest tile; never taken
+    if (ncols > (uint32_t)kCols) continue;  // the launcher sizes NB from the largest tile; never taken
+    if (lds_in_use) __syncthreads();  // the previous row's merge buffer has been read out
+    lds_in_use = true;
+    // Lane coordinates, re-derived per row from a value the optimiser cannot see through: nothing computed from
+    // them is loop-invariant, so no per-lane address survives from one row into the next row's register budget.
+    uint32_t tid = threadIdx.x;
+    asm volatile("" : "+v"(tid));
+    const uint32_t lane = tid & 63;
+    const uint32_t mt = lane & 15, mc = lane >> 4;
+    const uint32_t vsub = lane / kVLanesPerToken, vdl = lane % kVLanesPerToken;
     const uint32_t nb_total = (ncols + 15) / 16;
     // column blocks this wave works on: col_base + [0, nb_active)
     const uint32_t nb_active = nb_total > col_base ? min(nb_total - col_base, (uint32_t)NB) : 0u;
@@ -415,6 +434,7 @@ __global__ __launch_bounds__(64 * kTiledTileWaves * CG, (TiledOccupancy<NB, CG>:
         a.part_max[row] = col_max_lds[tid];
         a.part_sum[row] = col_sum_lds[tid];
     }
+    }  // rows of this workgroup
 }
 
 // Column blocks needed for tiles of up to `max_tile_tokens` query tokens and `group` heads per KV head.
@@ -423,7 +443,7 @@ inline int tiled_column_blocks(uint32_t max_tile_tokens, uint32_t group) { retur
 template <typename Tag, int D>
 inline int launch_tiled_map_typed(psi_hip_ctx* ctx, const Geometry& g, const MapArgs& a, uint32_t max_tile_tokens) {
     const int nb = tiled_column_blocks(max_tile_tokens, g.group);
-    const dim3 grid(a.num_total_kv_splits * g.hkv);
+    const dim3 grid((a.worker_cu ? a.num_workers : a.num_total_kv_splits) * g.hkv);
     const uint16_t* q = reinterpret_cast<const uint16_t*>(a.q);
     const uint16_t* pages = reinterpret_cast<const uint16_t*>(a.kv_pages);
 #define PSI_TILED_LAUNCH(NB, CG)                                                                                       \
@@ -431,11 +451,11 @@ inline int launch_tiled_map_typed(psi_hip_ctx* ctx, const Geometry& g, const Map
         if (g.tokens_per_page == 8)                                                                                    \
             hipLaunchKernelGGL((split_kv_tiled_map<Tag, D, NB, CG, true>), grid, dim3(64 * kTiledTileWaves * CG), 0,    \
                                ctx->stream, a, a.walk.page_ids, a.kv_splits, a.req_slots, q, pages, a.q_token_tiles,   \
-                               a.flat_token_indices);                                                                  \
+                               a.flat_token_indices, a.worker_cu);                                                     \
         else                                                                                                           \
             hipLaunchKernelGGL((split_kv_tiled_map<Tag, D, NB, CG, false>), grid, dim3(64 * kTiledTileWaves * CG), 0,   \
                                ctx->stream, a, a.walk.page_ids, a.kv_splits, a.req_slots, q, pages, a.q_token_tiles,   \
-                               a.flat_token_indices);                                                                  \
+                               a.flat_token_indices, a.worker_cu);                                                     \
     } while (0)
     if (nb == 1) PSI_TILED_LAUNCH(1, 1);
     else if (nb == 2) PSI_TILED_LAUNCH(2, 1);

@@ -49,7 +49,8 @@ static int tiled_q_map(psi_hip_ctx* ctx, const psi_hip_gqa_config* cfg, const ps
                        uint32_t gqa_layer_index, uint32_t num_total_tokens, uint32_t num_total_q_token_tiles,
                        uint32_t num_total_kv_splits, uint32_t num_active_tokens, uint32_t num_active_q_token_tiles,
                        uint32_t num_active_kv_splits, uint32_t max_active_q_tile_tokens, const uint32_t* row_groups,
-                       uint32_t group_tiles, uint32_t num_groups) {
+                       uint32_t group_tiles, uint32_t num_groups, const uint32_t* worker_cu = nullptr,
+                       uint32_t num_workers = 0) {
     PSI_REQUIRE(ctx != nullptr, "ctx must not be null");
     Geometry g;
     int rc = make_geometry(cfg, &g);
@@ -96,12 +97,16 @@ static int tiled_q_map(psi_hip_ctx* ctx, const psi_hip_gqa_config* cfg, const ps
     PSI_REQUIRE(max_active_q_tile_tokens <= q_token_tile_size,
                 "GQA SplitKV TiledQ largest active tile exceeds the Q-token tile size");
     a.max_q_tile_tokens = max_active_q_tile_tokens;
+    a.worker_cu = worker_cu;
+    a.num_workers = num_workers;
 
     LaunchScope scope(ctx, "tiled_q_map");
     rc = PSI_HIP_ERR_UNSUPPORTED;
     if (row_groups != nullptr && num_groups != 0) rc = launch_chunk_map(ctx, g, a, row_groups, group_tiles, num_groups);
     if (rc == PSI_HIP_ERR_UNSUPPORTED) rc = launch_tiled_map_fast(ctx, g, a);
     if (rc == PSI_HIP_ERR_UNSUPPORTED) {
+        a.worker_cu = nullptr;  // the generic kernel launches one workgroup per row
+        a.num_workers = 0;
         const uint64_t grid = (uint64_t)num_total_kv_splits * g.hq * q_token_tile_size * ((g.d + 63) / 64);
         PSI_REQUIRE(grid <= 0x7fffffffull, "GQA SplitKV TiledQ map grid exceeds the launch domain");
         launch_map_generic(ctx, g, a);
@@ -126,6 +131,22 @@ extern "C" int psi_hip_split_kv_tiled_q_map(psi_hip_ctx* ctx, const psi_hip_gqa_
                        flat_token_indices, q_token_tiles, kv_splits, scratch, scratch_bytes, gqa_layer_index,
                        num_total_tokens, num_total_q_token_tiles, num_total_kv_splits, num_active_tokens,
                        num_active_q_token_tiles, num_active_kv_splits, max_active_q_tile_tokens, nullptr, 0, 0);
+}
+
+extern "C" int psi_hip_split_kv_tiled_q_map_balanced(
+    psi_hip_ctx* ctx, const psi_hip_gqa_config* cfg, const psi_hip_page_table_layout* layout,
+    uint32_t q_token_tile_size, const void* q, const void* kv_pages, uint64_t kv_pages_bytes,
+    const uint32_t* req_slots, const uint32_t* page_ids, const uint32_t* flat_token_indices,
+    const uint32_t* q_token_tiles, const uint32_t* kv_splits, const uint32_t* worker_cu, uint32_t num_workers,
+    void* scratch, uint64_t scratch_bytes, uint32_t gqa_layer_index, uint32_t num_total_tokens,
+    uint32_t num_total_q_token_tiles, uint32_t num_total_kv_splits, uint32_t num_active_tokens,
+    uint32_t num_active_q_token_tiles, uint32_t num_active_kv_splits, uint32_t max_active_q_tile_tokens) {
+    PSI_REQUIRE(worker_cu != nullptr && num_workers > 0, "balanced map needs a worker table");
+    return tiled_q_map(ctx, cfg, layout, q_token_tile_size, q, kv_pages, kv_pages_bytes, req_slots, page_ids,
+                       flat_token_indices, q_token_tiles, kv_splits, scratch, scratch_bytes, gqa_layer_index,
+                       num_total_tokens, num_total_q_token_tiles, num_total_kv_splits, num_active_tokens,
+                       num_active_q_token_tiles, num_active_kv_splits, max_active_q_tile_tokens, nullptr, 0, 0,
+                       worker_cu, num_workers);
 }
 
 extern "C" int psi_hip_split_kv_tiled_q_map_grouped(

@@ -650,7 +650,8 @@ class GQAMetadataBuffers:
         workgroups per KV head (psi_hip_split_kv_balance_plan); adjacent pieces of one token inside a group
         become one row.  Returns the new replay shape."""
         s = self._shape
-        assert s is not None and not self._variant.is_tiled()
+        assert s is not None
+        groups = s.num_q_token_tiles if self._variant.is_tiled() else s.num_tokens  # what cu_kv_splits counts
         rows_in = s.num_sdpa_map_task_templates
         cap = max(rows_in + num_workers, self._max_kv_splits)  # the arrays are reused by the next update
         out_splits = np.full(cap * 3, L.SENTINEL, np.uint32)
@@ -662,7 +663,7 @@ class GQAMetadataBuffers:
             return a.ctypes.data_as(ctypes.POINTER(ctypes.c_uint32))
 
         L.check(L.load().psi_hip_split_kv_balance_plan(p(self.h_kv_splits), rows_in, p(self.h_cu_kv_splits),
-                                                       s.num_tokens, num_workers, p(out_splits), cap, p(out_cu),
+                                                       groups, num_workers, p(out_splits), cap, p(out_cu),
                                                        p(worker_cu), ctypes.byref(n_out)))
         self.h_kv_splits, self.h_cu_kv_splits, self.h_worker_cu = out_splits, out_cu, worker_cu
         self.num_workers = num_workers
@@ -927,6 +928,20 @@ class GQASplitKVTiledQKernels:
             _ptr(q_token_tiles), _ptr(sdpa_map_task_templates), _ptr(scratch.buffer), scratch.bytes,
             page_table_index, s.num_total_tokens, s.num_total_q_token_tiles, s.num_total_sdpa_map_task_templates,
             num_active_tokens, num_active_q_token_tiles, num_active_kv_splits, max_active_q_tile_tokens))
+
+    def invoke_map_balanced(self, q, kv_pages, req_slots, page_ids, flat_token_indices, q_token_tiles,
+                            sdpa_map_task_templates, worker_cu, num_workers: int, scratch, page_table_index: int,
+                            num_active_tokens: int, num_active_q_token_tiles: int, num_active_kv_splits: int,
+                            max_active_q_tile_tokens: int = 0):
+        """The map over a balanced plan: one workgroup per (worker, KV head) walks its row range."""
+        cfg, layout, s = self.config.struct(), self.config.page_table_layout.struct(), self.shape
+        L.check(self.device.lib.psi_hip_split_kv_tiled_q_map_balanced(
+            self.device.ctx, ctypes.byref(cfg), ctypes.byref(layout), self.config.q_token_tile_size, _ptr(q),
+            _ptr(kv_pages), _nbytes(kv_pages), _ptr(req_slots), _ptr(page_ids), _ptr(flat_token_indices),
+            _ptr(q_token_tiles), _ptr(sdpa_map_task_templates), _ptr(worker_cu), num_workers, _ptr(scratch.buffer),
+            scratch.bytes, page_table_index, s.num_total_tokens, s.num_total_q_token_tiles,
+            s.num_total_sdpa_map_task_templates, num_active_tokens, num_active_q_token_tiles, num_active_kv_splits,
+            max_active_q_tile_tokens))
 
     def invoke_map_grouped(self, q, kv_pages, req_slots, page_ids, flat_token_indices, q_token_tiles,
                            sdpa_map_task_templates, scratch, page_table_index: int, num_active_tokens: int,

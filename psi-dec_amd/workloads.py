@@ -191,7 +191,7 @@ class DeviceWorkload:
             self.shape = self.meta.update(w.req_slots, w.token_indices, w.cu_tokens, variant)
         if longest_first and not balanced:
             self.meta.order_longest_first()
-        self.balanced = balanced and not variant.is_tiled()
+        self.balanced = bool(balanced) and not grouped  # the prefill-chunk map has its own row grouping
         if self.balanced:
             workers = G.balanced_workers(G.GQASplitKVConfig(w.dtype, w.page_bytes, w.num_q_heads, w.num_kv_heads,
                                                             w.head_dim))
@@ -244,6 +244,13 @@ class DeviceWorkload:
                                             m.num_row_groups,
                                             min(int(np.diff(self.w.cu_tokens).max()),
                                                 self.variant.q_token_tile_size))
+        elif self.variant.is_tiled() and self.balanced:
+            self.kernels.invoke_map_balanced(self.q, self.pages, m.d_req_slots, self.page_ids,
+                                             m.d_flat_token_indices, m.d_q_token_tiles, m.d_kv_splits, m.d_worker_cu,
+                                             m.num_workers, self.scratch, self.w.layer, s.num_tokens,
+                                             s.num_q_token_tiles, s.num_sdpa_map_task_templates,
+                                             min(int(np.diff(self.w.cu_tokens).max()),
+                                                 self.variant.q_token_tile_size))
         elif self.variant.is_tiled():
             self.kernels.invoke_map_bucketed(self.q, self.pages, m.d_req_slots, self.page_ids,
                                              m.d_flat_token_indices, m.d_q_token_tiles, m.d_kv_splits, self.scratch,

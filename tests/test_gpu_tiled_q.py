@@ -277,3 +277,30 @@ def test_grouped_and_plain_maps_agree(psi, oracle, device):
         assert diff < 1e-3, diff
         if not expect_groups:
             assert diff == 0.0
+
+
+@pytest.mark.parametrize("dtype_name,hq,hkv,d,p,q_lens", [
+    ("Bfloat16", 24, 4, 256, 16, 2),                        # one-draft verify: one column block
+    ("Bfloat16", 24, 4, 256, 16, 4),                        # three drafts: two column blocks
+    ("Bfloat16", 24, 4, 256, 16, [8, 3, 1, 8, 5, 2, 7]),    # full tiles: four column blocks on eight waves
+    ("Float16", 16, 2, 256, 8, 3),                          # 8-token pages
+    ("Bfloat16", 32, 8, 128, 16, [20, 1, 9, 2, 1, 1, 12]),  # several Q-token tiles per request
+    ("Float32", 6, 2, 64, 8, 2),                            # generic kernels: one workgroup per row
+])
+def test_balanced_plan_for_multi_query_rows(psi, oracle, device, dtype_name, hq, hkv, d, p, q_lens):
+    """The multi-query map over equal worker shares (one workgroup per compute unit), a tile's adjacent pieces
+    inside a share merged into one row: outputs within tolerance of the oracle and, up to the order of
+    summation, equal to the row-per-workgroup launch; pages bit-exact."""
+    wl = importlib_workloads(psi)
+    dtype = getattr(psi.Dtype, dtype_name)
+    ctx = [30000, 40, 1025, 9000, 700, 33, 513]
+    w = wl.make_workload(53, ctx, hq, hkv, d, dtype, p, q_lens=q_lens)
+    variant = psi.GQASplitKVVariant.TiledQ(8, 16 if p >= 8 else 4, min(hq // hkv, 8))
+    what = f"balanced tiled {dtype_name} {hq}/{hkv}/{d} P={p} q={q_lens}"
+    stats, dw = run_and_check(psi, oracle, device, w, what, partition_tokens=512, variant=variant, balanced=True,
+                              max_tokens=64)
+    assert dw.balanced and dw.shape.num_sdpa_map_task_templates <= dw.meta.num_workers + dw.shape.num_q_token_tiles
+    plain = wl.DeviceWorkload(device, w, partition_tokens=512, variant=variant, f32_output=True, max_tokens=64)
+    plain.step()
+    # f16 probabilities are one 11-bit term: their rounding depends on where the rows are cut
+    assert np.abs(plain.output_f32() - dw.output_f32()).max() < (2e-4 if dtype_name == "Float16" else 2e-5)
