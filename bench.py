@@ -48,6 +48,8 @@ def parse_args():
                    help="dispatch the split rows in plan order instead of longest first")
     p.add_argument("--separate-append", action="store_true",
                    help="decode workload: launch the append as its own kernel instead of folding it into the map")
+    p.add_argument("--workers", type=int, default=0,
+                   help="balanced plan: workers per KV head (0 = one workgroup per compute unit over all KV heads)")
     p.add_argument("--row-per-workgroup", action="store_true",
                    help="decode workload: one workgroup per partition row instead of the balanced worker plan")
     p.add_argument("--kernel-only", action="store_true", help="time only the map kernel (for profiling runs)")
@@ -199,7 +201,7 @@ def main():
         arenas.append(wl.DeviceWorkload(device, w, partition_tokens=args.partition, balanced=not args.row_per_workgroup,
                                         longest_first=not args.plan_order,
                                         grouped=prefill and not args.no_row_groups,
-                                        fused_append=not args.separate_append))
+                                        fused_append=not args.separate_append, num_workers=args.workers or None))
     w = arenas[0].w
     shape = arenas[0].shape
     step_bytes = w.algorithmic_bytes()

@@ -146,7 +146,7 @@ class DeviceWorkload:
     def __init__(self, device: G.Device, w: Workload, partition_tokens: Optional[int] = None,
                  max_tokens: Optional[int] = None, variant: Optional[G.GQASplitKVVariant] = None,
                  f32_output: bool = False, balanced: bool = False, longest_first: bool = False,
-                 grouped: bool = False, fused_append: bool = False):
+                 grouped: bool = False, fused_append: bool = False, num_workers: Optional[int] = None):
         import torch
 
         self.device, self.w = device, w
@@ -193,8 +193,8 @@ class DeviceWorkload:
             self.meta.order_longest_first()
         self.balanced = bool(balanced) and not grouped  # the prefill-chunk map has its own row grouping
         if self.balanced:
-            workers = G.balanced_workers(G.GQASplitKVConfig(w.dtype, w.page_bytes, w.num_q_heads, w.num_kv_heads,
-                                                            w.head_dim))
+            workers = num_workers or G.balanced_workers(G.GQASplitKVConfig(w.dtype, w.page_bytes, w.num_q_heads,
+                                                                           w.num_kv_heads, w.head_dim))
             self.shape = self.meta.balance(workers)
         s = self.shape
         self.write = G.GQAKVPageWrite(device, G.GQAKVPageWriteConfig(w.num_kv_heads, w.head_dim, w.page_bytes,
