@@ -199,8 +199,8 @@ int psi_hip_split_kv_order_longest_first(uint32_t* kv_splits, uint32_t num_kv_sp
 
 /* Balanced decode plan (no counterpart in the reference, whose planner budgets partial states, not
  * device occupancy).  Re-cuts the rows of an existing SingleQ plan at 16-token tile boundaries into
- * `num_workers` consecutive groups that hold equal numbers of tiles; a decode-map workgroup then serves one
- * group per KV head and all workgroups finish together.  Inside a group, adjacent pieces of one token
+ * `num_workers` consecutive groups of equal cost (tiles, plus five tiles' worth for every row started); a map
+ * workgroup then serves one group per KV head and all workgroups finish together.  Inside a group, adjacent pieces of one token
  * are one row -- one pass through the keys, one partial state -- whatever the partition of the input plan,
  * so the output has at most num_workers + num_tokens rows (fewer row starts and partial states than a
  * workgroup per input row: the launch streams faster and the combine reads less).
@@ -211,7 +211,8 @@ int psi_hip_split_kv_balance_plan(const uint32_t* kv_splits_in, uint32_t num_row
                                   uint32_t num_tokens, uint32_t num_workers, uint32_t* kv_splits_out,
                                   uint32_t rows_capacity, uint32_t* cu_out, uint32_t* worker_cu_out,
                                   uint32_t* out_num_rows);
-/* Workers per KV head that fill the device exactly once with decode-map workgroups. */
+/* Workers per KV head for the balanced plan: 256 / num_kv_heads, i.e. one map workgroup per compute unit over
+ * all KV heads (more workgroups mean more rows and partial states for the same bytes and measure slower). */
 int psi_hip_split_kv_balanced_workers(const psi_hip_gqa_config* cfg, uint32_t* out_num_workers);
 
 /* ------------------------------------------------------------------ projections around the attention
