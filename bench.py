@@ -207,14 +207,14 @@ def main():
     step_bytes = w.algorithmic_bytes()
     map_bytes = w.map_algorithmic_bytes()
 
-    def run_steps(n):
-        for i in range(n):
+    def run_steps(n, first=0):
+        for i in range(first, first + n):
             arenas[i % len(arenas)].step()
 
     run_steps_direct = run_steps
 
-    def run_maps(n):
-        for i in range(n):
+    def run_maps(n, first=0):
+        for i in range(first, first + n):
             arenas[i % len(arenas)].map()
 
     # Optional: one HIP graph per arena holds the step's three launches (append, map, combine).
@@ -238,8 +238,8 @@ def main():
             device.use_stream(main_stream)
         torch.cuda.synchronize()
 
-        def run_steps(n):  # noqa: F811
-            for i in range(n):
+        def run_steps(n, first=0):  # noqa: F811
+            for i in range(first, first + n):
                 graphs[i % len(graphs)].replay()
 
     body = run_maps if args.kernel_only else run_steps
@@ -250,6 +250,21 @@ def main():
     torch.cuda.synchronize()
     elapsed = time.perf_counter() - t0
     ms_per_step = elapsed * 1e3 / args.steps
+
+    # Spread of the step time: an event on the launch stream after every step of a further run, differences between
+    # neighbours (the queue stays full, so a difference is one step's device time plus its share of launch gaps).
+    n_spread = min(args.steps, 100)
+    body(4)
+    ticks = [torch.cuda.Event(enable_timing=True) for _ in range(n_spread + 1)]
+    ticks[0].record(device.stream)
+    for i in range(n_spread):
+        body(1, first=i)
+        ticks[i + 1].record(device.stream)
+    ticks[-1].synchronize()
+    step_us = sorted(ticks[i].elapsed_time(ticks[i + 1]) * 1e3 for i in range(n_spread))
+
+    def percentile(fraction):
+        return step_us[min(len(step_us) - 1, int(fraction * len(step_us)))]
 
     # Dominant kernel, timed by HIP events on the launch stream around every map launch.
     device.set_timing(True)
@@ -302,6 +317,7 @@ def main():
         "warmup": args.warmup,
         "ms_per_step": ms_per_step,
         "us_per_layer_step": ms_per_step * 1e3,
+        "us_per_layer_step_p10_median_p90": [percentile(0.1), percentile(0.5), percentile(0.9)],
         "hbm_frac_of_peak": (map_bytes if args.kernel_only else step_bytes) / (ms_per_step / 1e3) / 1e9 / HBM_PEAK_GBPS,
         "higher_is_better": True,
         "scaling": "weak",
