@@ -241,7 +241,13 @@ __global__ __launch_bounds__(64 * kTiledTileWaves * CG, (TiledOccupancy<NB, CG>:
             else
                 v_lane = head_base(p.a) + v_region +
                          (((tile * kTileTokens) & page_mask) + j * kVTokensPerLoad + vsub) * D + vdl * 8;
-            vreg[j] = stream_load_b128(v_lane);  // V rows are whole lines read once; K keeps ordinary loads (two loads share each line)
+            // V rows are whole lines that one column group reads once: non-temporal.  With two column groups the
+            // second group is meant to find the line in cache, so the loads stay ordinary.  K keeps ordinary loads
+            // either way (two loads share each line).
+            if (CG == 1)
+                vreg[j] = stream_load_b128(v_lane);
+            else
+                vreg[j] = *reinterpret_cast<const uint4*>(v_lane);
         }
     };
 
@@ -355,22 +361,51 @@ __global__ __launch_bounds__(64 * kTiledTileWaves * CG, (TiledOccupancy<NB, CG>:
     };
 
     uint32_t tile = tile_begin + tile_wave;
-    if (tile < tile_end && nb_active != 0) {
-        {
+    auto is_partial = [&](uint32_t t) { return t * kTileTokens < kv_begin || (t + 1) * kTileTokens > kv_end; };
+    if constexpr (CG == 1) {
+        if (tile < tile_end && nb_active != 0) {
+            {
+                const TilePages pid = load_page_id(tile);
+                issue_k(tile, pid);
+                issue_v(tile, pid);
+            }
+            TilePages pid_next = load_page_id(tile + kTileWaves);
+            while (tile + kTileWaves < tile_end) {
+                const uint32_t next = tile + kTileWaves;
+                const TilePages pid_after = load_page_id(next + kTileWaves);
+                process_tile(tile, is_partial(tile), std::true_type(), next, pid_next);
+                pid_next = pid_after;
+                tile = next;
+            }
+            process_tile(tile, is_partial(tile), std::false_type(), 0u, TilePages{0u, 0u});
+        }
+    } else {
+        // The column groups walk the tiles in step, a barrier per round of four tiles: wave w of every group then
+        // asks for the same K and V lines within a tile's time of each other, and all but the first find them in
+        // cache.  Left to themselves the groups drift apart and each fetches the tile from HBM again.  The round
+        // count is the same for every wave of the workgroup; a wave without a tile (or without columns) in a round
+        // only joins the barrier.
+        const uint32_t rounds = tile_end > tile_begin ? (tile_end - tile_begin + kTileWaves - 1) / kTileWaves : 0u;
+        const bool walks = tile < tile_end && nb_active != 0;
+        TilePages pid_next{0u, 0u};
+        if (walks) {
             const TilePages pid = load_page_id(tile);
             issue_k(tile, pid);
             issue_v(tile, pid);
+            pid_next = load_page_id(tile + kTileWaves);
         }
-        TilePages pid_next = load_page_id(tile + kTileWaves);
-        auto is_partial = [&](uint32_t t) { return t * kTileTokens < kv_begin || (t + 1) * kTileTokens > kv_end; };
-        while (tile + kTileWaves < tile_end) {
-            const uint32_t next = tile + kTileWaves;
-            const TilePages pid_after = load_page_id(next + kTileWaves);
-            process_tile(tile, is_partial(tile), std::true_type(), next, pid_next);
-            pid_next = pid_after;
-            tile = next;
+        for (uint32_t round = 0; round < rounds; ++round) {
+            __builtin_amdgcn_s_barrier();
+            if (walks && tile < tile_end) {
+                // past the last tile the page IDs read as 0 and the look-ahead loads fetch a tile of page 0 that
+                // nobody uses: one code path for every round
+                const uint32_t next = tile + kTileWaves;
+                const TilePages pid_after = load_page_id(next + kTileWaves);
+                process_tile(tile, is_partial(tile), std::true_type(), next, pid_next);
+                pid_next = pid_after;
+                tile = next;
+            }
         }
-        process_tile(tile, is_partial(tile), std::false_type(), 0u, TilePages{0u, 0u});
     }
 
     // ---- merge the four wave states of each column group.  Column statistics live in the S layout
