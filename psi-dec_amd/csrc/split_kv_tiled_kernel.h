@@ -241,13 +241,7 @@ __global__ __launch_bounds__(64 * kTiledTileWaves * CG, (TiledOccupancy<NB, CG>:
             else
                 v_lane = head_base(p.a) + v_region +
                          (((tile * kTileTokens) & page_mask) + j * kVTokensPerLoad + vsub) * D + vdl * 8;
-            // V rows are whole lines that one column group reads once: non-temporal.  With two column groups the
-            // second group is meant to find the line in cache, so the loads stay ordinary.  K keeps ordinary loads
-            // either way (two loads share each line).
-            if (CG == 1)
-                vreg[j] = stream_load_b128(v_lane);
-            else
-                vreg[j] = *reinterpret_cast<const uint4*>(v_lane);
+            vreg[j] = stream_load_b128(v_lane);  // V rows are whole lines read once; K keeps ordinary loads (two loads share each line)
         }
     };
 
@@ -273,60 +267,74 @@ __global__ __launch_bounds__(64 * kTiledTileWaves * CG, (TiledOccupancy<NB, CG>:
         if (has_next) issue_k(next, next_pid);
         __builtin_amdgcn_sched_barrier(0);
 
-        // ---- online softmax per column over this lane's tokens 4*mc + r
         ProbOperand<Tag> pa[NB];
         float alpha[NB];
         bool moved = false;
+        auto softmax = [&]() __attribute__((always_inline)) {
+            // ---- online softmax per column over this lane's tokens 4*mc + r
 #pragma unroll
-        for (int nb = 0; nb < NB; ++nb) {
-            alpha[nb] = 1.0f;
-            if ((uint32_t)nb < nb_active) {
-                float v[4];
-                bool valid[4];
-                float m = -INFINITY;
+            for (int nb = 0; nb < NB; ++nb) {
+                alpha[nb] = 1.0f;
+                if ((uint32_t)nb < nb_active) {
+                    float v[4];
+                    bool valid[4];
+                    float m = -INFINITY;
 #pragma unroll
-                for (int r = 0; r < 4; ++r) {
-                    const uint32_t token = tile * kTileTokens + mc * 4 + r;
-                    valid[r] = token >= kv_begin && token < lim[nb];
-                    v[r] = valid[r] ? s[nb][r] * a.scale_log2 : -INFINITY;
-                    m = fmaxf(m, v[r]);
+                    for (int r = 0; r < 4; ++r) {
+                        const uint32_t token = tile * kTileTokens + mc * 4 + r;
+                        valid[r] = token >= kv_begin && token < lim[nb];
+                        v[r] = valid[r] ? s[nb][r] * a.scale_log2 : -INFINITY;
+                        m = fmaxf(m, v[r]);
+                    }
+                    m = fmaxf(m, __shfl_xor(m, 16, 64));
+                    m = fmaxf(m, __shfl_xor(m, 32, 64));
+                    const float next_max = fmaxf(run_max[nb], m);
+                    // a column with no visible key so far keeps max = -inf, sum = 0, O = 0
+                    alpha[nb] = run_max[nb] > -INFINITY ? __builtin_amdgcn_exp2f(run_max[nb] - next_max) : 0.0f;
+                    moved = moved || next_max != run_max[nb];
+                    run_max[nb] = next_max;
+                    float p[4], tile_sum = 0.0f;
+#pragma unroll
+                    for (int r = 0; r < 4; ++r) {
+                        p[r] = valid[r] ? __builtin_amdgcn_exp2f(v[r] - next_max) : 0.0f;
+                        tile_sum += p[r];
+                    }
+                    lane_sum[nb] = lane_sum[nb] * alpha[nb] + tile_sum;
+                    pa[nb].set(p);
                 }
-                m = fmaxf(m, __shfl_xor(m, 16, 64));
-                m = fmaxf(m, __shfl_xor(m, 32, 64));
-                const float next_max = fmaxf(run_max[nb], m);
-                // a column with no visible key so far keeps max = -inf, sum = 0, O = 0
-                alpha[nb] = run_max[nb] > -INFINITY ? __builtin_amdgcn_exp2f(run_max[nb] - next_max) : 0.0f;
-                moved = moved || next_max != run_max[nb];
-                run_max[nb] = next_max;
-                float p[4], tile_sum = 0.0f;
-#pragma unroll
-                for (int r = 0; r < 4; ++r) {
-                    p[r] = valid[r] ? __builtin_amdgcn_exp2f(v[r] - next_max) : 0.0f;
-                    tile_sum += p[r];
-                }
-                lane_sum[nb] = lane_sum[nb] * alpha[nb] + tile_sum;
-                pa[nb].set(p);
             }
+        };
+        auto stage_v = [&]() __attribute__((always_inline)) {
+            // ---- V tile: registers -> this wave's LDS buffer (rows outside the split zeroed: their
+            // probability is 0 but their bytes may be NaN/Inf), then refill the registers for the next tile
+            wave_lds_fence();  // the previous tile's reads of the buffer are complete
+#pragma unroll
+            for (int j = 0; j < kVLoads; ++j) {
+                const uint32_t tok_in_tile = j * kVTokensPerLoad + vsub;
+                uint4 val = vreg[j];
+                if (partial) {
+                    const uint32_t vtoken = tile * kTileTokens + tok_in_tile;
+                    if (vtoken < kv_begin || vtoken >= kv_end) val = make_uint4(0, 0, 0, 0);
+                }
+                *reinterpret_cast<uint4*>(my_v + tok_in_tile * kVStride + vdl * 8) = val;
+            }
+            __builtin_amdgcn_sched_barrier(0);
+            if (has_next) issue_v(next, next_pid);
+            __builtin_amdgcn_sched_barrier(0);
+        };
+        // One column group: V goes to LDS, and the next tile's V loads go out, before the softmax - a tile's period is
+        // the memory latency plus the time from the tile's start to the issue of the next tile's last load (verify
+        // with 3 / 4 query tokens: 437 / 442 -> 420 / 431 us).  Two column groups, two waves per SIMD, measure faster
+        // the other way round (8 tokens: 721 against 747 us).
+        if constexpr (CG == 1) {
+            stage_v();
+            softmax();
+        } else {
+            softmax();
+            stage_v();
         }
         const bool rescale = __any(moved);
-
-        // ---- V tile: registers -> this wave's LDS buffer (rows outside the split zeroed: their
-        // probability is 0 but their bytes may be NaN/Inf), then refill the registers for the next tile
-        wave_lds_fence();  // the previous tile's reads of the buffer are complete
-#pragma unroll
-        for (int j = 0; j < kVLoads; ++j) {
-            const uint32_t tok_in_tile = j * kVTokensPerLoad + vsub;
-            uint4 val = vreg[j];
-            if (partial) {
-                const uint32_t vtoken = tile * kTileTokens + tok_in_tile;
-                if (vtoken < kv_begin || vtoken >= kv_end) val = make_uint4(0, 0, 0, 0);
-            }
-            *reinterpret_cast<uint4*>(my_v + tok_in_tile * kVStride + vdl * 8) = val;
-        }
-        __builtin_amdgcn_sched_barrier(0);
-        if (has_next) issue_v(next, next_pid);
-        __builtin_amdgcn_sched_barrier(0);
-        wave_lds_fence();
+        wave_lds_fence();  // the V tile is in LDS
 
         // ---- O[column][dim] = alpha * O + P^T V
         if (rescale) {
@@ -361,51 +369,22 @@ __global__ __launch_bounds__(64 * kTiledTileWaves * CG, (TiledOccupancy<NB, CG>:
     };
 
     uint32_t tile = tile_begin + tile_wave;
-    auto is_partial = [&](uint32_t t) { return t * kTileTokens < kv_begin || (t + 1) * kTileTokens > kv_end; };
-    if constexpr (CG == 1) {
-        if (tile < tile_end && nb_active != 0) {
-            {
-                const TilePages pid = load_page_id(tile);
-                issue_k(tile, pid);
-                issue_v(tile, pid);
-            }
-            TilePages pid_next = load_page_id(tile + kTileWaves);
-            while (tile + kTileWaves < tile_end) {
-                const uint32_t next = tile + kTileWaves;
-                const TilePages pid_after = load_page_id(next + kTileWaves);
-                process_tile(tile, is_partial(tile), std::true_type(), next, pid_next);
-                pid_next = pid_after;
-                tile = next;
-            }
-            process_tile(tile, is_partial(tile), std::false_type(), 0u, TilePages{0u, 0u});
-        }
-    } else {
-        // The column groups walk the tiles in step, a barrier per round of four tiles: wave w of every group then
-        // asks for the same K and V lines within a tile's time of each other, and all but the first find them in
-        // cache.  Left to themselves the groups drift apart and each fetches the tile from HBM again.  The round
-        // count is the same for every wave of the workgroup; a wave without a tile (or without columns) in a round
-        // only joins the barrier.
-        const uint32_t rounds = tile_end > tile_begin ? (tile_end - tile_begin + kTileWaves - 1) / kTileWaves : 0u;
-        const bool walks = tile < tile_end && nb_active != 0;
-        TilePages pid_next{0u, 0u};
-        if (walks) {
+    if (tile < tile_end && nb_active != 0) {
+        {
             const TilePages pid = load_page_id(tile);
             issue_k(tile, pid);
             issue_v(tile, pid);
-            pid_next = load_page_id(tile + kTileWaves);
         }
-        for (uint32_t round = 0; round < rounds; ++round) {
-            __builtin_amdgcn_s_barrier();
-            if (walks && tile < tile_end) {
-                // past the last tile the page IDs read as 0 and the look-ahead loads fetch a tile of page 0 that
-                // nobody uses: one code path for every round
-                const uint32_t next = tile + kTileWaves;
-                const TilePages pid_after = load_page_id(next + kTileWaves);
-                process_tile(tile, is_partial(tile), std::true_type(), next, pid_next);
-                pid_next = pid_after;
-                tile = next;
-            }
+        TilePages pid_next = load_page_id(tile + kTileWaves);
+        auto is_partial = [&](uint32_t t) { return t * kTileTokens < kv_begin || (t + 1) * kTileTokens > kv_end; };
+        while (tile + kTileWaves < tile_end) {
+            const uint32_t next = tile + kTileWaves;
+            const TilePages pid_after = load_page_id(next + kTileWaves);
+            process_tile(tile, is_partial(tile), std::true_type(), next, pid_next);
+            pid_next = pid_after;
+            tile = next;
         }
+        process_tile(tile, is_partial(tile), std::false_type(), 0u, TilePages{0u, 0u});
     }
 
     // ---- merge the four wave states of each column group.  Column statistics live in the S layout
