@@ -81,6 +81,7 @@ struct ProbOperand<F16Tag> {
     }
 };
 
+constexpr float kMaxSlack = 8.0f;   // see the softmax of split_kv_tiled_map
 constexpr int kTiledTileWaves = 4;  // waves that share the KV tiles of a split among them
 
 // Two workgroups per SIMD for every shape.  Three would hold the one-column-block variant to 168 registers, which
@@ -288,7 +289,10 @@ __global__ __launch_bounds__(64 * kTiledTileWaves * CG, (TiledOccupancy<NB, CG>:
                     }
                     m = fmaxf(m, __shfl_xor(m, 16, 64));
                     m = fmaxf(m, __shfl_xor(m, 32, 64));
-                    const float next_max = fmaxf(run_max[nb], m);
+                    // The reference maximum of a column moves only when a tile exceeds it by more than kMaxSlack
+                    // (log2 domain), a few times per range: probabilities stay below 2^kMaxSlack, and the rescaling
+                    // of the accumulators, which every move of any of the wave's columns triggers, becomes rare.
+                    const float next_max = m > run_max[nb] + kMaxSlack ? m : run_max[nb];
                     // a column with no visible key so far keeps max = -inf, sum = 0, O = 0
                     alpha[nb] = run_max[nb] > -INFINITY ? __builtin_amdgcn_exp2f(run_max[nb] - next_max) : 0.0f;
                     moved = moved || next_max != run_max[nb];
