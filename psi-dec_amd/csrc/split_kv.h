@@ -6,7 +6,9 @@
 namespace psi {
 
 // Partial state of one (kv_split, q_head [, q_token_in_tile]) row, private to this library:
-//   max2 : running maximum of the logits in the log2 domain (logit * scale * log2(e)), -inf if empty
+//   max2 : reference value of the row's logits in the log2 domain (logit * scale * log2(e)), -inf if empty: their
+//          maximum, or (multi-query and chunk maps) a value at most 8 below it - the combine only needs sum and acc
+//          to be relative to the same value
 //   sum  : sum of exp2(logit2 - max2) over the split's keys
 //   acc  : un-normalised sum of exp2(logit2 - max2) * V, f32 [head_dim]
 // Arrays are laid out [row][...] with row = (split * num_q_heads + q_head) * rows_per_split_head + r.
