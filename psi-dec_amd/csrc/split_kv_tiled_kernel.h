@@ -87,7 +87,8 @@ constexpr int kTiledTileWaves = 4;  // waves that share the KV tiles of a split 
 // Two workgroups per SIMD for every shape.  Three would hold the one-column-block variant to 168 registers, which
 // it overflows into a private segment since it walks a range of rows (at a great loss, and the balanced launch
 // keeps one workgroup per compute unit anyway); one would let the wider variants move their accumulators into
-// AGPRs, which measures slower than their 0-48 bytes of private segment (verify q_len 4: 521 vs 455 us).
+// AGPRs, which measured slower (verify q_len 4: 521 vs 455 us).  At two workgroups per SIMD only the two-group
+// variants at head_dim 256 keep a private segment (40-44 bytes, outside the tile loop).
 template <int NB, int CG>
 struct TiledOccupancy {
     static constexpr int value = 2;
