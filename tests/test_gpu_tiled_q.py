@@ -54,6 +54,24 @@ def test_tiled_geometries(psi, oracle, device, dtype_name, hq, hkv, d, p, q_len)
                   variant=variant)
 
 
+@pytest.mark.parametrize("scale", [1.0, 0.25, 1.0 / 256.0])
+@pytest.mark.parametrize("dtype_name", ["Bfloat16", "Float16"])
+def test_sharp_and_flat_softmax(psi, oracle, device, scale, dtype_name):
+    """Logits from very peaked (scale 1: log2-domain spread of tens of units, a new maximum every few
+    tiles) to almost flat (1/256).  The maps move a column's reference maximum only when a tile
+    exceeds it by more than 2^8 and carry probabilities up to that size as 2-byte matrix operands;
+    the outputs must stay inside the tolerance either way - through the multi-query map (short
+    tiles) and through the chunk map (a 150-token chunk in row groups)."""
+    wl = importlib_workloads(psi)
+    dtype = getattr(psi.Dtype, dtype_name)
+    w = wl.make_workload(81, [700, 333, 64, 1200], 24, 4, 256, dtype, 16, q_lens=[3, 4, 2, 1], scale=scale)
+    run_and_check(psi, oracle, device, w, f"verify scale {scale} {dtype_name}", max_tokens=64)
+    w = wl.make_workload(82, [650, 40], 24, 4, 256, dtype, 16, q_lens=[150, 2], scale=scale)
+    stats, dw = run_and_check(psi, oracle, device, w, f"chunk scale {scale} {dtype_name}", partition_tokens=256,
+                              max_tokens=512, grouped=True)
+    assert dw.grouped
+
+
 def test_sentinel_split_rows_are_skipped(psi, oracle, device):
     """The split list is padded to its capacity with 0xFFFFFFFF rows; they must not touch anything:
     the scratch behind the active rows keeps its fill pattern."""
