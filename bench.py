@@ -39,6 +39,7 @@ def parse_args():
     p.add_argument("--arenas", type=int, default=2, help="independent page arenas rotated between steps")
     p.add_argument("--q-heads", type=int, default=24, help="decode workload: query heads (24; 16 for the long-context shape)")
     p.add_argument("--kv-heads", type=int, default=4, help="decode workload: KV heads (4; 2 for the long-context shape)")
+    p.add_argument("--dtype", choices=["bf16", "f16"], default="bf16", help="K/V/Q element type (f16 for the 1 x 512 shape)")
     p.add_argument("--seed", type=int, default=2)
     p.add_argument("--cpu-seconds", type=float, default=12.0, help="budget of the CPU baseline sample")
     p.add_argument("--no-cpu-baseline", action="store_true")
@@ -186,16 +187,17 @@ def main():
     if verify and args.batch == 32 and args.ctx_lo == 1024 and args.ctx_hi == 8192:
         args.batch, args.ctx_lo, args.ctx_hi = 64, 2048, 16384
     map_kernel = "tiled_q_map" if verify else "split_kv_map"
+    elem = psi.Dtype.Bfloat16 if args.dtype == "bf16" else psi.Dtype.Float16
     arenas = []
     for i in range(max(1, args.arenas)):
         if verify:
             ctx = ([args.prefix + args.chunk] if prefill else
                    wl.config_c2_context_lens(args.seed, args.batch, args.ctx_lo, args.ctx_hi) + args.q_len)
-            w = wl.make_workload(args.seed, ctx, 24, 4, 256, psi.Dtype.Bfloat16, 16, q_lens=args.q_len,
+            w = wl.make_workload(args.seed, ctx, 24, 4, 256, elem, 16, q_lens=args.q_len,
                                  host_pages=False, shuffle_pages=not args.identity_pages)
         else:
             ctx = wl.config_c2_context_lens(args.seed, args.batch, args.ctx_lo, args.ctx_hi) + 1
-            w = wl.make_workload(args.seed, ctx, args.q_heads, args.kv_heads, 256, psi.Dtype.Bfloat16, 16,
+            w = wl.make_workload(args.seed, ctx, args.q_heads, args.kv_heads, 256, elem, 16,
                                  host_pages=False, shuffle_pages=not args.identity_pages)
         w.seed = args.seed + 1000 * i  # same geometry, different page contents
         arenas.append(wl.DeviceWorkload(device, w, partition_tokens=args.partition, balanced=not args.row_per_workgroup,
@@ -307,7 +309,7 @@ def main():
     achieved = map_bytes / map_avg_s / 1e9
 
     workload_key = (f"{'verify_q%d' % args.q_len if verify else 'decode'}_b{args.batch}_ctx{args.ctx_lo}-{args.ctx_hi}"
-                    f"_{w.num_q_heads}q{w.num_kv_heads}kv_d256_bf16_p16_part{args.partition}_seed{args.seed}")
+                    f"_{w.num_q_heads}q{w.num_kv_heads}kv_d256_{args.dtype}_p16_part{args.partition}_seed{args.seed}")
     result = {
         "metric": "decode attn achieved HBM GB/s per layer-step (B=32, ctx 1k-8k); us/layer-step alongside",
         "value": (map_bytes if args.kernel_only else step_bytes) / (ms_per_step / 1e3) / 1e9,
@@ -322,7 +324,7 @@ def main():
         "higher_is_better": True,
         "scaling": "weak",
         "vs_baseline": None,
-        "dtype": "bf16",
+        "dtype": args.dtype,
         "data": "synthetic",
         "config": {
             "workload": workload_key,
@@ -359,7 +361,7 @@ def main():
         # multi-query chunk: priced against the matrix cores as well (4 * Hq * D flops per visible (query, key) pair)
         pairs = sum(args.prefix + i + 1 for i in range(args.chunk))
         flops = 4 * w.num_q_heads * w.head_dim * pairs
-        result["config"]["workload"] = f"prefill_chunk{args.chunk}_on_prefix{args.prefix}_24q4kv_d256_bf16_p16_part{args.partition}"
+        result["config"]["workload"] = f"prefill_chunk{args.chunk}_on_prefix{args.prefix}_24q4kv_d256_{args.dtype}_p16_part{args.partition}"
         result["config"]["row_groups"] = arenas[0].meta.num_row_groups
         result["mfma"] = {"bound": "mfma", "flops_per_launch": flops, "achieved": flops / map_avg_s / 1e12,
                           "peak": 2500.0, "unit": "TFLOP/s", "frac": flops / map_avg_s / 1e12 / 2500.0}
