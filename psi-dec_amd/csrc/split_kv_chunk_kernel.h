@@ -39,9 +39,13 @@
 //        operand read (16 rows, one chunk) then hit 16 different bank groups, and a row-wise store
 //        stays a permutation of its row.
 //   V^T  [D dims][32 keys] elements: 64-byte rows, 64 bytes of padding after every 8 rows, the 16-byte
-//        slot of keys 8s .. 8s+7 at position s XOR (row/4)%4.  Operand reads (16 consecutive rows, one
-//        slot) and transposing stores (4 rows 8 apart, all 16 key pairs) both cover 256 bytes of
-//        distinct banks.
+//        slot of keys 8s .. 8s+7 at position (s + 2 * (row/4)) % 4.  A 128-bit read is served in four
+//        rounds of 16 lanes, and the rounds are not the quarters of the wave: lanes 0-3, 12-15 and 20-27
+//        go together, then 4-11, 16-19 and 28-31, and the same in the upper half.  With this slot
+//        function the operand read (lane = row % 16 + 16 * slot) puts the 16 lanes of every round on 16
+//        different bank groups (480 bytes per ns and CU measured, the rate of the K reads; an XOR of the
+//        slot with (row/4)%4, conflict-free over plain quarters, measures 288).  Transposing stores (4 rows
+//        8 apart, all 16 key pairs) cover 256 bytes of distinct banks.
 //   page IDs of up to 4096 pages of the range, refilled for longer ranges.
 #pragma once
 #include "split_kv_tiled_kernel.h"
@@ -276,8 +280,8 @@ __global__ __launch_bounds__(64 * kChunkWaves, 2) void split_kv_chunk_map(
             const int word = e / 2;
             const uint32_t out = e % 2 == 0 ? ((w0[word] & 0xffffu) | (w1[word] << 16))
                                             : ((w0[word] >> 16) | (w1[word] & 0xffff0000u));
-            // row = 8 * v_chunk + e; its 16-byte slot v_pair / 4 is swizzled with (row / 4) % 4
-            const uint32_t slot = (v_pair >> 2) ^ ((2 * v_chunk + e / 4) & 3);
+            // row = 8 * v_chunk + e; its 16-byte slot v_pair / 4 is rotated by 2 * (row / 4): 2 * (e / 4) mod 4
+            const uint32_t slot = ((v_pair >> 2) + 2 * (e / 4)) & 3;
             *reinterpret_cast<uint32_t*>(vbuf + (8 * v_chunk + e) * 64 + v_chunk * 64 + slot * 16 + (v_pair & 3) * 4) = out;
         }
     };
@@ -287,7 +291,7 @@ __global__ __launch_bounds__(64 * kChunkWaves, 2) void split_kv_chunk_map(
     const uint32_t k_swz = mt;  // = key % 4 + 4 * (key / 8) for both key blocks
     const uint32_t k_row0 = (8 * (mt >> 2) + (mt & 3)) * (D * 2);
     // V^T row of (dim block db, lane row mt): dim 16 * db + mt, keys 8 * mc .. +7
-    const uint32_t vt_row0 = mt * 64 + (mt >> 3) * 64 + ((mc ^ ((mt >> 2) & 3)) * 16);
+    const uint32_t vt_row0 = mt * 64 + (mt >> 3) * 64 + (((mc + 2 * (mt >> 2)) & 3) * 16);
 
     float run_max = -INFINITY, lane_sum = 0.0f;
     f32x4_t o[kDimBlocks];
