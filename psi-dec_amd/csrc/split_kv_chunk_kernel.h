@@ -207,7 +207,9 @@ __global__ __launch_bounds__(64 * kChunkWaves, 2) void split_kv_chunk_map(
     uint32_t id_page0 = 0;  // page behind id_lds[0]
     auto refill_ids = [&](uint32_t first_tile) {
         id_page0 = (key_base0 + first_tile * kChunkKeys) >> log2p;
-        for (uint32_t i = tid; i < (uint32_t)kIdCap + 8; i += 64 * kChunkWaves) id_lds[i] = table_row[min(id_page0 + i, last_page)];
+        // only the pages the range still has: every later lookup is clamped to last_page
+        const uint32_t count = min((uint32_t)kIdCap + 8, last_page - id_page0 + 1);
+        for (uint32_t i = tid; i < count; i += 64 * kChunkWaves) id_lds[i] = table_row[id_page0 + i];
     };
     struct TileIds {
         uint32_t a, b;  // page of keys 0..15 and of keys 16..31 of a tile (the same value in every lane)
