@@ -309,8 +309,8 @@ __global__ __launch_bounds__(64 * kChunkWaves, 2) void split_kv_chunk_map(
         // ---- logits S[key][column]: two key blocks
         // The K operands are read kAhead k-steps before the products that take them, and the order is pinned: left
         // to itself the compiler keeps two operands in flight, and every product then waits out the LDS latency
-        // (452 -> 434 us on the 2048-on-4096 chunk).  The same treatment of the V^T operands measures slower than
-        // the compiler's own order (447 us; 453 us with the first reads issued ahead of the softmax).
+        // (450 -> 441 us on the 2048-on-4096 chunk, side by side).  The same treatment of the V^T operands measures
+        // slower than the compiler's own order (+3 %; +4 % with the first reads issued ahead of the softmax).
         f32x4_t s0 = f32x4_t{0.0f, 0.0f, 0.0f, 0.0f}, s1 = s0;
         constexpr int kAhead = 4;
         uint4 k0[kKSteps], k1[kKSteps];
