@@ -35,7 +35,7 @@ def parse_args():
     p.add_argument("--ctx-lo", type=int, default=1024)
     p.add_argument("--ctx-hi", type=int, default=8192)
     p.add_argument("--partition", type=int, default=None,
-                   help="split-KV partition length in tokens (default 512; 2048 for the prefill workload)")
+                   help="split-KV partition length in tokens (default 512; the whole context for the prefill workload)")
     p.add_argument("--arenas", type=int, default=2, help="independent page arenas rotated between steps")
     p.add_argument("--q-heads", type=int, default=24, help="decode workload: query heads (24; 16 for the long-context shape)")
     p.add_argument("--kv-heads", type=int, default=4, help="decode workload: KV heads (4; 2 for the long-context shape)")
@@ -181,7 +181,8 @@ def main():
     verify = args.workload in ("verify", "prefill")
     prefill = args.workload == "prefill"
     if args.partition is None:
-        args.partition = 2048 if prefill else 512
+        # prefill: one kv_split row per query tile (no split of the context) measures best for a single chunk
+        args.partition = max(2048, 1 << (args.prefix + args.chunk - 1).bit_length()) if prefill else 512
     if prefill:
         args.batch, args.q_len = 1, args.chunk
     if verify and args.batch == 32 and args.ctx_lo == 1024 and args.ctx_hi == 8192:
