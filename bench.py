@@ -44,7 +44,6 @@ def parse_args():
     p.add_argument("--cpu-seconds", type=float, default=12.0, help="budget of the CPU baseline sample")
     p.add_argument("--no-cpu-baseline", action="store_true")
     p.add_argument("--identity-pages", action="store_true", help="unshuffled page pool (diagnostic)")
-    p.add_argument("--decode-waves", type=int, default=0, help="waves per decode workgroup (0 = automatic)")
     p.add_argument("--plan-order", action="store_true",
                    help="dispatch the split rows in plan order instead of longest first")
     p.add_argument("--separate-append", action="store_true",
@@ -134,27 +133,40 @@ def cpu_baseline(psi, wl, w, dw, budget_s):
 
 
 def calibrate_copy(device, args):
-    """Copies (and separately just reads) a buffer of known size with the library's probe kernels.
-    Under `rocprofv3 --pmc FETCH_SIZE` / `WRITE_SIZE` the counter value of these launches against the
-    known byte count gives the scale factor applied to the attention kernels' counter readings."""
+    """Copies (and separately just reads) a buffer of known size with the probe kernels of
+    psi-dec_amd/lib/libpsi_hip_probe.so.  Under `rocprofv3 --pmc FETCH_SIZE` / `WRITE_SIZE` the counter value of
+    these launches against the known byte count gives the scale factor applied to the attention kernels'
+    counter readings."""
+    import ctypes
+
     import torch
 
+    probe = ctypes.CDLL(os.path.join(ROOT, "psi-dec_amd", "lib", "libpsi_hip_probe.so"))
+    probe.psi_probe_copy.restype = ctypes.c_int
+    probe.psi_probe_copy.argtypes = [ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p, ctypes.c_uint64, ctypes.c_int]
     nbytes = args.probe_mib << 20
     src = torch.empty(nbytes, dtype=torch.uint8, device="cuda").random_(0, 255)
     dst = torch.empty_like(src)
+    stream = ctypes.c_void_p(device.stream.cuda_stream)
     out = {"probe_bytes": nbytes, "launches": args.steps}
+
+    def launch(read_only):
+        rc = probe.psi_probe_copy(stream, dst.data_ptr(), src.data_ptr(), nbytes, int(read_only))
+        if rc != 0:
+            raise RuntimeError(f"psi_probe_copy failed: {rc}")
+
     for name, read_only in (("copy_probe", False), ("read_probe", True)):
         for _ in range(args.warmup):
-            device.copy_probe(dst, src, nbytes, read_only)
-        device.set_timing(True)
-        device.reset_timing()
+            launch(read_only)
+        start, stop = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        start.record(device.stream)
         for _ in range(args.steps):
-            device.copy_probe(dst, src, nbytes, read_only)
-        ms, n = device.kernel_time_ms(name)
-        device.set_timing(False)
+            launch(read_only)
+        stop.record(device.stream)
+        stop.synchronize()
+        us = start.elapsed_time(stop) * 1e3 / args.steps
         moved = nbytes if read_only else 2 * nbytes
-        out[name] = {"avg_launch_us": ms / n * 1e3, "bytes_moved_per_launch": moved,
-                     "GB/s": moved / (ms / n / 1e3) / 1e9}
+        out[name] = {"avg_launch_us": us, "bytes_moved_per_launch": moved, "GB/s": moved / (us / 1e6) / 1e9}
     print(json.dumps(out))
 
 
@@ -173,7 +185,6 @@ def main():
         print("bench.py needs a GPU", file=sys.stderr)
         sys.exit(1)
     device = psi.Device(0)
-    device.decode_waves(args.decode_waves)
     if args.calibrate_copy:
         calibrate_copy(device, args)
         return

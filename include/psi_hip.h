@@ -114,12 +114,6 @@ int psi_hip_ctx_reset_timing(psi_hip_ctx* ctx);
 /* F32_OUTPUT makes the combine kernels store the attention output as f32 [tokens, Hq, D] instead of
  * the io dtype, so a harness can check the f32-accumulated result before output rounding. */
 #define PSI_HIP_FLAG_F32_OUTPUT 2u
-/* DECODE_VALU_QK selects the decode map variant that computes QK^T with packed dot products on the
- * vector ALU instead of MFMA tiles (kept for counter comparisons; same results within tolerance). */
-#define PSI_HIP_FLAG_DECODE_VALU_QK 3u
-/* DECODE_WAVES fixes the number of waves per decode-map workgroup (1, 2 or 4); 0 restores the
- * automatic choice from the grid size. */
-#define PSI_HIP_FLAG_DECODE_WAVES 4u
 int psi_hip_ctx_set_flag(psi_hip_ctx* ctx, uint32_t flag, uint32_t value);
 
 /* Device-side active counts for captured launches: the counterpart of `ReplayU32::Parameter`
@@ -430,7 +424,9 @@ int psi_hip_split_kv_tiled_q_scratch_bytes(const psi_hip_gqa_config* cfg, uint32
  * kv_splits rows index q-token tiles.  Causal mask: key position > flat_token_indices[q] is hidden.
  * max_active_q_tile_tokens (no counterpart in the reference): the largest number of tokens any active
  * tile holds, e.g. 2 for a verify step with one draft; it sizes the kernel's query-column blocks.
- * 0 = unknown, any tile may hold q_token_tile_size tokens. */
+ * 0 = unknown, any tile may hold q_token_tile_size tokens.  It is a contract, not a hint: it must bound every
+ * batch the launch serves, including every batch later replayed on a graph captured from this call.  A row whose
+ * tile holds more tokens is entered as an empty partial state (its keys are not attended). */
 int psi_hip_split_kv_tiled_q_map(psi_hip_ctx* ctx, const psi_hip_gqa_config* cfg,
                                  const psi_hip_page_table_layout* layout, uint32_t q_token_tile_size,
                                  const void* q, const void* kv_pages, uint64_t kv_pages_bytes,
@@ -518,11 +514,6 @@ int psi_hip_page_table_start_index(const psi_hip_page_table_layout* layout, uint
  * num_gqa_layers * num_page_ids_per_block entries, out_by_layer the same count (layer-major). */
 int psi_hip_page_ids_by_layer(const uint32_t* block_ids, uint32_t block_ids_len, uint32_t num_gqa_layers,
                               uint32_t num_page_ids_per_block, uint32_t* out_by_layer);
-
-/* Measurement aid with no counterpart in the reference: a plain copy (read_only = 0: `bytes` read and
- * `bytes` written) or a pure read (read_only = 1) of known size, timed under the names "copy_probe" /
- * "read_probe".  HBM traffic counters are calibrated against it.  bytes must be a multiple of 16. */
-int psi_hip_copy_probe(psi_hip_ctx* ctx, void* dst, const void* src, uint64_t bytes, int read_only);
 
 /* ---------------------------------------------------------------------------------------------
  * Cache ownership on the host: page-ID allocator and the per-request token window.  No device work.

@@ -22,8 +22,6 @@ VARIANT_SINGLE_Q, VARIANT_TILED_Q = 0, 1
 CAPACITY_EXACT, CAPACITY_BUCKETED, CAPACITY_CALLER_TOKENS, CAPACITY_FIXED_PARTITION = 0, 1, 2, 3
 FLAG_FORCE_GENERIC = 1
 FLAG_F32_OUTPUT = 2
-FLAG_DECODE_VALU_QK = 3
-FLAG_DECODE_WAVES = 4
 
 
 class PsiHipError(RuntimeError):
@@ -254,7 +252,6 @@ PROTOTYPES = {
     "psi_hip_page_table_reset_req_slot": (c_int, [c_void_p, _LAYOUT, c_void_p, c_uint32]),
     "psi_hip_page_table_start_index": (c_int, [_LAYOUT, c_uint32, c_uint32, c_uint32, POINTER(c_uint64)]),
     "psi_hip_page_ids_by_layer": (c_int, [_U32P, c_uint32, c_uint32, c_uint32, _U32P]),
-    "psi_hip_copy_probe": (c_int, [c_void_p, c_void_p, c_void_p, c_uint64, c_int]),
     "psi_hip_id_allocator_create": (c_int, [c_uint64, POINTER(c_void_p)]),
     "psi_hip_id_allocator_destroy": (c_int, [c_void_p]),
     "psi_hip_id_allocator_alloc_one": (c_int, [c_void_p, _U32P]),

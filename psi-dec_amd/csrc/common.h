@@ -57,8 +57,6 @@ struct psi_hip_ctx {
     bool timing = false;
     bool force_generic = false;  // route every launch to the shape-generic kernels
     bool f32_output = false;     // combine kernels store f32 instead of the io dtype
-    bool decode_valu_qk = false; // decode map computes QK^T on the vector ALU instead of MFMA
-    int decode_waves_override = 0;  // 0 = choose waves per decode workgroup from the grid size
     // Device u32[4] = {active tokens, active Q-token tiles, active KV splits, reserved} read by every
     // kernel when it runs (graph replay); null: the counts passed by value apply.
     const uint32_t* replay_counts = nullptr;

@@ -140,12 +140,6 @@ int psi_hip_ctx_set_flag(psi_hip_ctx* ctx, uint32_t flag, uint32_t value) {
     switch (flag) {
         case PSI_HIP_FLAG_FORCE_GENERIC: ctx->force_generic = value != 0; break;
         case PSI_HIP_FLAG_F32_OUTPUT: ctx->f32_output = value != 0; break;
-        case PSI_HIP_FLAG_DECODE_VALU_QK: ctx->decode_valu_qk = value != 0; break;
-        case PSI_HIP_FLAG_DECODE_WAVES:
-            PSI_REQUIRE(value == 0 || value == 1 || value == 2 || value == 4,
-                        "decode waves per workgroup must be 0 (automatic), 1, 2 or 4");
-            ctx->decode_waves_override = (int)value;
-            break;
         default: return psi::fail(PSI_HIP_ERR_INVALID_ARGUMENT, "unknown context flag %u", flag);
     }
     return PSI_HIP_OK;

@@ -152,8 +152,6 @@ void fill_walk(PageWalk* walk, const Geometry& g, const psi_hip_page_table_layou
 int launch_decode_map_fast(psi_hip_ctx* ctx, const Geometry& g, const MapArgs& a);
 bool decode_map_takes_append(const psi_hip_ctx* ctx, const Geometry& g, const MapArgs& a);
 int launch_reduce_fast(psi_hip_ctx* ctx, const Geometry& g, const ReduceArgs& a);
-// The same decode map with the QK^T contraction on the vector ALU (comparison variant).
-int launch_decode_map_valu(psi_hip_ctx* ctx, const Geometry& g, const MapArgs& a);
 // MFMA TiledQ map for bf16 / f16, head_dim 256 / 128; PSI_HIP_ERR_UNSUPPORTED outside its domain.
 int launch_tiled_map_fast(psi_hip_ctx* ctx, const Geometry& g, const MapArgs& a);
 // MFMA prefill-chunk map over row groups; PSI_HIP_ERR_UNSUPPORTED outside chunk_map_supported().

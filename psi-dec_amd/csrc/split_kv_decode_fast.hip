@@ -74,6 +74,10 @@ __global__ __launch_bounds__(64 * kWideWaves) void split_kv_reduce_wide(ReduceAr
     const uint32_t lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const uint64_t row_out = blockIdx.x;
     const uint32_t token = (uint32_t)(row_out / a.hq), q_head = (uint32_t)(row_out % a.hq);
+    // The grid is cut for the by-value count; with device-side counts bound that is the bucket's capacity, and a
+    // workgroup beyond the active tokens must touch nothing (its cu_kv_splits entries are stale).  Uniform over
+    // the workgroup and ahead of the first barrier.
+    if (token >= a.num_active_tokens) return;
     const uint32_t begin = a.cu_kv_splits[token], end = a.cu_kv_splits[token + 1];
     const uint32_t* row_index = a.row_index;
     float global_max = -INFINITY;
@@ -188,7 +192,7 @@ __global__ __launch_bounds__(256) void split_kv_reduce_tiled_fast(ReduceArgs a) 
 
 // Shapes and pointers for which the MFMA decode map runs, i.e. for which the append can be folded into it.
 bool decode_map_takes_append(const psi_hip_ctx* ctx, const Geometry& g, const MapArgs& a) {
-    if (ctx->force_generic || ctx->decode_valu_qk) return false;
+    if (ctx->force_generic) return false;
     const bool two_byte = g.dtype == PSI_HIP_BF16 || g.dtype == PSI_HIP_F16;
     const uint32_t p = g.tokens_per_page;
     const bool page_ok = p >= 8 && (p & (p - 1)) == 0;
@@ -199,11 +203,6 @@ bool decode_map_takes_append(const psi_hip_ctx* ctx, const Geometry& g, const Ma
 
 int launch_decode_map_fast(psi_hip_ctx* ctx, const Geometry& g, const MapArgs& a) {
     if (ctx->force_generic) return PSI_HIP_ERR_UNSUPPORTED;
-    if (ctx->decode_valu_qk) {
-        // the comparison variant is row-per-workgroup and needs a tile inside one page
-        if (a.worker_cu != nullptr || g.tokens_per_page < 16) return PSI_HIP_ERR_UNSUPPORTED;
-        return launch_decode_map_valu(ctx, g, a);
-    }
     const bool two_byte = g.dtype == PSI_HIP_BF16 || g.dtype == PSI_HIP_F16;
     const uint32_t p = g.tokens_per_page;
     const bool page_ok = p >= 8 && (p & (p - 1)) == 0;

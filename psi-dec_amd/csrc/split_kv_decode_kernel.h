@@ -2,10 +2,10 @@
 // head_dim 128 or 256, pages of 8 or 16*2^k tokens.
 //
 // Work decomposition
-//   one workgroup (W = 1, 2 or 4 waves) = one (kv_split, kv_head); it serves all G query heads of
-//   that KV head.  One wave = every W-th 16-token tile of the split, with its own online-softmax
-//   state; the wave states are merged through LDS once, at the end.  W defaults to 4 and can be
-//   fixed per context for experiments.
+//   one workgroup (4 waves) = one (kv_split, kv_head); it serves all G query heads of that KV head.
+//   One wave = every 4th 16-token tile of the split, with its own online-softmax state; the wave
+//   states are merged through LDS once, at the end.  (1- and 2-wave workgroups measured no faster
+//   at any grid size: they only add partial rows per byte read.)
 //
 // Per 16-token tile and wave
 //   QK^T  one 16x16 MFMA tile: A = the K tile (16 tokens x head_dim, read straight from the page
@@ -101,9 +101,6 @@ __global__ __launch_bounds__(64 * kWaves, decode_waves_per_simd(G)) void split_k
     const uint32_t tid = threadIdx.x;
     const uint32_t lane = tid & 63;
     const uint32_t wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-#ifdef PSI_DECODE_TIMESTAMPS
-    const uint64_t t_start = wall_clock64();
-#endif
 
     __shared__ __attribute__((aligned(16))) float p_lds[kWaves][kTileTokens * kPStride];
     __shared__ __attribute__((aligned(16))) float alpha_lds[kWaves][8];
@@ -125,9 +122,6 @@ __global__ __launch_bounds__(64 * kWaves, decode_waves_per_simd(G)) void split_k
         row_begin = worker_cu[blockIdx.x / a.walk.hkv];
         row_end = worker_cu[blockIdx.x / a.walk.hkv + 1];
     }
-#ifdef PSI_DECODE_TIMESTAMPS
-    uint64_t t_loop = 0;
-#endif
     for (uint32_t split = row_begin; split < row_end; ++split) {
     if (split >= a.num_active_kv_splits) break;
     const uint32_t q_token = kv_splits[split * 3];
@@ -383,9 +377,6 @@ __global__ __launch_bounds__(64 * kWaves, decode_waves_per_simd(G)) void split_k
         }
     }
 
-#ifdef PSI_DECODE_TIMESTAMPS
-    t_loop = wall_clock64();
-#endif
     // ---- wave epilogue: fold the V token sub-lanes together, reduce the per-lane sums.
 #pragma unroll
     for (int h = 0; h < G; ++h)
@@ -441,58 +432,29 @@ __global__ __launch_bounds__(64 * kWaves, decode_waves_per_simd(G)) void split_k
     }
     if (split + 1 < row_end) __syncthreads();  // the LDS staging areas are reused by the next row
     }  // rows of this workgroup
-#ifdef PSI_DECODE_TIMESTAMPS
-    // experiment builds only: per-wave start / loop-end / end times and the hardware id, placed
-    // after the partial region (the harness over-allocates the scratch buffer)
-    if (lane == 0) {
-        uint64_t* dbg = reinterpret_cast<uint64_t*>(a.part_acc + (uint64_t)a.num_total_kv_splits * a.hq * D) + 64 +
-                        ((uint64_t)blockIdx.x * kWaves + wave) * 4;
-        dbg[0] = t_start;
-        dbg[1] = t_loop;
-        dbg[2] = wall_clock64();
-        dbg[3] = __builtin_amdgcn_s_getreg((4 << 0) | (0 << 6) | (31 << 11)) | ((uint64_t)__builtin_amdgcn_s_getreg((20 << 0) | (0 << 6) | (31 << 11)) << 32);
-    }
-#endif
 }
 
-
-// Waves per workgroup for a grid of `items` (kv_split, kv_head) workgroups.
-inline int decode_waves_per_item(uint64_t items) {
-    // Measured on MI355X: 4-wave workgroups are as fast as or faster than 2- and 1-wave ones at
-    // every grid size tried (fewer partial rows per byte read), so width only drops for tiny grids
-    // where 4-wave workgroups could not cover the compute units.
-    (void)items;
-    return 4;
-}
 
 template <typename Tag, int D, int G>
-inline void launch_decode_map_w(psi_hip_ctx* ctx, const Geometry& g, const MapArgs& a, int waves) {
+inline void launch_decode_map_w(psi_hip_ctx* ctx, const Geometry& g, const MapArgs& a) {
     const dim3 grid((a.worker_cu ? a.num_workers : a.num_total_kv_splits) * g.hkv);
     const uint16_t* q = reinterpret_cast<const uint16_t*>(a.q);
     const uint16_t* pages = reinterpret_cast<const uint16_t*>(a.kv_pages);
-    if (g.tokens_per_page == 8)  // a tile spans two pages; one workgroup width is built for this case
+    if (g.tokens_per_page == 8)  // a tile spans two pages
         hipLaunchKernelGGL((split_kv_decode_map<Tag, D, G, 4, true>), grid, dim3(256), 0, ctx->stream, a,
                            a.walk.page_ids, a.kv_splits, a.req_slots, q, pages, a.worker_cu);
-    else if (waves == 4)
-        hipLaunchKernelGGL((split_kv_decode_map<Tag, D, G, 4, false>), grid, dim3(256), 0, ctx->stream, a,
-                           a.walk.page_ids, a.kv_splits, a.req_slots, q, pages, a.worker_cu);
-    else if (waves == 2)
-        hipLaunchKernelGGL((split_kv_decode_map<Tag, D, G, 2, false>), grid, dim3(128), 0, ctx->stream, a,
-                           a.walk.page_ids, a.kv_splits, a.req_slots, q, pages, a.worker_cu);
     else
-        hipLaunchKernelGGL((split_kv_decode_map<Tag, D, G, 1, false>), grid, dim3(64), 0, ctx->stream, a,
+        hipLaunchKernelGGL((split_kv_decode_map<Tag, D, G, 4, false>), grid, dim3(256), 0, ctx->stream, a,
                            a.walk.page_ids, a.kv_splits, a.req_slots, q, pages, a.worker_cu);
 }
 
 // One translation unit per (element type, head_dim) instantiates every group size 1..8.
 template <typename Tag, int D>
 inline int launch_decode_map_group(psi_hip_ctx* ctx, const Geometry& g, const MapArgs& a) {
-    const uint64_t items = (uint64_t)(a.worker_cu ? a.num_workers : a.num_total_kv_splits) * g.hkv;
-    const int waves = ctx->decode_waves_override > 0 ? ctx->decode_waves_override : decode_waves_per_item(items);
     switch (g.group) {
 #define PSI_CASE(G)                                        \
     case G:                                                \
-        launch_decode_map_w<Tag, D, G>(ctx, g, a, waves);  \
+        launch_decode_map_w<Tag, D, G>(ctx, g, a);         \
         return PSI_HIP_OK;
         PSI_CASE(1)
         PSI_CASE(2)

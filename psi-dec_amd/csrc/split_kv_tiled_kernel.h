@@ -151,7 +151,23 @@ __global__ __launch_bounds__(64 * kTiledTileWaves * CG, (TiledOccupancy<NB, CG>:
     if (flat_begin >= a.num_active_tokens || flat_end > a.num_active_tokens || flat_end <= flat_begin) continue;
     const uint32_t tile_tokens = flat_end - flat_begin;
     const uint32_t ncols = tile_tokens * G;
-    if (ncols > (uint32_t)kCols) continue;  // the launcher sizes NB from the largest tile; never taken
+    if (ncols > (uint32_t)kCols) {
+        // A tile wider than the launch was sized for (the caller's largest-tile bound was too small, e.g. a
+        // capture made for two-token tiles replayed on a four-token batch).  The row cannot be computed here;
+        // it is entered as an empty state, so that the combine merges nothing stale, and the tile's output is
+        // then wrong in a visible way (zeros for a tile with no other row) rather than silently mixed.
+        const uint32_t rows = a.rows_per_split_head;
+        for (uint32_t idx = threadIdx.x; idx < ncols * (D / 4); idx += 64 * kWaves) {
+            const uint32_t c = idx / (D / 4), d4 = idx % (D / 4);
+            const uint64_t row = ((uint64_t)split * a.hq + (uint64_t)kv_head * G + c % G) * rows + c / G;
+            *reinterpret_cast<float4*>(&a.part_acc[row * D + d4 * 4]) = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
+            if (d4 == 0) {
+                a.part_max[row] = -INFINITY;
+                a.part_sum[row] = 0.0f;
+            }
+        }
+        continue;
+    }
     if (lds_in_use) __syncthreads();  // the previous row's merge buffer has been read out
     lds_in_use = true;
     // Lane coordinates, re-derived per row from a value the optimiser cannot see through: nothing computed from

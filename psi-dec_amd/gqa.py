@@ -98,20 +98,8 @@ class Device:
                                                     ctypes.byref(launches)))
         return total.value, launches.value
 
-    def copy_probe(self, dst, src, nbytes: int, read_only: bool = False):
-        """Plain copy (or pure read) of `nbytes`: the calibration load for HBM traffic counters."""
-        L.check(self.lib.psi_hip_copy_probe(self.ctx, _ptr(dst), _ptr(src), nbytes, int(read_only)))
-
     def force_generic(self, on: bool):
         L.check(self.lib.psi_hip_ctx_set_flag(self.ctx, L.FLAG_FORCE_GENERIC, int(on)))
-
-    def decode_valu_qk(self, on: bool):
-        """Decode map variant with QK^T on the vector ALU instead of MFMA (for comparisons)."""
-        L.check(self.lib.psi_hip_ctx_set_flag(self.ctx, L.FLAG_DECODE_VALU_QK, int(on)))
-
-    def decode_waves(self, waves: int):
-        """Waves per decode-map workgroup: 1, 2 or 4; 0 = chosen from the grid size."""
-        L.check(self.lib.psi_hip_ctx_set_flag(self.ctx, L.FLAG_DECODE_WAVES, int(waves)))
 
     def f32_output(self, on: bool):
         """Combine kernels then store f32 outputs (for checking the result before output rounding)."""

@@ -1,7 +1,10 @@
-// A plain device-to-device copy of known size.  It exists for measurement only: the HBM traffic
-// counters of this GPU are calibrated against it (bytes the counter reports for a copy of N bytes),
-// and its rate is the practical read+write ceiling the attention kernels are compared with.
-#include "common.h"
+// A plain device-to-device copy and a pure read of known size.  Measurement only, built into its own
+// library (lib/libpsi_hip_probe.so) so that the attention library ships nothing it does not need: the HBM
+// traffic counters of this GPU are calibrated against the copy (bytes the counter reports for a copy of N
+// bytes), and the rates are the practical ceilings the attention kernels are compared with.
+#include <hip/hip_runtime.h>
+
+#include <cstdint>
 
 namespace {
 
@@ -29,21 +32,19 @@ __global__ void __launch_bounds__(256) psi_read_probe(const uint4* __restrict__ 
 
 }  // namespace
 
-extern "C" int psi_hip_copy_probe(psi_hip_ctx* ctx, void* dst, const void* src, uint64_t bytes, int read_only) {
-    PSI_REQUIRE(ctx != nullptr && dst != nullptr && src != nullptr, "ctx, dst and src must not be null");
-    PSI_REQUIRE(bytes != 0 && bytes % 16 == 0, "probe size must be a positive multiple of 16 bytes");
-    PSI_REQUIRE((reinterpret_cast<uintptr_t>(dst) | reinterpret_cast<uintptr_t>(src)) % 16 == 0,
-                "probe buffers must be 16-byte aligned");
+// stream: a hipStream_t.  Returns 0, -1 for a bad argument, or the positive hipError_t of the launch.
+extern "C" int psi_probe_copy(void* stream, void* dst, const void* src, uint64_t bytes, int read_only) {
+    if (dst == nullptr || src == nullptr || bytes == 0 || bytes % 16 != 0) return -1;
+    if ((reinterpret_cast<uintptr_t>(dst) | reinterpret_cast<uintptr_t>(src)) % 16 != 0) return -1;
     const uint64_t count = bytes / 16;
     const uint64_t want = (count + 255) / 256;
     const unsigned grid = static_cast<unsigned>(want < 256ull * 16 ? want : 256ull * 16);
-    psi::LaunchScope scope(ctx, read_only ? "read_probe" : "copy_probe");
+    hipStream_t s = static_cast<hipStream_t>(stream);
     if (read_only)
-        hipLaunchKernelGGL(psi_read_probe, dim3(grid), dim3(256), 0, ctx->stream, static_cast<const uint4*>(src),
+        hipLaunchKernelGGL(psi_read_probe, dim3(grid), dim3(256), 0, s, static_cast<const uint4*>(src),
                            static_cast<uint4*>(dst), count);
     else
-        hipLaunchKernelGGL(psi_copy_probe, dim3(grid), dim3(256), 0, ctx->stream, static_cast<const uint4*>(src),
+        hipLaunchKernelGGL(psi_copy_probe, dim3(grid), dim3(256), 0, s, static_cast<const uint4*>(src),
                            static_cast<uint4*>(dst), count);
-    PSI_HIP_CHECK(hipGetLastError());
-    return PSI_HIP_OK;
+    return static_cast<int>(hipGetLastError());
 }

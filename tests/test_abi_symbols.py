@@ -32,6 +32,68 @@ def test_prototype_table_matches_header(psi):
     assert sorted(psi.PROTOTYPES) == declared_functions()
 
 
+_SCALARS = {"int": ctypes.c_int, "uint32_t": ctypes.c_uint32, "uint64_t": ctypes.c_uint64, "size_t": ctypes.c_size_t,
+            "float": ctypes.c_float, "double": ctypes.c_double}
+
+
+def declared_signatures():
+    """name -> (return is pointer, [argument kinds]) parsed from the header; an argument kind is "ptr" or the
+    ctypes scalar type its C type maps to."""
+    text = open(os.path.join(ROOT, "include", "psi_hip.h")).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    text = re.sub(r"^\s*#.*$", "", text, flags=re.M)
+    out = {}
+    for ret, name, args in re.findall(r"([A-Za-z_][\w \*]*?)\b(psi_hip_[a-z0-9_]+)\s*\(([^;{]*?)\)\s*;", text, flags=re.S):
+        kinds = []
+        args = " ".join(args.split())
+        if args and args != "void":
+            for arg in args.split(","):
+                arg = arg.strip()
+                if "*" in arg:
+                    kinds.append("ptr")
+                    continue
+                words = [w for w in arg.split() if w != "const"]
+                assert len(words) == 2, (name, arg)
+                kinds.append(_SCALARS[words[0]])
+        out[name] = ("*" in ret, kinds)
+    return out
+
+
+def _is_pointer_type(t):
+    return t in (ctypes.c_void_p, ctypes.c_char_p) or hasattr(t, "contents")
+
+
+def test_prototype_signatures_match_header(psi):
+    """The hand-kept ctypes table against the declarations: argument count, pointer vs scalar, and the exact
+    scalar type of every argument and of the return value."""
+    declared = declared_signatures()
+    assert sorted(declared) == sorted(psi.PROTOTYPES)
+    for name, (restype, argtypes) in psi.PROTOTYPES.items():
+        ret_is_ptr, kinds = declared[name]
+        assert _is_pointer_type(restype) == ret_is_ptr and (ret_is_ptr or restype is ctypes.c_int), name
+        assert len(argtypes) == len(kinds), f"{name}: {len(argtypes)} ctypes arguments, {len(kinds)} declared"
+        for i, (have, want) in enumerate(zip(argtypes, kinds)):
+            if want == "ptr":
+                assert _is_pointer_type(have), f"{name} argument {i}: declared a pointer, bound as {have}"
+            else:
+                assert have is want, f"{name} argument {i}: declared {want}, bound as {have}"
+
+
+def test_header_is_plain_c11_and_links(psi, tmp_path):
+    """include/psi_hip.h compiled as C11 (not through the library's own C++ sources), linked against the
+    built library; the program calls entry points that need no GPU."""
+    import subprocess
+
+    exe = tmp_path / "abi_c11"
+    lib_dir = os.path.dirname(psi.LIB_PATH)
+    subprocess.run(["gcc", "-std=c11", "-Wall", "-Wextra", "-Werror", "-pedantic", "-I", os.path.join(ROOT, "include"),
+                    os.path.join(ROOT, "tests", "abi", "abi_c11.c"), "-o", str(exe), "-L", lib_dir, "-lpsi_hip",
+                    f"-Wl,-rpath,{lib_dir}", "-Wl,-rpath,/opt/rocm/lib"], check=True)
+    done = subprocess.run([str(exe)], capture_output=True, text=True)
+    assert done.returncode == 0, done.stderr
+    assert "abi_c11 ok" in done.stdout
+
+
 def test_every_declaration_cites_the_reference():
     """Each entry point's comment names the reference file it stands in for (or says it has none)."""
     text = open(os.path.join(ROOT, "include", "psi_hip.h")).read()

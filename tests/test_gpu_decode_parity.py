@@ -79,18 +79,6 @@ def test_fast_and_generic_variants_agree(psi, oracle, device):
     assert np.abs(a - b).max() < 1e-5
 
 
-@pytest.mark.parametrize("waves", [1, 2, 4])
-def test_workgroup_widths_agree_with_oracle(psi, oracle, device, waves):
-    """The decode map with 1, 2 and 4 waves per workgroup (chosen from the grid size in production)."""
-    wl = importlib_workloads(psi)
-    w = wl.make_workload(19, [1500, 31, 530, 512], 24, 4, 256, psi.Dtype.Bfloat16, 16)
-    device.decode_waves(waves)
-    try:
-        run_and_check(psi, oracle, device, w, f"waves={waves}", partition_tokens=512, check_rounded=False)
-    finally:
-        device.decode_waves(0)
-
-
 def test_balanced_plan_matches_oracle(psi, oracle, device):
     """Equal-work worker plan: rows re-cut at tile boundaries, several rows per workgroup."""
     wl = importlib_workloads(psi)

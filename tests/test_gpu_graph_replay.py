@@ -236,3 +236,46 @@ def test_one_captured_step_serves_every_layer_of_the_table(psi, device):
         assert torch.equal(dw.output.view(torch.int16), eager[layer][0].view(torch.int16)), (word, layer)
         assert torch.equal(dw.pages.view(torch.int16), eager[layer][1].view(torch.int16)), (word, layer)
         _ = dw.output.float().sum().item()  # eager work between replays
+
+
+def test_wide_combine_leaves_inactive_tokens_alone(psi, oracle, device):
+    """Device-side counts below the capacity on a split list long enough for the workgroup-per-row combine
+    (40 rows per token of capacity): the batch holds one of two tokens, the metadata beyond it is what the
+    previous, full batch left behind.  The active token matches the oracle; the inactive token's output row
+    keeps its canary and the map writes no partial row beyond the active splits."""
+    import torch
+
+    from parity_util import assert_outputs_close, layout_tuple, oracle_dtype
+
+    wl = importlib_workloads(psi)
+    w = wl.make_workload(131, [3000, 2000], 16, 2, 256, psi.Dtype.Bfloat16, 16)
+    variant = psi.GQASplitKVVariant.SingleQ(16, 256, 8)
+    dw = wl.DeviceWorkload(device, w, partition_tokens=64, variant=variant, f32_output=True)
+    s = dw.shape
+    rows_first = -(-3000 // 64)
+    assert s.num_sdpa_map_task_templates == rows_first + -(-2000 // 64)
+    assert s.num_total_sdpa_map_task_templates // s.num_total_tokens >= 32  # the wide combine's domain
+    dw.step()  # the full batch: leaves its rows in the scratch and its entries in cu_kv_splits
+    full = dw.output_f32().reshape(2, -1)
+    row = w.num_q_heads * w.head_dim
+    counts = torch.tensor([1, 1, rows_first, 0], dtype=torch.int32, device=device.torch_device)
+    dw.output.fill_(-768.0)
+    scratch_before = dw.scratch.buffer.clone()
+    device.bind_replay_counts(counts)
+    try:
+        dw.step()  # by-value counts stay at the capacity (2 tokens, all rows)
+        device.sync()
+    finally:
+        device.bind_replay_counts(None)
+    got = dw.output.float().cpu().numpy().reshape(2, row)
+    assert (got[1] == -768.0).all(), "the combine wrote the output row of an inactive token"
+    assert np.array_equal(got[0], full[0])
+    # partial rows of the inactive token are untouched
+    acc_rows = dw.scratch.buffer.view(torch.float32)[-s.num_total_sdpa_map_task_templates * row:].view(-1, row)
+    acc_before = scratch_before.view(torch.float32)[-s.num_total_sdpa_map_task_templates * row:].view(-1, row)
+    assert torch.equal(acc_rows[rows_first:], acc_before[rows_first:])
+    dt = oracle_dtype(oracle, w)
+    exp = oracle.paged_gqa(w.num_q_heads, w.num_kv_heads, w.head_dim, w.scale, w.page_bytes, dt, layout_tuple(w),
+                           w.layer, w.req_slots[:1], w.token_indices[:1], np.arange(2, dtype=np.uint32),
+                           w.q.reshape(2, -1)[:1].reshape(-1), dw.pages_host(), w.page_ids, num_threads=8)
+    assert_outputs_close(got[0], exp, "wide combine under device-side counts")
