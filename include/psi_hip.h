@@ -493,6 +493,106 @@ int psi_hip_split_kv_tiled_q_reduce(psi_hip_ctx* ctx, const psi_hip_gqa_config* 
                                     uint32_t num_active_q_token_tiles, const uint32_t* partial_row_index,
                                     const psi_hip_output_gate* gate);
 
+/* ------------------------------------------------------------------ the attention layer
+ *
+ * `GQA::record(GQAInput)` / `UngatedGQA::record` (crates/inference-executor-metal/src/attn/gqa/backend.rs:394-658,
+ * ungated_backend.rs:182-380; `ReplayLayer`, src/def/layer.rs:12-23) without the two quantised matmuls around it:
+ * one call takes the QGKV projection output and the batch metadata and issues, on the context's stream, what the
+ * reference records between them -- QGKV split, Q / K RMSNorm + RoPE, KV page write, SplitKV map of the batch's
+ * variant, combine, sigmoid gate -- in this library's fused form: one prepare launch (Q and K normalised and
+ * rotated from strided views of the projection output, K and V written straight into their page lines), the map,
+ * and the combine with the gate applied to each element as it is stored.  Stream order stands for the barriers the
+ * reference records.  Results equal the operator-by-operator sequence bit for bit in the arena and in the output. */
+
+/* Device copies of one batch's `GQAMetadataBuffers` arrays (batch_metadata.rs:22-46) with the shape and variant
+ * psi_hip_gqa_metadata_update returned for them, plus this library's optional launch plans for the same rows. */
+typedef struct psi_hip_gqa_batch_metadata {
+    psi_hip_gqa_replay_shape shape;
+    psi_hip_split_kv_variant variant;
+    const uint32_t* req_slots;          /* u32[num_total_tokens] */
+    const uint32_t* flat_token_indices; /* u32[num_total_tokens] */
+    const uint32_t* q_token_tiles;      /* u32[num_total_q_token_tiles][2]; TiledQ only */
+    const uint32_t* kv_splits;          /* u32[num_total_kv_splits][3] */
+    const uint32_t* cu_kv_splits;       /* u32[num_total_tokens + 1] (SingleQ) / [num_total_q_token_tiles + 1] */
+    const uint32_t* partial_row_index;  /* null, or the row order of psi_hip_split_kv_order_longest_first */
+    const uint32_t* worker_cu;          /* null, or the worker table of psi_hip_split_kv_balance_plan */
+    uint32_t num_workers;
+    const uint32_t* row_groups;         /* null, or the table of psi_hip_split_kv_tiled_q_group_rows (TiledQ) */
+    uint32_t group_tiles;
+    uint32_t num_row_groups;
+    uint32_t max_active_q_tile_tokens;  /* TiledQ: bound on the tokens of any tile (0 = q_token_tile_size) */
+} psi_hip_gqa_batch_metadata;
+
+/* `GQACore` + `GQAMetalConfig` (backend.rs:114-146) as far as the attention needs them. */
+typedef struct psi_hip_gqa_layer_config {
+    psi_hip_gqa_config attention;
+    uint32_t gated; /* 1: `GQA`, projection rows [q_0|g_0|q_1|g_1|...|k|v]; 0: `UngatedGQA`, rows [q|k|v] */
+    uint32_t rope_dim;
+    float norm_eps;
+    float rope_theta;
+    psi_hip_rope_scaling rope_scaling;
+} psi_hip_gqa_layer_config;
+
+#define PSI_HIP_REPLAY_EXACT 0u    /* `GQAReplayMode::Exact`: active counts equal the recorded capacities */
+#define PSI_HIP_REPLAY_BUCKETED 1u /* `GQAReplayMode::Bucketed`: active counts within the capacities */
+
+/* `GQAInput` (backend.rs:169-182).  Activations come either as `qgkv`, the projection output the reference keeps in
+ * `scratch.qgkv` ([num_total_tokens] rows in the layer's layout), or -- qgkv null -- as rows that are already
+ * split, normalised and rotated: q [T][Hq][D], k and v [T][Hkv][D], optionally gates g [T][Hq][D] (the attention
+ * core alone: append, map, combine [, gate]; the decode step then folds the append into the map launch). */
+typedef struct psi_hip_gqa_layer_input {
+    psi_hip_page_table_layout page_table_layout;
+    uint32_t gqa_layer_index;
+    uint32_t replay_mode; /* PSI_HIP_REPLAY_* */
+    const psi_hip_gqa_batch_metadata* batch_metadata;
+    const void* qgkv;
+    const void* q;
+    const void* k;
+    const void* v;
+    const void* g;
+    void* kv_pages; /* `GQAKVCacheBindings` */
+    uint64_t kv_pages_bytes;
+    const uint32_t* page_ids;
+    const void* q_norm_weight; /* `GQAWeights::{q,k}_norm_weight`: bf16[head_dim]; unused with split inputs */
+    const void* k_norm_weight;
+    void* q_norm_rope;     /* `scratch.q_norm_rope` [num_total_tokens][Hq][D]; unused with split inputs */
+    void* partial_scratch; /* the `scratch.sdpa_partial_*` buffers as one, sized by psi_hip_gqa_layer_scratch_bytes */
+    uint64_t partial_scratch_bytes;
+    void* output; /* `scratch.gated_attention_output` / `scratch.attention_output`: [num_total_tokens][Hq][D] */
+} psi_hip_gqa_layer_input;
+
+/* Bytes of `partial_scratch` for a variant and split capacity (`GQAScratch::new`, scratch.rs:48-92). */
+int psi_hip_gqa_layer_scratch_bytes(const psi_hip_gqa_layer_config* cfg, const psi_hip_split_kv_variant* variant,
+                                    uint32_t num_total_kv_splits, uint64_t* out_bytes);
+
+/* `GQA::record` (backend.rs:394-658).  With device-side counts bound to the context the launches are valid for
+ * every batch of the capacity bucket (psi_hip_ctx_bind_replay_counts). */
+int psi_hip_gqa_layer_record(psi_hip_ctx* ctx, const psi_hip_gqa_layer_config* cfg,
+                             const psi_hip_gqa_layer_input* input);
+
+/* One recorded program per capacity bucket: the counterpart of the reference's replay-program store, which keeps a
+ * recorded program per `(variant, total tokens, total Q-token tiles, total KV splits)` key and binds the active
+ * counts at submission (crates/inference-executor-core/src/replay.rs:4-87; parameter keys backend.rs:55-57;
+ * `Stream::submit_replay_with_arguments`).  Here a program is a HIP graph captured from psi_hip_gqa_layer_record
+ * with the counts block bound.  The context's stream must be a created stream (capture is not possible on the
+ * null stream).  device_counts: caller-owned device u32[4], written by the cache at every submission.
+ * max_programs: programs kept; the least recently used one is dropped beyond that. */
+typedef struct psi_hip_gqa_replay_cache psi_hip_gqa_replay_cache;
+int psi_hip_gqa_replay_cache_create(psi_hip_ctx* ctx, const psi_hip_gqa_layer_config* cfg, uint32_t* device_counts,
+                                    uint32_t max_programs, psi_hip_gqa_replay_cache** out_cache);
+int psi_hip_gqa_replay_cache_destroy(psi_hip_gqa_replay_cache* cache);
+/* Replays the program of the input's bucket, recording it first if the cache has none: key = variant and geometry,
+ * the three capacities of input->batch_metadata->shape, the layer index (when by value), and every buffer address
+ * of the input (a program holds addresses).  The active counts of the shape go to the counts block, stream-ordered
+ * ahead of the program; gqa_layer_parameter > 0 binds the page-table layer gqa_layer_parameter - 1 the same way
+ * (`ReplayU32::Parameter`) instead of the input's gqa_layer_index.  *out_recorded (may be null): 1 if this call
+ * recorded. */
+int psi_hip_gqa_replay_cache_submit(psi_hip_gqa_replay_cache* cache, const psi_hip_gqa_layer_input* input,
+                                    uint32_t gqa_layer_parameter, int* out_recorded);
+/* Programs held, recordings and replays so far; any out pointer may be null. */
+int psi_hip_gqa_replay_cache_stats(const psi_hip_gqa_replay_cache* cache, uint32_t* programs, uint64_t* recordings,
+                                   uint64_t* replays);
+
 /* ------------------------------------------------------------------ request page table */
 
 /* `GQARequestPageTable::write_page_ids` (crates/inference-executor-metal/src/attn/gqa/request_page_table.rs:58-69):

@@ -438,7 +438,7 @@ class DecoderBlocks:
     # -- helpers (blocks/util.rs)
     def _pop_front_queued(self, num):
         num = min(len(self.queued) - (self.lanes - 1), num)
-        tokens = list(self.queued)[:num + self.lanes - 1]
+        tokens = [self.queued[i] for i in range(num + self.lanes - 1)]  # the head of the deque: O(num)
         for _ in range(num):
             self.queued.popleft()
         return tokens

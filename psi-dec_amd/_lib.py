@@ -22,6 +22,7 @@ VARIANT_SINGLE_Q, VARIANT_TILED_Q = 0, 1
 CAPACITY_EXACT, CAPACITY_BUCKETED, CAPACITY_CALLER_TOKENS, CAPACITY_FIXED_PARTITION = 0, 1, 2, 3
 FLAG_FORCE_GENERIC = 1
 FLAG_F32_OUTPUT = 2
+REPLAY_EXACT, REPLAY_BUCKETED = 0, 1
 
 
 class PsiHipError(RuntimeError):
@@ -100,6 +101,59 @@ class ReplayShapeStruct(ctypes.Structure):
         ("num_kv_splits", c_uint32),
         ("num_total_kv_splits", c_uint32),
         ("reduce_sdpa_partial_outputs", c_uint32),
+    ]
+
+
+class BatchMetadataStruct(ctypes.Structure):
+    _fields_ = [
+        ("shape", ReplayShapeStruct),
+        ("variant", VariantStruct),
+        ("req_slots", c_void_p),
+        ("flat_token_indices", c_void_p),
+        ("q_token_tiles", c_void_p),
+        ("kv_splits", c_void_p),
+        ("cu_kv_splits", c_void_p),
+        ("partial_row_index", c_void_p),
+        ("worker_cu", c_void_p),
+        ("num_workers", c_uint32),
+        ("row_groups", c_void_p),
+        ("group_tiles", c_uint32),
+        ("num_row_groups", c_uint32),
+        ("max_active_q_tile_tokens", c_uint32),
+    ]
+
+
+class LayerConfigStruct(ctypes.Structure):
+    _fields_ = [
+        ("attention", GQAConfigStruct),
+        ("gated", c_uint32),
+        ("rope_dim", c_uint32),
+        ("norm_eps", c_float),
+        ("rope_theta", c_float),
+        ("rope_scaling", RopeScalingStruct),
+    ]
+
+
+class LayerInputStruct(ctypes.Structure):
+    _fields_ = [
+        ("page_table_layout", PageTableLayoutStruct),
+        ("gqa_layer_index", c_uint32),
+        ("replay_mode", c_uint32),
+        ("batch_metadata", POINTER(BatchMetadataStruct)),
+        ("qgkv", c_void_p),
+        ("q", c_void_p),
+        ("k", c_void_p),
+        ("v", c_void_p),
+        ("g", c_void_p),
+        ("kv_pages", c_void_p),
+        ("kv_pages_bytes", c_uint64),
+        ("page_ids", c_void_p),
+        ("q_norm_weight", c_void_p),
+        ("k_norm_weight", c_void_p),
+        ("q_norm_rope", c_void_p),
+        ("partial_scratch", c_void_p),
+        ("partial_scratch_bytes", c_uint64),
+        ("output", c_void_p),
     ]
 
 
@@ -247,6 +301,13 @@ PROTOTYPES = {
         [c_void_p, _CFG, c_uint32, c_void_p, c_uint64, c_void_p, c_void_p, c_void_p, c_uint32, c_uint32, c_uint32,
          c_uint32, c_void_p, POINTER(OutputGateStruct)],
     ),
+    "psi_hip_gqa_layer_scratch_bytes": (c_int, [POINTER(LayerConfigStruct), _VARIANT, c_uint32, POINTER(c_uint64)]),
+    "psi_hip_gqa_layer_record": (c_int, [c_void_p, POINTER(LayerConfigStruct), POINTER(LayerInputStruct)]),
+    "psi_hip_gqa_replay_cache_create": (
+        c_int, [c_void_p, POINTER(LayerConfigStruct), c_void_p, c_uint32, POINTER(c_void_p)]),
+    "psi_hip_gqa_replay_cache_destroy": (c_int, [c_void_p]),
+    "psi_hip_gqa_replay_cache_submit": (c_int, [c_void_p, POINTER(LayerInputStruct), c_uint32, POINTER(c_int)]),
+    "psi_hip_gqa_replay_cache_stats": (c_int, [c_void_p, _U32P, _U64P, _U64P]),
     "psi_hip_page_table_write_page_ids": (
         c_int, [c_void_p, _LAYOUT, c_void_p, c_uint32, c_uint32, c_uint32, _U32P, c_uint32, c_uint32]),
     "psi_hip_page_table_reset_req_slot": (c_int, [c_void_p, _LAYOUT, c_void_p, c_uint32]),

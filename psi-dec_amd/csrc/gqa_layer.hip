@@ -1,0 +1,385 @@
+// The attention layer as one call, and one recorded program per capacity bucket.
+//
+// psi_hip_gqa_layer_record mirrors `GQA::record` / `UngatedGQA::record`
+// (crates/inference-executor-metal/src/attn/gqa/backend.rs:394-658, ungated_backend.rs:182-380) between the two
+// matmuls: QGKV split -> Q / K RMSNorm + RoPE -> KV page write -> SplitKV map of the batch's variant -> combine ->
+// gate, issued in this library's fused form (prepare launch, map, combine with gate).  It only sequences the
+// component entry points of include/psi_hip.h; every check and kernel lives with them.
+//
+// psi_hip_gqa_replay_cache_* keeps one HIP graph per `(variant, total tokens, total Q-token tiles, total KV
+// splits)` key, captured from that call with the device-side count block bound, as the reference keeps one
+// recorded program per key and binds `gqa.num_active_*` at submission
+// (crates/inference-executor-core/src/replay.rs:4-87, backend.rs:55-57).
+#include <cstring>
+#include <list>
+#include <vector>
+
+#include "common.h"
+#include "device_types.h"
+
+namespace psi {
+
+namespace {
+
+struct LayerPlan {
+    Geometry g;
+    psi_hip_rms_norm_rope_config q_norm, k_norm;
+    uint64_t token_width = 0;   // elements per projection row
+    uint64_t q_head_stride = 0; // elements between the q rows of neighbouring heads
+    uint64_t k_offset = 0, v_offset = 0;
+};
+
+int make_layer_plan(const psi_hip_gqa_layer_config* cfg, LayerPlan* plan) {
+    PSI_REQUIRE(cfg != nullptr, "GQA layer config must not be null");
+    int rc = make_geometry(&cfg->attention, &plan->g);
+    if (rc != PSI_HIP_OK) return rc;
+    const Geometry& g = plan->g;
+    PSI_REQUIRE(cfg->gated <= 1, "GQA layer `gated` must be 0 or 1");
+    psi_hip_rms_norm_rope_config n;
+    n.num_heads = g.hq;
+    n.head_dim = g.d;
+    n.rope_dim = cfg->rope_dim;
+    n.eps = cfg->norm_eps;
+    n.rope_theta = cfg->rope_theta;
+    n.scaling = cfg->rope_scaling;
+    n.dtype = g.dtype;
+    plan->q_norm = n;
+    n.num_heads = g.hkv;
+    plan->k_norm = n;
+    if (cfg->gated) {  // [q_0|g_0|q_1|g_1|...|k|v], metal/gqa_qgkv_split.metal:5-43
+        plan->token_width = 2ull * ((uint64_t)g.hq + g.hkv) * g.d;
+        plan->q_head_stride = 2ull * g.d;
+        plan->k_offset = 2ull * g.hq * g.d;
+    } else {  // [q|k|v], metal/gqa_qkv_split.metal
+        plan->token_width = ((uint64_t)g.hq + 2ull * g.hkv) * g.d;
+        plan->q_head_stride = g.d;
+        plan->k_offset = (uint64_t)g.hq * g.d;
+    }
+    plan->v_offset = plan->k_offset + (uint64_t)g.hkv * g.d;
+    return PSI_HIP_OK;
+}
+
+const void* offset_elems(const void* base, uint64_t elems, uint32_t elem_bytes) {
+    return static_cast<const char*>(base) + elems * elem_bytes;
+}
+
+// `GQAReplayShape::validate` (crates/inference-executor-core/src/attn/gqa/core.rs:135-142) and
+// `GQA::validate_input` (backend.rs:231-252).
+int check_input(const psi_hip_gqa_layer_input* in) {
+    PSI_REQUIRE(in != nullptr, "GQA layer input must not be null");
+    PSI_REQUIRE(in->batch_metadata != nullptr, "GQA batch metadata must be updated before recording");
+    const psi_hip_gqa_replay_shape& s = in->batch_metadata->shape;
+    PSI_REQUIRE(s.num_tokens > 0 && s.num_tokens <= s.num_total_tokens, "GQA replay shape: 0 < tokens <= capacity");
+    PSI_REQUIRE(s.num_q_token_tiles > 0 && s.num_q_token_tiles <= s.num_tokens &&
+                    s.num_q_token_tiles <= s.num_total_q_token_tiles,
+                "GQA replay shape: 0 < Q-token tiles <= tokens, capacity");
+    PSI_REQUIRE(s.num_kv_splits >= s.num_q_token_tiles && s.num_kv_splits <= s.num_total_kv_splits,
+                "GQA replay shape: Q-token tiles <= KV splits <= capacity");
+    PSI_REQUIRE(in->replay_mode == PSI_HIP_REPLAY_EXACT || in->replay_mode == PSI_HIP_REPLAY_BUCKETED,
+                "unknown GQA replay mode %u", in->replay_mode);
+    if (in->replay_mode == PSI_HIP_REPLAY_EXACT)
+        PSI_REQUIRE(s.num_tokens == s.num_total_tokens && s.num_q_token_tiles == s.num_total_q_token_tiles,
+                    "GQA exact replay requires active counts equal to the recorded capacities");
+    int rc = check_layout(&in->page_table_layout);
+    if (rc != PSI_HIP_OK) return rc;
+    PSI_REQUIRE(in->gqa_layer_index < in->page_table_layout.num_gqa_layers, "GQA page-table index exceeds layer count");
+    const uint32_t kind = in->batch_metadata->variant.kind;
+    PSI_REQUIRE(kind == PSI_HIP_VARIANT_SINGLE_Q || kind == PSI_HIP_VARIANT_TILED_Q, "unknown SplitKV variant %u", kind);
+    PSI_REQUIRE(in->kv_pages && in->page_ids && in->partial_scratch && in->output,
+                "GQA layer cache, scratch and output buffers must not be null");
+    return PSI_HIP_OK;
+}
+
+int record_layer(psi_hip_ctx* ctx, const psi_hip_gqa_layer_config* cfg, const psi_hip_gqa_layer_input* in) {
+    PSI_REQUIRE(ctx != nullptr, "ctx must not be null");
+    LayerPlan plan;
+    int rc = make_layer_plan(cfg, &plan);
+    if (rc != PSI_HIP_OK) return rc;
+    rc = check_input(in);
+    if (rc != PSI_HIP_OK) return rc;
+    const Geometry& g = plan.g;
+    const psi_hip_gqa_batch_metadata& md = *in->batch_metadata;
+    const psi_hip_gqa_replay_shape& s = md.shape;
+    const psi_hip_gqa_config* acfg = &cfg->attention;
+    const psi_hip_page_table_layout* layout = &in->page_table_layout;
+    const bool tiled = md.variant.kind == PSI_HIP_VARIANT_TILED_Q;
+    const uint32_t layer = in->gqa_layer_index;
+
+    const void* q = in->q;
+    psi_hip_output_gate gate_storage;
+    const psi_hip_output_gate* gate = nullptr;
+    bool append_with_map = false;
+    if (in->qgkv != nullptr) {
+        // split + Q norm/rope + K norm/rope + page write: one launch over strided views of the projection output
+        PSI_REQUIRE(in->q_norm_weight && in->k_norm_weight && in->q_norm_rope,
+                    "GQA layer norm weights and the q_norm_rope scratch must not be null");
+        rc = psi_hip_qk_norm_rope_kv_page_write(
+            ctx, acfg, layout, &plan.q_norm, &plan.k_norm, in->qgkv, plan.token_width, plan.q_head_stride,
+            in->q_norm_weight, in->q_norm_rope, in->kv_pages, in->kv_pages_bytes,
+            offset_elems(in->qgkv, plan.k_offset, g.elem), plan.token_width,
+            offset_elems(in->qgkv, plan.v_offset, g.elem), plan.token_width, in->k_norm_weight, md.req_slots,
+            md.flat_token_indices, in->page_ids, s.num_total_tokens, s.num_tokens, layer);
+        if (rc != PSI_HIP_OK) return rc;
+        q = in->q_norm_rope;
+        if (cfg->gated) {
+            gate_storage = psi_hip_output_gate{offset_elems(in->qgkv, g.d, g.elem), plan.token_width, 2ull * g.d};
+            gate = &gate_storage;
+        }
+    } else {
+        PSI_REQUIRE(in->q && in->k && in->v, "GQA layer needs the projection output or split q / k / v rows");
+        if (in->g != nullptr) {
+            gate_storage = psi_hip_output_gate{in->g, (uint64_t)g.hq * g.d, g.d};
+            gate = &gate_storage;
+        }
+        if (tiled) {
+            rc = psi_hip_kv_page_write(ctx, acfg, layout, in->kv_pages, in->kv_pages_bytes, in->k, in->v, md.req_slots,
+                                       md.flat_token_indices, in->page_ids, s.num_total_tokens, s.num_tokens, layer);
+            if (rc != PSI_HIP_OK) return rc;
+        } else {
+            append_with_map = true;  // the decode map writes each token's lines itself
+        }
+    }
+
+    if (tiled) {
+        const uint32_t ts = md.variant.q_token_tile_size;
+        PSI_REQUIRE(md.q_token_tiles != nullptr, "GQA SplitKV TiledQ needs the Q-token tile table");
+        if (md.row_groups != nullptr && md.num_row_groups != 0)
+            rc = psi_hip_split_kv_tiled_q_map_grouped(
+                ctx, acfg, layout, ts, q, in->kv_pages, in->kv_pages_bytes, md.req_slots, in->page_ids,
+                md.flat_token_indices, md.q_token_tiles, md.kv_splits, in->partial_scratch, in->partial_scratch_bytes,
+                layer, s.num_total_tokens, s.num_total_q_token_tiles, s.num_total_kv_splits, s.num_tokens,
+                s.num_q_token_tiles, s.num_kv_splits, md.max_active_q_tile_tokens, md.row_groups, md.group_tiles,
+                md.num_row_groups);
+        else if (md.worker_cu != nullptr)
+            rc = psi_hip_split_kv_tiled_q_map_balanced(
+                ctx, acfg, layout, ts, q, in->kv_pages, in->kv_pages_bytes, md.req_slots, in->page_ids,
+                md.flat_token_indices, md.q_token_tiles, md.kv_splits, md.worker_cu, md.num_workers,
+                in->partial_scratch, in->partial_scratch_bytes, layer, s.num_total_tokens, s.num_total_q_token_tiles,
+                s.num_total_kv_splits, s.num_tokens, s.num_q_token_tiles, s.num_kv_splits, md.max_active_q_tile_tokens);
+        else
+            rc = psi_hip_split_kv_tiled_q_map(
+                ctx, acfg, layout, ts, q, in->kv_pages, in->kv_pages_bytes, md.req_slots, in->page_ids,
+                md.flat_token_indices, md.q_token_tiles, md.kv_splits, in->partial_scratch, in->partial_scratch_bytes,
+                layer, s.num_total_tokens, s.num_total_q_token_tiles, s.num_total_kv_splits, s.num_tokens,
+                s.num_q_token_tiles, s.num_kv_splits, md.max_active_q_tile_tokens);
+        if (rc != PSI_HIP_OK) return rc;
+        return psi_hip_split_kv_tiled_q_reduce(ctx, acfg, ts, in->partial_scratch, in->partial_scratch_bytes,
+                                               md.q_token_tiles, md.cu_kv_splits, in->output, s.num_total_tokens,
+                                               s.num_total_q_token_tiles, s.num_total_kv_splits, s.num_q_token_tiles,
+                                               md.partial_row_index, gate);
+    }
+    if (append_with_map)
+        rc = psi_hip_kv_page_write_split_kv_single_q_map(
+            ctx, acfg, layout, q, in->kv_pages, in->kv_pages_bytes, in->k, in->v, md.req_slots, md.flat_token_indices,
+            in->page_ids, md.kv_splits, md.worker_cu, md.worker_cu ? md.num_workers : 0, in->partial_scratch,
+            in->partial_scratch_bytes, layer, s.num_total_tokens, s.num_total_kv_splits, s.num_tokens, s.num_kv_splits);
+    else if (md.worker_cu != nullptr)
+        rc = psi_hip_split_kv_single_q_map_balanced(
+            ctx, acfg, layout, q, in->kv_pages, in->kv_pages_bytes, md.req_slots, in->page_ids, md.kv_splits,
+            md.worker_cu, md.num_workers, in->partial_scratch, in->partial_scratch_bytes, layer, s.num_total_tokens,
+            s.num_total_kv_splits, s.num_tokens, s.num_kv_splits);
+    else
+        rc = psi_hip_split_kv_single_q_map(ctx, acfg, layout, q, in->kv_pages, in->kv_pages_bytes, md.req_slots,
+                                           in->page_ids, md.kv_splits, in->partial_scratch, in->partial_scratch_bytes,
+                                           layer, s.num_total_tokens, s.num_total_kv_splits, s.num_tokens,
+                                           s.num_kv_splits);
+    if (rc != PSI_HIP_OK) return rc;
+    return psi_hip_split_kv_single_q_reduce(ctx, acfg, in->partial_scratch, in->partial_scratch_bytes, md.cu_kv_splits,
+                                            in->output, s.num_total_tokens, s.num_total_kv_splits, s.num_tokens,
+                                            md.partial_row_index, gate);
+}
+
+// Writes the four words of the count block from kernel arguments: stream-ordered ahead of the program that reads
+// them, no host memory involved (a plain store; the block is ordinary device memory).
+__global__ void set_replay_counts_kernel(uint32_t* block, uint32_t tokens, uint32_t tiles, uint32_t splits,
+                                         uint32_t layer_plus_one) {
+    if (threadIdx.x == 0 && blockIdx.x == 0) {
+        block[kReplayTokens] = tokens;
+        block[kReplayTiles] = tiles;
+        block[kReplaySplits] = splits;
+        block[kReplayLayer] = layer_plus_one;
+    }
+}
+
+// What a recorded program depends on: everything that becomes a kernel argument or a grid size.
+struct ProgramKey {
+    psi_hip_split_kv_variant variant;
+    uint32_t totals[3];
+    psi_hip_page_table_layout layout;
+    uint32_t layer, replay_mode, layer_is_parameter;
+    uint32_t num_workers, group_tiles, num_row_groups, max_active_q_tile_tokens;
+    uint64_t kv_pages_bytes, partial_scratch_bytes;
+    const void* pointers[20];
+};
+
+ProgramKey make_key(const psi_hip_gqa_layer_input& in, bool layer_is_parameter) {
+    ProgramKey k;
+    std::memset(&k, 0, sizeof(k));  // padding bytes take part in the comparison
+    const psi_hip_gqa_batch_metadata& md = *in.batch_metadata;
+    k.variant = md.variant;
+    k.totals[0] = md.shape.num_total_tokens;
+    k.totals[1] = md.shape.num_total_q_token_tiles;
+    k.totals[2] = md.shape.num_total_kv_splits;
+    k.layout = in.page_table_layout;
+    k.layer = layer_is_parameter ? 0u : in.gqa_layer_index;
+    k.layer_is_parameter = layer_is_parameter;
+    k.replay_mode = in.replay_mode;
+    k.num_workers = md.worker_cu ? md.num_workers : 0;
+    k.group_tiles = md.row_groups ? md.group_tiles : 0;
+    k.num_row_groups = md.row_groups ? md.num_row_groups : 0;
+    k.max_active_q_tile_tokens = md.max_active_q_tile_tokens;
+    k.kv_pages_bytes = in.kv_pages_bytes;
+    k.partial_scratch_bytes = in.partial_scratch_bytes;
+    const void* p[20] = {in.qgkv, in.q, in.k, in.v, in.g, in.kv_pages, in.page_ids, in.q_norm_weight,
+                         in.k_norm_weight, in.q_norm_rope, in.partial_scratch, in.output, md.req_slots,
+                         md.flat_token_indices, md.q_token_tiles, md.kv_splits, md.cu_kv_splits,
+                         md.partial_row_index, md.worker_cu, md.row_groups};
+    std::memcpy(k.pointers, p, sizeof(p));
+    return k;
+}
+
+struct Program {
+    ProgramKey key;
+    hipGraphExec_t exec = nullptr;
+};
+
+}  // namespace
+}  // namespace psi
+
+struct psi_hip_gqa_replay_cache {
+    psi_hip_ctx* ctx = nullptr;
+    psi_hip_gqa_layer_config cfg;
+    uint32_t* device_counts = nullptr;
+    uint32_t max_programs = 0;
+    std::list<psi::Program> programs;  // most recently used first
+    uint64_t recordings = 0, replays = 0;
+};
+
+using namespace psi;
+
+extern "C" int psi_hip_gqa_layer_scratch_bytes(const psi_hip_gqa_layer_config* cfg,
+                                               const psi_hip_split_kv_variant* variant, uint32_t num_total_kv_splits,
+                                               uint64_t* out_bytes) {
+    PSI_REQUIRE(cfg != nullptr && variant != nullptr, "GQA layer config and variant must not be null");
+    if (variant->kind == PSI_HIP_VARIANT_TILED_Q)
+        return psi_hip_split_kv_tiled_q_scratch_bytes(&cfg->attention, variant->q_token_tile_size, num_total_kv_splits,
+                                                      out_bytes);
+    PSI_REQUIRE(variant->kind == PSI_HIP_VARIANT_SINGLE_Q, "unknown SplitKV variant %u", variant->kind);
+    return psi_hip_split_kv_single_q_scratch_bytes(&cfg->attention, num_total_kv_splits, out_bytes);
+}
+
+extern "C" int psi_hip_gqa_layer_record(psi_hip_ctx* ctx, const psi_hip_gqa_layer_config* cfg,
+                                        const psi_hip_gqa_layer_input* input) {
+    return record_layer(ctx, cfg, input);
+}
+
+extern "C" int psi_hip_gqa_replay_cache_create(psi_hip_ctx* ctx, const psi_hip_gqa_layer_config* cfg,
+                                               uint32_t* device_counts, uint32_t max_programs,
+                                               psi_hip_gqa_replay_cache** out_cache) {
+    PSI_REQUIRE(ctx != nullptr && out_cache != nullptr, "ctx and out_cache must not be null");
+    PSI_REQUIRE(device_counts != nullptr, "the replay cache needs a device count block (u32[4])");
+    PSI_REQUIRE(max_programs > 0, "the replay cache must hold at least one program");
+    LayerPlan plan;
+    int rc = make_layer_plan(cfg, &plan);
+    if (rc != PSI_HIP_OK) return rc;
+    auto* cache = new psi_hip_gqa_replay_cache();
+    cache->ctx = ctx;
+    cache->cfg = *cfg;
+    cache->device_counts = device_counts;
+    cache->max_programs = max_programs;
+    *out_cache = cache;
+    return PSI_HIP_OK;
+}
+
+extern "C" int psi_hip_gqa_replay_cache_destroy(psi_hip_gqa_replay_cache* cache) {
+    if (cache == nullptr) return PSI_HIP_OK;
+    for (auto& p : cache->programs)
+        if (p.exec) (void)hipGraphExecDestroy(p.exec);
+    delete cache;
+    return PSI_HIP_OK;
+}
+
+extern "C" int psi_hip_gqa_replay_cache_stats(const psi_hip_gqa_replay_cache* cache, uint32_t* programs,
+                                              uint64_t* recordings, uint64_t* replays) {
+    PSI_REQUIRE(cache != nullptr, "replay cache must not be null");
+    if (programs) *programs = (uint32_t)cache->programs.size();
+    if (recordings) *recordings = cache->recordings;
+    if (replays) *replays = cache->replays;
+    return PSI_HIP_OK;
+}
+
+// Records the layer at the capacities of `input` into a new program.
+static int record_program(psi_hip_gqa_replay_cache* cache, const psi_hip_gqa_layer_input* input, hipGraphExec_t* out) {
+    psi_hip_ctx* ctx = cache->ctx;
+    // by-value counts = the capacities (they cut the grids and bound the device-side counts)
+    psi_hip_gqa_batch_metadata md = *input->batch_metadata;
+    md.shape.num_tokens = md.shape.num_total_tokens;
+    md.shape.num_q_token_tiles = md.shape.num_total_q_token_tiles;
+    md.shape.num_kv_splits = md.shape.num_total_kv_splits;
+    psi_hip_gqa_layer_input at_capacity = *input;
+    at_capacity.batch_metadata = &md;
+
+    const uint32_t* bound_before = ctx->replay_counts;
+    const bool timing_before = ctx->timing;
+    ctx->replay_counts = cache->device_counts;
+    ctx->timing = false;  // event records would become nodes of the program
+    hipGraph_t graph = nullptr;
+    hipError_t e = hipStreamBeginCapture(ctx->stream, hipStreamCaptureModeThreadLocal);
+    int rc = PSI_HIP_OK;
+    if (e != hipSuccess) {
+        rc = fail(PSI_HIP_ERR_RUNTIME, "hipStreamBeginCapture failed: %s", hipGetErrorString(e));
+    } else {
+        rc = record_layer(ctx, &cache->cfg, &at_capacity);
+        e = hipStreamEndCapture(ctx->stream, &graph);  // always ends the capture, also after a failed recording
+        if (rc == PSI_HIP_OK && e != hipSuccess)
+            rc = fail(PSI_HIP_ERR_RUNTIME, "hipStreamEndCapture failed: %s", hipGetErrorString(e));
+    }
+    ctx->replay_counts = bound_before;
+    ctx->timing = timing_before;
+    if (rc == PSI_HIP_OK) {
+        e = hipGraphInstantiate(out, graph, nullptr, nullptr, 0);
+        if (e != hipSuccess) rc = fail(PSI_HIP_ERR_RUNTIME, "hipGraphInstantiate failed: %s", hipGetErrorString(e));
+    }
+    if (graph) (void)hipGraphDestroy(graph);
+    return rc;
+}
+
+extern "C" int psi_hip_gqa_replay_cache_submit(psi_hip_gqa_replay_cache* cache, const psi_hip_gqa_layer_input* input,
+                                               uint32_t gqa_layer_parameter, int* out_recorded) {
+    PSI_REQUIRE(cache != nullptr, "replay cache must not be null");
+    psi_hip_ctx* ctx = cache->ctx;
+    PSI_REQUIRE(ctx->stream != nullptr, "the replay cache records by stream capture: the context needs a created stream");
+    int rc = check_input(input);
+    if (rc != PSI_HIP_OK) return rc;
+    PSI_REQUIRE(gqa_layer_parameter <= input->page_table_layout.num_gqa_layers,
+                "GQA page-table index exceeds layer count");
+    if (out_recorded) *out_recorded = 0;
+    const ProgramKey key = make_key(*input, gqa_layer_parameter != 0);
+    auto it = cache->programs.begin();
+    for (; it != cache->programs.end(); ++it)
+        if (std::memcmp(&it->key, &key, sizeof(key)) == 0) break;
+    if (it == cache->programs.end()) {
+        Program p;
+        p.key = key;
+        rc = record_program(cache, input, &p.exec);
+        if (rc != PSI_HIP_OK) return rc;
+        cache->programs.push_front(p);
+        cache->recordings += 1;
+        if (out_recorded) *out_recorded = 1;
+        while (cache->programs.size() > cache->max_programs) {
+            // a dropped program may still be running: wait for the stream before its nodes go away
+            PSI_HIP_CHECK(hipStreamSynchronize(ctx->stream));
+            (void)hipGraphExecDestroy(cache->programs.back().exec);
+            cache->programs.pop_back();
+        }
+    } else if (it != cache->programs.begin()) {
+        cache->programs.splice(cache->programs.begin(), cache->programs, it);
+    }
+    const psi_hip_gqa_replay_shape& s = input->batch_metadata->shape;
+    hipLaunchKernelGGL(set_replay_counts_kernel, dim3(1), dim3(64), 0, ctx->stream, cache->device_counts, s.num_tokens,
+                       s.num_q_token_tiles, s.num_kv_splits, gqa_layer_parameter);
+    PSI_HIP_CHECK(hipGetLastError());
+    PSI_HIP_CHECK(hipGraphLaunch(cache->programs.front().exec, ctx->stream));
+    cache->replays += 1;
+    return PSI_HIP_OK;
+}

@@ -517,26 +517,74 @@ class GQAReplayShape:
 
 
 class GQAMetadataBuffers:
-    """Capacity-sized metadata refreshed per microbatch: host arrays plus device copies."""
+    """Capacity-sized metadata refreshed per microbatch (`GQAMetadataBuffers`, batch_metadata.rs:71-126).
 
-    def __init__(self, device: Optional[Device], max_tokens: int, max_kv_splits: Optional[int] = None):
+    With a device, the host arrays are views into one pinned staging buffer and the device arrays views into one
+    device buffer of the same layout: both keep their addresses for the object's lifetime (a recorded program
+    holds them), and `upload()` is one or two asynchronous copies on the device's stream.  Without a device
+    (`None`) only the host arrays exist.  `max_workers`: room for the rows a balanced worker plan may add."""
+
+    def __init__(self, device: Optional[Device], max_tokens: int, max_kv_splits: Optional[int] = None,
+                 max_workers: int = 256):
         assert max_tokens > 0, "GQA batch metadata requires tokens"
         self.device, self._max_tokens = device, max_tokens
         self._max_kv_splits = max_kv_splits if max_kv_splits is not None else max_tokens
-        self.h_req_slots = np.zeros(max_tokens, np.uint32)
-        self.h_flat_token_indices = np.zeros(max_tokens, np.uint32)
-        self.h_q_token_tiles = np.zeros(max_tokens * 2, np.uint32)
-        self.h_kv_splits = np.zeros(self._max_kv_splits * 3, np.uint32)
-        self.h_cu_kv_splits = np.zeros(max_tokens + 1, np.uint32)
+        self._max_workers = max_workers
+        rows = self._max_kv_splits + max_workers
+        sizes = (("req_slots", max_tokens), ("flat_token_indices", max_tokens), ("q_token_tiles", 2 * max_tokens),
+                 ("cu_kv_splits", max_tokens + 1), ("worker_cu", max_workers + 1), ("kv_splits", 3 * rows),
+                 ("partial_row_index", rows))
+        self._offsets, total = {}, 0
+        for name, n in sizes:
+            self._offsets[name] = (total, n)
+            total += n
+        self._words = total
+        if device is not None:
+            import torch
+
+            self._h_all_t = torch.zeros(total, dtype=torch.int32, pin_memory=True)
+            h_all = self._h_all_t.numpy().view(np.uint32)
+            self._d_all = torch.zeros(total, dtype=torch.int32, device=device.torch_device)
+        else:
+            h_all = np.zeros(total, np.uint32)
+            self._d_all = None
+
+        def host(name, used=None):
+            off, n = self._offsets[name]
+            return h_all[off:off + (n if used is None else used)]
+
+        def dev(name):
+            if self._d_all is None:
+                return None
+            off, n = self._offsets[name]
+            return self._d_all[off:off + n]
+
+        self.h_req_slots, self.d_req_slots = host("req_slots"), dev("req_slots")
+        self.h_flat_token_indices, self.d_flat_token_indices = host("flat_token_indices"), dev("flat_token_indices")
+        self.h_q_token_tiles, self.d_q_token_tiles = host("q_token_tiles"), dev("q_token_tiles")
+        self.h_cu_kv_splits, self.d_cu_kv_splits = host("cu_kv_splits"), dev("cu_kv_splits")
+        self._h_worker_cu_all, self._d_worker_cu_all = host("worker_cu"), dev("worker_cu")
+        self._h_kv_splits_all = host("kv_splits")
+        self.h_kv_splits = self._h_kv_splits_all[:3 * self._max_kv_splits]  # what the planner may fill
+        self.d_kv_splits = dev("kv_splits")
+        self._h_row_index_all, self._d_row_index_all = host("partial_row_index"), dev("partial_row_index")
         self._shape, self._variant = None, None
-        self.d_req_slots = self.d_flat_token_indices = self.d_q_token_tiles = None
-        self.d_kv_splits = self.d_cu_kv_splits = None
         self.h_partial_row_index = self.d_partial_row_index = None
+        self.h_worker_cu = self.d_worker_cu = None
+        self.num_workers = 0
         self.h_row_groups = self.d_row_groups = None
+        self._h_row_groups_t = self._d_row_groups_all = None
         self.group_tiles = self.num_row_groups = 0
+        self.max_active_q_tile_tokens = 0
+        self._uploaded = None  # event after the last upload: the staging buffer is free again once it has passed
 
     def max_tokens(self) -> int:
         return self._max_tokens
+
+    def _staging_free(self):
+        if self._uploaded is not None:
+            self._uploaded.synchronize()
+            self._uploaded = None
 
     def _update(self, req_slots, token_indices, cu_tokens, variant, mode, caller_tokens=0, boundaries=(),
                 partition_tokens=0):
@@ -547,6 +595,8 @@ class GQAMetadataBuffers:
         def p(a):
             return a.ctypes.data_as(ctypes.POINTER(ctypes.c_uint32))
 
+        self._staging_free()
+        self.h_kv_splits = self._h_kv_splits_all[:3 * self._max_kv_splits]
         L.check(L.load().psi_hip_gqa_metadata_update(
             self._max_tokens, L.u32_array(req_slots), L.u32_array(token_indices), L.u32_array(cu_tokens),
             len(req_slots), ctypes.byref(v), mode, caller_tokens, L.u32_array(boundaries), len(boundaries),
@@ -557,19 +607,34 @@ class GQAMetadataBuffers:
                                      bool(shape.reduce_sdpa_partial_outputs))
         self._variant = variant
         self.h_partial_row_index = self.d_partial_row_index = None  # rows are in plan order again
+        self.h_worker_cu = self.d_worker_cu = None
+        self.num_workers = 0
         self.h_row_groups = self.d_row_groups = None
         self.group_tiles = self.num_row_groups = 0
+        q_lens = np.diff(np.asarray(cu_tokens, dtype=np.int64))
+        self.max_active_q_tile_tokens = (int(min(q_lens.max(), variant.q_token_tile_size)) if variant.is_tiled()
+                                         else 0)
         if self.device is not None:
             self.upload()
         return self._shape
 
     def upload(self):
-        d = self.device
-        self.d_req_slots = d.from_numpy(self.h_req_slots)
-        self.d_flat_token_indices = d.from_numpy(self.h_flat_token_indices)
-        self.d_q_token_tiles = d.from_numpy(self.h_q_token_tiles)
-        self.d_kv_splits = d.from_numpy(self.h_kv_splits)
-        self.d_cu_kv_splits = d.from_numpy(self.h_cu_kv_splits)
+        """Host arrays -> their device copies, asynchronously on the device's stream (pinned staging, fixed
+        device addresses).  Everything up to the last planned row of kv_splits goes in one copy."""
+        if self.device is None:
+            return
+        import torch
+
+        rows = self._shape.num_total_sdpa_map_task_templates if self._shape is not None else 0
+        off, _ = self._offsets["kv_splits"]
+        end = off + 3 * rows
+        with torch.cuda.stream(self.device.stream):
+            self._d_all[:end].copy_(self._h_all_t[:end], non_blocking=True)
+            if self.h_partial_row_index is not None:
+                o, _ = self._offsets["partial_row_index"]
+                self._d_all[o:o + rows].copy_(self._h_all_t[o:o + rows], non_blocking=True)
+            self._uploaded = torch.cuda.Event()
+            self._uploaded.record(self.device.stream)
 
     def update(self, req_slots, token_indices, cu_tokens, split_kv_variant):
         return self._update(req_slots, token_indices, cu_tokens, split_kv_variant, L.CAPACITY_EXACT)
@@ -597,7 +662,8 @@ class GQAMetadataBuffers:
         rows first.  `d_partial_row_index` must then be passed to the combine."""
         s = self._shape
         n = s.num_sdpa_map_task_templates
-        self.h_partial_row_index = np.zeros(max(len(self.h_kv_splits) // 3, 1), np.uint32)
+        self._staging_free()
+        self.h_partial_row_index = self._h_row_index_all
         self.h_partial_row_index[:] = np.arange(len(self.h_partial_row_index), dtype=np.uint32)
 
         def p(a):
@@ -605,8 +671,8 @@ class GQAMetadataBuffers:
 
         L.check(L.load().psi_hip_split_kv_order_longest_first(p(self.h_kv_splits), n, p(self.h_partial_row_index)))
         if self.device is not None:
+            self.d_partial_row_index = self._d_row_index_all
             self.upload()
-            self.d_partial_row_index = self.device.from_numpy(self.h_partial_row_index)
         return self.h_partial_row_index
 
     def group_rows(self, config) -> int:
@@ -617,7 +683,17 @@ class GQAMetadataBuffers:
         s = self._shape
         assert s is not None and self._variant.is_tiled()
         n = s.num_sdpa_map_task_templates
-        table = np.full(max(n, 1) * 32, L.SENTINEL, np.uint32)
+        words = max(n, 1) * 32
+        if self.device is not None:
+            import torch
+
+            if self._h_row_groups_t is None or self._h_row_groups_t.numel() < words:
+                self._h_row_groups_t = torch.zeros(words, dtype=torch.int32, pin_memory=True)
+                self._d_row_groups_all = torch.zeros(words, dtype=torch.int32, device=self.device.torch_device)
+            table = self._h_row_groups_t.numpy().view(np.uint32)[:words]
+        else:
+            table = np.zeros(words, np.uint32)
+        table[:] = L.SENTINEL
         tiles, groups = ctypes.c_uint32(), ctypes.c_uint32()
         cfg = config.struct()
 
@@ -628,20 +704,27 @@ class GQAMetadataBuffers:
             ctypes.byref(cfg), config.q_token_tile_size, p(self.h_kv_splits), n, p(self.h_q_token_tiles),
             s.num_q_token_tiles, p(self.h_req_slots), p(table), len(table), ctypes.byref(tiles), ctypes.byref(groups)))
         self.group_tiles, self.num_row_groups = tiles.value, groups.value
-        self.h_row_groups = table[:max(tiles.value * groups.value, 1)].copy()
+        used = max(tiles.value * groups.value, 1)
+        self.h_row_groups = table[:used]
         if self.device is not None and groups.value:
-            self.d_row_groups = self.device.from_numpy(self.h_row_groups)
+            import torch
+
+            with torch.cuda.stream(self.device.stream):
+                self._d_row_groups_all[:used].copy_(self._h_row_groups_t[:used], non_blocking=True)
+            self.d_row_groups = self._d_row_groups_all
         return groups.value
 
     def balance(self, num_workers: int):
-        """Re-cuts the current SingleQ plan into rows grouped for `num_workers` equal-work decode
-        workgroups per KV head (psi_hip_split_kv_balance_plan); adjacent pieces of one token inside a group
-        become one row.  Returns the new replay shape."""
+        """Re-cuts the current plan into rows grouped for `num_workers` equal-work map workgroups per KV head
+        (psi_hip_split_kv_balance_plan); adjacent pieces of one token inside a group become one row.  Returns the
+        new replay shape."""
         s = self._shape
         assert s is not None
+        assert num_workers <= self._max_workers, "more workers than the metadata buffers reserve rows for"
         groups = s.num_q_token_tiles if self._variant.is_tiled() else s.num_tokens  # what cu_kv_splits counts
         rows_in = s.num_sdpa_map_task_templates
-        cap = max(rows_in + num_workers, self._max_kv_splits)  # the arrays are reused by the next update
+        cap = self._max_kv_splits + self._max_workers
+        assert rows_in + num_workers <= cap
         out_splits = np.full(cap * 3, L.SENTINEL, np.uint32)
         out_cu = np.zeros(self._max_tokens + 1, np.uint32)
         worker_cu = np.zeros(num_workers + 1, np.uint32)
@@ -653,13 +736,18 @@ class GQAMetadataBuffers:
         L.check(L.load().psi_hip_split_kv_balance_plan(p(self.h_kv_splits), rows_in, p(self.h_cu_kv_splits),
                                                        groups, num_workers, p(out_splits), cap, p(out_cu),
                                                        p(worker_cu), ctypes.byref(n_out)))
-        self.h_kv_splits, self.h_cu_kv_splits, self.h_worker_cu = out_splits, out_cu, worker_cu
+        self._staging_free()
+        self.h_kv_splits = self._h_kv_splits_all
+        self.h_kv_splits[:] = out_splits
+        self.h_cu_kv_splits[:] = out_cu
+        self.h_worker_cu = self._h_worker_cu_all[:num_workers + 1]
+        self.h_worker_cu[:] = worker_cu
         self.num_workers = num_workers
         self._shape = GQAReplayShape(s.num_tokens, s.num_total_tokens, s.num_q_token_tiles,
                                      s.num_total_q_token_tiles, n_out.value, n_out.value, True)
         if self.device is not None:
+            self.d_worker_cu = self._d_worker_cu_all
             self.upload()
-            self.d_worker_cu = self.device.from_numpy(worker_cu)
         return self._shape
 
     def replay_shape(self) -> GQAReplayShape:
@@ -669,6 +757,20 @@ class GQAMetadataBuffers:
     def split_kv_variant(self) -> GQASplitKVVariant:
         assert self._variant is not None, "GQA batch metadata must be updated before recording"
         return self._variant
+
+    def struct(self, shape: Optional[GQAReplayShape] = None):
+        """The batch as the layer entry points take it (psi_hip_gqa_batch_metadata): device addresses of the
+        arrays, the shape (`shape` overrides the capacities, e.g. a replay bucket) and the launch plans."""
+        assert self.device is not None and self._shape is not None
+        s = shape or self._shape
+        return L.BatchMetadataStruct(
+            L.ReplayShapeStruct(s.num_tokens, s.num_total_tokens, s.num_q_token_tiles, s.num_total_q_token_tiles,
+                                s.num_sdpa_map_task_templates, s.num_total_sdpa_map_task_templates,
+                                int(s.reduce_sdpa_partial_outputs)),
+            self._variant.struct(), _ptr(self.d_req_slots), _ptr(self.d_flat_token_indices),
+            _ptr(self.d_q_token_tiles), _ptr(self.d_kv_splits), _ptr(self.d_cu_kv_splits),
+            _ptr(self.d_partial_row_index), _ptr(self.d_worker_cu), self.num_workers, _ptr(self.d_row_groups),
+            self.group_tiles, self.num_row_groups, self.max_active_q_tile_tokens)
 
 
 # ------------------------------------------------------------------ request page table
@@ -959,3 +1061,241 @@ class GQASplitKVTiledQKernels:
             _ptr(q_token_tiles), _ptr(cu_sdpa_partial_outputs), _ptr(output), s.num_total_tokens,
             s.num_total_q_token_tiles, s.num_total_sdpa_map_task_templates, num_active_q_token_tiles,
             _ptr(partial_row_index), _gate_ref(gate)))
+
+
+# ------------------------------------------------------------------ the attention layer
+
+
+@dataclass(frozen=True)
+class GQACore:
+    """`GQACore` (crates/inference-executor-core/src/attn/gqa/core.rs:3-91)."""
+    model_layer_index: int
+    hidden_dim: int
+    head_dim: int
+    num_q_heads: int
+    num_kv_heads: int
+    scale: float
+
+    def validate(self):
+        assert self.hidden_dim > 0 and self.head_dim > 0 and self.num_q_heads > 0 and self.num_kv_heads > 0
+        assert self.num_q_heads % self.num_kv_heads == 0 and self.scale > 0.0
+
+    def q_dim(self) -> int:
+        return self.num_q_heads * self.head_dim
+
+    def k_dim(self) -> int:
+        return self.num_kv_heads * self.head_dim
+
+    def qgkv_dim(self) -> int:
+        return 2 * self.q_dim() + 2 * self.k_dim()
+
+    def qkv_dim(self) -> int:
+        return self.q_dim() + 2 * self.k_dim()
+
+
+@dataclass(frozen=True)
+class GQAMetalConfig:
+    """`GQAMetalConfig` (attn/gqa/backend.rs:114-146) without the matmul quantisation fields; the name is the
+    reference's, the device is not."""
+    page_bytes: int
+    rope_dim: int
+    norm_eps: float
+    rope_theta: float
+    rope_scaling: RopeScaling = RopeScaling()
+    io_dtype: Dtype = Dtype.Bfloat16
+
+
+class GQAReplayMode(IntEnum):
+    Exact = L.REPLAY_EXACT
+    Bucketed = L.REPLAY_BUCKETED
+
+
+@dataclass
+class GQAKVCacheBindings:
+    kv_pages: object
+    page_ids: object
+
+
+@dataclass
+class GQAWeights:
+    """The norm weights of `GQAWeights` (backend.rs:156-166); the projection weights stay with the caller."""
+    q_norm_weight: object
+    k_norm_weight: object
+
+
+class GQAScratch:
+    """`GQAScratch` (attn/gqa/scratch.rs:17-92) as far as this path uses it: the projection output, the
+    normalised queries, the partial states (one buffer, sized by the library) and the layer's output."""
+
+    def __init__(self, device: Device, gqa: "GQA", max_tokens: int, max_kv_splits: Optional[int] = None):
+        import torch
+
+        core, dt = gqa.core, gqa.config.io_dtype.torch()
+        dev = device.torch_device
+        self.max_tokens = max_tokens
+        self.max_kv_splits = max_kv_splits if max_kv_splits is not None else max_tokens
+        width = core.qgkv_dim() if gqa.gated else core.qkv_dim()
+        self.qgkv = torch.zeros(max_tokens * width, dtype=dt, device=dev)
+        self.q_norm_rope = torch.zeros(max_tokens * core.q_dim(), dtype=dt, device=dev)
+        # the wider of the two variants' layouts for the split capacity
+        nbytes = 0
+        for variant in (GQASplitKVVariant.SingleQ(256, 256, 1), GQASplitKVVariant.TiledQ(8, 16, 1)):
+            nbytes = max(nbytes, gqa.scratch_bytes(variant, self.max_kv_splits))
+        self.sdpa_partial = torch.zeros(nbytes, dtype=torch.uint8, device=dev)
+        self.attention_output = torch.zeros(max_tokens * core.q_dim(), dtype=dt, device=dev)
+
+
+@dataclass
+class GQAInput:
+    """`GQAInput` (backend.rs:169-182).  `qgkv`: the projection output (defaults to `scratch.qgkv`); or pass
+    rows already split, normalised and rotated as `q`, `k`, `v` (and optionally gates `g`).  `output`: defaults
+    to `scratch.attention_output`."""
+    page_table_layout: GQAPageTableLayout
+    gqa_layer_index: int
+    batch_metadata: GQAMetadataBuffers
+    kv_cache: GQAKVCacheBindings
+    scratch: GQAScratch
+    weights: Optional[GQAWeights] = None
+    replay_mode: GQAReplayMode = GQAReplayMode.Bucketed
+    qgkv: object = None
+    q: object = None
+    k: object = None
+    v: object = None
+    g: object = None
+    output: object = None
+    shape: Optional[GQAReplayShape] = None  # overrides batch_metadata.replay_shape() (e.g. wider capacities)
+
+
+class GQA:
+    """`GQA` / `UngatedGQA` (attn/gqa/backend.rs:214-392, ungated_backend.rs:104-180): the attention part of a
+    layer behind `record`.  `gated`: projection rows [q_0|g_0|...|k|v] and a sigmoid gate on the output."""
+
+    def __init__(self, device: Device, core: GQACore, config: GQAMetalConfig, gated: bool = True):
+        core.validate()
+        self.device, self.core, self.config, self.gated = device, core, config, gated
+        self.split_kv = GQASplitKV.new(GQASplitKVConfig(config.io_dtype, config.page_bytes, core.num_q_heads,
+                                                        core.num_kv_heads, core.head_dim))
+
+    @staticmethod
+    def new(device, core, config, gated=True):
+        return GQA(device, core, config, gated)
+
+    def struct(self):
+        c, k = self.core, self.config
+        return L.LayerConfigStruct(_cfg_struct(c.num_q_heads, c.num_kv_heads, c.head_dim, c.scale, k.page_bytes,
+                                               k.io_dtype),
+                                   int(self.gated), k.rope_dim, k.norm_eps, k.rope_theta, k.rope_scaling.struct())
+
+    def num_tokens_per_page(self) -> int:
+        return self.split_kv.config.num_tokens_per_page()
+
+    def scratch_bytes(self, variant: GQASplitKVVariant, num_total_kv_splits: int) -> int:
+        out, cfg, v = ctypes.c_uint64(), self.struct(), variant.struct()
+        L.check(L.load().psi_hip_gqa_layer_scratch_bytes(ctypes.byref(cfg), ctypes.byref(v), num_total_kv_splits,
+                                                         ctypes.byref(out)))
+        return out.value
+
+    def new_scratch(self, max_tokens: int, max_kv_splits: Optional[int] = None) -> GQAScratch:
+        return GQAScratch(self.device, self, max_tokens, max_kv_splits)
+
+    def select_variant(self, batch_metadata, token_indices, cu_tokens, policy=None) -> GQASplitKVVariant:
+        return select_split_kv_variant(self.split_kv, batch_metadata.max_tokens(), policy, token_indices, cu_tokens)
+
+    def prepare(self, batch_metadata: GQAMetadataBuffers, req_slots, token_indices, cu_tokens) -> GQAReplayShape:
+        """`GQA::prepare` (backend.rs:289-304)."""
+        variant = self.select_variant(batch_metadata, token_indices, cu_tokens)
+        return batch_metadata.update(req_slots, token_indices, cu_tokens, variant)
+
+    def prepare_bucketed(self, batch_metadata, req_slots, token_indices, cu_tokens,
+                         policy: GQAReplayBucketPolicy) -> GQAReplayShape:
+        """`GQA::prepare_bucketed` (backend.rs:306-323)."""
+        variant = self.select_variant(batch_metadata, token_indices, cu_tokens, policy)
+        return batch_metadata.update_bucketed(req_slots, token_indices, cu_tokens, variant, policy)
+
+    def prepare_fixed_partition(self, batch_metadata, req_slots, token_indices, cu_tokens, partition_tokens: int,
+                                balanced: bool = True, grouped: bool = False,
+                                variant: Optional[GQASplitKVVariant] = None) -> GQAReplayShape:
+        """Not in the reference: partitions of fixed length instead of the greedy budget, then (by default) the
+        balanced worker plan that gives every compute unit an equal share of the batch's tiles; `grouped`
+        selects the row-group plan of the prefill-chunk map instead."""
+        if variant is None:
+            variant = self.select_variant(batch_metadata, token_indices, cu_tokens)
+        shape = batch_metadata.update_fixed_partition(req_slots, token_indices, cu_tokens, variant, partition_tokens)
+        if grouped and variant.is_tiled():
+            c, k = self.core, self.config
+            tiled_cfg = GQASplitKVTiledQConfig(c.num_q_heads, c.num_kv_heads, c.head_dim, variant.q_head_tile_size,
+                                               variant.q_token_tile_size, variant.kv_token_tile_size, c.scale,
+                                               k.page_bytes, k.io_dtype, None)
+            if batch_metadata.group_rows(tiled_cfg):
+                return shape
+        if balanced:
+            shape = batch_metadata.balance(balanced_workers(self.split_kv.config))
+        return shape
+
+    def input_struct(self, inp: GQAInput):
+        """(psi_hip_gqa_layer_input, keep-alive objects) for an input."""
+        md = inp.batch_metadata.struct(inp.shape)
+        sc = inp.scratch
+        qgkv = inp.qgkv if (inp.qgkv is not None or inp.q is not None) else sc.qgkv
+        out = inp.output if inp.output is not None else sc.attention_output
+        w = inp.weights
+        s = L.LayerInputStruct(
+            inp.page_table_layout.struct(), inp.gqa_layer_index, int(inp.replay_mode), ctypes.pointer(md),
+            _ptr(qgkv if inp.q is None else None), _ptr(inp.q), _ptr(inp.k), _ptr(inp.v), _ptr(inp.g),
+            _ptr(inp.kv_cache.kv_pages), _nbytes(inp.kv_cache.kv_pages), _ptr(inp.kv_cache.page_ids),
+            _ptr(w.q_norm_weight if w else None), _ptr(w.k_norm_weight if w else None), _ptr(sc.q_norm_rope),
+            _ptr(sc.sdpa_partial), _nbytes(sc.sdpa_partial), _ptr(out))
+        return s, (md, out)
+
+    def record(self, inp: GQAInput):
+        """`GQA::record` (backend.rs:394-658): issues the layer's launches on the device's stream and returns
+        the output buffer (the reference returns the caller-owned buffer it was given, too)."""
+        cfg = self.struct()
+        s, keep = self.input_struct(inp)
+        L.check(self.device.lib.psi_hip_gqa_layer_record(self.device.ctx, ctypes.byref(cfg), ctypes.byref(s)))
+        return keep[1]
+
+
+class GQAReplayCache:
+    """One recorded program (HIP graph) per capacity bucket of a layer: the reference's replay-program store keyed
+    by `(variant, total tokens, total Q-token tiles, total KV splits)` with the active counts bound at submission
+    (crates/inference-executor-core/src/replay.rs:4-87, backend.rs:55-57).  The device must launch on a created
+    stream (not the null stream)."""
+
+    def __init__(self, device: Device, gqa: GQA, max_programs: int = 32):
+        import torch
+
+        self.device, self.gqa = device, gqa
+        self.counts = torch.zeros(4, dtype=torch.int32, device=device.torch_device)
+        handle, cfg = ctypes.c_void_p(), gqa.struct()
+        L.check(device.lib.psi_hip_gqa_replay_cache_create(device.ctx, ctypes.byref(cfg), _ptr(self.counts),
+                                                           max_programs, ctypes.byref(handle)))
+        self.handle = handle
+
+    def submit(self, inp: GQAInput, gqa_layer_parameter: int = 0) -> bool:
+        """Replays the program of the input's bucket (recording it first when there is none); True if this call
+        recorded.  `gqa_layer_parameter` n > 0 binds page-table layer n - 1 at submission."""
+        s, _keep = self.gqa.input_struct(inp)
+        recorded = ctypes.c_int()
+        L.check(self.device.lib.psi_hip_gqa_replay_cache_submit(self.handle, ctypes.byref(s), gqa_layer_parameter,
+                                                                ctypes.byref(recorded)))
+        return bool(recorded.value)
+
+    def stats(self):
+        """(programs held, recordings, replays)."""
+        p, r, n = ctypes.c_uint32(), ctypes.c_uint64(), ctypes.c_uint64()
+        L.check(self.device.lib.psi_hip_gqa_replay_cache_stats(self.handle, ctypes.byref(p), ctypes.byref(r),
+                                                               ctypes.byref(n)))
+        return p.value, r.value, n.value
+
+    def close(self):
+        if self.handle:
+            self.device.sync()
+            self.device.lib.psi_hip_gqa_replay_cache_destroy(self.handle)
+            self.handle = None
+
+    def __del__(self):
+        try:
+            self.close()
+        except Exception:
+            pass

@@ -50,6 +50,9 @@ class Workload:
     flat_k: np.ndarray           # storage [tokens, Hkv, D]
     flat_v: np.ndarray
     seed: int
+    outlier_rate: float = 0.0    # K elements set to +-outlier_sigma * input_scale (applied on the device too)
+    outlier_sigma: float = 8.0
+    input_scale: float = 1.0
 
     @property
     def page_bytes(self) -> int:
@@ -137,7 +140,40 @@ def make_workload(seed: int, context_lens: Sequence[int], num_q_heads: int, num_
     if scale is None:
         scale = 1.0 / float(np.sqrt(head_dim))
     return Workload(num_q_heads, num_kv_heads, head_dim, dtype, float(scale), tokens_per_page, layout, layer,
-                    num_pages, req_slots, token_indices, cu_tokens, table, pages, q, flat_k, flat_v, seed)
+                    num_pages, req_slots, token_indices, cu_tokens, table, pages, q, flat_k, flat_v, seed,
+                    outlier_rate, outlier_sigma, input_scale)
+
+
+def device_pages(device: G.Device, w: Workload):
+    """The workload's page arena in HBM: uploaded when the workload carries host pages, else drawn on the device
+    from the workload's seed (same distribution, K outliers included)."""
+    import torch
+
+    dev = device.torch_device
+    torch_dtype = w.dtype.torch()
+    if w.pages is not None:
+        return device.from_numpy(w.pages.reshape(-1))
+    n = w.num_pages * 2 * w.num_kv_heads * w.tokens_per_page * w.head_dim
+    gen = torch.Generator(device=dev)
+    gen.manual_seed(w.seed)
+    pages = torch.empty(n, dtype=torch_dtype, device=dev)
+    chunk = 1 << 26
+    for start in range(0, n, chunk):
+        end = min(n, start + chunk)
+        pages[start:end] = (torch.randn(end - start, generator=gen, device=dev, dtype=torch.float32) *
+                            w.input_scale).to(torch_dtype)
+    if w.outlier_rate > 0:
+        # large-magnitude K outliers: the K half of each page comes first
+        half = w.num_kv_heads * w.tokens_per_page * w.head_dim
+        by_page = pages.view(w.num_pages, 2 * half)
+        rows = 1 << 12
+        for start in range(0, w.num_pages, rows):
+            k_part = by_page[start:start + rows, :half]
+            draw = torch.rand(k_part.shape, generator=gen, device=dev)
+            value = torch.where(draw < w.outlier_rate / 2, w.outlier_sigma * w.input_scale,
+                                -w.outlier_sigma * w.input_scale).to(torch_dtype)
+            k_part.copy_(torch.where(draw < w.outlier_rate, value, k_part))
+    return pages
 
 
 class DeviceWorkload:
@@ -146,28 +182,20 @@ class DeviceWorkload:
     def __init__(self, device: G.Device, w: Workload, partition_tokens: Optional[int] = None,
                  max_tokens: Optional[int] = None, variant: Optional[G.GQASplitKVVariant] = None,
                  f32_output: bool = False, balanced: bool = False, longest_first: bool = False,
-                 grouped: bool = False, fused_append: bool = False, num_workers: Optional[int] = None):
+                 grouped: bool = False, fused_append: bool = False, num_workers: Optional[int] = None,
+                 pages=None, page_ids=None):
+        """`pages` / `page_ids`: an arena and a page table already on the device (shared with another workload
+        of the same step) instead of this workload's own."""
         import torch
 
         self.device, self.w = device, w
         self.torch_dtype = w.dtype.torch()
         dev = device.torch_device
-        if w.pages is not None:
-            self.pages = device.from_numpy(w.pages.reshape(-1))
-        else:
-            n = w.num_pages * 2 * w.num_kv_heads * w.tokens_per_page * w.head_dim
-            gen = torch.Generator(device=dev)
-            gen.manual_seed(w.seed)
-            self.pages = torch.empty(n, dtype=self.torch_dtype, device=dev)
-            chunk = 1 << 26
-            for start in range(0, n, chunk):
-                end = min(n, start + chunk)
-                self.pages[start:end] = torch.randn(end - start, generator=gen, device=dev,
-                                                    dtype=torch.float32).to(self.torch_dtype)
+        self.pages = pages if pages is not None else device_pages(device, w)
         self.q = device.from_numpy(w.q.reshape(-1))
         self.flat_k = device.from_numpy(w.flat_k.reshape(-1))
         self.flat_v = device.from_numpy(w.flat_v.reshape(-1))
-        self.page_ids = device.from_numpy(w.page_ids)
+        self.page_ids = page_ids if page_ids is not None else device.from_numpy(w.page_ids)
         split_kv = G.GQASplitKV.new(G.GQASplitKVConfig(w.dtype, w.page_bytes, w.num_q_heads, w.num_kv_heads,
                                                        w.head_dim))
         q_lens = np.diff(w.cu_tokens)
@@ -225,6 +253,10 @@ class DeviceWorkload:
         self.grouped = bool(grouped) and variant.is_tiled()
         if self.grouped:
             self.meta.group_rows(self.cfg)
+        self.gqa = G.GQA(device, G.GQACore(0, w.num_q_heads * w.head_dim, w.head_dim, w.num_q_heads, w.num_kv_heads,
+                                           w.scale),
+                         G.GQAMetalConfig(w.page_bytes, 2, 1e-6, 10000.0, io_dtype=w.dtype), gated=False)
+        self._layer_input = None
 
     def append(self):
         m = self.meta
@@ -286,13 +318,36 @@ class DeviceWorkload:
                                                 worker_cu=m.d_worker_cu if self.balanced else None,
                                                 num_workers=m.num_workers if self.balanced else 0)
 
+    def layer_input(self) -> "G.GQAInput":
+        """The step as the layer entry takes it: split, normalised rows in; the workload's own buffers as scratch."""
+        if self._layer_input is None:
+            w = self.w
+
+            class _Scratch:  # the buffers of `GQAScratch` this path touches
+                qgkv = None
+                q_norm_rope = None
+                sdpa_partial = self.scratch.buffer
+                attention_output = self.output
+
+            self._layer_input = G.GQAInput(w.layout, w.layer, self.meta, G.GQAKVCacheBindings(self.pages, self.page_ids),
+                                           _Scratch, replay_mode=G.GQAReplayMode.Bucketed, q=self.q, k=self.flat_k,
+                                           v=self.flat_v, output=self.output)
+        self._layer_input.kv_cache = G.GQAKVCacheBindings(self.pages, self.page_ids)
+        return self._layer_input
+
     def step(self):
-        """One layer-step: append the new tokens, then attend (the new tokens see themselves)."""
-        if self.fused_append:
-            self.append_map()
-        else:
-            self.append()
-            self.map()
+        """One layer-step: append the new tokens, then attend (the new tokens see themselves).  Issued through
+        the layer entry (`GQA.record`) unless the decode step is asked to launch its append separately, which
+        exercises the component entry points one by one."""
+        if self.fused_append or self.variant.is_tiled():
+            self.device.f32_output(self.f32_output)
+            try:
+                self.gqa.record(self.layer_input())
+            finally:
+                self.device.f32_output(False)
+            return
+        self.append()
+        self.map()
         self.reduce()
 
     def output_f32(self) -> np.ndarray:
@@ -311,6 +366,65 @@ class DeviceWorkload:
         if t.dtype in (torch.bfloat16, torch.float16, torch.int16):
             return t.view(torch.int16).cpu().numpy().view(np.uint16)
         return t.cpu().numpy()
+
+
+class MixedStep:
+    """A step that holds prefill chunks and decode tokens at once, over one arena and one page table.  The
+    reference would run one SplitKV variant for the whole batch; here the requests with more than
+    `chunk_min_tokens` new tokens go through the multi-query kernels with the row-group plan and the others
+    through the decode kernels (balanced worker plan, append inside the map launch): two `GQA.record` calls on
+    the same stream.  The chunk requests must come first in the batch, so that either part's tokens are one
+    contiguous run of the flat q / k / v / output rows."""
+
+    def __init__(self, device: G.Device, w: Workload, decode_partition: int = 512,
+                 chunk_partition: Optional[int] = None, chunk_min_tokens: int = 8, f32_output: bool = False):
+        import dataclasses
+
+        import torch
+
+        q_lens = np.diff(w.cu_tokens).astype(np.int64)
+        is_chunk = q_lens > chunk_min_tokens
+        n_chunk = int(is_chunk.sum())
+        assert 0 < n_chunk < len(q_lens) and is_chunk[:n_chunk].all(), "chunk requests first, then decode requests"
+        self.device, self.w, self.f32_output = device, w, f32_output
+        self.pages, self.page_ids = device_pages(device, w), device.from_numpy(w.page_ids)
+        cut = int(w.cu_tokens[n_chunk])
+
+        def part(lo_req, hi_req, lo_tok, hi_tok):
+            return dataclasses.replace(
+                w, req_slots=w.req_slots[lo_req:hi_req], token_indices=w.token_indices[lo_req:hi_req],
+                cu_tokens=(w.cu_tokens[lo_req:hi_req + 1] - w.cu_tokens[lo_req]).astype(np.uint32),
+                q=w.q.reshape(w.num_tokens, -1)[lo_tok:hi_tok].reshape(-1),
+                flat_k=w.flat_k.reshape(w.num_tokens, -1)[lo_tok:hi_tok].reshape(-1),
+                flat_v=w.flat_v.reshape(w.num_tokens, -1)[lo_tok:hi_tok].reshape(-1))
+
+        chunk_w, decode_w = part(0, n_chunk, 0, cut), part(n_chunk, len(q_lens), cut, w.num_tokens)
+        if chunk_partition is None:  # one kv_split row per query tile: no split of the context
+            chunk_partition = max(2048, 1 << int(chunk_w.context_lens.max() - 1).bit_length())
+        group = w.num_q_heads // w.num_kv_heads
+        self.chunk = DeviceWorkload(device, chunk_w, partition_tokens=chunk_partition, f32_output=f32_output,
+                                    grouped=True, variant=G.GQASplitKVVariant.TiledQ(8, 16, min(group, 8)),
+                                    pages=self.pages, page_ids=self.page_ids)
+        self.decode = DeviceWorkload(device, decode_w, partition_tokens=decode_partition, f32_output=f32_output,
+                                     balanced=True, fused_append=True, pages=self.pages, page_ids=self.page_ids)
+        assert not self.decode.variant.is_tiled()
+
+    def step(self):
+        self.chunk.step()
+        self.decode.step()
+
+    def output_f32(self) -> np.ndarray:
+        return np.concatenate([self.chunk.output_f32(), self.decode.output_f32()])
+
+
+def config_c5(seed: int = 5, chunk: int = 2048, prefix: int = 4096, batch: int = 128, lo: int = 512,
+              hi: int = 32768) -> Workload:
+    """Mixed chunked-prefill + decode step: one sequence appends `chunk` tokens on a `prefix`-token history, `batch`
+    decode sequences with contexts uniform in [lo, hi] append one token each; 24 Q / 4 KV heads, D=256, bf16,
+    16-token pages of one shuffled pool."""
+    ctx = np.concatenate([[prefix + chunk], config_c2_context_lens(seed, batch, lo, hi) + 1])
+    return make_workload(seed, ctx, 24, 4, 256, G.Dtype.Bfloat16, 16, q_lens=[chunk] + [1] * batch,
+                         host_pages=False)
 
 
 def config_c1(seed: int = 1) -> Workload:

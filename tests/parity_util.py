@@ -75,3 +75,67 @@ def importlib_workloads(psi):
     import importlib
 
     return importlib.import_module(psi.__name__ + ".workloads")
+
+
+def oracle_sample(oracle, dw, picks, num_threads=16):
+    """Attention of the requests `picks` of a device workload recomputed by the scalar oracle from the device's
+    own pages (after the step's append): the picked requests' pages are gathered on the device into a compact
+    arena with a table of its own, so that a multi-gigabyte arena never crosses to the host.  Returns the f32
+    outputs [tokens of the picks][Hq * D] in pick order."""
+    import torch
+
+    w = dw.w
+    lay = w.layout
+    assert lay.num_page_ids_per_block == 1
+    per_slot = lay.num_gqa_layers * lay.num_blocks
+    page_elems = 2 * w.num_kv_heads * w.tokens_per_page * w.head_dim
+    table = dw.page_ids.cpu().numpy().view(np.uint32)
+    ctx = w.context_lens
+    counts = [-(-int(ctx[r]) // w.tokens_per_page) for r in picks]
+    blocks = max(counts)
+    ids, sub_table, cursor = [], np.zeros(len(picks) * blocks, np.uint32), 0
+    for i, (r, n) in enumerate(zip(picks, counts)):
+        start = int(w.req_slots[r]) * per_slot + w.layer * lay.num_blocks
+        ids.append(table[start:start + n].astype(np.int64))
+        sub_table[i * blocks:i * blocks + n] = np.arange(cursor, cursor + n)
+        cursor += n
+    index = torch.from_numpy(np.concatenate(ids)).to(dw.pages.device)
+    sub_pages = dw.pages.view(w.num_pages, page_elems).index_select(0, index)
+    dw.device.sync()
+    if sub_pages.dtype in (torch.bfloat16, torch.float16):
+        sub_pages = sub_pages.view(torch.int16).cpu().numpy().view(np.uint16)
+    else:
+        sub_pages = sub_pages.cpu().numpy()
+    q_lens = np.diff(w.cu_tokens)
+    rows = np.concatenate([np.arange(w.cu_tokens[r], w.cu_tokens[r + 1]) for r in picks])
+    q = w.q.reshape(w.num_tokens, -1)[rows].reshape(-1)
+    cu = np.concatenate([[0], np.cumsum([q_lens[r] for r in picks])]).astype(np.uint32)
+    out = oracle.paged_gqa(w.num_q_heads, w.num_kv_heads, w.head_dim, w.scale, w.page_bytes, oracle_dtype(oracle, w),
+                           (len(picks), 1, blocks, 1), 0, np.arange(len(picks), dtype=np.uint32),
+                           w.token_indices[list(picks)], cu, q, sub_pages.reshape(-1), sub_table,
+                           num_threads=num_threads)
+    return np.asarray(out).reshape(len(rows), -1), rows
+
+
+def assert_appended_lines(dw):
+    """Every K / V line of this step's new tokens sits in its page slot, bit for bit (checked on the device:
+    the arena does not cross to the host)."""
+    import torch
+
+    w = dw.w
+    lay = w.layout
+    assert lay.num_page_ids_per_block == 1
+    per_slot = lay.num_gqa_layers * lay.num_blocks
+    q_lens = np.diff(w.cu_tokens)
+    slots = np.repeat(w.req_slots, q_lens).astype(np.int64)
+    pos = np.concatenate([w.token_indices[r] + np.arange(n) for r, n in enumerate(q_lens)]).astype(np.int64)
+    table = dw.page_ids.cpu().numpy().view(np.uint32).astype(np.int64)
+    page = table[slots * per_slot + w.layer * lay.num_blocks + pos // w.tokens_per_page]
+    dev = dw.pages.device
+    arena = dw.pages.view(w.num_pages, 2, w.num_kv_heads, w.tokens_per_page, w.head_dim)
+    page_t, off_t = torch.from_numpy(page).to(dev), torch.from_numpy(pos % w.tokens_per_page).to(dev)
+    for kind, flat in ((0, dw.flat_k), (1, dw.flat_v)):
+        got = arena[page_t, kind, :, off_t, :]  # [tokens, Hkv, D]
+        exp = flat.view(w.num_tokens, w.num_kv_heads, w.head_dim)
+        assert torch.equal(got.view(torch.int16) if got.element_size() == 2 else got,
+                           exp.view(torch.int16) if exp.element_size() == 2 else exp), "appended lines differ"

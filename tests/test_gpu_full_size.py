@@ -7,7 +7,8 @@ Plus the long-context / large-magnitude-K case at a length the oracle still cove
 import numpy as np
 import pytest
 
-from parity_util import assert_outputs_close, importlib_workloads, layout_tuple, oracle_dtype, run_and_check
+from parity_util import (assert_appended_lines, assert_outputs_close, importlib_workloads, layout_tuple, oracle_dtype,
+                         oracle_sample, run_and_check)
 
 pytestmark = pytest.mark.gpu
 
@@ -95,32 +96,65 @@ def test_long_context_with_large_keys(psi, oracle, device):
         assert np.abs(out - first).max() < 2e-5
 
 
-def test_c3_full_length_split_invariance(psi, device):
-    """4 x 131072 tokens (1.07 GB of K/V), 32 vs 256 partitions per sequence."""
+# How `bench.py` launches a decode step (balanced worker plan, append inside the map launch) and a verify step
+# (balanced worker plan), next to the plain launch (one workgroup per plan row, separate append).
+DECODE_MODES = [pytest.param({}, id="row per workgroup"),
+                pytest.param({"balanced": True, "longest_first": True, "fused_append": True}, id="bench default")]
+VERIFY_MODES = [pytest.param({}, id="row per workgroup"), pytest.param({"balanced": True}, id="bench default")]
+
+
+def _sampled_check(oracle, dw, picks, what):
+    """Oracle on the picked requests from the device's own pages; appended K/V lines bit-exact for every token."""
+    exp, rows = oracle_sample(oracle, dw, picks)
+    got = dw.output_f32().reshape(dw.w.num_tokens, -1)[rows]
+    stats = assert_outputs_close(got.reshape(-1), exp.reshape(-1), what)
+    assert_appended_lines(dw)
+    return stats
+
+
+@pytest.mark.parametrize("how", DECODE_MODES)
+def test_c3_full_length_with_outliers(psi, oracle, device, how):
+    """4 x 131072 tokens (1.07 GB of K/V), 16 Q / 2 KV heads, K outliers of 8 sigma at rate 1e-4 across the whole
+    arena: 32 vs 256 partitions per sequence agree to f32 rounding, and one whole sequence (all 16 heads over
+    131072 keys) matches the scalar oracle run on the device's pages."""
+    import torch
+
     wl = importlib_workloads(psi)
-    w = wl.make_workload(33, [131072] * 4, 16, 2, 256, psi.Dtype.Bfloat16, 16, host_pages=False)
+    w = wl.make_workload(33, [131072] * 4, 16, 2, 256, psi.Dtype.Bfloat16, 16, host_pages=False, outlier_rate=1e-4,
+                         outlier_sigma=8.0)
     outs = []
     for partition in (4096, 512):
-        dw = wl.DeviceWorkload(device, w, partition_tokens=partition, f32_output=True)
+        dw = wl.DeviceWorkload(device, w, partition_tokens=partition, f32_output=True, **how)
         dw.step()
         outs.append(dw.output_f32())
+        if partition == 512:
+            k_half = dw.pages.view(w.num_pages, 2, -1)[:256, 0].float().abs()
+            rate = float((k_half >= 7.9).float().mean())
+            assert 0.5e-4 < rate < 2e-4, f"outlier rate {rate:.2e}"
+            _sampled_check(oracle, dw, [2], "C3 sampled sequence")
         del dw
     assert np.isfinite(outs[0]).all()
     assert np.abs(outs[0] - outs[1]).max() < 2e-5
 
 
-def test_verify_full_batch_split_and_placement(psi, device):
-    """C4's batch (64 sequences, contexts 2048..16384, 2 tokens each): partition invariance of the
-    multi-query kernels at full size."""
+@pytest.mark.parametrize("q_len", [2, 4])
+@pytest.mark.parametrize("how", VERIFY_MODES)
+def test_c4_verify_full_batch(psi, oracle, device, how, q_len):
+    """C4's batch (64 sequences, contexts 2048..16384, 24 Q / 4 KV heads) with one and with three drafts per
+    sequence, causal among the new tokens: 512- and 4096-token partitions agree to f32 rounding, the shortest,
+    median and longest sequence match the scalar oracle, every appended line is in its page slot."""
     wl = importlib_workloads(psi)
-    ctx = wl.config_c2_context_lens(4, 64, 2048, 16384) + 2
-    w = wl.make_workload(4, ctx, 24, 4, 256, psi.Dtype.Bfloat16, 16, q_lens=2, host_pages=False)
+    ctx = wl.config_c2_context_lens(4, 64, 2048, 16384) + q_len
+    w = wl.make_workload(4, ctx, 24, 4, 256, psi.Dtype.Bfloat16, 16, q_lens=q_len, host_pages=False)
     outs = []
     for partition in (512, 4096):
-        dw = wl.DeviceWorkload(device, w, partition_tokens=partition, f32_output=True)
-        assert dw.variant.is_tiled()
+        dw = wl.DeviceWorkload(device, w, partition_tokens=partition, f32_output=True, **how)
+        assert dw.variant.is_tiled() and dw.balanced == bool(how)
         dw.step()
         outs.append(dw.output_f32())
+        if partition == 512:
+            order = np.argsort(w.context_lens)
+            _sampled_check(oracle, dw, [int(order[0]), int(order[32]), int(order[-1])], f"C4 q_len {q_len} sampled")
         del dw
     assert np.isfinite(outs[0]).all()
     assert np.abs(outs[0] - outs[1]).max() < 2e-5
@@ -155,17 +189,174 @@ def test_c5_prefill_chunk_full_size(psi, oracle, device):
     assert_outputs_close(outs["grouped 2048"][picks].reshape(-1), exp, "C5 chunk sampled")
 
 
-def test_c5_decode_batch_full_size(psi, device):
-    """C5's decode side: 128 sequences with contexts 512..32768 (about 8.7 GB of K/V), split-count
-    invariance between 512- and 4096-token partitions."""
+@pytest.mark.parametrize("how", DECODE_MODES)
+def test_c5_decode_batch_full_size(psi, oracle, device, how):
+    """C5's decode side: 128 sequences with contexts 512..32768 (about 8.7 GB of K/V).  512- and 4096-token
+    partitions agree to f32 rounding; the shortest, median and longest sequence match the scalar oracle."""
     wl = importlib_workloads(psi)
     ctx = wl.config_c2_context_lens(55, 128, 512, 32768)
     w = wl.make_workload(55, ctx, 24, 4, 256, psi.Dtype.Bfloat16, 16, host_pages=False)
     outs = []
     for partition in (512, 4096):
-        dw = wl.DeviceWorkload(device, w, partition_tokens=partition, f32_output=True)
+        dw = wl.DeviceWorkload(device, w, partition_tokens=partition, f32_output=True, **how)
         dw.step()
         outs.append(dw.output_f32())
+        if partition == 512:
+            order = np.argsort(w.context_lens)
+            _sampled_check(oracle, dw, [int(order[0]), int(order[64]), int(order[-1])], "C5 decode sampled")
         del dw
     assert np.isfinite(outs[0]).all()
     assert np.abs(outs[0] - outs[1]).max() < 2e-5
+
+
+def test_c5_mixed_step(psi, oracle, device):
+    """C5 as one step: a 2048-token prefill chunk on a 4096-token prefix and 128 decode sequences with contexts
+    512..32768 over one arena and one page table -- the chunk through the row-group map, the decode tokens
+    through the balanced decode map, both appends included.  Sampled against the scalar oracle on the device's
+    pages: chunk tokens at the start, at a 512 boundary, in the middle and at the end; the shortest, median and
+    longest decode sequence.  Every appended line is in its page slot."""
+    wl = importlib_workloads(psi)
+    w = wl.config_c5()
+    step = wl.MixedStep(device, w, f32_output=True)
+    assert step.chunk.meta.num_row_groups > 0 and step.decode.balanced and step.decode.fused_append
+    step.step()
+    got = step.output_f32().reshape(w.num_tokens, -1)
+    assert np.isfinite(got).all()
+    # decode side: whole requests
+    order = 1 + np.argsort(w.context_lens[1:])
+    picks = [int(order[0]), int(order[64]), int(order[-1])]
+    dec = step.decode
+    exp, rows = oracle_sample(oracle, dec, [p - 1 for p in picks])
+    assert_outputs_close(dec.output_f32().reshape(dec.w.num_tokens, -1)[rows].reshape(-1), exp.reshape(-1),
+                         "C5 mixed, decode side")
+    assert_appended_lines(dec)
+    assert_appended_lines(step.chunk)
+    # chunk side: single query tokens of the chunk, each as a one-token request at its own position
+    import dataclasses
+
+    tokens = np.array([0, 1, 511, 512, 1023, 2040, 2047])
+    cw = step.chunk.w
+    probe_w = dataclasses.replace(cw, req_slots=np.repeat(cw.req_slots, len(tokens)),
+                                  token_indices=(cw.token_indices[0] + tokens).astype(np.uint32),
+                                  cu_tokens=np.arange(len(tokens) + 1, dtype=np.uint32),
+                                  q=cw.q.reshape(cw.num_tokens, -1)[tokens].reshape(-1))
+
+    class _Probe:  # what oracle_sample reads of a device workload
+        w, pages, page_ids, device = probe_w, step.pages, step.page_ids, step.device
+
+    exp, _ = oracle_sample(oracle, _Probe, list(range(len(tokens))))
+    assert_outputs_close(got[tokens].reshape(-1), exp.reshape(-1), "C5 mixed, chunk side")
+
+
+def test_c4_batch_accept_rollback_cycle(psi, oracle, host_oracle, device):
+    """C4 end to end on its full batch: 64 requests with 2048..16384 cached tokens, the library's allocator and
+    token window next to the Python restatement of the reference's (`oracle/host_oracle.py`), three drafts per
+    request.  Two verify steps (4 new tokens per request through the multi-query kernels, balanced plan): after
+    each, a seeded accept mask commits a prefix of the drafts, so the next step starts at the first rejected
+    position and overwrites it.  Checked: every query, block hand-over and token window of the two bookkeepers
+    agree at every step, the device page table equals the restatement's table bit for bit after the rollbacks,
+    cached lengths advance by 1 + accepted, no page is freed below block granularity, the appended lines are in
+    their page slots, and sampled sequences match the scalar oracle on the device's pages (so a step sees the
+    accepted history and none of the rejected drafts)."""
+    import dataclasses
+    import importlib
+
+    import torch
+    from test_runtime_blocks import OracleImpl, ProductImpl, public
+
+    wl = importlib_workloads(psi)
+    hq, hkv, d, p, spec = 24, 4, 256, 16, 3
+    rng = np.random.default_rng(404)
+    cached0 = wl.config_c2_context_lens(4, 64, 2048, 16384)
+    n_req = len(cached0)
+    blocks_per_req = [-(-(int(c) + 2 * (spec + 1) + p) // p) for c in cached0]
+    num_pages = sum(blocks_per_req) + 8
+    max_blocks = max(blocks_per_req)
+    layout = psi.GQAPageTableLayout(n_req, 1, max_blocks, 1)
+    table = psi.GQARequestPageTable(device, layout)
+    oracle_table = np.zeros(layout.num_page_ids(), np.uint32)
+    o, lib = OracleImpl(host_oracle), ProductImpl(psi)
+    ao, al = o.allocator(num_pages), lib.allocator(num_pages)
+    both = []
+
+    def sync(r, bo, bl):
+        so, sl = bo.prepare_blocks(), bl.prepare_blocks()
+        assert so == sl, f"request {r}: block hand-over differs"
+        for i, ids in enumerate(sl[1][0]):
+            table.write_page_ids(r, 0, sl[0] + i, ids, num_cache_pages=num_pages)
+            oracle_table[r * max_blocks + so[0] + i] = so[1][0][i][0]
+
+    for r, c in enumerate(cached0):
+        prompt = [100000 * r + i for i in range(int(c) + 1)]  # c cached tokens after the prefill + the decode input
+        bo, bl = o.blocks(ao, p, 1, 1, prompt), lib.blocks(al, p, 1, 1, prompt)
+        while True:
+            so, sl = bo.init(), bl.init()
+            assert so == sl
+            if so >= int(c):
+                break
+        qo, ql = bo.prepare(int(c)), bl.prepare(int(c))
+        assert public(qo) == public(ql) and qo["kind"] == "Prefill" and qo["token_index"] == 0
+        sync(r, bo, bl)
+        bo.commit_prefill(qo), bl.commit_prefill(ql)
+        drafts = [50000 + 10 * r + j for j in range(spec)]
+        bo.set_spec(drafts), bl.set_spec(drafts)
+        both.append((bo, bl))
+    assert (ao.used(), ao.free()) == (al.used(), al.free())
+
+    page_elems = 2 * hkv * p * d
+    base = wl.make_workload(44, [32] * 2, hq, hkv, d, psi.Dtype.Bfloat16, p, host_pages=False)  # a template
+    pages, accepted_total, used_before = None, 0, al.used()
+    for step in range(2):
+        queries = []
+        for r, (bo, bl) in enumerate(both):
+            _, _, _, ready, queued, drafts = bl.state()
+            budget = len(ready) + len(queued) + len(drafts)
+            while bl.b.ready_token_slots() < budget:
+                so, sl = bo.init(), bl.init()
+                assert so == sl and so != "ResourceLimitExceeded"
+            qo, ql = bo.prepare(budget), bl.prepare(budget)
+            assert public(qo) == public(ql)
+            assert ql["kind"] == "Decode" and len(ql["tokens"]) == 1 and len(ql["spec_tokens"]) == spec
+            sync(r, bo, bl)
+            queries.append((qo, ql))
+        starts = np.array([ql["token_index"] for _, ql in queries], np.uint32)
+        q_len = 1 + spec
+        total = n_req * q_len
+        w = dataclasses.replace(
+            base, layout=layout, num_pages=num_pages, req_slots=np.arange(n_req, dtype=np.uint32),
+            token_indices=starts, cu_tokens=(np.arange(n_req + 1) * q_len).astype(np.uint32),
+            page_ids=oracle_table.copy(), pages=None, seed=404,
+            q=wl.to_storage(rng.standard_normal((total, hq, d), dtype=np.float32), psi.Dtype.Bfloat16).reshape(-1),
+            flat_k=wl.to_storage(rng.standard_normal((total, hkv, d), dtype=np.float32), psi.Dtype.Bfloat16).reshape(-1),
+            flat_v=wl.to_storage(rng.standard_normal((total, hkv, d), dtype=np.float32), psi.Dtype.Bfloat16).reshape(-1))
+        # the device table is the one the library's hand-overs wrote; it must equal the restatement's
+        device.sync()
+        assert np.array_equal(table.page_ids_buffer().cpu().numpy().view(np.uint32), oracle_table), f"step {step}"
+        if pages is None:
+            pages = wl.device_pages(device, w)  # random history in every page
+        dw = wl.DeviceWorkload(device, w, partition_tokens=512, f32_output=True, balanced=True, pages=pages,
+                               page_ids=table.page_ids_buffer())
+        assert dw.variant.is_tiled()
+        dw.step()
+        order = np.argsort(w.context_lens)
+        _sampled_check(oracle, dw, [int(order[0]), int(order[31]), int(order[-1])], f"C4 cycle step {step}")
+        del dw
+        for r, ((bo, bl), (qo, ql)) in enumerate(zip(both, queries)):
+            accept = int(rng.integers(0, spec + 1))  # seeded accept mask: a prefix of the drafts
+            accepted_total += accept
+            before = len(bl.b.cached_tokens())
+            sampled = 70000 + 100 * step + r
+            new_drafts = [60000 + 100 * step + 10 * r + j for j in range(spec)]
+            bo.commit_decode(qo, qo["spec_tokens"][:accept], sampled, new_drafts)
+            bl.commit_decode(ql, ql["spec_tokens"][:accept], sampled, new_drafts)
+            assert len(bl.b.cached_tokens()) == before + 1 + accept
+            if r % 16 == 0:
+                assert bo.state() == bl.state()
+            assert bo.counts() == bl.counts()
+        # rejected drafts free nothing: pages are owned per block, and no block was released
+        assert al.used() >= used_before and (ao.used(), ao.free()) == (al.used(), al.free())
+    assert 0 < accepted_total < 2 * n_req * spec
+    assert o.bitmap(ao) == lib.bitmap(al)
+    for bo, bl in both:
+        bo.drop(), bl.drop()
+    assert (ao.used(), al.used()) == (0, 0)

@@ -5,21 +5,26 @@ active counts as kernel arguments and use no memset, so a captured step is self-
 import numpy as np
 import pytest
 
-from parity_util import importlib_workloads
+from parity_util import assert_outputs_close, importlib_workloads, oracle_step
 
 pytestmark = pytest.mark.gpu
 
 
 @pytest.mark.parametrize("q_len,fused_append", [(1, False), (2, False), (1, True)])
-def test_captured_layer_step_replays(psi, device, q_len, fused_append):
-    """`fused_append`: the append rides in the decode map launch (two nodes in the graph instead of three)."""
+def test_captured_layer_step_replays(psi, oracle, device, q_len, fused_append):
+    """`fused_append`: the append rides in the decode map launch (two nodes in the graph instead of three).
+    Every replay equals the eager step bit for bit, and the eager step matches the CPU oracle on the inputs of
+    that replay."""
+    import dataclasses
+
     import torch
 
     wl = importlib_workloads(psi)
     w = wl.make_workload(101 + q_len, [700, 33, 1500, 512, 64], 24, 4, 256, psi.Dtype.Bfloat16, 16, q_lens=q_len)
-    dw = wl.DeviceWorkload(device, w, partition_tokens=512, fused_append=fused_append)
+    dw = wl.DeviceWorkload(device, w, partition_tokens=512, fused_append=fused_append, f32_output=True)
     assert dw.fused_append == fused_append
     pristine = dw.pages.clone()
+    current = w
 
     def eager():
         dw.pages.copy_(pristine)
@@ -49,29 +54,34 @@ def test_captured_layer_step_replays(psi, device, q_len, fused_append):
         # new inputs each time: queries and the new tokens' K/V change, the history is restored
         dw.pages.copy_(pristine)
         if replay:
-            for t in (dw.q, dw.flat_k, dw.flat_v):
-                t.copy_(device.from_numpy(wl.to_storage(rng.standard_normal(t.numel(), dtype=np.float32),
-                                                       w.dtype)))
+            fresh = {}
+            for name, t in (("q", dw.q), ("flat_k", dw.flat_k), ("flat_v", dw.flat_v)):
+                fresh[name] = wl.to_storage(rng.standard_normal(t.numel(), dtype=np.float32), w.dtype)
+                t.copy_(device.from_numpy(fresh[name]))
+            current = dataclasses.replace(w, **fresh)
         expected = eager()
+        n = w.num_tokens * w.num_q_heads * w.head_dim
+        assert_outputs_close(expected[:n].cpu().numpy(), oracle_step(oracle, current)[1], f"eager step of replay {replay}")
         dw.pages.copy_(pristine)
         dw.output.zero_()
         torch.cuda.synchronize()
         graph.replay()
         torch.cuda.synchronize()
-        assert torch.equal(dw.output.view(torch.int16), expected.view(torch.int16)), f"replay {replay}"
+        assert torch.equal(dw.output.view(torch.int32), expected.view(torch.int32)), f"replay {replay}"
         if replay == 0:
-            assert torch.equal(dw.output.view(torch.int16), base.view(torch.int16))
+            assert torch.equal(dw.output.view(torch.int32), base.view(torch.int32))
         # eager work of the program between replays
         _ = (dw.output.float() * 2).sum().item()
 
 
 @pytest.mark.parametrize("balanced", [False, True])
-def test_one_captured_step_serves_every_batch_of_its_bucket(psi, device, balanced):
+def test_one_captured_step_serves_every_batch_of_its_bucket(psi, oracle, device, balanced):
     """Device-side active counts (`ReplayU32::Parameter` of the reference): a decode step captured once at the
     capacity of its bucket (5 tokens, 16 splits) with the counts bound, then replayed for batches of 5, 3, 1 and
     4 requests after refreshing only the metadata arrays, the inputs and the 16-byte count block.  Each replay
-    equals the eager step with by-value counts, bit for bit, in the output rows and in the page arena; rows
-    beyond the active count keep a canary.  `balanced`: the plan is re-cut into equal worker shares on the host
+    equals the eager step with by-value counts, bit for bit, in the output rows (f32, before output rounding) and
+    in the page arena, and that eager step matches the CPU oracle on the batch; rows beyond the active count keep
+    a canary.  `balanced`: the plan is re-cut into equal worker shares on the host
     for every batch and the append rides in the map launch; the grid (workers x KV heads) is the same for all."""
     import torch
 
@@ -95,8 +105,9 @@ def test_one_captured_step_serves_every_batch_of_its_bucket(psi, device, balance
     d_counts = torch.zeros(4, **i32)
     d_workers = torch.zeros(workers + 1, **i32)
     q, fk, fv = torch.zeros_like(dw.q), torch.zeros_like(dw.flat_k), torch.zeros_like(dw.flat_v)
-    out = torch.zeros(cap_tokens * row, dtype=torch.bfloat16, device=device.torch_device)
+    out = torch.zeros(cap_tokens * row, dtype=torch.float32, device=device.torch_device)
     host_meta = psi.GQAMetadataBuffers(None, cap_tokens, max_kv_splits=cap_splits)
+    device.f32_output(True)  # taken when a combine is launched or captured
 
     def load_batch(picks):
         n = len(picks)
@@ -104,16 +115,16 @@ def test_one_captured_step_serves_every_batch_of_its_bucket(psi, device, balance
                                                  512)
         if balanced:
             shape = host_meta.balance(workers)
-            d_workers.copy_(device.from_numpy(host_meta.h_worker_cu))
+            d_workers.copy_(device.from_numpy(host_meta.h_worker_cu.copy()))
             d_splits.fill_(-1)
-            d_splits[:len(host_meta.h_kv_splits)].copy_(device.from_numpy(host_meta.h_kv_splits))
-            d_slots.copy_(device.from_numpy(host_meta.h_req_slots))
-            d_pos.copy_(device.from_numpy(host_meta.h_flat_token_indices))
-            d_cu.copy_(device.from_numpy(host_meta.h_cu_kv_splits))
+            d_splits.copy_(device.from_numpy(host_meta.h_kv_splits[:cap_splits * 3].copy()))
+            d_slots.copy_(device.from_numpy(host_meta.h_req_slots.copy()))
+            d_pos.copy_(device.from_numpy(host_meta.h_flat_token_indices.copy()))
+            d_cu.copy_(device.from_numpy(host_meta.h_cu_kv_splits.copy()))
         if not balanced:
             for dst, src in ((d_slots, host_meta.h_req_slots), (d_pos, host_meta.h_flat_token_indices),
-                             (d_splits, host_meta.h_kv_splits), (d_cu, host_meta.h_cu_kv_splits)):
-                dst.copy_(device.from_numpy(src))
+                             (d_splits, host_meta.h_kv_splits[:cap_splits * 3]), (d_cu, host_meta.h_cu_kv_splits)):
+                dst.copy_(device.from_numpy(src.copy()))
         for dst, src, width in ((q, dw.q, row), (fk, dw.flat_k, kv_row), (fv, dw.flat_v, kv_row)):
             dst.zero_()
             for i, r in enumerate(picks):
@@ -150,25 +161,38 @@ def test_one_captured_step_serves_every_batch_of_its_bucket(psi, device, balance
     finally:
         device.bind_replay_counts(None)
         device.use_stream(main)
+        device.f32_output(False)
     torch.cuda.synchronize()
+
+    import dataclasses
 
     for picks in ([0, 1, 2, 3, 4], [2, 0, 4], [3], [4, 3, 1, 0]):
         shape = load_batch(picks)
         n = shape.num_tokens
         dw.pages.copy_(pristine)
         out.fill_(-768.0)
+        device.f32_output(True)
         step(shape.num_tokens, shape.num_sdpa_map_task_templates)  # eager, counts by value
+        device.f32_output(False)
         device.sync()
         eager_out, eager_pages = out.clone(), dw.pages.clone()
+        sub = dataclasses.replace(w, req_slots=w.req_slots[picks], token_indices=w.token_indices[picks],
+                                  cu_tokens=np.arange(len(picks) + 1, dtype=np.uint32),
+                                  q=w.q.reshape(-1, row)[picks].reshape(-1),
+                                  flat_k=w.flat_k.reshape(-1, kv_row)[picks].reshape(-1),
+                                  flat_v=w.flat_v.reshape(-1, kv_row)[picks].reshape(-1))
+        exp_pages, exp = oracle_step(oracle, sub)
+        assert_outputs_close(eager_out[:n * row].cpu().numpy(), exp, f"eager step {picks}")
+        assert np.array_equal(eager_pages.view(torch.int16).cpu().numpy().view(np.uint16).reshape(exp_pages.shape), exp_pages)
         dw.pages.copy_(pristine)
         out.fill_(-768.0)
         scratch.buffer.zero_()
         torch.cuda.synchronize()
         graph.replay()
         torch.cuda.synchronize()
-        assert torch.equal(out.view(torch.int16), eager_out.view(torch.int16)), picks
+        assert torch.equal(out.view(torch.int32), eager_out.view(torch.int32)), picks
         assert torch.equal(dw.pages.view(torch.int16), eager_pages.view(torch.int16)), picks
-        assert (out[n * row:].float() == -768.0).all() and (out[:n * row].float() != -768.0).any()
+        assert (out[n * row:] == -768.0).all() and (out[:n * row] != -768.0).any()
         _ = out.float().sum().item()  # eager work between replays
 
 
