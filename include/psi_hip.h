@@ -570,6 +570,20 @@ int psi_hip_gqa_layer_scratch_bytes(const psi_hip_gqa_layer_config* cfg, const p
 int psi_hip_gqa_layer_record(psi_hip_ctx* ctx, const psi_hip_gqa_layer_config* cfg,
                              const psi_hip_gqa_layer_input* input);
 
+/* psi_hip_gqa_layer_record with the partial states in a buffer built into the library instead of
+ * input->partial_scratch (which is ignored, as is partial_scratch_bytes).  No counterpart in the reference.  It is
+ * for callers that cannot allocate device memory: code under HIP graph capture, tight serving loops, harnesses
+ * that forbid allocation.  The call allocates nothing on the host or the device and only launches kernels; the
+ * buffer is a static device array of PSI_HIP_STATIC_SCRATCH_BYTES that every GPU the library runs on holds until
+ * the process ends (its address is looked up when a context is created on that GPU).  A batch whose partial
+ * states need more (psi_hip_gqa_layer_scratch_bytes for the variant and num_total_kv_splits) is rejected with
+ * PSI_HIP_ERR_INVALID_ARGUMENT.  All calls on one GPU share the one buffer, which keeps the previous call's
+ * contents: nothing in it has to start at zero (the combine only reads rows the same call's map wrote), but two
+ * calls that overlap on one GPU -- on different streams or from different contexts -- race. */
+#define PSI_HIP_STATIC_SCRATCH_BYTES (16u << 20)
+int psi_hip_gqa_layer_record_static_scratch(psi_hip_ctx* ctx, const psi_hip_gqa_layer_config* cfg,
+                                            const psi_hip_gqa_layer_input* input);
+
 /* One recorded program per capacity bucket: the counterpart of the reference's replay-program store, which keeps a
  * recorded program per `(variant, total tokens, total Q-token tiles, total KV splits)` key and binds the active
  * counts at submission (crates/inference-executor-core/src/replay.rs:4-87; parameter keys backend.rs:55-57;

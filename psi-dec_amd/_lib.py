@@ -23,6 +23,7 @@ CAPACITY_EXACT, CAPACITY_BUCKETED, CAPACITY_CALLER_TOKENS, CAPACITY_FIXED_PARTIT
 FLAG_FORCE_GENERIC = 1
 FLAG_F32_OUTPUT = 2
 REPLAY_EXACT, REPLAY_BUCKETED = 0, 1
+STATIC_SCRATCH_BYTES = 16 << 20
 
 
 class PsiHipError(RuntimeError):
@@ -303,6 +304,8 @@ PROTOTYPES = {
     ),
     "psi_hip_gqa_layer_scratch_bytes": (c_int, [POINTER(LayerConfigStruct), _VARIANT, c_uint32, POINTER(c_uint64)]),
     "psi_hip_gqa_layer_record": (c_int, [c_void_p, POINTER(LayerConfigStruct), POINTER(LayerInputStruct)]),
+    "psi_hip_gqa_layer_record_static_scratch": (
+        c_int, [c_void_p, POINTER(LayerConfigStruct), POINTER(LayerInputStruct)]),
     "psi_hip_gqa_replay_cache_create": (
         c_int, [c_void_p, POINTER(LayerConfigStruct), c_void_p, c_uint32, POINTER(c_void_p)]),
     "psi_hip_gqa_replay_cache_destroy": (c_int, [c_void_p]),

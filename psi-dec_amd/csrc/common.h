@@ -41,6 +41,8 @@ struct Geometry {
 };
 
 int make_geometry(const psi_hip_gqa_config* cfg, Geometry* g);
+// Device address of the library's built-in partial-state array on `device` (the calling thread's current device).
+int resolve_static_scratch(int device);
 int check_layout(const psi_hip_page_table_layout* layout);
 
 struct KernelTimer {

@@ -98,6 +98,10 @@ int psi_hip_ctx_create(int device, void* stream, psi_hip_ctx** out_ctx) {
     if (strncmp(prop.gcnArchName, "gfx950", 6) != 0)
         return psi::fail(PSI_HIP_ERR_UNSUPPORTED, "device %d is %s; this library is built for gfx950 only", device,
                          prop.gcnArchName);
+    // the built-in scratch of psi_hip_gqa_layer_record_static_scratch: its address on this GPU, looked up here,
+    // with this GPU current, so that the entry point itself only launches
+    int rc = psi::resolve_static_scratch(device);
+    if (rc != PSI_HIP_OK) return rc;
     auto* ctx = new psi_hip_ctx();
     ctx->device = device;
     ctx->stream = (hipStream_t)stream;

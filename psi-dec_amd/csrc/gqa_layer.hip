@@ -17,7 +17,28 @@
 #include "common.h"
 #include "device_types.h"
 
+// Partial-state storage for callers that cannot allocate: one array per GPU, inside the library's code object,
+// held from the moment the library is loaded on that GPU until the process ends.  In host code `scratch` is only
+// a stand-in for the symbol: the device address comes from hipGetSymbolAddress, once per device, and that address
+// is what kernels and checks use.
+constexpr uint64_t kStaticScratchBytes = PSI_HIP_STATIC_SCRATCH_BYTES;
+static __device__ __align__(256) unsigned char scratch[kStaticScratchBytes];
+
 namespace psi {
+
+constexpr int kMaxStaticScratchDevices = 64;
+static void* g_static_scratch[kMaxStaticScratchDevices] = {};  // device address of `scratch` on each GPU
+
+// Looks up this GPU's copy of the array.  `device` must be the current device of the calling thread.
+int resolve_static_scratch(int device) {
+    PSI_REQUIRE(device >= 0 && device < kMaxStaticScratchDevices, "device %d has no static scratch slot", device);
+    if (g_static_scratch[device] != nullptr) return PSI_HIP_OK;
+    void* ptr = nullptr;
+    PSI_HIP_CHECK(hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch)));
+    PSI_REQUIRE(ptr != nullptr && reinterpret_cast<uintptr_t>(ptr) % 256 == 0, "static scratch address is not usable");
+    g_static_scratch[device] = ptr;
+    return PSI_HIP_OK;
+}
 
 namespace {
 
@@ -271,6 +292,31 @@ extern "C" int psi_hip_gqa_layer_scratch_bytes(const psi_hip_gqa_layer_config* c
 extern "C" int psi_hip_gqa_layer_record(psi_hip_ctx* ctx, const psi_hip_gqa_layer_config* cfg,
                                         const psi_hip_gqa_layer_input* input) {
     return record_layer(ctx, cfg, input);
+}
+
+extern "C" int psi_hip_gqa_layer_record_static_scratch(psi_hip_ctx* ctx, const psi_hip_gqa_layer_config* cfg,
+                                                       const psi_hip_gqa_layer_input* input) {
+    PSI_REQUIRE(ctx != nullptr && cfg != nullptr && input != nullptr && input->batch_metadata != nullptr,
+                "ctx, config, input and batch metadata must not be null");
+    PSI_REQUIRE(ctx->device >= 0 && ctx->device < kMaxStaticScratchDevices && g_static_scratch[ctx->device] != nullptr,
+                "the static scratch of device %d was not resolved when the context was created", ctx->device);
+    uint64_t need = 0;
+    int rc = psi_hip_gqa_layer_scratch_bytes(cfg, &input->batch_metadata->variant,
+                                             input->batch_metadata->shape.num_total_kv_splits, &need);
+    if (rc != PSI_HIP_OK) return rc;
+    PSI_REQUIRE(need <= kStaticScratchBytes,
+                "GQA partial states of %u KV splits need %llu bytes; the built-in scratch holds %llu (use "
+                "psi_hip_gqa_layer_record with a buffer of your own)",
+                input->batch_metadata->shape.num_total_kv_splits, (unsigned long long)need,
+                (unsigned long long)kStaticScratchBytes);
+    psi_hip_gqa_layer_input with_scratch = *input;
+    with_scratch.partial_scratch = g_static_scratch[ctx->device];
+    with_scratch.partial_scratch_bytes = kStaticScratchBytes;
+    const bool timing_before = ctx->timing;
+    ctx->timing = false;  // per-kernel timing creates events
+    rc = record_layer(ctx, cfg, &with_scratch);
+    ctx->timing = timing_before;
+    return rc;
 }
 
 extern "C" int psi_hip_gqa_replay_cache_create(psi_hip_ctx* ctx, const psi_hip_gqa_layer_config* cfg,

@@ -50,7 +50,7 @@ def _ptr(t):
 
 
 def _nbytes(t):
-    return t.numel() * t.element_size()
+    return t.numel() * t.element_size() if t is not None else 0
 
 
 class Device:
@@ -1254,6 +1254,21 @@ class GQA:
         s, keep = self.input_struct(inp)
         L.check(self.device.lib.psi_hip_gqa_layer_record(self.device.ctx, ctypes.byref(cfg), ctypes.byref(s)))
         return keep[1]
+
+
+def _record_static_scratch(self, inp: GQAInput):
+    """`record` with the partial states in the library's built-in buffer (psi_hip_gqa_layer_record_static_scratch):
+    for callers that cannot allocate.  `inp.scratch.sdpa_partial` is not used; batches whose partial states exceed
+    `STATIC_SCRATCH_BYTES` are rejected."""
+    cfg = self.struct()
+    s, keep = self.input_struct(inp)
+    s.partial_scratch, s.partial_scratch_bytes = None, 0
+    L.check(self.device.lib.psi_hip_gqa_layer_record_static_scratch(self.device.ctx, ctypes.byref(cfg), ctypes.byref(s)))
+    return keep[1]
+
+
+GQA.record_static_scratch = _record_static_scratch
+STATIC_SCRATCH_BYTES = L.STATIC_SCRATCH_BYTES
 
 
 class GQAReplayCache:
