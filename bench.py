@@ -1,17 +1,26 @@
 #!/usr/bin/env python3
 """Benchmark of the paged KV-cache attention path on one MI355X.
 
-A step is one decode layer-step over one batch of synthetic input resident in HBM:
-KV append (one token per sequence) -> split-KV grouped-query decode map -> log-sum-exp combine; the
-append rides in the map launch unless --separate-append is given.
-Default workload: batch 32, contexts uniform in [1024, 8192], 24 Q / 4 KV heads, head_dim 256,
-bf16 K/V in 16-token pages from a shuffled pool, 512-token partitions.
+A step is one attention layer-step over one batch of synthetic input resident in HBM, issued through the layer
+entry (`GQA.record`): KV append -> split-KV map -> log-sum-exp combine (decode: the append rides in the map
+launch).  Headline workload (`C2`): batch 32, contexts uniform in [1024, 8192], 24 Q / 4 KV heads, head_dim
+256, bf16 K/V in 16-token pages from a shuffled pool, 512-token partitions re-cut into equal worker shares.
 
-Prints ONE JSON line.  `value` is the achieved HBM bandwidth of the whole layer-step (algorithmic
-bytes / wall time); `us_per_layer_step` is the time itself.  `roofline` prices the dominant kernel
-(the split-KV map) against the 8 TB/s HBM3E peak from HIP events on the launch stream around a run of
-back-to-back launches (the figure with one event pair per launch is reported next to it); `cpu_baseline`
-times the scalar CPU oracle on a bounded sample of the same workload on this box's host cores.
+Prints ONE JSON line.  Top level = the headline workload: `value` is the achieved HBM bandwidth of the whole
+layer-step (algorithmic bytes / wall time), `us_per_layer_step` the time itself; `roofline` prices the dominant
+kernel (the split-KV map) against the 8 TB/s HBM3E peak from HIP events on the launch stream; `cpu_baseline` times
+the scalar CPU oracle on a bounded sample of the same workload on this box's host cores.  `configs` carries the
+same figures for the other benchmark configurations (C1, C3, C4 with one and three drafts, C5's decode side, its
+prefill chunk, and the mixed step), each timed in this run with the same step and warm-up counts.
+
+Clocks.  `ms_per_step` / `us_per_layer_step`: host wall clock around K queued steps, device synchronised on both
+sides -- steps run back to back, as the layers of a decoder do.  `us_per_layer_step_p10_median_p90`: a HIP event
+after every single step of a further run; the event between two steps keeps the next step's first kernel from
+starting under the previous step's tail, so these read a few microseconds higher than the back-to-back figure.
+`host_plan_us`: what the host does per step before it can launch -- metadata update, worker plan, upload -- and is
+not part of the step time (the launches of step n overlap the planning of step n + 1 only if the caller
+pipelines them).  Before the W warm-up steps every workload runs untimed for about 30 ms (`settle_steps_before_warmup`):
+set-up, so that the clocks have settled after the arena was generated.
 """
 import argparse
 import importlib
@@ -24,6 +33,8 @@ ROOT = os.path.dirname(os.path.abspath(__file__))
 sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBPS = 8000.0
+MFMA_BF16_PEAK_TFLOPS = 2500.0
+CONFIG_NAMES = ["C1", "C3", "C4_q2", "C4_q4", "C5_decode", "C5_prefill", "C5_mixed"]
 
 
 def parse_args():
@@ -31,39 +42,30 @@ def parse_args():
     p.add_argument("--gpus", type=int, default=1)
     p.add_argument("--steps", type=int, default=200)
     p.add_argument("--warmup", type=int, default=20)
+    p.add_argument("--only", default=None,
+                   help="time one workload only: C2 (the headline), " + ", ".join(CONFIG_NAMES) + ", or `custom`")
+    p.add_argument("--no-configs", action="store_true", help="headline workload only")
+    p.add_argument("--kernel-only", action="store_true", help="time only the map kernel (for profiling runs)")
+    p.add_argument("--cpu-seconds", type=float, default=12.0, help="budget of the CPU baseline sample")
+    p.add_argument("--no-cpu-baseline", action="store_true")
+    p.add_argument("--seed", type=int, default=2)
+    # the `custom` decode workload (and overrides of the headline's launch mode, for comparisons)
     p.add_argument("--batch", type=int, default=32)
     p.add_argument("--ctx-lo", type=int, default=1024)
     p.add_argument("--ctx-hi", type=int, default=8192)
-    p.add_argument("--partition", type=int, default=None,
-                   help="split-KV partition length in tokens (default 512; the whole context for the prefill workload)")
-    p.add_argument("--arenas", type=int, default=2, help="independent page arenas rotated between steps")
-    p.add_argument("--q-heads", type=int, default=24, help="decode workload: query heads (24; 16 for the long-context shape)")
-    p.add_argument("--kv-heads", type=int, default=4, help="decode workload: KV heads (4; 2 for the long-context shape)")
-    p.add_argument("--dtype", choices=["bf16", "f16"], default="bf16", help="K/V/Q element type (f16 for the 1 x 512 shape)")
-    p.add_argument("--seed", type=int, default=2)
-    p.add_argument("--cpu-seconds", type=float, default=12.0, help="budget of the CPU baseline sample")
-    p.add_argument("--no-cpu-baseline", action="store_true")
+    p.add_argument("--q-heads", type=int, default=24)
+    p.add_argument("--kv-heads", type=int, default=4)
+    p.add_argument("--q-len", type=int, default=1, help="custom workload: new tokens per sequence")
+    p.add_argument("--dtype", choices=["bf16", "f16"], default="bf16")
+    p.add_argument("--partition", type=int, default=512)
+    p.add_argument("--arenas", type=int, default=0, help="page arenas rotated between steps (0 = per workload)")
     p.add_argument("--identity-pages", action="store_true", help="unshuffled page pool (diagnostic)")
-    p.add_argument("--plan-order", action="store_true",
-                   help="dispatch the split rows in plan order instead of longest first")
-    p.add_argument("--separate-append", action="store_true",
-                   help="decode workload: launch the append as its own kernel instead of folding it into the map")
-    p.add_argument("--workers", type=int, default=0,
-                   help="balanced plan: workers per KV head (0 = one workgroup per compute unit over all KV heads)")
-    p.add_argument("--row-per-workgroup", action="store_true",
-                   help="decode workload: one workgroup per partition row instead of the balanced worker plan")
-    p.add_argument("--kernel-only", action="store_true", help="time only the map kernel (for profiling runs)")
+    p.add_argument("--plan-order", action="store_true", help="row-per-workgroup launch in plan order, not longest first")
+    p.add_argument("--separate-append", action="store_true", help="decode: launch the append as its own kernel")
+    p.add_argument("--workers", type=int, default=0, help="balanced plan: workers per KV head (0 = one workgroup per CU)")
+    p.add_argument("--row-per-workgroup", action="store_true", help="one workgroup per partition row, no worker plan")
     p.add_argument("--graph", action="store_true",
-                   help="replay a captured HIP graph per step instead of launching its three kernels one by one "
-                        "(measured slower on this stack: 133 vs 126 us per step)")
-    p.add_argument("--workload", choices=["decode", "verify", "prefill"], default="decode",
-                   help="decode: one new token per sequence (the headline workload); verify: --q-len tokens per "
-                        "sequence through the multi-query kernels (batch 64, contexts 2048-16384 unless overridden)")
-    p.add_argument("--q-len", type=int, default=2)
-    p.add_argument("--prefix", type=int, default=4096, help="prefill workload: cached tokens before the chunk")
-    p.add_argument("--chunk", type=int, default=2048, help="prefill workload: new tokens of the one sequence")
-    p.add_argument("--no-row-groups", action="store_true",
-                   help="prefill workload: one workgroup per (row, KV head) instead of the row-group map")
+                   help="submit every step through the per-bucket program cache (HIP graph replay) instead of launching")
     p.add_argument("--calibrate-copy", action="store_true",
                    help="run only the plain copy / read probes of known size (counter calibration, practical ceiling)")
     p.add_argument("--probe-mib", type=int, default=1024)
@@ -71,8 +73,8 @@ def parse_args():
 
 
 def read_profile_traffic(workload_key):
-    """HBM bytes per launch of the dominant kernel measured with rocprofv3 --pmc (FETCH_SIZE +
-    WRITE_SIZE, scaled by the copy calibration), if a committed summary covers this workload."""
+    """HBM bytes per launch of the dominant kernel measured with rocprofv3 --pmc (FETCH_SIZE + WRITE_SIZE, scaled by
+    the copy calibration), if a committed summary under profiles/ covers this workload."""
     folder = os.path.join(ROOT, "profiles")
     try:
         names = sorted(os.listdir(folder))
@@ -83,17 +85,261 @@ def read_profile_traffic(workload_key):
             continue
         with open(os.path.join(folder, name)) as f:
             text = f.read()
-        if f"workload={workload_key}" not in text:
-            continue
-        for line in text.splitlines():
-            if line.startswith("traffic_bytes_per_launch="):
-                return float(line.split("=", 1)[1])
+        blocks = text.split("workload=")
+        for block in blocks[1:]:
+            if block.split()[0] != workload_key:
+                continue
+            for line in block.splitlines():
+                if line.startswith("traffic_bytes_per_launch="):
+                    return float(line.split("=", 1)[1])
     return None
 
 
+class Case:
+    """One workload: page arenas rotated between steps, how a step and its dominant launch are issued."""
+
+    def __init__(self, name, key, arenas, kind, map_kernel, roof_kernel, description):
+        self.name, self.key, self.arenas, self.kind = name, key, arenas, kind
+        self.map_kernel, self.roof_kernel, self.description = map_kernel, roof_kernel, description
+        self.flops = None  # per map launch, for MFMA-priced workloads
+
+
+def build_case(psi, wl, device, name, args):
+    import numpy as np
+
+    bf16 = psi.Dtype.Bfloat16
+    decode_how = dict(balanced=not args.row_per_workgroup, longest_first=not args.plan_order,
+                      fused_append=not args.separate_append, num_workers=args.workers or None)
+    verify_how = dict(balanced=not args.row_per_workgroup, longest_first=not args.plan_order)
+
+    def decode_case(key, ctxs, hq, hkv, dtype, partition, arenas, seed, kernel="split_kv_decode_map", **kw):
+        out = []
+        for i in range(arenas):
+            w = wl.make_workload(seed, ctxs, hq, hkv, 256, dtype, 16, host_pages=False,
+                                 shuffle_pages=not args.identity_pages, **kw)
+            w.seed = seed + 1000 * i  # same geometry, different page contents
+            out.append(wl.DeviceWorkload(device, w, partition_tokens=partition, **decode_how))
+        return Case(name, key, out, "decode", "split_kv_map", kernel, "kv append + split-KV map (one launch) -> LSE combine")
+
+    def verify_case(key, ctxs, q_len, partition, arenas, seed):
+        out = []
+        for i in range(arenas):
+            w = wl.make_workload(seed, ctxs, 24, 4, 256, bf16, 16, q_lens=q_len, host_pages=False,
+                                 shuffle_pages=not args.identity_pages)
+            w.seed = seed + 1000 * i
+            out.append(wl.DeviceWorkload(device, w, partition_tokens=partition, **verify_how))
+        return Case(name, key, out, "verify", "tiled_q_map", "split_kv_tiled_map",
+                    "kv append -> multi-query split-KV map -> LSE combine")
+
+    if name == "C2":
+        ctx = wl.config_c2_context_lens(args.seed, 32, 1024, 8192) + 1
+        key = f"decode_b32_ctx1024-8192_24q4kv_d256_bf16_p16_part{args.partition}_seed{args.seed}"
+        return decode_case(key, ctx, 24, 4, bf16, args.partition, args.arenas or 2, args.seed)
+    if name == "custom":
+        elem = bf16 if args.dtype == "bf16" else psi.Dtype.Float16
+        ctx = wl.config_c2_context_lens(args.seed, args.batch, args.ctx_lo, args.ctx_hi) + args.q_len
+        key = (f"{'decode' if args.q_len == 1 else 'verify_q%d' % args.q_len}_b{args.batch}_ctx{args.ctx_lo}-{args.ctx_hi}"
+               f"_{args.q_heads}q{args.kv_heads}kv_d256_{args.dtype}_p16_part{args.partition}_seed{args.seed}")
+        if args.q_len == 1:
+            return decode_case(key, ctx, args.q_heads, args.kv_heads, elem, args.partition, args.arenas or 2, args.seed)
+        return verify_case(key, ctx, args.q_len, args.partition, args.arenas or 1, args.seed)
+    if name == "C1":
+        # 1 MB per arena: enough arenas that a page comes back only after 300 MB of other pages went through the
+        # 256 MB last-level cache
+        key = "decode_b1_ctx512_16q2kv_d256_f16_p16_part512_seed1"
+        return decode_case(key, [512], 16, 2, psi.Dtype.Float16, 512, args.arenas or 300, 1, input_scale=1.0 / 16.0,
+                           spare_pages=0, shuffle_slots=False)
+    if name == "C3":
+        key = "decode_b4_ctx131072_16q2kv_d256_bf16_p16_part512_outliers1e-4_seed33"
+        return decode_case(key, [131072] * 4, 16, 2, bf16, 512, args.arenas or 1, 33, outlier_rate=1e-4, outlier_sigma=8.0)
+    if name in ("C4_q2", "C4_q4"):
+        q_len = 2 if name == "C4_q2" else 4
+        ctx = wl.config_c2_context_lens(4, 64, 2048, 16384) + q_len
+        return verify_case(f"verify_q{q_len}_b64_ctx2048-16384_24q4kv_d256_bf16_p16_part512_seed4", ctx, q_len, 512,
+                           args.arenas or 1, 4)
+    if name == "C5_decode":
+        ctx = wl.config_c2_context_lens(5, 128, 512, 32768) + 1
+        return decode_case("decode_b128_ctx512-32768_24q4kv_d256_bf16_p16_part512_seed5", ctx, 24, 4, bf16, 512,
+                           args.arenas or 1, 5)
+    if name == "C5_prefill":
+        w = wl.make_workload(5, [4096 + 2048], 24, 4, 256, bf16, 16, q_lens=2048, host_pages=False)
+        dw = wl.DeviceWorkload(device, w, partition_tokens=8192, grouped=True,
+                               variant=psi.GQASplitKVVariant.TiledQ(8, 16, 6))
+        case = Case(name, "prefill_chunk2048_on_prefix4096_24q4kv_d256_bf16_p16_unsplit_seed5", [dw], "prefill",
+                    "tiled_q_map", "split_kv_chunk_map", "kv append -> row-group (prefill-chunk) map -> LSE combine")
+        case.flops = 4 * 24 * 256 * sum(4096 + i + 1 for i in range(2048))
+        return case
+    if name == "C5_mixed":
+        step = wl.MixedStep(device, wl.config_c5())
+        case = Case(name, "mixed_chunk2048_on_prefix4096_plus_decode_b128_ctx512-32768_24q4kv_d256_bf16_p16_seed5",
+                    [step], "mixed", None, None,
+                    "chunk: kv append -> row-group map -> combine; decode: append + map (one launch) -> combine; "
+                    "one arena, one page table, one stream")
+        return case
+    raise SystemExit(f"unknown workload {name}")
+
+
+def algorithmic_bytes(case):
+    a = case.arenas[0]
+    if case.kind == "mixed":
+        return a.chunk.w.algorithmic_bytes() + a.decode.w.algorithmic_bytes()
+    return a.w.algorithmic_bytes()
+
+
+def host_plan_us(psi, wl, case, repeats=15):
+    """Median host time of one step's planning for the workload: metadata update (+ worker plan / dispatch order /
+    row groups) and the upload of the arrays to their fixed device buffers, as the Python mirror issues it."""
+    parts = [case.arenas[0]] if case.kind != "mixed" else [case.arenas[0].chunk, case.arenas[0].decode]
+    times = []
+    for _ in range(repeats):
+        t0 = time.perf_counter()
+        for dw in parts:
+            dw.plan()
+        times.append((time.perf_counter() - t0) * 1e6)
+    for dw in parts:
+        dw.device.sync()
+    return sorted(times)[len(times) // 2]
+
+
+def time_case(psi, wl, device, case, args, with_spread=True):
+    import torch
+
+    arenas = case.arenas
+    step_bytes = algorithmic_bytes(case)
+    graph_cache = None
+    if args.graph and case.kind != "mixed":
+        graph_cache = psi.GQAReplayCache(device, arenas[0].gqa, max_programs=2 * len(arenas) + 2)
+
+    def run_steps(n, first=0):
+        for i in range(first, first + n):
+            a = arenas[i % len(arenas)]
+            if graph_cache is not None:
+                graph_cache.submit(a.layer_input())
+            else:
+                a.step()
+
+    def run_maps(n, first=0):
+        for i in range(first, first + n):
+            arenas[i % len(arenas)].map()
+
+    kernel_only = args.kernel_only and case.kind != "mixed"
+    body = run_maps if kernel_only else run_steps
+    # Set-up, not measurement: generating a workload's arena leaves the GPU's clocks unsettled for some 20 ms of
+    # attention work (step times drift by 5-10 % over the first 40 steps), and an arena's first step pays for the
+    # first touch of its buffers.  Every arena is run once and the workload for at least 30 ms before the W
+    # warm-up steps and the K timed ones.
+    settle_steps, t_settle = 0, time.perf_counter()
+    while settle_steps < len(arenas) or (time.perf_counter() - t_settle < 0.03 and settle_steps < 2000):
+        body(1, first=settle_steps)
+        settle_steps += 1
+        if settle_steps % 8 == 0:
+            device.sync()
+    device.sync()
+    body(args.warmup)
+    device.sync()
+    t0 = time.perf_counter()
+    body(args.steps)
+    device.sync()
+    ms_per_step = (time.perf_counter() - t0) * 1e3 / args.steps
+    out = {"workload": case.key, "step": "map kernel only" if kernel_only else case.description,
+           "us_per_layer_step": ms_per_step * 1e3, "settle_steps_before_warmup": settle_steps,
+           "algorithmic_bytes_per_step": step_bytes,
+           "step_GBps": step_bytes / (ms_per_step / 1e3) / 1e9,
+           "step_frac_of_hbm_peak": step_bytes / (ms_per_step / 1e3) / 1e9 / HBM_PEAK_GBPS}
+    if with_spread:
+        n_spread = min(args.steps, 100)
+        body(4)
+        ticks = [torch.cuda.Event(enable_timing=True) for _ in range(n_spread + 1)]
+        ticks[0].record(device.stream)
+        for i in range(n_spread):
+            body(1, first=i)
+            ticks[i + 1].record(device.stream)
+        ticks[-1].synchronize()
+        step_us = sorted(ticks[i].elapsed_time(ticks[i + 1]) * 1e3 for i in range(n_spread))
+        out["us_per_layer_step_p10_median_p90"] = [step_us[int(f * (len(step_us) - 1))] for f in (0.1, 0.5, 0.9)]
+    if case.kind == "mixed":
+        m = arenas[0]
+        device.set_timing(True)
+        device.reset_timing()
+        run_steps(min(args.steps, 20))
+        kernels = {}
+        for k in ("kv_page_write", "tiled_q_map", "tiled_q_reduce", "split_kv_map", "split_kv_reduce"):
+            ms, n = device.kernel_time_ms(k)
+            kernels[k] = ms / max(n, 1) * 1e3
+        device.set_timing(False)
+        out["kernel_us_in_step"] = kernels
+        out["roofline"] = None  # two dominant kernels with two bounds: see C5_prefill and C5_decode
+        out["chunk_rows"] = m.chunk.shape.num_sdpa_map_task_templates
+        out["decode_rows"] = m.decode.shape.num_sdpa_map_task_templates
+        return out
+
+    # Dominant kernel: HIP events on the launch stream around every map launch ...
+    device.set_timing(True)
+    device.reset_timing()
+    run_maps(min(args.steps, 100))
+    map_ms, map_launches = device.kernel_time_ms(case.map_kernel)
+    device.set_timing(False)
+    map_pair_us = map_ms / max(map_launches, 1) * 1e3
+    # ... and the same launches back to back with an event after every group: a pair of events per launch adds the
+    # events' own record latency to every launch, a group adds the gap between two launches instead.  The median
+    # group is taken, so that a host-side hiccup inside one group does not pass for kernel time.
+    est = max(map_pair_us, 1.0)
+    group_launches = int(min(40, max(4, 4000.0 / est)))
+    n_groups = 5 if args.steps >= 100 else (3 if args.steps >= 20 else 1)
+    run_maps(4)
+    marks = [torch.cuda.Event(enable_timing=True) for _ in range(n_groups + 1)]
+    marks[0].record(device.stream)
+    for g in range(n_groups):
+        run_maps(group_launches)
+        marks[g + 1].record(device.stream)
+    marks[-1].synchronize()
+    group_us = sorted(marks[g].elapsed_time(marks[g + 1]) * 1e3 / group_launches for g in range(n_groups))
+    map_b2b_us = group_us[len(group_us) // 2]
+    # Both bound the kernel's own duration from above; the roofline takes the smaller.  Unprofiled that is the
+    # back-to-back average, which a profiler's kernel trace reproduces (End - Start per launch).
+    map_us = min(map_b2b_us, map_pair_us)
+    a0 = arenas[0]
+    map_bytes = a0.w.map_algorithmic_bytes()
+    device.set_timing(True)
+    device.reset_timing()
+    run_steps(min(args.steps, 50))
+    kernels = {}
+    names = ("kv_page_write", case.map_kernel, "tiled_q_reduce" if case.kind != "decode" else "split_kv_reduce")
+    for k in names:
+        ms, n = device.kernel_time_ms(k)
+        kernels[k] = ms / max(n, 1) * 1e3
+    device.set_timing(False)
+    timing = {"avg_launch_us": map_us, "back_to_back_launch_us": map_b2b_us, "event_pair_per_launch_us": map_pair_us,
+              "launches_timed": int(n_groups * group_launches if map_b2b_us <= map_pair_us else map_launches),
+              "timing": "HIP events on the launch stream; the smaller of the back-to-back and per-launch figures"}
+    hbm = {"bound": "hbm", "kernel": case.roof_kernel, "achieved": map_bytes / (map_us / 1e6) / 1e9,
+           "peak": HBM_PEAK_GBPS, "unit": "GB/s", "frac": map_bytes / (map_us / 1e6) / 1e9 / HBM_PEAK_GBPS,
+           "traffic": read_profile_traffic(case.key), "algorithmic_bytes_per_launch": map_bytes, **timing}
+    if case.flops:
+        tflops = case.flops / (map_us / 1e6) / 1e12
+        out["roofline"] = {"bound": "mfma", "kernel": case.roof_kernel, "achieved": tflops, "peak": MFMA_BF16_PEAK_TFLOPS,
+                           "unit": "TFLOP/s", "frac": tflops / MFMA_BF16_PEAK_TFLOPS,
+                           "traffic": read_profile_traffic(case.key), "flops_per_launch": case.flops, **timing}
+        out["hbm_view"] = {k: hbm[k] for k in ("achieved", "peak", "unit", "frac", "algorithmic_bytes_per_launch")}
+    else:
+        out["roofline"] = hbm
+    out["kernel_us_in_step"] = kernels
+    out["kv_split_rows"] = a0.shape.num_sdpa_map_task_templates
+    out["context_tokens_total"] = int(a0.w.context_lens.astype("int64").sum())
+    out["dispatch"] = (("row groups of the prefill-chunk map" if a0.grouped else
+                        "one workgroup per compute unit and KV head over equal shares of the plan's tiles")
+                       if (a0.balanced or a0.grouped) else
+                       "one workgroup per plan row, " + ("plan order" if args.plan_order else "longest first"))
+    out["launch"] = "per-bucket program cache (HIP graph replay)" if graph_cache is not None else "direct launches"
+    if graph_cache is not None:
+        out["replay_cache_programs_recordings_replays"] = list(graph_cache.stats())
+        graph_cache.close()
+    return out
+
+
 def cpu_baseline(psi, wl, w, dw, budget_s):
-    """Scalar oracle (a C restatement of the reference's sequential f32 oracle) on the first
-    requests of the batch, one thread, on this box's host cores."""
+    """Scalar oracle (a C restatement of the reference's sequential f32 oracle) on the first requests of the
+    batch, one thread, on this box's host cores."""
     import numpy as np
 
     from oracle import binding as oracle
@@ -176,7 +422,6 @@ def main():
         print(f"bench.py measures one GPU only (got --gpus {args.gpus}); the path does not shard in this build",
               file=sys.stderr)
         sys.exit(2)
-    import numpy as np
     import torch
 
     psi = importlib.import_module("psi-dec_amd")
@@ -184,208 +429,64 @@ def main():
     if not torch.cuda.is_available():
         print("bench.py needs a GPU", file=sys.stderr)
         sys.exit(1)
-    device = psi.Device(0)
+    # a created stream: the program cache records by stream capture, which the null stream does not allow
+    stream = torch.cuda.Stream()
+    torch.cuda.set_stream(stream)
+    device = psi.Device(0, stream)
     if args.calibrate_copy:
         calibrate_copy(device, args)
         return
 
-    verify = args.workload in ("verify", "prefill")
-    prefill = args.workload == "prefill"
-    if args.partition is None:
-        # prefill: one kv_split row per query tile (no split of the context) measures best for a single chunk
-        args.partition = max(2048, 1 << (args.prefix + args.chunk - 1).bit_length()) if prefill else 512
-    if prefill:
-        args.batch, args.q_len = 1, args.chunk
-    if verify and args.batch == 32 and args.ctx_lo == 1024 and args.ctx_hi == 8192:
-        args.batch, args.ctx_lo, args.ctx_hi = 64, 2048, 16384
-    map_kernel = "tiled_q_map" if verify else "split_kv_map"
-    elem = psi.Dtype.Bfloat16 if args.dtype == "bf16" else psi.Dtype.Float16
-    arenas = []
-    for i in range(max(1, args.arenas)):
-        if verify:
-            ctx = ([args.prefix + args.chunk] if prefill else
-                   wl.config_c2_context_lens(args.seed, args.batch, args.ctx_lo, args.ctx_hi) + args.q_len)
-            w = wl.make_workload(args.seed, ctx, 24, 4, 256, elem, 16, q_lens=args.q_len,
-                                 host_pages=False, shuffle_pages=not args.identity_pages)
-        else:
-            ctx = wl.config_c2_context_lens(args.seed, args.batch, args.ctx_lo, args.ctx_hi) + 1
-            w = wl.make_workload(args.seed, ctx, args.q_heads, args.kv_heads, 256, elem, 16,
-                                 host_pages=False, shuffle_pages=not args.identity_pages)
-        w.seed = args.seed + 1000 * i  # same geometry, different page contents
-        arenas.append(wl.DeviceWorkload(device, w, partition_tokens=args.partition, balanced=not args.row_per_workgroup,
-                                        longest_first=not args.plan_order,
-                                        grouped=prefill and not args.no_row_groups,
-                                        fused_append=not args.separate_append, num_workers=args.workers or None))
-    w = arenas[0].w
-    shape = arenas[0].shape
-    step_bytes = w.algorithmic_bytes()
-    map_bytes = w.map_algorithmic_bytes()
-
-    def run_steps(n, first=0):
-        for i in range(first, first + n):
-            arenas[i % len(arenas)].step()
-
-    run_steps_direct = run_steps
-
-    def run_maps(n, first=0):
-        for i in range(first, first + n):
-            arenas[i % len(arenas)].map()
-
-    # Optional: one HIP graph per arena holds the step's three launches (append, map, combine).
-    graphs = []
-    if args.graph and not args.kernel_only:
-        main_stream = device.stream
-        side = torch.cuda.Stream()
-        side.wait_stream(torch.cuda.current_stream())
-        try:
-            with torch.cuda.stream(side):
-                device.use_stream(side)
-                for a in arenas:
-                    a.step()
-                side.synchronize()
-                for a in arenas:
-                    g = torch.cuda.CUDAGraph()
-                    with torch.cuda.graph(g, stream=side):
-                        a.step()
-                    graphs.append(g)
-        finally:
-            device.use_stream(main_stream)
-        torch.cuda.synchronize()
-
-        def run_steps(n, first=0):  # noqa: F811
-            for i in range(first, first + n):
-                graphs[i % len(graphs)].replay()
-
-    body = run_maps if args.kernel_only else run_steps
-    body(args.warmup)
-    torch.cuda.synchronize()
-    t0 = time.perf_counter()
-    body(args.steps)
-    torch.cuda.synchronize()
-    elapsed = time.perf_counter() - t0
-    ms_per_step = elapsed * 1e3 / args.steps
-
-    # Spread of the step time: an event on the launch stream after every step of a further run, differences between
-    # neighbours (the queue stays full, so a difference is one step's device time plus its share of launch gaps).
-    n_spread = min(args.steps, 100)
-    body(4)
-    ticks = [torch.cuda.Event(enable_timing=True) for _ in range(n_spread + 1)]
-    ticks[0].record(device.stream)
-    for i in range(n_spread):
-        body(1, first=i)
-        ticks[i + 1].record(device.stream)
-    ticks[-1].synchronize()
-    step_us = sorted(ticks[i].elapsed_time(ticks[i + 1]) * 1e3 for i in range(n_spread))
-
-    def percentile(fraction):
-        return step_us[min(len(step_us) - 1, int(fraction * len(step_us)))]
-
-    # Dominant kernel, timed by HIP events on the launch stream around every map launch.
-    device.set_timing(True)
-    device.reset_timing()
-    run_maps(min(args.steps, 100))
-    map_ms, map_launches = device.kernel_time_ms(map_kernel)
-    device.set_timing(False)
-    map_avg_s = map_ms / max(map_launches, 1) / 1e3
-    # The same launches back to back, an event on the launch stream after every 40 of them: the
-    # per-launch pairs above add the record latency of two events to every launch, a group adds the gap between two
-    # launches instead.  The median group is reported, so that a host-side hiccup inside one group (a profiler
-    # flushing its buffers, say) does not pass for kernel time.
-    group_launches = 40
-    n_groups = 5 if args.steps >= 100 else 1
-    run_maps(4)  # the queue is full when the first event is recorded
-    marks = [torch.cuda.Event(enable_timing=True) for _ in range(n_groups + 1)]
-    marks[0].record(device.stream)
-    for g in range(n_groups):
-        run_maps(group_launches)
-        marks[g + 1].record(device.stream)
-    marks[-1].synchronize()
-    group_us = [marks[g].elapsed_time(marks[g + 1]) * 1e3 / group_launches for g in range(n_groups)]
-    map_back_to_back_us = sorted(group_us)[len(group_us) // 2]
-    n_back_to_back = n_groups * group_launches
-    map_pair_us = map_avg_s * 1e6
-    # Both figures bound the kernel's own duration from above (one adds launch gaps, the other event latency); the
-    # roofline uses the smaller one.  Unprofiled that is the back-to-back average, which the profiler's kernel
-    # trace reproduces (End - Start per launch); under a profiler, which instruments every dispatch, the per-launch
-    # pairs are the tighter bound.
-    map_avg_s = min(map_back_to_back_us, map_pair_us) / 1e6
-    # the other two kernels of the step, for the record
-    device.set_timing(True)
-    device.reset_timing()
-    run_steps_direct(min(args.steps, 50))
-    kernels_us = {}
-    for name in ("kv_page_write", map_kernel, "tiled_q_reduce" if verify else "split_kv_reduce"):
-        ms, n = device.kernel_time_ms(name)
-        kernels_us[name] = ms / max(n, 1) * 1e3
-    device.set_timing(False)
-    achieved = map_bytes / map_avg_s / 1e9
-
-    workload_key = (f"{'verify_q%d' % args.q_len if verify else 'decode'}_b{args.batch}_ctx{args.ctx_lo}-{args.ctx_hi}"
-                    f"_{w.num_q_heads}q{w.num_kv_heads}kv_d256_{args.dtype}_p16_part{args.partition}_seed{args.seed}")
+    headline_name = args.only if args.only else "C2"
+    case = build_case(psi, wl, device, headline_name, args)
+    head = time_case(psi, wl, device, case, args)
+    head["host_plan_us"] = host_plan_us(psi, wl, case)
     result = {
-        "metric": "decode attn achieved HBM GB/s per layer-step (B=32, ctx 1k-8k); us/layer-step alongside",
-        "value": (map_bytes if args.kernel_only else step_bytes) / (ms_per_step / 1e3) / 1e9,
+        "metric": ("decode attn achieved HBM GB/s per layer-step (B=32, ctx 1k-8k); us/layer-step alongside"
+                   if headline_name == "C2" else f"attention layer-step of workload {headline_name}: achieved HBM GB/s; "
+                   "us/layer-step alongside"),
+        "value": head["step_GBps"],
         "unit": "GB/s",
         "n_gpus": 1,
         "steps": args.steps,
         "warmup": args.warmup,
-        "ms_per_step": ms_per_step,
-        "us_per_layer_step": ms_per_step * 1e3,
-        "us_per_layer_step_p10_median_p90": [percentile(0.1), percentile(0.5), percentile(0.9)],
-        "hbm_frac_of_peak": (map_bytes if args.kernel_only else step_bytes) / (ms_per_step / 1e3) / 1e9 / HBM_PEAK_GBPS,
+        "ms_per_step": head["us_per_layer_step"] / 1e3,
+        "us_per_layer_step": head["us_per_layer_step"],
+        "us_per_layer_step_p10_median_p90": head.get("us_per_layer_step_p10_median_p90"),
+        "hbm_frac_of_peak": head["step_frac_of_hbm_peak"],
         "higher_is_better": True,
         "scaling": "weak",
         "vs_baseline": None,
-        "dtype": args.dtype,
+        "dtype": "f16" if headline_name == "C1" or (headline_name == "custom" and args.dtype == "f16") else "bf16",
         "data": "synthetic",
-        "config": {
-            "workload": workload_key,
-            "step": "map kernel only" if args.kernel_only else "kv append -> split-KV map -> LSE combine",
-            "launch": "hip graph replay" if graphs else "direct launches",
-            "batch": args.batch,
-            "context_tokens_total": int(w.context_lens.astype(np.int64).sum()),
-            "kv_splits": shape.num_sdpa_map_task_templates,
-            "algorithmic_bytes_per_step": step_bytes,
-            "arenas_rotated": len(arenas),
-            "kernel_us_in_step": kernels_us,
-            "dispatch": ("one workgroup per compute unit and KV head over equal shares of the tiles of the "
-                         "512-token plan" if arenas[0].balanced else
-                         "one workgroup per plan row, " + ("plan order" if args.plan_order else "longest first")),
-            "append": "folded into the map launch" if arenas[0].fused_append else "separate kernel",
-        },
-        "roofline": {
-            "bound": "hbm",
-            "kernel": "split_kv_tiled_map" if verify else "split_kv_decode_map",
-            "achieved": achieved,
-            "peak": HBM_PEAK_GBPS,
-            "unit": "GB/s",
-            "frac": achieved / HBM_PEAK_GBPS,
-            "traffic": read_profile_traffic(workload_key),
-            "algorithmic_bytes_per_launch": map_bytes,
-            "avg_launch_us": map_avg_s * 1e6,
-            "launches_timed": int(n_back_to_back if map_back_to_back_us <= map_pair_us else map_launches),
-            "timing": "HIP events on the launch stream; the smaller of the two figures below",
-            "back_to_back_launch_us": map_back_to_back_us,
-            "event_pair_per_launch_us": map_pair_us,
-        },
+        "config": {k: v for k, v in head.items() if k not in ("roofline", "step_GBps", "step_frac_of_hbm_peak",
+                                                              "us_per_layer_step", "us_per_layer_step_p10_median_p90",
+                                                              "hbm_view")},
+        "roofline": head["roofline"],
     }
-    if prefill:
-        # multi-query chunk: priced against the matrix cores as well (4 * Hq * D flops per visible (query, key) pair)
-        pairs = sum(args.prefix + i + 1 for i in range(args.chunk))
-        flops = 4 * w.num_q_heads * w.head_dim * pairs
-        result["config"]["workload"] = f"prefill_chunk{args.chunk}_on_prefix{args.prefix}_24q4kv_d256_{args.dtype}_p16_part{args.partition}"
-        result["config"]["row_groups"] = arenas[0].meta.num_row_groups
-        # the chunk map is bound by the matrix cores: that is its roofline; the HBM view stays alongside
-        hbm_view = result["roofline"]
-        result["roofline"] = {"bound": "mfma", "kernel": "split_kv_chunk_map" if arenas[0].grouped else "split_kv_tiled_map",
-                              "achieved": flops / map_avg_s / 1e12, "peak": 2500.0, "unit": "TFLOP/s",
-                              "frac": flops / map_avg_s / 1e12 / 2500.0, "traffic": None, "flops_per_launch": flops,
-                              "avg_launch_us": hbm_view["avg_launch_us"], "launches_timed": hbm_view["launches_timed"],
-                              "timing": hbm_view["timing"], "back_to_back_launch_us": hbm_view["back_to_back_launch_us"],
-                              "event_pair_per_launch_us": hbm_view["event_pair_per_launch_us"]}
-        result["hbm"] = {k: hbm_view[k] for k in ("achieved", "peak", "unit", "frac", "algorithmic_bytes_per_launch")}
-    if not args.no_cpu_baseline:
-        result["cpu_baseline"] = cpu_baseline(psi, wl, w, arenas[0], args.cpu_seconds)
+    result["config"]["arenas_rotated"] = len(case.arenas)
+    result["config"]["clocks"] = {
+        "ms_per_step": "host wall clock over the K queued steps, device synchronised before and after",
+        "us_per_layer_step_p10_median_p90": "one HIP event after every step of a further run (adds an event per step)",
+        "roofline.avg_launch_us": "HIP events on the launch stream around runs of map launches",
+        "host_plan_us": "host time to plan and upload one step's metadata; not inside ms_per_step"}
+    if "hbm_view" in head:
+        result["hbm"] = head["hbm_view"]
+    if not args.no_cpu_baseline and case.kind != "mixed":
+        result["cpu_baseline"] = cpu_baseline(psi, wl, case.arenas[0].w, case.arenas[0], args.cpu_seconds)
+    del case, head
+    torch.cuda.empty_cache()
+    if not args.only and not args.no_configs and not args.kernel_only:
+        configs = {}
+        for name in CONFIG_NAMES:
+            c = build_case(psi, wl, device, name, args)
+            r = time_case(psi, wl, device, c, args)
+            r["host_plan_us"] = host_plan_us(psi, wl, c)
+            r["arenas_rotated"] = len(c.arenas)
+            configs[name] = r
+            del c
+            torch.cuda.empty_cache()
+        result["configs"] = configs
     print(json.dumps(result))
 
 

@@ -561,6 +561,54 @@ typedef struct psi_hip_gqa_layer_input {
     void* output; /* `scratch.gated_attention_output` / `scratch.attention_output`: [num_total_tokens][Hq][D] */
 } psi_hip_gqa_layer_input;
 
+/* How the planned rows are dispatched (this library's launch plans; PLAN_ORDER is the reference's). */
+#define PSI_HIP_DISPATCH_PLAN_ORDER 0u    /* one workgroup per row, rows as planned */
+#define PSI_HIP_DISPATCH_LONGEST_FIRST 1u /* psi_hip_split_kv_order_longest_first */
+#define PSI_HIP_DISPATCH_BALANCED 2u      /* psi_hip_split_kv_balance_plan */
+#define PSI_HIP_DISPATCH_ROW_GROUPS 3u    /* psi_hip_split_kv_tiled_q_group_rows (TiledQ; SingleQ batches get BALANCED) */
+
+typedef struct psi_hip_gqa_plan_options {
+    uint32_t capacity_mode;           /* PSI_HIP_CAPACITY_* */
+    uint32_t partition_tokens;        /* FIXED_PARTITION */
+    uint32_t caller_num_total_tokens; /* CALLER_TOKENS */
+    uint32_t dispatch;                /* PSI_HIP_DISPATCH_* */
+    uint32_t num_workers;             /* BALANCED: workers per KV head, 0 = psi_hip_split_kv_balanced_workers */
+    uint32_t bucket_max_tokens;       /* variant selection: `GQAReplayBucketPolicy::max_tokens`, 0 = none */
+    const uint32_t* topology_boundaries;
+    uint32_t num_boundaries;
+} psi_hip_gqa_plan_options;
+
+/* Host arrays of one batch's metadata with their capacities (e.g. views of one pinned staging block that is then
+ * uploaded in one copy).  partial_row_index / worker_cu / row_groups may be null when the dispatch does not use
+ * them. */
+typedef struct psi_hip_gqa_host_metadata {
+    uint32_t max_tokens;          /* req_slots_by_token, flat_token_indices [max_tokens]; q_token_tiles [max_tokens][2];
+                                     cu_kv_splits [max_tokens + 1] */
+    uint32_t kv_splits_capacity;  /* rows of kv_splits ([rows][3]) and of partial_row_index */
+    uint32_t max_workers;         /* worker_cu [max_workers + 1] */
+    uint64_t row_groups_capacity; /* words of row_groups */
+    uint32_t* req_slots_by_token;
+    uint32_t* flat_token_indices;
+    uint32_t* q_token_tiles;
+    uint32_t* kv_splits;
+    uint32_t* cu_kv_splits;
+    uint32_t* partial_row_index;
+    uint32_t* worker_cu;
+    uint32_t* row_groups;
+} psi_hip_gqa_host_metadata;
+
+/* `GQA::prepare` / `prepare_bucketed` / `prepare_bucketed_with_token_capacity` (backend.rs:289-364): selects the
+ * batch's SplitKV variant (`select_split_kv_variant`, variant null) or takes the caller's, updates the metadata
+ * arrays, and -- beyond the reference -- adds the dispatch plan, all on the host in one call.  out_plan receives
+ * shape, variant, num_workers, group_tiles, num_row_groups and max_active_q_tile_tokens; its pointer fields are
+ * left to the caller (they name the device copies).  out_uses (may be null): bit 0 partial_row_index is in use,
+ * bit 1 worker_cu, bit 2 row_groups. */
+int psi_hip_gqa_layer_prepare(const psi_hip_gqa_layer_config* cfg, const psi_hip_gqa_plan_options* options,
+                              const uint32_t* req_slots, const uint32_t* token_indices, const uint32_t* cu_tokens,
+                              uint32_t num_reqs, const psi_hip_split_kv_variant* variant,
+                              const psi_hip_gqa_host_metadata* host, psi_hip_gqa_batch_metadata* out_plan,
+                              uint32_t* out_uses);
+
 /* Bytes of `partial_scratch` for a variant and split capacity (`GQAScratch::new`, scratch.rs:48-92). */
 int psi_hip_gqa_layer_scratch_bytes(const psi_hip_gqa_layer_config* cfg, const psi_hip_split_kv_variant* variant,
                                     uint32_t num_total_kv_splits, uint64_t* out_bytes);

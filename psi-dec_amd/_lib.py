@@ -23,6 +23,7 @@ CAPACITY_EXACT, CAPACITY_BUCKETED, CAPACITY_CALLER_TOKENS, CAPACITY_FIXED_PARTIT
 FLAG_FORCE_GENERIC = 1
 FLAG_F32_OUTPUT = 2
 REPLAY_EXACT, REPLAY_BUCKETED = 0, 1
+DISPATCH_PLAN_ORDER, DISPATCH_LONGEST_FIRST, DISPATCH_BALANCED, DISPATCH_ROW_GROUPS = 0, 1, 2, 3
 STATIC_SCRATCH_BYTES = 16 << 20
 
 
@@ -132,6 +133,36 @@ class LayerConfigStruct(ctypes.Structure):
         ("norm_eps", c_float),
         ("rope_theta", c_float),
         ("rope_scaling", RopeScalingStruct),
+    ]
+
+
+class PlanOptionsStruct(ctypes.Structure):
+    _fields_ = [
+        ("capacity_mode", c_uint32),
+        ("partition_tokens", c_uint32),
+        ("caller_num_total_tokens", c_uint32),
+        ("dispatch", c_uint32),
+        ("num_workers", c_uint32),
+        ("bucket_max_tokens", c_uint32),
+        ("topology_boundaries", POINTER(c_uint32)),
+        ("num_boundaries", c_uint32),
+    ]
+
+
+class HostMetadataStruct(ctypes.Structure):
+    _fields_ = [
+        ("max_tokens", c_uint32),
+        ("kv_splits_capacity", c_uint32),
+        ("max_workers", c_uint32),
+        ("row_groups_capacity", c_uint64),
+        ("req_slots_by_token", c_void_p),
+        ("flat_token_indices", c_void_p),
+        ("q_token_tiles", c_void_p),
+        ("kv_splits", c_void_p),
+        ("cu_kv_splits", c_void_p),
+        ("partial_row_index", c_void_p),
+        ("worker_cu", c_void_p),
+        ("row_groups", c_void_p),
     ]
 
 
@@ -303,6 +334,9 @@ PROTOTYPES = {
          c_uint32, c_void_p, POINTER(OutputGateStruct)],
     ),
     "psi_hip_gqa_layer_scratch_bytes": (c_int, [POINTER(LayerConfigStruct), _VARIANT, c_uint32, POINTER(c_uint64)]),
+    "psi_hip_gqa_layer_prepare": (
+        c_int, [POINTER(LayerConfigStruct), POINTER(PlanOptionsStruct), c_void_p, c_void_p, c_void_p, c_uint32,
+                _VARIANT, POINTER(HostMetadataStruct), POINTER(BatchMetadataStruct), _U32P]),
     "psi_hip_gqa_layer_record": (c_int, [c_void_p, POINTER(LayerConfigStruct), POINTER(LayerInputStruct)]),
     "psi_hip_gqa_layer_record_static_scratch": (
         c_int, [c_void_p, POINTER(LayerConfigStruct), POINTER(LayerInputStruct)]),

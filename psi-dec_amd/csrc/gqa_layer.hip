@@ -289,6 +289,108 @@ extern "C" int psi_hip_gqa_layer_scratch_bytes(const psi_hip_gqa_layer_config* c
     return psi_hip_split_kv_single_q_scratch_bytes(&cfg->attention, num_total_kv_splits, out_bytes);
 }
 
+extern "C" int psi_hip_gqa_layer_prepare(const psi_hip_gqa_layer_config* cfg, const psi_hip_gqa_plan_options* options,
+                                         const uint32_t* req_slots, const uint32_t* token_indices,
+                                         const uint32_t* cu_tokens, uint32_t num_reqs,
+                                         const psi_hip_split_kv_variant* variant,
+                                         const psi_hip_gqa_host_metadata* host, psi_hip_gqa_batch_metadata* out_plan,
+                                         uint32_t* out_uses) {
+    PSI_REQUIRE(cfg && options && host && out_plan, "GQA prepare: config, options, host arrays and out_plan must not be null");
+    PSI_REQUIRE(req_slots && token_indices && cu_tokens && num_reqs > 0, "GQA prepare needs a batch");
+    PSI_REQUIRE(host->req_slots_by_token && host->flat_token_indices && host->q_token_tiles && host->kv_splits &&
+                    host->cu_kv_splits,
+                "GQA prepare: the metadata arrays must not be null");
+    PSI_REQUIRE(options->dispatch <= PSI_HIP_DISPATCH_ROW_GROUPS, "unknown dispatch plan %u", options->dispatch);
+    psi_hip_split_kv_variant chosen;
+    int rc;
+    if (variant != nullptr) {
+        chosen = *variant;
+    } else {
+        rc = psi_hip_split_kv_select_batch(&cfg->attention, host->max_tokens, options->bucket_max_tokens, token_indices,
+                                           cu_tokens, num_reqs, &chosen);
+        if (rc != PSI_HIP_OK) return rc;
+    }
+    const bool tiled = chosen.kind == PSI_HIP_VARIANT_TILED_Q;
+    uint32_t dispatch = options->dispatch;
+    if (dispatch == PSI_HIP_DISPATCH_ROW_GROUPS && !tiled) dispatch = PSI_HIP_DISPATCH_BALANCED;
+    uint32_t workers = 0;
+    if (dispatch == PSI_HIP_DISPATCH_BALANCED || dispatch == PSI_HIP_DISPATCH_ROW_GROUPS) {
+        workers = options->num_workers;
+        if (workers == 0) {
+            rc = psi_hip_split_kv_balanced_workers(&cfg->attention, &workers);
+            if (rc != PSI_HIP_OK) return rc;
+        }
+    }
+    // With a worker plan the planner's rows are an intermediate: they go to a side buffer and the re-cut rows to
+    // the caller's array.
+    thread_local std::vector<uint32_t> planned, planned_cu;
+    const bool recut = dispatch == PSI_HIP_DISPATCH_BALANCED;
+    uint32_t* plan_rows = host->kv_splits;
+    uint32_t* plan_cu = host->cu_kv_splits;
+    uint32_t plan_capacity = host->kv_splits_capacity;
+    if (recut) {
+        PSI_REQUIRE(host->worker_cu != nullptr && workers <= host->max_workers,
+                    "GQA prepare: the worker table holds %u workers, the plan needs %u", host->max_workers, workers);
+        PSI_REQUIRE(host->kv_splits_capacity > workers, "GQA prepare: kv_splits has no room for a worker plan");
+        plan_capacity = host->kv_splits_capacity - workers;
+        planned.resize((size_t)plan_capacity * 3);
+        planned_cu.resize((size_t)host->max_tokens + 1);
+        plan_rows = planned.data();
+        plan_cu = planned_cu.data();
+    }
+    psi_hip_gqa_replay_shape shape;
+    rc = psi_hip_gqa_metadata_update(host->max_tokens, req_slots, token_indices, cu_tokens, num_reqs, &chosen,
+                                     options->capacity_mode, options->caller_num_total_tokens,
+                                     options->topology_boundaries, options->num_boundaries, options->partition_tokens,
+                                     plan_capacity, host->req_slots_by_token, host->flat_token_indices,
+                                     host->q_token_tiles, plan_rows, plan_cu, &shape);
+    if (rc != PSI_HIP_OK) return rc;
+    uint32_t uses = 0, group_tiles = 0, num_groups = 0;
+    if (dispatch == PSI_HIP_DISPATCH_ROW_GROUPS) {
+        PSI_REQUIRE(host->row_groups != nullptr, "GQA prepare: row groups need their table");
+        rc = psi_hip_split_kv_tiled_q_group_rows(&cfg->attention, chosen.q_token_tile_size, host->kv_splits,
+                                                 shape.num_kv_splits, host->q_token_tiles, shape.num_q_token_tiles,
+                                                 host->req_slots_by_token, host->row_groups, host->row_groups_capacity,
+                                                 &group_tiles, &num_groups);
+        if (rc != PSI_HIP_OK) return rc;
+        if (num_groups != 0) uses |= 4u;
+        // a geometry without the grouped kernel keeps the plain plan (one workgroup per row)
+    } else if (recut) {
+        uint32_t rows_out = 0;
+        const uint32_t groups = tiled ? shape.num_q_token_tiles : shape.num_tokens;
+        rc = psi_hip_split_kv_balance_plan(plan_rows, shape.num_kv_splits, plan_cu, groups, workers, host->kv_splits,
+                                           host->kv_splits_capacity, host->cu_kv_splits, host->worker_cu, &rows_out);
+        if (rc != PSI_HIP_OK) return rc;
+        for (uint64_t i = (uint64_t)rows_out * 3; i < (uint64_t)host->kv_splits_capacity * 3; ++i)
+            host->kv_splits[i] = PSI_HIP_SENTINEL;
+        shape.num_kv_splits = shape.num_total_kv_splits = rows_out;
+        shape.reduce_sdpa_partial_outputs = 1;
+        uses |= 2u;
+    } else if (dispatch == PSI_HIP_DISPATCH_LONGEST_FIRST) {
+        PSI_REQUIRE(host->partial_row_index != nullptr, "GQA prepare: the dispatch order needs partial_row_index");
+        for (uint32_t i = 0; i < host->kv_splits_capacity; ++i) host->partial_row_index[i] = i;
+        rc = psi_hip_split_kv_order_longest_first(host->kv_splits, shape.num_kv_splits, host->partial_row_index);
+        if (rc != PSI_HIP_OK) return rc;
+        uses |= 1u;
+    }
+    uint32_t max_tile_tokens = 0;
+    if (tiled) {
+        for (uint32_t r = 0; r < num_reqs; ++r) {
+            const uint32_t n = cu_tokens[r + 1] - cu_tokens[r];
+            max_tile_tokens = n > max_tile_tokens ? n : max_tile_tokens;
+        }
+        if (max_tile_tokens > chosen.q_token_tile_size) max_tile_tokens = chosen.q_token_tile_size;
+    }
+    out_plan->shape = shape;
+    out_plan->variant = chosen;
+    out_plan->num_workers = (uses & 2u) ? workers : 0;
+    out_plan->group_tiles = group_tiles;
+    out_plan->num_row_groups = num_groups;
+    out_plan->max_active_q_tile_tokens = max_tile_tokens;
+    if (out_uses) *out_uses = uses;
+    return PSI_HIP_OK;
+}
+
 extern "C" int psi_hip_gqa_layer_record(psi_hip_ctx* ctx, const psi_hip_gqa_layer_config* cfg,
                                         const psi_hip_gqa_layer_input* input) {
     return record_layer(ctx, cfg, input);

@@ -573,7 +573,8 @@ class GQAMetadataBuffers:
         self.h_worker_cu = self.d_worker_cu = None
         self.num_workers = 0
         self.h_row_groups = self.d_row_groups = None
-        self._h_row_groups_t = self._d_row_groups_all = None
+        self._h_row_groups_t = self._d_row_groups_all = self._h_row_groups_all = None
+        self._host_struct = None
         self.group_tiles = self.num_row_groups = 0
         self.max_active_q_tile_tokens = 0
         self._uploaded = None  # event after the last upload: the staging buffer is free again once it has passed
@@ -684,15 +685,9 @@ class GQAMetadataBuffers:
         assert s is not None and self._variant.is_tiled()
         n = s.num_sdpa_map_task_templates
         words = max(n, 1) * 32
-        if self.device is not None:
-            import torch
-
-            if self._h_row_groups_t is None or self._h_row_groups_t.numel() < words:
-                self._h_row_groups_t = torch.zeros(words, dtype=torch.int32, pin_memory=True)
-                self._d_row_groups_all = torch.zeros(words, dtype=torch.int32, device=self.device.torch_device)
-            table = self._h_row_groups_t.numpy().view(np.uint32)[:words]
-        else:
-            table = np.zeros(words, np.uint32)
+        if self._row_groups_words() < words:
+            self._alloc_row_groups(words)
+        table = self._h_row_groups_all[:words]
         table[:] = L.SENTINEL
         tiles, groups = ctypes.c_uint32(), ctypes.c_uint32()
         cfg = config.struct()
@@ -749,6 +744,77 @@ class GQAMetadataBuffers:
             self.d_worker_cu = self._d_worker_cu_all
             self.upload()
         return self._shape
+
+    def prepare(self, layer_struct, req_slots, token_indices, cu_tokens, capacity_mode=L.CAPACITY_EXACT,
+                partition_tokens: int = 0, dispatch: int = L.DISPATCH_PLAN_ORDER, num_workers: int = 0,
+                variant: Optional[GQASplitKVVariant] = None, policy: Optional[GQAReplayBucketPolicy] = None,
+                caller_num_total_tokens: int = 0) -> GQAReplayShape:
+        """One host call for the whole of a step's planning (psi_hip_gqa_layer_prepare): variant selection when
+        `variant` is None, metadata update, dispatch plan; then one upload.  `layer_struct`: `GQA.struct()`."""
+        self._staging_free()
+        rs = np.ascontiguousarray(req_slots, dtype=np.uint32)
+        ti = np.ascontiguousarray(token_indices, dtype=np.uint32)
+        cu = np.ascontiguousarray(cu_tokens, dtype=np.uint32)
+        assert len(rs) == len(ti) and len(cu) == len(rs) + 1
+        boundaries = L.u32_array(policy.token_topology_boundaries) if policy is not None else None
+        options = L.PlanOptionsStruct(capacity_mode, partition_tokens, caller_num_total_tokens, dispatch, num_workers,
+                                      policy.max_tokens() if policy is not None else 0, boundaries,
+                                      len(policy.token_topology_boundaries) if policy is not None else 0)
+        if dispatch == L.DISPATCH_ROW_GROUPS and self._row_groups_words() == 0:
+            self._alloc_row_groups((self._max_kv_splits + self._max_workers) * 32)
+        if self._host_struct is None or self._host_struct.row_groups_capacity != self._row_groups_words():
+            def addr(a):
+                return ctypes.c_void_p(a.ctypes.data) if a is not None else None
+
+            self._host_struct = L.HostMetadataStruct(
+                self._max_tokens, self._max_kv_splits + self._max_workers, self._max_workers, self._row_groups_words(),
+                addr(self.h_req_slots), addr(self.h_flat_token_indices), addr(self.h_q_token_tiles),
+                addr(self._h_kv_splits_all), addr(self.h_cu_kv_splits), addr(self._h_row_index_all),
+                addr(self._h_worker_cu_all), addr(self._h_row_groups_all))
+        plan, uses = L.BatchMetadataStruct(), ctypes.c_uint32()
+        v = variant.struct() if variant is not None else None
+        L.check(L.load().psi_hip_gqa_layer_prepare(
+            ctypes.byref(layer_struct), ctypes.byref(options), rs.ctypes.data, ti.ctypes.data, cu.ctypes.data, len(rs),
+            ctypes.byref(v) if v is not None else None, ctypes.byref(self._host_struct), ctypes.byref(plan),
+            ctypes.byref(uses)))
+        sh = plan.shape
+        self._shape = GQAReplayShape(sh.num_tokens, sh.num_total_tokens, sh.num_q_token_tiles, sh.num_total_q_token_tiles,
+                                     sh.num_kv_splits, sh.num_total_kv_splits, bool(sh.reduce_sdpa_partial_outputs))
+        self._variant = GQASplitKVVariant.from_struct(plan.variant)
+        self.h_kv_splits = self._h_kv_splits_all
+        use_index, use_workers, use_groups = bool(uses.value & 1), bool(uses.value & 2), bool(uses.value & 4)
+        self.h_partial_row_index = self._h_row_index_all if use_index else None
+        self.d_partial_row_index = self._d_row_index_all if use_index else None
+        self.num_workers = plan.num_workers
+        self.h_worker_cu = self._h_worker_cu_all[:plan.num_workers + 1] if use_workers else None
+        self.d_worker_cu = self._d_worker_cu_all if use_workers else None
+        self.group_tiles, self.num_row_groups = plan.group_tiles, plan.num_row_groups
+        self.h_row_groups = (self._h_row_groups_all[:max(plan.group_tiles * plan.num_row_groups, 1)]
+                             if use_groups else None)
+        self.d_row_groups = self._d_row_groups_all if use_groups else None
+        self.max_active_q_tile_tokens = plan.max_active_q_tile_tokens
+        if self.device is not None:
+            if use_groups:
+                import torch
+
+                used = plan.group_tiles * plan.num_row_groups
+                with torch.cuda.stream(self.device.stream):
+                    self._d_row_groups_all[:used].copy_(self._h_row_groups_t[:used], non_blocking=True)
+            self.upload()
+        return self._shape
+
+    def _row_groups_words(self) -> int:
+        return 0 if self._h_row_groups_all is None else len(self._h_row_groups_all)
+
+    def _alloc_row_groups(self, words: int):
+        if self.device is not None:
+            import torch
+
+            self._h_row_groups_t = torch.zeros(words, dtype=torch.int32, pin_memory=True)
+            self._d_row_groups_all = torch.zeros(words, dtype=torch.int32, device=self.device.torch_device)
+            self._h_row_groups_all = self._h_row_groups_t.numpy().view(np.uint32)
+        else:
+            self._h_row_groups_all = np.zeros(words, np.uint32)
 
     def replay_shape(self) -> GQAReplayShape:
         assert self._shape is not None, "GQA batch metadata must be updated before recording"
@@ -1202,35 +1268,27 @@ class GQA:
         return select_split_kv_variant(self.split_kv, batch_metadata.max_tokens(), policy, token_indices, cu_tokens)
 
     def prepare(self, batch_metadata: GQAMetadataBuffers, req_slots, token_indices, cu_tokens) -> GQAReplayShape:
-        """`GQA::prepare` (backend.rs:289-304)."""
-        variant = self.select_variant(batch_metadata, token_indices, cu_tokens)
-        return batch_metadata.update(req_slots, token_indices, cu_tokens, variant)
+        """`GQA::prepare` (backend.rs:289-304): variant selection and metadata update, one host call."""
+        return batch_metadata.prepare(self.struct(), req_slots, token_indices, cu_tokens)
 
     def prepare_bucketed(self, batch_metadata, req_slots, token_indices, cu_tokens,
                          policy: GQAReplayBucketPolicy) -> GQAReplayShape:
         """`GQA::prepare_bucketed` (backend.rs:306-323)."""
-        variant = self.select_variant(batch_metadata, token_indices, cu_tokens, policy)
-        return batch_metadata.update_bucketed(req_slots, token_indices, cu_tokens, variant, policy)
+        assert policy.max_tokens() == batch_metadata.max_tokens(), \
+            "GQA replay bucket policy must match metadata token capacity"
+        return batch_metadata.prepare(self.struct(), req_slots, token_indices, cu_tokens,
+                                      capacity_mode=L.CAPACITY_BUCKETED, policy=policy)
 
     def prepare_fixed_partition(self, batch_metadata, req_slots, token_indices, cu_tokens, partition_tokens: int,
                                 balanced: bool = True, grouped: bool = False,
-                                variant: Optional[GQASplitKVVariant] = None) -> GQAReplayShape:
+                                variant: Optional[GQASplitKVVariant] = None, num_workers: int = 0) -> GQAReplayShape:
         """Not in the reference: partitions of fixed length instead of the greedy budget, then (by default) the
         balanced worker plan that gives every compute unit an equal share of the batch's tiles; `grouped`
-        selects the row-group plan of the prefill-chunk map instead."""
-        if variant is None:
-            variant = self.select_variant(batch_metadata, token_indices, cu_tokens)
-        shape = batch_metadata.update_fixed_partition(req_slots, token_indices, cu_tokens, variant, partition_tokens)
-        if grouped and variant.is_tiled():
-            c, k = self.core, self.config
-            tiled_cfg = GQASplitKVTiledQConfig(c.num_q_heads, c.num_kv_heads, c.head_dim, variant.q_head_tile_size,
-                                               variant.q_token_tile_size, variant.kv_token_tile_size, c.scale,
-                                               k.page_bytes, k.io_dtype, None)
-            if batch_metadata.group_rows(tiled_cfg):
-                return shape
-        if balanced:
-            shape = batch_metadata.balance(balanced_workers(self.split_kv.config))
-        return shape
+        selects the row-group plan of the prefill-chunk map instead.  One host call and one upload."""
+        dispatch = (L.DISPATCH_ROW_GROUPS if grouped else L.DISPATCH_BALANCED if balanced else L.DISPATCH_PLAN_ORDER)
+        return batch_metadata.prepare(self.struct(), req_slots, token_indices, cu_tokens,
+                                      capacity_mode=L.CAPACITY_FIXED_PARTITION, partition_tokens=partition_tokens,
+                                      dispatch=dispatch, num_workers=num_workers, variant=variant)
 
     def input_struct(self, inp: GQAInput):
         """(psi_hip_gqa_layer_input, keep-alive objects) for an input."""

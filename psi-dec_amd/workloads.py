@@ -212,18 +212,16 @@ class DeviceWorkload:
                 splits_cap = int(sum(-(-(int(t) + i + 1) // partition_tokens)
                                      for t, n in zip(w.token_indices, q_lens) for i in range(int(n))))
             self.meta = G.GQAMetadataBuffers(device, max(w.num_tokens, 1), max_kv_splits=splits_cap)
-            self.shape = self.meta.update_fixed_partition(w.req_slots, w.token_indices, w.cu_tokens, variant,
-                                                          partition_tokens)
         else:
             self.meta = G.GQAMetadataBuffers(device, max_tokens or max(w.num_tokens, 1))
-            self.shape = self.meta.update(w.req_slots, w.token_indices, w.cu_tokens, variant)
-        if longest_first and not balanced:
-            self.meta.order_longest_first()
+        self._partition_tokens, self._longest_first, self._num_workers = partition_tokens, longest_first, num_workers
         self.balanced = bool(balanced) and not grouped  # the prefill-chunk map has its own row grouping
-        if self.balanced:
-            workers = num_workers or G.balanced_workers(G.GQASplitKVConfig(w.dtype, w.page_bytes, w.num_q_heads,
-                                                                           w.num_kv_heads, w.head_dim))
-            self.shape = self.meta.balance(workers)
+        self.grouped = bool(grouped) and variant.is_tiled()
+        self.gqa = G.GQA(device, G.GQACore(0, w.num_q_heads * w.head_dim, w.head_dim, w.num_q_heads, w.num_kv_heads,
+                                           w.scale),
+                         G.GQAMetalConfig(w.page_bytes, 2, 1e-6, 10000.0, io_dtype=w.dtype), gated=False)
+        self._layer_struct = self.gqa.struct()
+        self.plan()
         s = self.shape
         self.write = G.GQAKVPageWrite(device, G.GQAKVPageWriteConfig(w.num_kv_heads, w.head_dim, w.page_bytes,
                                                                      w.dtype))
@@ -250,13 +248,21 @@ class DeviceWorkload:
         self._rows = rows
         # decode only: the append rides in the map launch (one launch fewer per step)
         self.fused_append = bool(fused_append) and not variant.is_tiled()
-        self.grouped = bool(grouped) and variant.is_tiled()
-        if self.grouped:
-            self.meta.group_rows(self.cfg)
-        self.gqa = G.GQA(device, G.GQACore(0, w.num_q_heads * w.head_dim, w.head_dim, w.num_q_heads, w.num_kv_heads,
-                                           w.scale),
-                         G.GQAMetalConfig(w.page_bytes, 2, 1e-6, 10000.0, io_dtype=w.dtype), gated=False)
         self._layer_input = None
+
+    def plan(self):
+        """The host side of one step: batch metadata, split plan, dispatch plan (worker shares, row order or row
+        groups) in one library call, and one upload into the metadata buffers' fixed device arrays."""
+        w = self.w
+        L = G.L
+        dispatch = (L.DISPATCH_ROW_GROUPS if self.grouped else L.DISPATCH_BALANCED if self.balanced else
+                    L.DISPATCH_LONGEST_FIRST if self._longest_first else L.DISPATCH_PLAN_ORDER)
+        fixed = self._partition_tokens is not None
+        self.shape = self.meta.prepare(self._layer_struct, w.req_slots, w.token_indices, w.cu_tokens,
+                                       capacity_mode=L.CAPACITY_FIXED_PARTITION if fixed else L.CAPACITY_EXACT,
+                                       partition_tokens=self._partition_tokens or 0, dispatch=dispatch,
+                                       num_workers=self._num_workers or 0, variant=self.variant)
+        return self.shape
 
     def append(self):
         m = self.meta

@@ -577,3 +577,66 @@ def test_row_group_table_capacity_is_checked(psi):
                                                    10, ctypes.byref(n_tiles), ctypes.byref(n_groups)) == 0
     assert (n_tiles.value, n_groups.value) == (5, 2)  # two requests never share a group
     assert table.tolist() == [0, MAX, MAX, MAX, MAX, 1, MAX, MAX, MAX, MAX]
+
+
+# ------------------------------------------------------------------ the whole plan in one call
+
+
+@pytest.mark.parametrize("seed", range(12))
+def test_single_call_prepare_equals_the_step_by_step_plan(psi, seed):
+    """psi_hip_gqa_layer_prepare (variant selection, metadata update and dispatch plan in one host call) writes,
+    array for array, what the separate entry points write: the reference's exact plan, the fixed-partition plan,
+    and the three dispatch plans on top of it."""
+    import importlib
+
+    L = importlib.import_module("psi-dec_amd._lib")
+    rng = np.random.default_rng(500 + seed)
+    n = int(rng.integers(1, 9))
+    q_len = int(rng.choice([1, 1, 2, 4, 11]))
+    q_lens = np.full(n, q_len) if rng.random() < 0.6 else rng.integers(1, 12, size=n)
+    starts = rng.integers(0, 5000, size=n).astype(np.uint32)
+    slots = rng.permutation(16)[:n].astype(np.uint32)
+    cu = np.concatenate([[0], np.cumsum(q_lens)]).astype(np.uint32)
+    core = psi.GQACore(0, 24 * 256, 256, 24, 4, 0.0625)
+    gqa = psi.GQA(None, core, psi.GQAMetalConfig(65536, 64, 1e-6, 1e6))
+    max_tokens, max_splits, workers = 128, 2048, 8
+
+    def arrays(md):
+        s = md.replay_shape()
+        out = dict(shape=s, variant=md.split_kv_variant(), slots=md.h_req_slots[:s.num_tokens].tolist(),
+                   pos=md.h_flat_token_indices[:s.num_tokens].tolist(),
+                   tiles=md.h_q_token_tiles[:2 * s.num_q_token_tiles].tolist() if md.split_kv_variant().is_tiled() else None,
+                   splits=md.h_kv_splits[:3 * s.num_total_sdpa_map_task_templates].tolist(),
+                   cu=md.h_cu_kv_splits[:(s.num_q_token_tiles if md.split_kv_variant().is_tiled() else s.num_tokens) + 1].tolist(),
+                   index=None if md.h_partial_row_index is None else md.h_partial_row_index[:s.num_sdpa_map_task_templates].tolist(),
+                   workers=None if md.h_worker_cu is None else md.h_worker_cu.tolist(),
+                   groups=None if md.h_row_groups is None or not md.num_row_groups else
+                   (md.group_tiles, md.h_row_groups[:md.group_tiles * md.num_row_groups].tolist()))
+        return out
+
+    variant = psi.select_split_kv_variant(gqa.split_kv, max_tokens, None, starts.tolist(), cu.tolist())
+    # the reference's plan
+    a = psi.GQAMetadataBuffers(None, max_tokens)
+    a.update(slots, starts, cu, variant)
+    b = psi.GQAMetadataBuffers(None, max_tokens)
+    assert gqa.prepare(b, slots, starts, cu) == a.replay_shape()
+    assert arrays(a) == arrays(b)
+    for dispatch in ("plan", "longest", "balanced", "groups"):
+        a = psi.GQAMetadataBuffers(None, max_tokens, max_kv_splits=max_splits, max_workers=workers)
+        a.update_fixed_partition(slots, starts, cu, variant, 256)
+        if dispatch == "longest":
+            a.order_longest_first()
+        elif dispatch == "balanced" or (dispatch == "groups" and not variant.is_tiled()):
+            a.balance(workers)
+        elif dispatch == "groups":
+            cfg = psi.GQASplitKVTiledQConfig(24, 4, 256, variant.q_head_tile_size, variant.q_token_tile_size,
+                                             variant.kv_token_tile_size, 0.0625, 65536, psi.Dtype.Bfloat16, None)
+            a.group_rows(cfg)
+        b = psi.GQAMetadataBuffers(None, max_tokens, max_kv_splits=max_splits, max_workers=workers)
+        b.prepare(gqa.struct(), slots, starts, cu, capacity_mode=L.CAPACITY_FIXED_PARTITION, partition_tokens=256,
+                  dispatch={"plan": L.DISPATCH_PLAN_ORDER, "longest": L.DISPATCH_LONGEST_FIRST,
+                            "balanced": L.DISPATCH_BALANCED, "groups": L.DISPATCH_ROW_GROUPS}[dispatch],
+                  num_workers=workers)
+        assert arrays(a) == arrays(b), dispatch
+        if variant.is_tiled():
+            assert b.max_active_q_tile_tokens == min(int(q_lens.max()), variant.q_token_tile_size)
