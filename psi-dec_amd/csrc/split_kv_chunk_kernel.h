@@ -15,37 +15,31 @@
 //   barrier per tile; global loads run two tiles ahead in two register sets).
 //
 // Per 32-key tile and wave (16 columns)
-//   QK^T  S[key][column] on v_mfma_f32_16x16x32: A = K rows from LDS, B = the query columns, held
-//         in registers for the whole kernel.  Row i of key block b is key 8*(i/4) + 4*b + i%4, so
-//         that a lane ends up with keys 8*(lane/16) .. +7 of its column: the B-operand layout of
-//         the next contraction.
-//   softmax  per column, in-lane over 8 keys; masks only on tiles that touch the start of the range
+//   QK^T  S[key][column] on v_mfma_f32_16x16x32 of the storage type: A = K rows from LDS (key 16 * b + i in row i of
+//         key block b), B = the query columns, held in registers for the whole kernel.  A lane ends up with keys
+//         16 * b + 4 * (lane / 16) + r, r = 0..3, b = 0, 1, of its column.
+//   softmax  per column, in-lane over those 8 keys; masks only on tiles that touch the start of the range
 //         or a column's causal limit.  The reference maximum of a column moves only when a tile
 //         exceeds it by more than 2^8; a wave-wide vote guards the cross-lane maximum and the
 //         rescaling of the accumulators, which therefore run a handful of times per range.
 //         Probabilities stay below 2^8.
-//   PV    O^T[dim][column] += V^T[dim][key] * P^T[key][column] on v_mfma_f32_16x16x32: A = V^T
-//         from LDS (the tile is transposed once, on its way into LDS, so that a lane reads its 8
-//         keys of one dim as one 128-bit word), B = the probabilities from registers.  The
-//         accumulators keep a column per lane, so rescaling needs no cross-lane traffic.  bf16
-//         probabilities are two truncated bf16 terms (two MFMAs), f16 one rounded term.
-//
-// What bounds it: every wave reads the whole K and V^T tile from LDS (8 x 32 KB per 32 keys), which is
-// about as long as the MFMA work of the tile; 16 columns per wave is what fits next to the query
-// operands in 256 registers.
+//   PV    O^T[dim][column] += V^T[dim][key] * P^T[key][column] on v_mfma_f32_16x16x32_f16: B = the probabilities,
+//         rounded once to f16 (11 significant bits; one bf16 term alone, 8 bits, costs the whole output tolerance,
+//         and two bf16 terms cost half as many matrix instructions again), A = V^T read straight out of the
+//         row-major V tile with the transposing LDS read of gfx950 (ds_read_b64_tr_b16: the 16 lanes of a quarter
+//         wave hand in 16 addresses of 4 elements each, a 16 x 4 block, and get it back transposed - lane 4a + c
+//         receives element c of the addresses a, a + 4, a + 8, a + 12), so no instruction of the kernel
+//         transposes V.  The V tile is kept as f16 in LDS: bf16 pages are converted once per tile on their way
+//         from the load registers into LDS (exact for 6.1e-5 <= |v| <= 65504; smaller magnitudes lose bits or
+//         flush to zero, larger ones saturate - neither occurs in a KV cache, and both stay far inside the output
+//         tolerance for values that do).  The accumulators keep a column per lane, so rescaling needs no
+//         cross-lane traffic.
 //
 // LDS layout per buffer
-//   K    [32 keys][D] elements, 16-byte chunk index XOR (key%4 + 4*(key/8)): the 16 lanes of an
-//        operand read (16 rows, one chunk) then hit 16 different bank groups, and a row-wise store
-//        stays a permutation of its row.
-//   V^T  [D dims][32 keys] elements: 64-byte rows, 64 bytes of padding after every 8 rows, the 16-byte
-//        slot of keys 8s .. 8s+7 at position (s + 2 * (row/4)) % 4.  A 128-bit read is served in four
-//        rounds of 16 lanes, and the rounds are not the quarters of the wave: lanes 0-3, 12-15 and 20-27
-//        go together, then 4-11, 16-19 and 28-31, and the same in the upper half.  With this slot
-//        function the operand read (lane = row % 16 + 16 * slot) puts the 16 lanes of every round on 16
-//        different bank groups (480 bytes per ns and CU measured, the rate of the K reads; an XOR of the
-//        slot with (row/4)%4, conflict-free over plain quarters, measures 288).  Transposing stores (4 rows
-//        8 apart, all 16 key pairs) cover 256 bytes of distinct banks.
+//   K    [32 keys][D] elements, 16-byte chunk index XOR (key % 16): the 16 lanes of an operand read (16 rows, one
+//        chunk) then hit 16 different bank groups, and a row-wise store stays a permutation of its row.
+//   V    [32 keys][D] f16, rows padded to D * 2 + 32 bytes: the four keys of a quarter wave's transposing read
+//        (32 bytes each, 16 dims) then fall into different bank groups, and so do the eight keys of two quarters.
 //   page IDs of up to 4096 pages of the range, refilled for longer ranges.
 #pragma once
 #include "split_kv_tiled_kernel.h"
@@ -60,35 +54,37 @@ static_assert(kChunkWaves * kChunkWaveCols == kChunkCols, "128 query columns per
 constexpr uint32_t kNoRow = 0xffffffffu;
 typedef __attribute__((ext_vector_type(4))) uint32_t u32x4_t;  // 128-bit word that stays in registers
 
-// Probabilities of 8 keys -> B operand(s) of the 16x16x32 contraction.
+// Probabilities of 8 keys -> B operand of the 16x16x32 f16 contraction: one term, rounded to nearest.
+__device__ __forceinline__ uint4 prob_operand_f16(const float (&p)[8]) {
+    const f16x8_t h = {(_Float16)p[0], (_Float16)p[1], (_Float16)p[2], (_Float16)p[3],
+                       (_Float16)p[4], (_Float16)p[5], (_Float16)p[6], (_Float16)p[7]};
+    return __builtin_bit_cast(uint4, h);
+}
+
+// 8 elements of the storage type -> 8 f16.  bf16: widening is exact, the narrowing truncates (exact inside the
+// f16 range, see the header).
 template <typename Tag>
-struct ProbOperand8;
+__device__ __forceinline__ u32x4_t to_f16x8(u32x4_t w);
 template <>
-struct ProbOperand8<BF16Tag> {
-    static constexpr int kTerms = 2;
-    uint4 term[2];
-    __device__ __forceinline__ void set(const float (&p)[8]) {
-        uint32_t hi[8], lo[8];
+__device__ __forceinline__ u32x4_t to_f16x8<F16Tag>(u32x4_t w) { return w; }
+template <>
+__device__ __forceinline__ u32x4_t to_f16x8<BF16Tag>(u32x4_t w) {
+    u32x4_t out;
 #pragma unroll
-        for (int j = 0; j < 8; ++j) {
-            hi[j] = __float_as_uint(p[j]) & 0xffff0000u;
-            lo[j] = __float_as_uint(p[j] - __uint_as_float(hi[j]));
-        }
-        term[0] = make_uint4((hi[0] >> 16) | hi[1], (hi[2] >> 16) | hi[3], (hi[4] >> 16) | hi[5], (hi[6] >> 16) | hi[7]);
-        term[1] = make_uint4((lo[0] >> 16) | (lo[1] & 0xffff0000u), (lo[2] >> 16) | (lo[3] & 0xffff0000u),
-                             (lo[4] >> 16) | (lo[5] & 0xffff0000u), (lo[6] >> 16) | (lo[7] & 0xffff0000u));
+    for (int i = 0; i < 4; ++i) {
+        const float lo = __uint_as_float(w[i] << 16), hi = __uint_as_float(w[i] & 0xffff0000u);
+        out[i] = __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_pkrtz(lo, hi));
     }
-};
-template <>
-struct ProbOperand8<F16Tag> {
-    static constexpr int kTerms = 1;
-    uint4 term[1];
-    __device__ __forceinline__ void set(const float (&p)[8]) {
-        const f16x8_t h = {(_Float16)p[0], (_Float16)p[1], (_Float16)p[2], (_Float16)p[3],
-                           (_Float16)p[4], (_Float16)p[5], (_Float16)p[6], (_Float16)p[7]};
-        term[0] = __builtin_bit_cast(uint4, h);
-    }
-};
+    return out;
+}
+
+typedef __attribute__((ext_vector_type(4))) short tr_s16x4_t;
+// Transposing LDS read: see the header.  `p` is this lane's address of 4 consecutive 2-byte elements.
+__device__ __forceinline__ uint2 lds_read_tr16_b64(const unsigned char* p) {
+    const tr_s16x4_t v = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
+        (__attribute__((address_space(3))) tr_s16x4_t*)(const_cast<unsigned char*>(p)));
+    return __builtin_bit_cast(uint2, v);
+}
 
 __device__ __forceinline__ uint32_t wave_min_u32(uint32_t v) {
 #pragma unroll
@@ -104,7 +100,8 @@ __device__ __forceinline__ uint32_t wave_max_u32(uint32_t v) {
 template <int D>
 struct ChunkLds {
     static constexpr int kKBytes = kChunkKeys * D * 2;
-    static constexpr int kVtBytes = D * kChunkKeys * 2 + (D / 8) * 64;
+    static constexpr int kVStride = D * 2 + 32;  // bytes per key row of the V tile
+    static constexpr int kVtBytes = kChunkKeys * kVStride;
     static constexpr int kIdCap = 4096;  // page IDs of a stretch of the KV range kept in LDS (+8: two tiles of look-ahead)
     static constexpr int bytes = 2 * (kKBytes + kVtBytes) + (kIdCap + 8) * 4;
 };
@@ -123,6 +120,7 @@ __global__ __launch_bounds__(64 * kChunkWaves, 2) void split_kv_chunk_map(
     constexpr int kLoads = kChunkKeys * kRowChunks / (64 * kChunkWaves);  // 128-bit loads per thread and operand (2)
     constexpr int kKBytes = ChunkLds<D>::kKBytes;
     constexpr int kVtBytes = ChunkLds<D>::kVtBytes;
+    constexpr int kVStride = ChunkLds<D>::kVStride;
     constexpr int kBufBytes = kKBytes + kVtBytes;
     constexpr int CB = kChunkColBlocks;
     constexpr float kSlack = 8.0f;
@@ -233,67 +231,55 @@ __global__ __launch_bounds__(64 * kChunkWaves, 2) void split_kv_chunk_map(
                          base + __builtin_amdgcn_readfirstlane(ids.b) * page_bytes + in_page};
     };
 
-    // ---- cooperative tile loaders: per-thread byte offsets inside a page are fixed for the kernel
+    // ---- cooperative tile loaders: per-thread byte offsets inside a page are fixed for the kernel.  Thread
+    // (ld_sub, ld_chunk) takes the 16-byte chunk ld_chunk of keys ld_sub and 16 + ld_sub, of K and of V.
     constexpr int kSubs = 64 * kChunkWaves / kRowChunks;  // 16
-    const uint32_t ld_chunk = tid % kRowChunks;   // K: 16-byte chunk of a row (8 dims)
-    const uint32_t ld_sub = tid / kRowChunks;     // K: load j takes key kSubs * j + ld_sub
-    // V goes the other way round: 16 adjacent lanes take the 16 key pairs of one chunk, so that a
-    // transposing store instruction covers whole 64-byte rows of V^T.
-    const uint32_t v_pair = tid % kSubs;          // V: load j takes key 2 * v_pair + j
-    const uint32_t v_chunk = tid / kSubs;
-    const bool small_page = a.walk.tokens_per_page == 16;  // keys 16..31 of a tile then start their own page
-    uint32_t k_off[kLoads], v_off[kLoads];
-#pragma unroll
-    for (int j = 0; j < kLoads; ++j) {
-        const uint32_t k_key = kSubs * j + ld_sub, v_key = kLoads * v_pair + j;
-        k_off[j] = ((kv_head * a.walk.tokens_per_page + (small_page ? (k_key & 15) : k_key)) * D + ld_chunk * 8) * 2;
-        v_off[j] = (((a.walk.hkv + kv_head) * a.walk.tokens_per_page + (small_page ? (v_key & 15) : v_key)) * D + v_chunk * 8) * 2;
-    }
+    const uint32_t ld_chunk = tid % kRowChunks;
+    const uint32_t ld_sub = tid / kRowChunks;
+    const uint32_t k_off = ((kv_head * a.walk.tokens_per_page + ld_sub) * D + ld_chunk * 8) * 2;
+    const uint32_t v_off = (((a.walk.hkv + kv_head) * a.walk.tokens_per_page + ld_sub) * D + ld_chunk * 8) * 2;
+    // keys 16..31 sit 16 rows further on in a page that holds the whole tile, and at the same offset of the next
+    // page otherwise (tile_bases then points at that page)
+    const uint32_t second_half = a.walk.tokens_per_page == 16 ? 0u : 16u * D * 2u;
     struct Staging {
         u32x4_t k[kLoads], v[kLoads];
     };
     auto issue_loads = [&](TileBases tb) __attribute__((always_inline)) -> Staging {
         Staging st;
-        st.k[0] = *reinterpret_cast<const u32x4_t*>(tb.a + k_off[0]);  // keys 0..15
-        st.k[1] = *reinterpret_cast<const u32x4_t*>(tb.b + k_off[1]);  // keys 16..31
-        const unsigned char* vb = v_pair < 8 ? tb.a : tb.b;
-#pragma unroll
-        for (int j = 0; j < kLoads; ++j) st.v[j] = *reinterpret_cast<const u32x4_t*>(vb + v_off[j]);
+        st.k[0] = *reinterpret_cast<const u32x4_t*>(tb.a + k_off);                // keys 0..15
+        st.k[1] = *reinterpret_cast<const u32x4_t*>(tb.b + k_off + second_half);  // keys 16..31
+        st.v[0] = *reinterpret_cast<const u32x4_t*>(tb.a + v_off);
+        st.v[1] = *reinterpret_cast<const u32x4_t*>(tb.b + v_off + second_half);
         return st;
     };
     // Registers -> LDS buffer `buf`.  V rows outside [kv_begin, kv_end_max) are zeroed: their
     // probability is 0 but their bytes may be NaN / Inf.
-    const uint32_t k_store0 = ld_sub * (D * 2) + ((ld_chunk ^ ((ld_sub & 3) + 4 * (ld_sub >> 3))) * 16);
-    const uint32_t k_store1 = (kSubs + ld_sub) * (D * 2) + ((ld_chunk ^ ((ld_sub & 3) + 4 * ((kSubs + ld_sub) >> 3))) * 16);
+    const uint32_t k_store0 = ld_sub * (D * 2) + ((ld_chunk ^ ld_sub) * 16);
+    const uint32_t k_store1 = k_store0 + kSubs * (D * 2);
+    const uint32_t v_store0 = ld_sub * kVStride + ld_chunk * 16;
+    const uint32_t v_store1 = v_store0 + kSubs * kVStride;
     auto store_tile = [&](uint32_t it, uint32_t buf, const Staging& st) __attribute__((always_inline)) {
         unsigned char* kbuf = lds + buf * kBufBytes;
         unsigned char* vbuf = kbuf + kKBytes;
         const uint32_t kb = key_base0 + min(it, num_kv_tiles - 1) * kChunkKeys;
         *reinterpret_cast<u32x4_t*>(kbuf + k_store0) = st.k[0];
         *reinterpret_cast<u32x4_t*>(kbuf + k_store1) = st.k[1];
-        u32x4_t w0 = st.v[0], w1 = st.v[1];
+        u32x4_t w0 = to_f16x8<Tag>(st.v[0]), w1 = to_f16x8<Tag>(st.v[1]);
         if (kb < kv_begin || kb + kChunkKeys > kv_end_max) {  // first or last tile of the range
-            const uint32_t token = kb + kLoads * v_pair;
+            const uint32_t token = kb + ld_sub;
             if (token < kv_begin || token >= kv_end_max) w0 = u32x4_t{0u, 0u, 0u, 0u};
-            if (token + 1 < kv_begin || token + 1 >= kv_end_max) w1 = u32x4_t{0u, 0u, 0u, 0u};
+            if (token + kSubs < kv_begin || token + kSubs >= kv_end_max) w1 = u32x4_t{0u, 0u, 0u, 0u};
         }
-#pragma unroll
-        for (int e = 0; e < 8; ++e) {
-            const int word = e / 2;
-            const uint32_t out = e % 2 == 0 ? ((w0[word] & 0xffffu) | (w1[word] << 16))
-                                            : ((w0[word] >> 16) | (w1[word] & 0xffff0000u));
-            // row = 8 * v_chunk + e; its 16-byte slot v_pair / 4 is rotated by 2 * (row / 4): 2 * (e / 4) mod 4
-            const uint32_t slot = ((v_pair >> 2) + 2 * (e / 4)) & 3;
-            *reinterpret_cast<uint32_t*>(vbuf + (8 * v_chunk + e) * 64 + v_chunk * 64 + slot * 16 + (v_pair & 3) * 4) = out;
-        }
+        *reinterpret_cast<u32x4_t*>(vbuf + v_store0) = w0;
+        *reinterpret_cast<u32x4_t*>(vbuf + v_store1) = w1;
     };
 
     // ---- operand read addresses of this lane
-    // K row of (block b, lane row mt): key 8 * (mt / 4) + 4 * b + mt % 4, chunk (4 * ks + mc) ^ swizzle
-    const uint32_t k_swz = mt;  // = key % 4 + 4 * (key / 8) for both key blocks
-    const uint32_t k_row0 = (8 * (mt >> 2) + (mt & 3)) * (D * 2);
-    // V^T row of (dim block db, lane row mt): dim 16 * db + mt, keys 8 * mc .. +7
-    const uint32_t vt_row0 = mt * 64 + (mt >> 3) * 64 + (((mc + 2 * (mt >> 2)) & 3) * 16);
+    // K row of (block b, lane row mt): key 16 * b + mt, chunk (4 * ks + mc) ^ mt
+    const uint32_t k_row0 = mt * (D * 2);
+    // V^T operand of (dim block db, key block b): the lane hands in the address of key 16 * b + 4 * mc + mt / 4,
+    // dims 16 * db + 4 * (mt % 4) .. + 3, and receives keys 16 * b + 4 * mc + 0..3 of dim 16 * db + mt
+    const uint32_t vt_base = (4 * mc + (mt >> 2)) * kVStride + (mt & 3) * 8;
 
     float run_max = -INFINITY, lane_sum = 0.0f;
     f32x4_t o[kDimBlocks];
@@ -315,9 +301,9 @@ __global__ __launch_bounds__(64 * kChunkWaves, 2) void split_kv_chunk_map(
         constexpr int kAhead = 4;
         uint4 k0[kKSteps], k1[kKSteps];
         auto read_k = [&](int ks) __attribute__((always_inline)) {
-            const uint32_t off = k_row0 + (((4 * ks + mc) ^ k_swz) * 16);
+            const uint32_t off = k_row0 + (((4 * ks + mc) ^ mt) * 16);
             k0[ks] = *reinterpret_cast<const uint4*>(kbuf + off);
-            k1[ks] = *reinterpret_cast<const uint4*>(kbuf + off + 4 * (D * 2));
+            k1[ks] = *reinterpret_cast<const uint4*>(kbuf + off + 16 * (D * 2));
         };
         __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
@@ -336,7 +322,7 @@ __global__ __launch_bounds__(64 * kChunkWaves, 2) void split_kv_chunk_map(
         }
         __builtin_amdgcn_sched_group_barrier(0x008, 2 * kAhead, 0);
         __builtin_amdgcn_sched_barrier(0);
-        // ---- online softmax; this lane holds keys kb + 8 * mc + j, j = 4 * b + r, of column mt.
+        // ---- online softmax; this lane holds keys kb + 16 * b + 4 * mc + r, j = 4 * b + r, of column mt.
         // Logits relative to the column's reference maximum; masked keys at -inf.
         float v[8];  // raw logits; masked keys at -inf
 #pragma unroll
@@ -344,7 +330,7 @@ __global__ __launch_bounds__(64 * kChunkWaves, 2) void split_kv_chunk_map(
         if (masked) {
 #pragma unroll
             for (int j = 0; j < 8; ++j) {
-                const uint32_t token = kb + 8 * mc + j;
+                const uint32_t token = kb + 16 * (j >> 2) + 4 * mc + (j & 3);
                 if (token < kv_begin || token >= lim) v[j] = -INFINITY;
             }
         }
@@ -376,19 +362,19 @@ __global__ __launch_bounds__(64 * kChunkWaves, 2) void split_kv_chunk_map(
             tile_sum += p[j];
         }
         lane_sum += tile_sum;
-        ProbOperand8<Tag> pb;
-        pb.set(p);
-        // ---- O^T[dim][column] += V^T * P^T
-        // four dim blocks at a time: four independent accumulators between the two terms of one block
+        const uint4 pb = prob_operand_f16(p);
+        // ---- O^T[dim][column] += V^T * P^T, four dim blocks at a time
 #pragma unroll
         for (int g = 0; g < kDimBlocks; g += 4) {
             uint4 vt[4];
 #pragma unroll
-            for (int i = 0; i < 4; ++i) vt[i] = *reinterpret_cast<const uint4*>(vbuf + vt_row0 + (g + i) * (16 * 64 + 2 * 64));
+            for (int i = 0; i < 4; ++i) {
+                const unsigned char* src = vbuf + vt_base + (g + i) * 32;
+                const uint2 lo = lds_read_tr16_b64(src), hi = lds_read_tr16_b64(src + 16 * kVStride);
+                vt[i] = make_uint4(lo.x, lo.y, hi.x, hi.y);
+            }
 #pragma unroll
-            for (int t = 0; t < ProbOperand8<Tag>::kTerms; ++t)
-#pragma unroll
-                for (int i = 0; i < 4; ++i) o[g + i] = mfma_16x16x32<Tag>(vt[i], pb.term[t], o[g + i]);
+            for (int i = 0; i < 4; ++i) o[g + i] = mfma_16x16x32<F16Tag>(vt[i], pb, o[g + i]);
         }
     };
 

@@ -523,20 +523,20 @@ def check_groups(meta, shape, tile_size, max_tiles):
 
 def test_row_groups_of_a_prefill_chunk(psi):
     """A 70-token chunk on a 300-token prefix, 256-token partitions, next to two decode requests:
-    24 Q / 4 KV heads deal 3 heads to a workgroup, so a group holds 5 tiles of 8 tokens."""
+    24 Q / 4 KV heads deal 2 heads to a workgroup, so a group holds 8 tiles of 8 tokens."""
     meta = psi.GQAMetadataBuffers(None, 128, max_kv_splits=64)
     variant = psi.GQASplitKVVariant.TiledQ(8, 16, 6)
     shape = meta.update_fixed_partition([3, 1, 5], [300, 40, 999], [0, 70, 71, 72], variant, 256)
     assert meta.group_rows(tiled_config(psi, 24, 4)) == meta.num_row_groups > 0
-    table = check_groups(meta, shape, 8, 5)
+    table = check_groups(meta, shape, 8, 8)
     rows = meta.h_kv_splits.reshape(-1, 3)
-    # the chunk has 9 tiles; partition 0 is seen by all of them -> groups of 5 + 4
+    # the chunk has 9 tiles; partition 0 is seen by all of them -> groups of 8 + 1
     sizes = sorted(int((g != MAX).sum()) for g in table if rows[g[0]][1] == 0 and rows[g[0]][0] < 9)
-    assert sizes == [4, 5]
+    assert sizes == [1, 8]
     # the groups survive a re-ordering of the rows (positions change, membership does not)
     meta.order_longest_first()
     meta.group_rows(tiled_config(psi, 24, 4))
-    check_groups(meta, shape, 8, 5)
+    check_groups(meta, shape, 8, 8)
 
 
 @pytest.mark.parametrize("hq,hkv,expected", [(16, 2, 4), (8, 2, 4), (4, 4, 16), (10, 2, 3), (14, 2, 4)])
@@ -572,11 +572,11 @@ def test_row_group_table_capacity_is_checked(psi):
     rc = lib.psi_hip_split_kv_tiled_q_group_rows(ctypes.byref(cfg), 8, p(rows), 2, p(tiles), 2, p(slots), p(table), 5,
                                                  ctypes.byref(n_tiles), ctypes.byref(n_groups))
     assert rc != 0 and b"row-group table too small" in lib.psi_hip_last_error()
-    table = np.zeros(10, np.uint32)
+    table = np.zeros(16, np.uint32)
     assert lib.psi_hip_split_kv_tiled_q_group_rows(ctypes.byref(cfg), 8, p(rows), 2, p(tiles), 2, p(slots), p(table),
-                                                   10, ctypes.byref(n_tiles), ctypes.byref(n_groups)) == 0
-    assert (n_tiles.value, n_groups.value) == (5, 2)  # two requests never share a group
-    assert table.tolist() == [0, MAX, MAX, MAX, MAX, 1, MAX, MAX, MAX, MAX]
+                                                   16, ctypes.byref(n_tiles), ctypes.byref(n_groups)) == 0
+    assert (n_tiles.value, n_groups.value) == (8, 2)  # two requests never share a group
+    assert table.tolist() == [0] + [MAX] * 7 + [1] + [MAX] * 7
 
 
 # ------------------------------------------------------------------ the whole plan in one call
