@@ -163,9 +163,11 @@ def build_case(psi, wl, device, name, args):
                            args.arenas or 1, 5)
     if name == "C5_prefill":
         w = wl.make_workload(5, [4096 + 2048], 24, 4, 256, bf16, 16, q_lens=2048, host_pages=False)
-        dw = wl.DeviceWorkload(device, w, partition_tokens=8192, grouped=True,
+        # 4096-token partitions: two rows per query tile, twice as many work items of half the size, which fill
+        # the 256 compute units evenly (unsplit, 384 items make one and a half rounds: 375 against 323 us)
+        dw = wl.DeviceWorkload(device, w, partition_tokens=4096, grouped=True,
                                variant=psi.GQASplitKVVariant.TiledQ(8, 16, 6))
-        case = Case(name, "prefill_chunk2048_on_prefix4096_24q4kv_d256_bf16_p16_unsplit_seed5", [dw], "prefill",
+        case = Case(name, "prefill_chunk2048_on_prefix4096_24q4kv_d256_bf16_p16_part4096_seed5", [dw], "prefill",
                     "tiled_q_map", "split_kv_chunk_map", "kv append -> row-group (prefill-chunk) map -> LSE combine")
         case.flops = 4 * 24 * 256 * sum(4096 + i + 1 for i in range(2048))
         return case

@@ -78,14 +78,6 @@ __device__ __forceinline__ u32x4_t to_f16x8<BF16Tag>(u32x4_t w) {
     return out;
 }
 
-typedef __attribute__((ext_vector_type(4))) short tr_s16x4_t;
-// Transposing LDS read: see the header.  `p` is this lane's address of 4 consecutive 2-byte elements.
-__device__ __forceinline__ uint2 lds_read_tr16_b64(const unsigned char* p) {
-    const tr_s16x4_t v = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
-        (__attribute__((address_space(3))) tr_s16x4_t*)(const_cast<unsigned char*>(p)));
-    return __builtin_bit_cast(uint2, v);
-}
-
 __device__ __forceinline__ uint32_t wave_min_u32(uint32_t v) {
 #pragma unroll
     for (int s = 1; s < 64; s <<= 1) v = min(v, (uint32_t)__shfl_xor((int)v, s, 64));

@@ -81,6 +81,16 @@ struct ProbOperand<F16Tag> {
     }
 };
 
+typedef __attribute__((ext_vector_type(4))) short tr_s16x4_t;
+// Transposing LDS read of gfx950 (ds_read_b64_tr_b16): the 16 lanes of a quarter wave hand in 16 addresses of 4
+// consecutive 2-byte elements each, a 16 x 4 block, and get it back transposed: lane 4 * a + c receives element c of
+// the addresses a, a + 4, a + 8, a + 12.
+__device__ __forceinline__ uint2 lds_read_tr16_b64(const void* p) {
+    const tr_s16x4_t v = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
+        (__attribute__((address_space(3))) tr_s16x4_t*)(const_cast<void*>(p)));
+    return __builtin_bit_cast(uint2, v);
+}
+
 constexpr float kMaxSlack = 8.0f;   // see the softmax of split_kv_tiled_map
 constexpr int kTiledTileWaves = 4;  // waves that share the KV tiles of a split among them
 
@@ -109,7 +119,8 @@ __global__ __launch_bounds__(64 * kTiledTileWaves * CG, (TiledOccupancy<NB, CG>:
     constexpr int kVLoads = kTileTokens / kVTokensPerLoad;  // 8 or 4
     constexpr int kKSteps = D / 32;                         // MFMA k-steps of QK^T
     constexpr int kDimBlocks = D / 16;                      // 16-dim output blocks of PV
-    constexpr int kVStride = D + 8;                         // elements per token row of the V buffer (bank spread)
+    constexpr int kVStride = D + 16;                        // elements per token row of the V buffer: the four rows of a
+                                                            // quarter wave's transposing read fall into different banks
     constexpr int kCols = CG * NB * 16;
     constexpr int kMergeStride = D + 4;                     // floats per column row of the merge buffer
 
@@ -264,8 +275,10 @@ __global__ __launch_bounds__(64 * kTiledTileWaves * CG, (TiledOccupancy<NB, CG>:
     };
 
     uint16_t* my_v = v_lds + wave * kTileTokens * kVStride;
-    // B operand of PV for dim block db: 4 consecutive tokens of this lane's token quad, one dim.
-    const uint16_t* my_v_read = my_v + (mc * 4) * kVStride + mt;
+    // B operand of PV for dim block db (tokens 4 * mc .. + 3 of dim 16 * db + mt) through the transposing LDS read:
+    // the lane hands in the address of token 4 * mc + mt / 4, dims 16 * db + 4 * (mt % 4) .. + 3, and the 16 lanes of
+    // a quarter wave get their 16 x 4 block back transposed.
+    const uint16_t* my_v_read = my_v + (mc * 4 + (mt >> 2)) * kVStride + (mt & 3) * 4;
 
     auto process_tile = [&](uint32_t tile, bool partial, auto has_next_tag, uint32_t next, TilePages next_pid)
                             __attribute__((always_inline)) {
@@ -374,9 +387,7 @@ __global__ __launch_bounds__(64 * kTiledTileWaves * CG, (TiledOccupancy<NB, CG>:
         }
 #pragma unroll
         for (int db = 0; db < kDimBlocks; ++db) {
-            const uint16_t* src = my_v_read + db * 16;
-            const uint32_t v0 = src[0], v1 = src[kVStride], v2 = src[2 * kVStride], v3 = src[3 * kVStride];
-            const uint2 b = make_uint2(v0 | (v1 << 16), v2 | (v3 << 16));
+            const uint2 b = lds_read_tr16_b64(my_v_read + db * 16);
 #pragma unroll
             for (int nb = 0; nb < NB; ++nb) {
                 if ((uint32_t)nb < nb_active) {
