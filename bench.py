@@ -63,6 +63,7 @@ def parse_args():
     p.add_argument("--plan-order", action="store_true", help="row-per-workgroup launch in plan order, not longest first")
     p.add_argument("--separate-append", action="store_true", help="decode: launch the append as its own kernel")
     p.add_argument("--workers", type=int, default=0, help="balanced plan: workers per KV head (0 = one workgroup per CU)")
+    p.add_argument("--grouped", action="store_true", help="custom multi-query workload: row-group (prefill-chunk) map")
     p.add_argument("--row-per-workgroup", action="store_true", help="one workgroup per partition row, no worker plan")
     p.add_argument("--graph", action="store_true",
                    help="submit every step through the per-bucket program cache (HIP graph replay) instead of launching")
@@ -110,7 +111,8 @@ def build_case(psi, wl, device, name, args):
     bf16 = psi.Dtype.Bfloat16
     decode_how = dict(balanced=not args.row_per_workgroup, longest_first=not args.plan_order,
                       fused_append=not args.separate_append, num_workers=args.workers or None)
-    verify_how = dict(balanced=not args.row_per_workgroup, longest_first=not args.plan_order)
+    verify_how = dict(balanced=not args.row_per_workgroup, longest_first=not args.plan_order,
+                      num_workers=args.workers or None)
 
     def decode_case(key, ctxs, hq, hkv, dtype, partition, arenas, seed, kernel="split_kv_decode_map", **kw):
         out = []
@@ -142,6 +144,13 @@ def build_case(psi, wl, device, name, args):
                f"_{args.q_heads}q{args.kv_heads}kv_d256_{args.dtype}_p16_part{args.partition}_seed{args.seed}")
         if args.q_len == 1:
             return decode_case(key, ctx, args.q_heads, args.kv_heads, elem, args.partition, args.arenas or 2, args.seed)
+        if args.grouped:
+            w = wl.make_workload(args.seed, ctx, args.q_heads, args.kv_heads, 256, elem, 16, q_lens=args.q_len,
+                                 host_pages=False)
+            dw = wl.DeviceWorkload(device, w, partition_tokens=args.partition, grouped=True,
+                                   variant=psi.GQASplitKVVariant.TiledQ(8, 16, args.q_heads // args.kv_heads))
+            return Case(name, key + "_grouped", [dw], "verify", "tiled_q_map", "split_kv_chunk_map",
+                        "kv append -> row-group (prefill-chunk) map -> LSE combine")
         return verify_case(key, ctx, args.q_len, args.partition, args.arenas or 1, args.seed)
     if name == "C1":
         # 1 MB per arena: enough arenas that a page comes back only after 300 MB of other pages went through the

@@ -483,6 +483,470 @@ __global__ __launch_bounds__(64 * kTiledTileWaves * CG, (TiledOccupancy<NB, CG>:
     }  // rows of this workgroup
 }
 
+// ---------------------------------------------------------------------------------------------------------------
+// The streaming variant: up to three column blocks per wave, KV tiles brought into LDS by the load unit itself.
+//
+// A 16-token tile of K (and of V) is 16 rows of D elements.  `global_load_lds_dwordx4` moves 16 bytes per lane from
+// a per-lane global address to LDS address M0 + instruction offset + 16 * lane, with no register in between, so a
+// wave keeps two tiles of K and two of V in flight or in use without holding any of them in registers: the loads of
+// tile i + 2 go out as soon as tile i has been multiplied.  One instruction covers 8 rows x 128 bytes (whole lines):
+// lane p = 8 * c + t fetches chunk c (8 elements) of row t, and lands at slot p of a 1 KiB block; a tile is
+// 2 * D / 64 such blocks, [row half][line of the row].  Read back, the A operand of K * Q^T (16 rows x 8 elements
+// per quarter wave) and the transposed V block of a quarter wave both gather whole 16-byte slots, conflict-free.
+//
+// The loads are inline assembly, and so are the waits for them: the compiler does not know that they write LDS, and
+// where it does (the builtin) it waits for every outstanding one before any LDS read, which would undo the prefetch.
+// ---------------------------------------------------------------------------------------------------------------
+
+// Maximum over the four lanes l % 16 == const of a wave, in every one of them, on the vector ALU: the two swaps
+// exchange the odd 16-lane (32-lane) rows of one operand with the even rows of the other.
+__device__ __forceinline__ float quarter_wave_max(float x) {
+    const uint32_t u = __float_as_uint(x);
+    const auto h = __builtin_amdgcn_permlane32_swap(u, u, false, false);
+    const uint32_t m = __float_as_uint(fmaxf(__uint_as_float(h[0]), __uint_as_float(h[1])));
+    const auto q = __builtin_amdgcn_permlane16_swap(m, m, false, false);
+    return fmaxf(__uint_as_float(q[0]), __uint_as_float(q[1]));
+}
+
+// Line `kLine` (64 elements) of the 8 + 8 rows of a tile: two loads of 1 KiB, one per half tile.  The instruction
+// offset is added to the global and to the LDS address alike, hence 1024 - 128 between the M0 values of consecutive
+// lines.  `tie` is an accumulator that the matrix cores have just written from the last LDS operand read out of the
+// bytes these loads replace: LDS reads return in order, so once that product could be issued the stage's old
+// contents have been read, and naming it here keeps the loads behind that product.
+template <int kLine, int kHalfBytes>
+__device__ __forceinline__ void dma_tile_line(uint32_t lds_tile, const void* rows0, const void* rows1, f32x4_t& tie) {
+    asm volatile(
+        "s_add_u32 m0, %1, %4\n\ts_nop 0\n\t"
+        "global_load_lds_dwordx4 %2, off offset:%6 nt\n\t"
+        "s_add_u32 m0, %1, %5\n\ts_nop 0\n\t"
+        "global_load_lds_dwordx4 %3, off offset:%6 nt"
+        : "+a"(tie)
+        : "s"(lds_tile), "v"(rows0), "v"(rows1), "n"(kLine * 896), "n"(kHalfBytes + kLine * 896), "n"(kLine * 128)
+        : "memory", "m0", "scc");
+}
+template <int kLine, int kHalfBytes>
+__device__ __forceinline__ void dma_tile_line(uint32_t lds_tile, const void* rows0, const void* rows1) {
+    asm volatile(
+        "s_add_u32 m0, %0, %3\n\ts_nop 0\n\t"
+        "global_load_lds_dwordx4 %1, off offset:%5 nt\n\t"
+        "s_add_u32 m0, %0, %4\n\ts_nop 0\n\t"
+        "global_load_lds_dwordx4 %2, off offset:%5 nt"
+        :
+        : "s"(lds_tile), "v"(rows0), "v"(rows1), "n"(kLine * 896), "n"(kHalfBytes + kLine * 896), "n"(kLine * 128)
+        : "memory", "m0", "scc");
+}
+template <int kDQ, int kHalfBytes>
+__device__ __forceinline__ void dma_tile(uint32_t lds_tile, const void* rows0, const void* rows1) {
+    dma_tile_line<0, kHalfBytes>(lds_tile, rows0, rows1);
+    dma_tile_line<1, kHalfBytes>(lds_tile, rows0, rows1);
+    if constexpr (kDQ == 4) {
+        dma_tile_line<2, kHalfBytes>(lds_tile, rows0, rows1);
+        dma_tile_line<3, kHalfBytes>(lds_tile, rows0, rows1);
+    }
+}
+
+#ifndef PSI_Q_REGS_NB
+#define PSI_Q_REGS_NB 2
+#endif
+template <int N, typename F, int I = 0>
+__device__ __forceinline__ void static_for(F&& f) {
+    if constexpr (I < N) {
+        f(std::integral_constant<int, I>());
+        static_for<N, F, I + 1>(static_cast<F&&>(f));
+    }
+}
+
+// Waits until at most `kLoads * groups` of the wave's loads are outstanding (they complete in order).
+template <int kLoads>
+__device__ __forceinline__ void wait_load_groups(uint32_t groups) {
+    if (groups >= 3) asm volatile("s_waitcnt vmcnt(%0)" ::"n"(3 * kLoads) : "memory");
+    else if (groups == 2) asm volatile("s_waitcnt vmcnt(%0)" ::"n"(2 * kLoads) : "memory");
+    else if (groups == 1) asm volatile("s_waitcnt vmcnt(%0)" ::"n"(kLoads) : "memory");
+    else asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+}
+
+constexpr int tiled_stream_lds_bytes(int D, int NB) {
+    return kTiledTileWaves * 4 * (kTileTokens * D * 2) + NB * (D / 32) * 64 * 16;
+}
+
+template <typename Tag, int D, int NB, bool kHalfPage>
+__global__ __launch_bounds__(64 * kTiledTileWaves, 1) void split_kv_tiled_stream_map(
+    MapArgs a, const uint32_t* __restrict__ page_ids, const uint32_t* __restrict__ kv_splits,
+    const uint32_t* __restrict__ req_slots, const uint16_t* __restrict__ q, const uint16_t* __restrict__ pages,
+    const uint32_t* __restrict__ q_token_tiles, const uint32_t* __restrict__ flat_token_indices,
+    const uint32_t* __restrict__ worker_cu) {
+    resolve_active(a);
+    constexpr int kWaves = kTiledTileWaves;
+    constexpr int kKSteps = D / 32;             // MFMA k-steps of QK^T
+    constexpr int kDimBlocks = D / 16;          // 16-dim output blocks of PV
+    constexpr int kDQ = D / 64;                 // 128-byte lines per row
+    constexpr int kTileLoads = 2 * kDQ;         // load instructions per tile of K (or of V)
+    constexpr int kTileBytes = kTileTokens * D * 2;
+    constexpr int kHalfBytes = kTileBytes / 2;
+    constexpr int kWaveBytes = 4 * kTileBytes;  // K stage 0, K stage 1, V stage 0, V stage 1
+    constexpr int kCols = NB * 16;
+    constexpr int kMergeStride = D + 4;         // floats per column row of the merge buffer
+    constexpr int kStageBytes = kWaves * kWaveBytes;
+    constexpr int kQBytes = NB * kKSteps * 64 * 16;
+    static_assert(kCols * kMergeStride * 4 <= kStageBytes, "the merge buffer reuses the tile stages");
+
+    __shared__ __attribute__((aligned(1024))) unsigned char lds_union[kStageBytes + kQBytes];
+    __shared__ float wave_max_lds[kWaves][kCols];
+    __shared__ float col_max_lds[kCols];
+    __shared__ float col_sum_lds[kCols];
+    uint4* qb_lds = reinterpret_cast<uint4*>(lds_union + kStageBytes);  // [NB][kKSteps][64]
+    float* merge = reinterpret_cast<float*>(lds_union);
+
+    const uint32_t G = a.group;
+    const uint32_t kv_head = blockIdx.x % a.walk.hkv;
+    const uint32_t wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    unsigned char* my_stages = lds_union + wave * kWaveBytes;
+    const uint32_t my_stages_lds =
+        (uint32_t)(size_t)(__attribute__((address_space(3))) unsigned char*)(lds_union) + wave * kWaveBytes;
+
+    uint32_t row_begin = blockIdx.x / a.walk.hkv, row_end = row_begin + 1;
+    if (worker_cu != nullptr) {
+        row_begin = worker_cu[blockIdx.x / a.walk.hkv];
+        row_end = worker_cu[blockIdx.x / a.walk.hkv + 1];
+    }
+    bool lds_in_use = false;
+    for (uint32_t split = row_begin; split < row_end; ++split) {
+    if (split >= a.num_active_kv_splits) break;
+    const uint32_t q_tile = kv_splits[split * 3];
+    if (q_tile >= a.num_active_q_token_tiles) continue;  // sentinel padding
+    const uint32_t kv_begin = kv_splits[split * 3 + 1];
+    const uint32_t kv_end = kv_splits[split * 3 + 2];
+    const uint32_t flat_begin = q_token_tiles[q_tile * 2], flat_end = q_token_tiles[q_tile * 2 + 1];
+    if (flat_begin >= a.num_active_tokens || flat_end > a.num_active_tokens || flat_end <= flat_begin) continue;
+    const uint32_t tile_tokens = flat_end - flat_begin;
+    const uint32_t ncols = tile_tokens * G;
+    if (ncols > (uint32_t)kCols) {
+        // A tile wider than the launch was sized for: entered as an empty state (see split_kv_tiled_map).
+        const uint32_t rows = a.rows_per_split_head;
+        for (uint32_t idx = threadIdx.x; idx < ncols * (D / 4); idx += 64 * kWaves) {
+            const uint32_t c = idx / (D / 4), d4 = idx % (D / 4);
+            const uint64_t row = ((uint64_t)split * a.hq + (uint64_t)kv_head * G + c % G) * rows + c / G;
+            *reinterpret_cast<float4*>(&a.part_acc[row * D + d4 * 4]) = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
+            if (d4 == 0) {
+                a.part_max[row] = -INFINITY;
+                a.part_sum[row] = 0.0f;
+            }
+        }
+        continue;
+    }
+    if (lds_in_use) __syncthreads();  // the previous row's merge buffer has been read out
+    lds_in_use = true;
+    uint32_t tid = threadIdx.x;
+    asm volatile("" : "+v"(tid));  // lane coordinates re-derived per row (see split_kv_tiled_map)
+    const uint32_t lane = tid & 63;
+    const uint32_t mt = lane & 15, mc = lane >> 4;
+    const uint32_t nb_total = (ncols + 15) / 16;
+    const uint32_t nb_active = min(nb_total, (uint32_t)NB);
+    const uint32_t req_slot = req_slots[flat_begin];
+
+    uint32_t lim[NB];  // keys [kv_begin, lim) are visible to the column (0: column unused)
+#pragma unroll
+    for (int nb = 0; nb < NB; ++nb) {
+        const uint32_t c = nb * 16 + mt;
+        lim[nb] = 0;
+        if (c < ncols) lim[nb] = min(kv_end, flat_token_indices[flat_begin + c / G] + 1);
+    }
+
+    // Keys below `open_until` are visible to every column in use (the unused ones are never stored).
+    uint32_t open_until = kv_end;
+#pragma unroll
+    for (int nb = 0; nb < NB; ++nb)
+        if (lim[nb] != 0) open_until = min(open_until, lim[nb]);
+#pragma unroll
+    for (int sh = 1; sh < 64; sh <<= 1) open_until = min(open_until, (uint32_t)__shfl_xor((int)open_until, sh, 64));
+    open_until = __builtin_amdgcn_readfirstlane(open_until);
+
+    // Query columns as MFMA B operands [nb][k-step][lane]; unused columns are zero.
+    for (uint32_t nb = wave; nb < (uint32_t)NB; nb += kWaves) {
+        const uint32_t c = nb * 16 + mt;
+        const bool used = c < ncols;
+        const uint32_t cc = used ? c : 0;
+        const uint16_t* q_row =
+            q + ((uint64_t)(flat_begin + cc / G) * a.hq + (uint64_t)kv_head * G + cc % G) * D + mc * 8;
+#pragma unroll
+        for (int i = 0; i < kKSteps; ++i) {
+            const uint4 v = *reinterpret_cast<const uint4*>(q_row + i * 32);
+            qb_lds[(nb * kKSteps + i) * 64 + lane] = used ? v : make_uint4(0, 0, 0, 0);
+        }
+    }
+    __syncthreads();
+
+    // Up to two column blocks keep their query operands in registers for the whole row.
+    constexpr bool kQInRegs = NB <= PSI_Q_REGS_NB;
+    uint4 q_reg[kQInRegs ? NB * kKSteps : 1];
+    if (kQInRegs) {
+#pragma unroll
+        for (int j = 0; j < NB * kKSteps; ++j) q_reg[j] = qb_lds[j * 64 + lane];
+    }
+
+    const uint32_t log2p = 31 - __builtin_clz(a.walk.tokens_per_page);
+    const uint32_t page_mask = a.walk.tokens_per_page - 1;
+    const uint32_t* table_row = page_ids + ((uint64_t)req_slot * a.walk.num_layers + a.layer) *
+                                                      a.walk.num_blocks * a.walk.ids_per_block;
+    const uint64_t v_region = (uint64_t)a.walk.hkv * a.walk.tokens_per_page * D;
+    const uint32_t tile_begin = kv_begin / kTileTokens;
+    const uint32_t tile_end = (kv_end + kTileTokens - 1) / kTileTokens;
+
+    float run_max[NB], lane_sum[NB];
+    f32x4_t o[NB][kDimBlocks];
+#pragma unroll
+    for (int nb = 0; nb < NB; ++nb) {
+        run_max[nb] = -INFINITY;
+        lane_sum[nb] = 0.0f;
+#pragma unroll
+        for (int db = 0; db < kDimBlocks; ++db) o[nb][db] = f32x4_t{0.0f, 0.0f, 0.0f, 0.0f};
+    }
+
+    // The accumulators live in the accumulation registers across the tile loop: the matrix cores add into them in
+    // place, and only the rare rescaling moves them through the vector registers.
+    auto anchor_accumulators = [&]() __attribute__((always_inline)) {
+#pragma unroll
+        for (int nb = 0; nb < NB; ++nb)
+#pragma unroll
+            for (int db = 0; db < kDimBlocks; ++db) asm volatile("" : "+a"(o[nb][db]));
+    };
+
+    const uint32_t last_page = (kv_end - 1) >> log2p;
+    auto load_page_id = [&](uint32_t tile) -> TilePages {
+        TilePages p{0u, 0u};
+        if (tile < tile_end) {
+            const uint32_t first = (tile * kTileTokens) >> log2p;
+            p.a = table_row[first];
+            if (kHalfPage) p.b = table_row[min(first + 1, last_page)];
+        }
+        return p;
+    };
+    // This lane's share of a load: chunk `lane / 8` of row `lane % 8` of the half tile.
+    const uint32_t lane_elem = (lane & 7) * D + (lane >> 3) * 8;
+    auto half_rows = [&](uint32_t tile, TilePages p, int half) -> const uint16_t* {
+        if (kHalfPage)
+            return pages + (uint64_t)(half ? p.b : p.a) * a.walk.page_elems +
+                   (uint64_t)kv_head * a.walk.tokens_per_page * D + lane_elem;
+        return pages + (uint64_t)p.a * a.walk.page_elems + (uint64_t)kv_head * a.walk.tokens_per_page * D +
+               (((tile * kTileTokens) & page_mask) + half * 8) * D + lane_elem;
+    };
+    auto issue_k = [&](uint32_t tile, TilePages p, uint32_t stage) {
+        dma_tile<kDQ, kHalfBytes>(my_stages_lds + stage * kTileBytes, half_rows(tile, p, 0), half_rows(tile, p, 1));
+    };
+    auto issue_v = [&](uint32_t tile, TilePages p, uint32_t stage) {
+        dma_tile<kDQ, kHalfBytes>(my_stages_lds + (2 + stage) * kTileBytes, half_rows(tile, p, 0) + v_region,
+                                  half_rows(tile, p, 1) + v_region);
+    };
+
+    // A operand of QK^T, k-step i: row mt, elements 32 * i + 8 * mc .. + 7 -> half mt / 8, line i / 2, chunk
+    // 4 * (i % 2) + mc, row mt % 8: the k-steps lie 512 bytes apart.
+    const uint32_t k_read = (mt >> 3) * kHalfBytes + mc * 128 + (mt & 7) * 16;
+    // B operand of PV, dim block db (tokens 4 * mc .. + 3 of dim 16 * db + mt) through the transposing read: the lane
+    // hands in token 4 * mc + mt / 4, dims 16 * db + 4 * (mt % 4) .. + 3 -> half mc / 2, row 4 * (mc % 2) + mt / 4,
+    // line db / 4, chunk 2 * (db % 4) + (mt % 4) / 2, its upper or lower 8 bytes: the dim blocks lie 256 bytes apart.
+    const uint32_t v_read =
+        (mc >> 1) * kHalfBytes + (((mt & 3) >> 1) * 8 + (mc & 1) * 4 + (mt >> 2)) * 16 + (mt & 1) * 8;
+
+    const uint32_t first_tile = tile_begin + wave;
+    const uint32_t my_tiles = first_tile < tile_end && nb_active != 0 ? (tile_end - first_tile + kWaves - 1) / kWaves : 0u;
+    auto is_partial = [&](uint32_t t) { return t * kTileTokens < kv_begin || (t + 1) * kTileTokens > kv_end; };
+
+    TilePages pid_ahead{0u, 0u};  // of tile i + 2
+    if (my_tiles != 0) {
+        const TilePages p0 = load_page_id(first_tile);
+        issue_k(first_tile, p0, 0);
+        issue_v(first_tile, p0, 0);
+        if (my_tiles > 1) {
+            const TilePages p1 = load_page_id(first_tile + kWaves);
+            issue_k(first_tile + kWaves, p1, 1);
+            issue_v(first_tile + kWaves, p1, 1);
+        }
+        pid_ahead = load_page_id(first_tile + 2 * kWaves);
+    }
+    for (uint32_t i = 0; i < my_tiles; ++i) {
+        const uint32_t tile = first_tile + i * kWaves;
+        const uint32_t stage = i & 1;
+        anchor_accumulators();
+        const bool has1 = i + 1 < my_tiles, has2 = i + 2 < my_tiles;
+        const TilePages pid2 = pid_ahead;
+        pid_ahead = load_page_id(tile + 3 * kWaves);
+        const unsigned char* k_tile = my_stages + stage * kTileBytes;
+        unsigned char* v_tile = my_stages + (2 + stage) * kTileBytes;
+
+        // ---- logits S[token][column]: K(i) has landed once only V(i), K(i+1), V(i+1) are outstanding
+        wait_load_groups<kTileLoads>(has1 ? 3u : 1u);
+        f32x4_t s[NB];
+#pragma unroll
+        for (int nb = 0; nb < NB; ++nb) s[nb] = f32x4_t{0.0f, 0.0f, 0.0f, 0.0f};
+        // The loads of tile i + 2 go out line by line, each as soon as the products that read the line of tile i
+        // it replaces have been issued: a stage is then free again after a quarter of the phase, not all of it.
+        const uint16_t* next_rows0 = half_rows(tile + 2 * kWaves, pid2, 0);
+        const uint16_t* next_rows1 = half_rows(tile + 2 * kWaves, pid2, 1);
+        static_for<kDQ>([&](auto line_tag) __attribute__((always_inline)) {
+            constexpr int line = decltype(line_tag)::value;
+#pragma unroll
+            for (int ks = 2 * line; ks < 2 * line + 2; ++ks) {
+                const uint4 ka = *reinterpret_cast<const uint4*>(k_tile + k_read + ks * 512);
+#pragma unroll
+                for (int nb = 0; nb < NB; ++nb)
+                    s[nb] = mfma_16x16x32<Tag>(ka, kQInRegs ? q_reg[kQInRegs ? nb * kKSteps + ks : 0]
+                                                            : qb_lds[(nb * kKSteps + ks) * 64 + lane], s[nb]);
+            }
+            if (has2)
+                dma_tile_line<line, kHalfBytes>(my_stages_lds + stage * kTileBytes, next_rows0, next_rows1, s[NB - 1]);
+        });
+
+        // ---- online softmax per column over this lane's tokens 4*mc + r (see split_kv_tiled_map).  Nearly every
+        // tile lies inside the range of every column and needs no mask.
+        ProbOperand<Tag> pa[NB];
+        float alpha[NB];
+        bool moved = false;
+        auto softmax = [&](auto masked_tag) __attribute__((always_inline)) {
+            constexpr bool masked = decltype(masked_tag)::value;
+#pragma unroll
+            for (int nb = 0; nb < NB; ++nb) {
+                float v[4];
+                bool valid[4];
+                float m = -INFINITY;
+#pragma unroll
+                for (int r = 0; r < 4; ++r) {
+                    const uint32_t token = tile * kTileTokens + mc * 4 + r;
+                    valid[r] = !masked || (token >= kv_begin && token < lim[nb]);
+                    v[r] = valid[r] ? s[nb][r] * a.scale_log2 : -INFINITY;
+                    m = fmaxf(m, v[r]);
+                }
+                m = quarter_wave_max(m);
+                const float next_max = m > run_max[nb] + kMaxSlack ? m : run_max[nb];
+                alpha[nb] = run_max[nb] > -INFINITY ? __builtin_amdgcn_exp2f(run_max[nb] - next_max) : 0.0f;
+                moved = moved || next_max != run_max[nb];
+                run_max[nb] = next_max;
+                float p[4], tile_sum = 0.0f;
+#pragma unroll
+                for (int r = 0; r < 4; ++r) {
+                    p[r] = valid[r] ? __builtin_amdgcn_exp2f(v[r] - next_max) : 0.0f;
+                    tile_sum += p[r];
+                }
+                lane_sum[nb] = lane_sum[nb] * alpha[nb] + tile_sum;
+                pa[nb].set(p);
+            }
+        };
+        if (tile * kTileTokens >= kv_begin && (tile + 1) * kTileTokens <= open_until) softmax(std::false_type());
+        else softmax(std::true_type());
+        const bool rescale = __any(moved);
+        if (rescale) {
+            // rare (a column's reference maximum moved): through the vector registers and back, inside the branch
+#pragma unroll
+            for (int nb = 0; nb < NB; ++nb) {
+                float al[4];
+#pragma unroll
+                for (int r = 0; r < 4; ++r) al[r] = __shfl(alpha[nb], mc * 4 + r, 64);
+#pragma unroll
+                for (int db = 0; db < kDimBlocks; ++db) {
+                    f32x4_t t = o[nb][db];
+                    asm volatile("" : "+v"(t));
+#pragma unroll
+                    for (int r = 0; r < 4; ++r) t[r] *= al[r];
+                    asm volatile("" : "+a"(t));
+                    o[nb][db] = t;
+                }
+            }
+        }
+        anchor_accumulators();
+
+        // ---- O[column][dim] += P^T V: V(i) has landed once only K(i+1), V(i+1), K(i+2) are outstanding
+        wait_load_groups<kTileLoads>((has1 ? 2u : 0u) + (has2 ? 1u : 0u));
+        if (is_partial(tile)) {
+            // rows outside the split have probability 0, but their bytes may be NaN or Inf: zero them in LDS
+            for (uint32_t idx = lane; idx < kTileTokens * kDQ * 8; idx += 64) {
+                const uint32_t slot = idx & 63, block = idx >> 6;  // block = half * kDQ + line
+                const uint32_t vtoken = tile * kTileTokens + (block / kDQ) * 8 + (slot & 7);
+                if (vtoken < kv_begin || vtoken >= kv_end)
+                    *reinterpret_cast<uint4*>(v_tile + idx * 16) = make_uint4(0, 0, 0, 0);
+            }
+            wave_lds_fence();
+        }
+        static_for<kDQ>([&](auto line_tag) __attribute__((always_inline)) {
+            constexpr int line = decltype(line_tag)::value;
+#pragma unroll
+            for (int db = 4 * line; db < 4 * line + 4; ++db) {
+                const uint2 b = lds_read_tr16_b64(v_tile + v_read + db * 256);
+#pragma unroll
+                for (int nb = 0; nb < NB; ++nb) {
+#pragma unroll
+                    for (int t = 0; t < ProbOperand<Tag>::kTerms; ++t)
+                        o[nb][db] = mfma_16x16x16<Tag>(pa[nb].term[t], b, o[nb][db]);
+                }
+            }
+            if (has2)
+                dma_tile_line<line, kHalfBytes>(my_stages_lds + (2 + stage) * kTileBytes, next_rows0 + v_region,
+                                                next_rows1 + v_region, o[NB - 1][4 * line + 3]);
+        });
+    }
+
+    // ---- merge the four wave states.  Column statistics live in the S layout (lane <-> column mt), the
+    // accumulators in the MFMA output layout (lane <-> columns 4*mc + r, dim mt).
+#pragma unroll
+    for (int nb = 0; nb < NB; ++nb) {
+        lane_sum[nb] += __shfl_xor(lane_sum[nb], 16, 64);
+        lane_sum[nb] += __shfl_xor(lane_sum[nb], 32, 64);
+        if (mc == 0) wave_max_lds[wave][nb * 16 + mt] = run_max[nb];
+    }
+    __syncthreads();  // every wave has left the main loop: the tile stages may now be reused
+#pragma unroll
+    for (int nb = 0; nb < NB; ++nb) {
+        const uint32_t c = nb * 16 + mt;
+        float gm = wave_max_lds[0][c];
+#pragma unroll
+        for (int w = 1; w < kWaves; ++w) gm = fmaxf(gm, wave_max_lds[w][c]);
+        const float f = run_max[nb] > -INFINITY ? __builtin_amdgcn_exp2f(run_max[nb] - gm) : 0.0f;
+        lane_sum[nb] *= f;
+        if (wave == 0 && mc == 0) col_max_lds[c] = gm;
+        float fr[4];
+#pragma unroll
+        for (int r = 0; r < 4; ++r) fr[r] = __shfl(f, mc * 4 + r, 64);
+#pragma unroll
+        for (int db = 0; db < kDimBlocks; ++db)
+#pragma unroll
+            for (int r = 0; r < 4; ++r) o[nb][db][r] *= fr[r];
+    }
+    for (uint32_t w = 0; w < (uint32_t)kWaves; ++w) {
+        if (wave == w) {
+#pragma unroll
+            for (int nb = 0; nb < NB; ++nb) {
+                if ((uint32_t)nb < nb_active) {
+                    if (mc == 0) {
+                        const uint32_t c = nb * 16 + mt;
+                        col_sum_lds[c] = (w == 0 ? 0.0f : col_sum_lds[c]) + lane_sum[nb];
+                    }
+#pragma unroll
+                    for (int db = 0; db < kDimBlocks; ++db)
+#pragma unroll
+                        for (int r = 0; r < 4; ++r) {
+                            float* dst = merge + (nb * 16 + mc * 4 + r) * kMergeStride + db * 16 + mt;
+                            *dst = (w == 0 ? 0.0f : *dst) + o[nb][db][r];
+                        }
+                }
+            }
+        }
+        __syncthreads();
+    }
+
+    // ---- emit: partial row of (split, q_head, token_in_tile); 1 KiB of contiguous f32 per wave store
+    const uint32_t rows = a.rows_per_split_head;
+    for (uint32_t idx = tid; idx < ncols * (D / 4); idx += 64 * kWaves) {
+        const uint32_t c = idx / (D / 4), d4 = idx % (D / 4);
+        const uint64_t row = ((uint64_t)split * a.hq + (uint64_t)kv_head * G + c % G) * rows + c / G;
+        const float4 val = *reinterpret_cast<const float4*>(merge + c * kMergeStride + d4 * 4);
+        *reinterpret_cast<float4*>(&a.part_acc[row * D + d4 * 4]) = val;
+    }
+    if (tid < ncols) {
+        const uint64_t row = ((uint64_t)split * a.hq + (uint64_t)kv_head * G + tid % G) * rows + tid / G;
+        a.part_max[row] = col_max_lds[tid];
+        a.part_sum[row] = col_sum_lds[tid];
+    }
+    }  // rows of this workgroup
+}
+
 // Column blocks needed for tiles of up to `max_tile_tokens` query tokens and `group` heads per KV head.
 inline int tiled_column_blocks(uint32_t max_tile_tokens, uint32_t group) { return (int)((max_tile_tokens * group + 15) / 16); }
 
@@ -503,11 +967,24 @@ inline int launch_tiled_map_typed(psi_hip_ctx* ctx, const Geometry& g, const Map
                                ctx->stream, a, a.walk.page_ids, a.kv_splits, a.req_slots, q, pages, a.q_token_tiles,   \
                                a.flat_token_indices, a.worker_cu);                                                     \
     } while (0)
-    if (nb == 1) PSI_TILED_LAUNCH(1, 1);
-    else if (nb == 2) PSI_TILED_LAUNCH(2, 1);
+#define PSI_TILED_STREAM_LAUNCH(NB)                                                                                    \
+    do {                                                                                                               \
+        if (g.tokens_per_page == 8)                                                                                    \
+            hipLaunchKernelGGL((split_kv_tiled_stream_map<Tag, D, NB, true>), grid, dim3(64 * kTiledTileWaves), 0,      \
+                               ctx->stream, a, a.walk.page_ids, a.kv_splits, a.req_slots, q, pages, a.q_token_tiles,   \
+                               a.flat_token_indices, a.worker_cu);                                                     \
+        else                                                                                                           \
+            hipLaunchKernelGGL((split_kv_tiled_stream_map<Tag, D, NB, false>), grid, dim3(64 * kTiledTileWaves), 0,     \
+                               ctx->stream, a, a.walk.page_ids, a.kv_splits, a.req_slots, q, pages, a.q_token_tiles,   \
+                               a.flat_token_indices, a.worker_cu);                                                     \
+    } while (0)
+    if (nb == 1) PSI_TILED_STREAM_LAUNCH(1);
+    else if (nb == 2) PSI_TILED_STREAM_LAUNCH(2);
+    else if (nb == 3) PSI_TILED_STREAM_LAUNCH(3);
     else if (nb <= 4) PSI_TILED_LAUNCH(2, 2);
     else return PSI_HIP_ERR_UNSUPPORTED;
 #undef PSI_TILED_LAUNCH
+#undef PSI_TILED_STREAM_LAUNCH
     return PSI_HIP_OK;
 }
 
