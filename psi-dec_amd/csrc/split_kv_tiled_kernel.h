@@ -3,28 +3,26 @@
 // crates/inference-backend-metal/src/components/metal/gqa_split_kv_tiled_q.metal:49-319.
 //
 // Work decomposition
-//   one workgroup (4 waves) = one (kv_split row, kv_head).  The row names a request-local tile of
-//   up to 8 query tokens; with the G query heads that share the KV head this gives up to 8*G
-//   query columns, column c = token_in_tile * G + head, handled as blocks of 16 columns.  Every
-//   K and V byte of the split is therefore fetched from HBM once for all of them.  One wave =
-//   every 4th 16-token KV tile for NB column blocks, with its own online-softmax state per column;
-//   wave states merge through LDS at the end.  Up to 32 columns fit one wave's registers (NB <= 2);
-//   wider tiles use a second group of four waves for columns 32..63 (CG = 2), which walks the same
-//   KV tiles a moment later and finds them in cache.
+//   one workgroup = one (kv_split row, kv_head), or a worker's range of rows in the balanced launch.  The row
+//   names a request-local tile of up to 8 query tokens; with the G query heads that share the KV head this gives
+//   up to 8*G query columns, column c = token_in_tile * G + head, handled as blocks of 16 columns.  Every K and V
+//   byte of the split is therefore fetched from HBM once for all of them.  Four streams of KV tiles per workgroup
+//   (stream p takes the 16-token tiles p, p + 4, ...), each with its own online-softmax state per column; the
+//   states merge through LDS at the end of the row.
+//   Up to 48 columns (three blocks): split_kv_tiled_paired_map, two waves per stream, KV tiles through LDS by
+//   global_load_lds.  49 to 64 columns: split_kv_tiled_map with two groups of four waves (CG = 2), one per 32
+//   columns, each wave with its tile in registers; the second group finds most tiles in cache.
 //
-// Per 16-token KV tile and wave
-//   QK^T  S[token][column] on v_mfma_f32_16x16x32: A = the K tile straight from the page (lane =
-//         token lane%16, 8 contiguous dims per 128-bit load), B = the query columns staged once
-//         per workgroup in LDS in operand order.
-//   softmax  the MFMA leaves each lane with 4 tokens of one column; causal / range masks per
-//         column; probabilities stay in registers: that register layout is exactly the A operand
-//         of v_mfma_f32_16x16x16 (row = column, k = 4 tokens).
-//   PV    O[column][dim] += P^T * V on v_mfma_f32_16x16x16.  The contraction runs over tokens, the
-//         strided axis of V, so the V tile goes through a per-wave LDS buffer: written with
-//         128-bit stores as loaded, read back as 4 tokens x 1 dim per lane.  bf16 probabilities
-//         are split into two bf16 terms (two MFMAs) so that P carries 16 mantissa bits; f16
+// Per 16-token KV tile
+//   QK^T  S[token][column] on v_mfma_f32_16x16x32: A = the K tile (lane = token lane%16, 8 contiguous dims), B =
+//         the query columns staged once per row in LDS in operand order (or kept in registers).
+//   softmax  the MFMA leaves each lane with 4 tokens of one column; causal / range masks per column;
+//         probabilities stay in registers: that register layout is exactly the A operand of
+//         v_mfma_f32_16x16x16 (row = column, k = 4 tokens).
+//   PV    O[column][dim] += P^T * V on v_mfma_f32_16x16x16.  The contraction runs over tokens, the strided axis
+//         of V, so the V tile is read out of LDS with the transposing read (4 tokens x 1 dim per lane).  bf16
+//         probabilities are split into two bf16 terms (two MFMAs) so that P carries 16 mantissa bits; f16
 //         carries 11 in one.
-//   K and V loads run one tile ahead, as in the decode kernel.
 //
 // Algorithmic bytes per (kv token, kv head): 2 * head_dim * 2, read once per (Q tile, split).
 #pragma once
@@ -484,15 +482,14 @@ __global__ __launch_bounds__(64 * kTiledTileWaves * CG, (TiledOccupancy<NB, CG>:
 }
 
 // ---------------------------------------------------------------------------------------------------------------
-// The streaming variant: up to three column blocks per wave, KV tiles brought into LDS by the load unit itself.
+// KV tiles through LDS without registers (tiles of up to 48 query columns; see split_kv_tiled_paired_map below).
 //
 // A 16-token tile of K (and of V) is 16 rows of D elements.  `global_load_lds_dwordx4` moves 16 bytes per lane from
-// a per-lane global address to LDS address M0 + instruction offset + 16 * lane, with no register in between, so a
-// wave keeps two tiles of K and two of V in flight or in use without holding any of them in registers: the loads of
-// tile i + 2 go out as soon as tile i has been multiplied.  One instruction covers 8 rows x 128 bytes (whole lines):
-// lane p = 8 * c + t fetches chunk c (8 elements) of row t, and lands at slot p of a 1 KiB block; a tile is
-// 2 * D / 64 such blocks, [row half][line of the row].  Read back, the A operand of K * Q^T (16 rows x 8 elements
-// per quarter wave) and the transposed V block of a quarter wave both gather whole 16-byte slots, conflict-free.
+// a per-lane global address to LDS address M0 + instruction offset + 16 * lane, with no register in between.  One
+// instruction covers 8 rows x 128 bytes (whole lines): lane p = 8 * c + t fetches chunk c (8 elements) of row t, and
+// lands at slot p of a 1 KiB block; a tile is 2 * D / 64 such blocks, [row half][line of the row].  Read back, the A
+// operand of K * Q^T (16 rows x 8 elements per quarter wave) and the transposed V block of a quarter wave both
+// gather whole 16-byte slots, conflict-free.
 //
 // The loads are inline assembly, and so are the waits for them: the compiler does not know that they write LDS, and
 // where it does (the builtin) it waits for every outstanding one before any LDS read, which would undo the prefetch.
@@ -510,20 +507,7 @@ __device__ __forceinline__ float quarter_wave_max(float x) {
 
 // Line `kLine` (64 elements) of the 8 + 8 rows of a tile: two loads of 1 KiB, one per half tile.  The instruction
 // offset is added to the global and to the LDS address alike, hence 1024 - 128 between the M0 values of consecutive
-// lines.  `tie` is an accumulator that the matrix cores have just written from the last LDS operand read out of the
-// bytes these loads replace: LDS reads return in order, so once that product could be issued the stage's old
-// contents have been read, and naming it here keeps the loads behind that product.
-template <int kLine, int kHalfBytes>
-__device__ __forceinline__ void dma_tile_line(uint32_t lds_tile, const void* rows0, const void* rows1, f32x4_t& tie) {
-    asm volatile(
-        "s_add_u32 m0, %1, %4\n\ts_nop 0\n\t"
-        "global_load_lds_dwordx4 %2, off offset:%6 nt\n\t"
-        "s_add_u32 m0, %1, %5\n\ts_nop 0\n\t"
-        "global_load_lds_dwordx4 %3, off offset:%6 nt"
-        : "+a"(tie)
-        : "s"(lds_tile), "v"(rows0), "v"(rows1), "n"(kLine * 896), "n"(kHalfBytes + kLine * 896), "n"(kLine * 128)
-        : "memory", "m0", "scc");
-}
+// lines.
 template <int kLine, int kHalfBytes>
 __device__ __forceinline__ void dma_tile_line(uint32_t lds_tile, const void* rows0, const void* rows1) {
     asm volatile(
@@ -545,17 +529,6 @@ __device__ __forceinline__ void dma_tile(uint32_t lds_tile, const void* rows0, c
     }
 }
 
-#ifndef PSI_Q_REGS_NB
-#define PSI_Q_REGS_NB 2
-#endif
-template <int N, typename F, int I = 0>
-__device__ __forceinline__ void static_for(F&& f) {
-    if constexpr (I < N) {
-        f(std::integral_constant<int, I>());
-        static_for<N, F, I + 1>(static_cast<F&&>(f));
-    }
-}
-
 // Waits until at most `kLoads * groups` of the wave's loads are outstanding (they complete in order).
 template <int kLoads>
 __device__ __forceinline__ void wait_load_groups(uint32_t groups) {
@@ -565,61 +538,147 @@ __device__ __forceinline__ void wait_load_groups(uint32_t groups) {
     else asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
 }
 
-constexpr int tiled_stream_lds_bytes(int D, int NB) {
-    return kTiledTileWaves * 4 * (kTileTokens * D * 2) + NB * (D / 32) * 64 * 16;
-}
-
+// ---------------------------------------------------------------------------------------------------------------
+// The multi-query map for tiles of up to 48 query columns: two waves per SIMD on each stream of KV tiles.
+//
+// A wave stands at a load until the memory pipeline takes it, and at a product until the matrix cores take it: one
+// wave alone does the one or the other, and its time per tile is the sum (by the cycle counter, the K * Q^T phase of
+// one column block took 1800 cycles with the tile's eight K loads in it and 200 without).  Here eight waves form
+// four pairs; the waves p and p + 4 of a pair
+// (on one SIMD) walk the tiles p, p + 4, ... of the row together through one set of LDS stages.  The second wave of
+// the pair issues every load, announces each tile of K and of V in LDS as it lands and takes the smaller share of
+// the query columns (none of one block, one of two or three); the first wave takes the larger share and says in LDS
+// when it has read a stage, so that the second may refill it.  While one of them stands at a load the other
+// multiplies.  All of it is bounded: a wait on the other wave's progress gives up after 2^16 polls (the row's
+// results are then wrong, which the parity tests see, but no wave stays behind).
+// ---------------------------------------------------------------------------------------------------------------
 template <typename Tag, int D, int NB, bool kHalfPage>
-__global__ __launch_bounds__(64 * kTiledTileWaves, 1) void split_kv_tiled_stream_map(
+__global__ __launch_bounds__(128 * kTiledTileWaves, 1) void split_kv_tiled_paired_map(
     MapArgs a, const uint32_t* __restrict__ page_ids, const uint32_t* __restrict__ kv_splits,
     const uint32_t* __restrict__ req_slots, const uint16_t* __restrict__ q, const uint16_t* __restrict__ pages,
     const uint32_t* __restrict__ q_token_tiles, const uint32_t* __restrict__ flat_token_indices,
     const uint32_t* __restrict__ worker_cu) {
     resolve_active(a);
-    constexpr int kWaves = kTiledTileWaves;
+    constexpr int kPairs = kTiledTileWaves;
+    constexpr int kWaves = 2 * kPairs;
     constexpr int kKSteps = D / 32;             // MFMA k-steps of QK^T
     constexpr int kDimBlocks = D / 16;          // 16-dim output blocks of PV
     constexpr int kDQ = D / 64;                 // 128-byte lines per row
     constexpr int kTileLoads = 2 * kDQ;         // load instructions per tile of K (or of V)
     constexpr int kTileBytes = kTileTokens * D * 2;
     constexpr int kHalfBytes = kTileBytes / 2;
-    constexpr int kWaveBytes = 4 * kTileBytes;  // K stage 0, K stage 1, V stage 0, V stage 1
+    constexpr int kPairBytes = 4 * kTileBytes;  // K stage 0, K stage 1, V stage 0, V stage 1
     constexpr int kCols = NB * 16;
     constexpr int kMergeStride = D + 4;         // floats per column row of the merge buffer
-    constexpr int kStageBytes = kWaves * kWaveBytes;
+    constexpr int kStageBytes = kPairs * kPairBytes;
     constexpr int kQBytes = NB * kKSteps * 64 * 16;
+    constexpr int kBlocksSecond = NB > 2 ? NB - 2 : 0;  // column blocks of the loading wave
+    constexpr int kBlocksFirst = NB - kBlocksSecond;
     static_assert(kCols * kMergeStride * 4 <= kStageBytes, "the merge buffer reuses the tile stages");
 
     __shared__ __attribute__((aligned(1024))) unsigned char lds_union[kStageBytes + kQBytes];
-    __shared__ float wave_max_lds[kWaves][kCols];
+    __shared__ float wave_max_lds[kPairs][kCols];
     __shared__ float col_max_lds[kCols];
     __shared__ float col_sum_lds[kCols];
+    // tiles of the row so far, per pair: [K landed, V landed, K read by the first wave, V read by the first wave]
+    __shared__ uint32_t progress[4][kPairs];
     uint4* qb_lds = reinterpret_cast<uint4*>(lds_union + kStageBytes);  // [NB][kKSteps][64]
     float* merge = reinterpret_cast<float*>(lds_union);
 
     const uint32_t G = a.group;
     const uint32_t kv_head = blockIdx.x % a.walk.hkv;
     const uint32_t wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
-    unsigned char* my_stages = lds_union + wave * kWaveBytes;
+    const uint32_t pair = wave % kPairs;
+    const bool second = wave >= (uint32_t)kPairs;
+    unsigned char* my_stages = lds_union + pair * kPairBytes;
     const uint32_t my_stages_lds =
-        (uint32_t)(size_t)(__attribute__((address_space(3))) unsigned char*)(lds_union) + wave * kWaveBytes;
+        (uint32_t)(size_t)(__attribute__((address_space(3))) unsigned char*)(lds_union) + pair * kPairBytes;
+    volatile uint32_t* landed_k = &progress[0][pair];
+    volatile uint32_t* landed_v = &progress[1][pair];
+    volatile uint32_t* read_k = &progress[2][pair];
+    volatile uint32_t* read_v = &progress[3][pair];
+    auto wait_until_above = [&](volatile uint32_t* counter, uint32_t value) __attribute__((always_inline)) {
+        for (uint32_t polls = 0; *counter <= value && polls < (1u << 16); ++polls) __builtin_amdgcn_s_sleep(1);
+        asm volatile("" ::: "memory");
+    };
 
     uint32_t row_begin = blockIdx.x / a.walk.hkv, row_end = row_begin + 1;
     if (worker_cu != nullptr) {
         row_begin = worker_cu[blockIdx.x / a.walk.hkv];
         row_end = worker_cu[blockIdx.x / a.walk.hkv + 1];
     }
+    const uint32_t log2p = 31 - __builtin_clz(a.walk.tokens_per_page);
+    const uint32_t page_mask = a.walk.tokens_per_page - 1;
+    const uint64_t v_region = (uint64_t)a.walk.hkv * a.walk.tokens_per_page * D;
+    const uint32_t lane_id = threadIdx.x & 63;
+
+    // What a wave must know of a row before it can start on it: a chain of four dependent reads (the row of the
+    // split table, its query tile, the tile's request slot and token positions, the first page ids).
+    struct RowStart {
+        uint32_t step;                                 // links done
+        uint32_t valid, kv_begin, kv_end, flat_begin, ncols, req_slot;
+        uint32_t q_tile;
+        uint32_t position[NB];                         // per lane: position of the query token of column 16 * nb + lane % 16
+        TilePages page[3];                             // of this pair's first three tiles
+    };
+    auto page_of_tile = [&](const uint32_t* table_row, uint32_t tile, uint32_t kv_end_) -> TilePages {
+        TilePages pg{0u, 0u};
+        if (tile * kTileTokens < kv_end_) {
+            const uint32_t first = (tile * kTileTokens) >> log2p;
+            pg.a = table_row[first];
+            if (kHalfPage) pg.b = table_row[min(first + 1, (kv_end_ - 1) >> log2p)];
+        }
+        return pg;
+    };
+    auto table_row_of = [&](uint32_t req_slot_) {
+        return page_ids + ((uint64_t)req_slot_ * a.walk.num_layers + a.layer) * a.walk.num_blocks * a.walk.ids_per_block;
+    };
+    // One link of the chain for row `row`.
+    auto advance = [&](RowStart& r, uint32_t row) __attribute__((always_inline)) {
+        if (r.step == 0) {
+            r.valid = row < row_end && row < a.num_active_kv_splits;
+            if (r.valid) {
+                r.q_tile = kv_splits[row * 3];
+                r.kv_begin = kv_splits[row * 3 + 1];
+                r.kv_end = kv_splits[row * 3 + 2];
+                r.valid = r.q_tile < a.num_active_q_token_tiles;
+            }
+        } else if (r.step == 1) {
+            if (r.valid) {
+                uint32_t fb = q_token_tiles[r.q_tile * 2], fe = q_token_tiles[r.q_tile * 2 + 1];
+                r.valid = !(fb >= a.num_active_tokens || fe > a.num_active_tokens || fe <= fb);
+                r.flat_begin = fb;
+                r.ncols = r.valid ? (fe - fb) * G : 0u;
+            }
+        } else if (r.step == 2) {
+            if (r.valid) {
+                r.req_slot = req_slots[r.flat_begin];
+#pragma unroll
+                for (int nb = 0; nb < NB; ++nb) {
+                    const uint32_t c = nb * 16 + (lane_id & 15);
+                    r.position[nb] = c < r.ncols ? flat_token_indices[r.flat_begin + c / G] : 0xffffffffu;
+                }
+            }
+        } else if (r.step == 3) {
+            if (r.valid && r.ncols <= (uint32_t)kCols) {
+                const uint32_t* table_row = table_row_of(r.req_slot);
+                const uint32_t first = r.kv_begin / kTileTokens + pair;
+#pragma unroll
+                for (int j = 0; j < 3; ++j) {
+                    r.page[j] = page_of_tile(table_row, first + j * kPairs, r.kv_end);
+                }
+            }
+        }
+        ++r.step;
+    };
     bool lds_in_use = false;
     for (uint32_t split = row_begin; split < row_end; ++split) {
     if (split >= a.num_active_kv_splits) break;
-    const uint32_t q_tile = kv_splits[split * 3];
-    if (q_tile >= a.num_active_q_token_tiles) continue;  // sentinel padding
-    const uint32_t kv_begin = kv_splits[split * 3 + 1];
-    const uint32_t kv_end = kv_splits[split * 3 + 2];
-    const uint32_t flat_begin = q_token_tiles[q_tile * 2], flat_end = q_token_tiles[q_tile * 2 + 1];
-    if (flat_begin >= a.num_active_tokens || flat_end > a.num_active_tokens || flat_end <= flat_begin) continue;
-    const uint32_t tile_tokens = flat_end - flat_begin;
-    const uint32_t ncols = tile_tokens * G;
+    RowStart cur;
+    cur.step = 0;
+    while (cur.step < 4) advance(cur, split);
+    if (!cur.valid) continue;  // sentinel padding or a tile outside the active ones
+    const uint32_t kv_begin = cur.kv_begin, kv_end = cur.kv_end, flat_begin = cur.flat_begin, ncols = cur.ncols;
     if (ncols > (uint32_t)kCols) {
         // A tile wider than the launch was sized for: entered as an empty state (see split_kv_tiled_map).
         const uint32_t rows = a.rows_per_split_head;
@@ -640,87 +699,20 @@ __global__ __launch_bounds__(64 * kTiledTileWaves, 1) void split_kv_tiled_stream
     asm volatile("" : "+v"(tid));  // lane coordinates re-derived per row (see split_kv_tiled_map)
     const uint32_t lane = tid & 63;
     const uint32_t mt = lane & 15, mc = lane >> 4;
-    const uint32_t nb_total = (ncols + 15) / 16;
-    const uint32_t nb_active = min(nb_total, (uint32_t)NB);
-    const uint32_t req_slot = req_slots[flat_begin];
-
-    uint32_t lim[NB];  // keys [kv_begin, lim) are visible to the column (0: column unused)
-#pragma unroll
-    for (int nb = 0; nb < NB; ++nb) {
-        const uint32_t c = nb * 16 + mt;
-        lim[nb] = 0;
-        if (c < ncols) lim[nb] = min(kv_end, flat_token_indices[flat_begin + c / G] + 1);
-    }
 
     // Keys below `open_until` are visible to every column in use (the unused ones are never stored).
     uint32_t open_until = kv_end;
 #pragma unroll
     for (int nb = 0; nb < NB; ++nb)
-        if (lim[nb] != 0) open_until = min(open_until, lim[nb]);
+        if (cur.position[nb] != 0xffffffffu) open_until = min(open_until, cur.position[nb] + 1);
 #pragma unroll
     for (int sh = 1; sh < 64; sh <<= 1) open_until = min(open_until, (uint32_t)__shfl_xor((int)open_until, sh, 64));
     open_until = __builtin_amdgcn_readfirstlane(open_until);
 
-    // Query columns as MFMA B operands [nb][k-step][lane]; unused columns are zero.
-    for (uint32_t nb = wave; nb < (uint32_t)NB; nb += kWaves) {
-        const uint32_t c = nb * 16 + mt;
-        const bool used = c < ncols;
-        const uint32_t cc = used ? c : 0;
-        const uint16_t* q_row =
-            q + ((uint64_t)(flat_begin + cc / G) * a.hq + (uint64_t)kv_head * G + cc % G) * D + mc * 8;
-#pragma unroll
-        for (int i = 0; i < kKSteps; ++i) {
-            const uint4 v = *reinterpret_cast<const uint4*>(q_row + i * 32);
-            qb_lds[(nb * kKSteps + i) * 64 + lane] = used ? v : make_uint4(0, 0, 0, 0);
-        }
-    }
-    __syncthreads();
-
-    // Up to two column blocks keep their query operands in registers for the whole row.
-    constexpr bool kQInRegs = NB <= PSI_Q_REGS_NB;
-    uint4 q_reg[kQInRegs ? NB * kKSteps : 1];
-    if (kQInRegs) {
-#pragma unroll
-        for (int j = 0; j < NB * kKSteps; ++j) q_reg[j] = qb_lds[j * 64 + lane];
-    }
-
-    const uint32_t log2p = 31 - __builtin_clz(a.walk.tokens_per_page);
-    const uint32_t page_mask = a.walk.tokens_per_page - 1;
-    const uint32_t* table_row = page_ids + ((uint64_t)req_slot * a.walk.num_layers + a.layer) *
-                                                      a.walk.num_blocks * a.walk.ids_per_block;
-    const uint64_t v_region = (uint64_t)a.walk.hkv * a.walk.tokens_per_page * D;
+    const uint32_t* table_row = table_row_of(cur.req_slot);
     const uint32_t tile_begin = kv_begin / kTileTokens;
     const uint32_t tile_end = (kv_end + kTileTokens - 1) / kTileTokens;
-
-    float run_max[NB], lane_sum[NB];
-    f32x4_t o[NB][kDimBlocks];
-#pragma unroll
-    for (int nb = 0; nb < NB; ++nb) {
-        run_max[nb] = -INFINITY;
-        lane_sum[nb] = 0.0f;
-#pragma unroll
-        for (int db = 0; db < kDimBlocks; ++db) o[nb][db] = f32x4_t{0.0f, 0.0f, 0.0f, 0.0f};
-    }
-
-    // The accumulators live in the accumulation registers across the tile loop: the matrix cores add into them in
-    // place, and only the rare rescaling moves them through the vector registers.
-    auto anchor_accumulators = [&]() __attribute__((always_inline)) {
-#pragma unroll
-        for (int nb = 0; nb < NB; ++nb)
-#pragma unroll
-            for (int db = 0; db < kDimBlocks; ++db) asm volatile("" : "+a"(o[nb][db]));
-    };
-
-    const uint32_t last_page = (kv_end - 1) >> log2p;
-    auto load_page_id = [&](uint32_t tile) -> TilePages {
-        TilePages p{0u, 0u};
-        if (tile < tile_end) {
-            const uint32_t first = (tile * kTileTokens) >> log2p;
-            p.a = table_row[first];
-            if (kHalfPage) p.b = table_row[min(first + 1, last_page)];
-        }
-        return p;
-    };
+    auto load_page_id = [&](uint32_t tile) -> TilePages { return page_of_tile(table_row, tile, kv_end); };
     // This lane's share of a load: chunk `lane / 8` of row `lane % 8` of the half tile.
     const uint32_t lane_elem = (lane & 7) * D + (lane >> 3) * 8;
     auto half_rows = [&](uint32_t tile, TilePages p, int half) -> const uint16_t* {
@@ -737,199 +729,258 @@ __global__ __launch_bounds__(64 * kTiledTileWaves, 1) void split_kv_tiled_stream
         dma_tile<kDQ, kHalfBytes>(my_stages_lds + (2 + stage) * kTileBytes, half_rows(tile, p, 0) + v_region,
                                   half_rows(tile, p, 1) + v_region);
     };
+    const uint32_t first_tile = tile_begin + pair;
+    const uint32_t my_tiles = first_tile < tile_end ? (tile_end - first_tile + kPairs - 1) / kPairs : 0u;
+    // The row's first loads go out before anything else of it: the query columns are staged while they fly.
+    if (second && my_tiles != 0) {
+        issue_k(first_tile, cur.page[0], 0);
+        issue_v(first_tile, cur.page[0], 0);
+        if (my_tiles > 1) {
+            issue_k(first_tile + kPairs, cur.page[1], 1);
+            issue_v(first_tile + kPairs, cur.page[1], 1);
+        }
+    }
+
+    // Query columns as MFMA B operands [nb][k-step][lane]; unused columns are zero.
+    for (uint32_t nb = wave; nb < (uint32_t)NB; nb += kWaves) {
+        const uint32_t c = nb * 16 + mt;
+        const bool used = c < ncols;
+        const uint32_t cc = used ? c : 0;
+        const uint16_t* q_row =
+            q + ((uint64_t)(flat_begin + cc / G) * a.hq + (uint64_t)kv_head * G + cc % G) * D + mc * 8;
+#pragma unroll
+        for (int i = 0; i < kKSteps; ++i) {
+            const uint4 v = *reinterpret_cast<const uint4*>(q_row + i * 32);
+            qb_lds[(nb * kKSteps + i) * 64 + lane] = used ? v : make_uint4(0, 0, 0, 0);
+        }
+    }
+    if (tid < 4 * kPairs) (&progress[0][0])[tid] = 0;
+    __syncthreads();
 
     // A operand of QK^T, k-step i: row mt, elements 32 * i + 8 * mc .. + 7 -> half mt / 8, line i / 2, chunk
     // 4 * (i % 2) + mc, row mt % 8: the k-steps lie 512 bytes apart.
-    const uint32_t k_read = (mt >> 3) * kHalfBytes + mc * 128 + (mt & 7) * 16;
     // B operand of PV, dim block db (tokens 4 * mc .. + 3 of dim 16 * db + mt) through the transposing read: the lane
     // hands in token 4 * mc + mt / 4, dims 16 * db + 4 * (mt % 4) .. + 3 -> half mc / 2, row 4 * (mc % 2) + mt / 4,
     // line db / 4, chunk 2 * (db % 4) + (mt % 4) / 2, its upper or lower 8 bytes: the dim blocks lie 256 bytes apart.
+    const uint32_t k_read = (mt >> 3) * kHalfBytes + mc * 128 + (mt & 7) * 16;
     const uint32_t v_read =
         (mc >> 1) * kHalfBytes + (((mt & 3) >> 1) * 8 + (mc & 1) * 4 + (mt >> 2)) * 16 + (mt & 1) * 8;
-
-    const uint32_t first_tile = tile_begin + wave;
-    const uint32_t my_tiles = first_tile < tile_end && nb_active != 0 ? (tile_end - first_tile + kWaves - 1) / kWaves : 0u;
     auto is_partial = [&](uint32_t t) { return t * kTileTokens < kv_begin || (t + 1) * kTileTokens > kv_end; };
 
-    TilePages pid_ahead{0u, 0u};  // of tile i + 2
-    if (my_tiles != 0) {
-        const TilePages p0 = load_page_id(first_tile);
-        issue_k(first_tile, p0, 0);
-        issue_v(first_tile, p0, 0);
-        if (my_tiles > 1) {
-            const TilePages p1 = load_page_id(first_tile + kWaves);
-            issue_k(first_tile + kWaves, p1, 1);
-            issue_v(first_tile + kWaves, p1, 1);
+    // One wave's part of the row: the column blocks kBlock0 .. + kBlocks - 1, and the loads if it is the second
+    // wave of its pair.  Both instances pass the same workgroup barriers.
+    auto walk_row = [&](auto blocks_tag, auto block0_tag, auto loads_tag) __attribute__((always_inline)) {
+        constexpr int kBlocks = decltype(blocks_tag)::value;
+        constexpr int kBlock0 = decltype(block0_tag)::value;
+        constexpr bool kLoads = decltype(loads_tag)::value;
+        constexpr int kB = kBlocks > 0 ? kBlocks : 1;  // array extents
+
+        uint32_t lim[kB];  // keys [kv_begin, lim) are visible to the column (0: column unused)
+#pragma unroll
+        for (int nb = 0; nb < kBlocks; ++nb) {
+            const uint32_t position = cur.position[kBlock0 + nb];
+            lim[nb] = position != 0xffffffffu ? min(kv_end, position + 1) : 0u;
         }
-        pid_ahead = load_page_id(first_tile + 2 * kWaves);
-    }
-    for (uint32_t i = 0; i < my_tiles; ++i) {
-        const uint32_t tile = first_tile + i * kWaves;
-        const uint32_t stage = i & 1;
-        anchor_accumulators();
-        const bool has1 = i + 1 < my_tiles, has2 = i + 2 < my_tiles;
-        const TilePages pid2 = pid_ahead;
-        pid_ahead = load_page_id(tile + 3 * kWaves);
-        const unsigned char* k_tile = my_stages + stage * kTileBytes;
-        unsigned char* v_tile = my_stages + (2 + stage) * kTileBytes;
-
-        // ---- logits S[token][column]: K(i) has landed once only V(i), K(i+1), V(i+1) are outstanding
-        wait_load_groups<kTileLoads>(has1 ? 3u : 1u);
-        f32x4_t s[NB];
+        // One column block per wave keeps its query operands in registers for the whole row.
+        constexpr bool kQInRegs = kBlocks == 1;
+        uint4 q_reg[kQInRegs ? kKSteps : 1];
+        if (kQInRegs) {
 #pragma unroll
-        for (int nb = 0; nb < NB; ++nb) s[nb] = f32x4_t{0.0f, 0.0f, 0.0f, 0.0f};
-        // The loads of tile i + 2 go out line by line, each as soon as the products that read the line of tile i
-        // it replaces have been issued: a stage is then free again after a quarter of the phase, not all of it.
-        const uint16_t* next_rows0 = half_rows(tile + 2 * kWaves, pid2, 0);
-        const uint16_t* next_rows1 = half_rows(tile + 2 * kWaves, pid2, 1);
-        static_for<kDQ>([&](auto line_tag) __attribute__((always_inline)) {
-            constexpr int line = decltype(line_tag)::value;
-#pragma unroll
-            for (int ks = 2 * line; ks < 2 * line + 2; ++ks) {
-                const uint4 ka = *reinterpret_cast<const uint4*>(k_tile + k_read + ks * 512);
-#pragma unroll
-                for (int nb = 0; nb < NB; ++nb)
-                    s[nb] = mfma_16x16x32<Tag>(ka, kQInRegs ? q_reg[kQInRegs ? nb * kKSteps + ks : 0]
-                                                            : qb_lds[(nb * kKSteps + ks) * 64 + lane], s[nb]);
-            }
-            if (has2)
-                dma_tile_line<line, kHalfBytes>(my_stages_lds + stage * kTileBytes, next_rows0, next_rows1, s[NB - 1]);
-        });
-
-        // ---- online softmax per column over this lane's tokens 4*mc + r (see split_kv_tiled_map).  Nearly every
-        // tile lies inside the range of every column and needs no mask.
-        ProbOperand<Tag> pa[NB];
-        float alpha[NB];
-        bool moved = false;
-        auto softmax = [&](auto masked_tag) __attribute__((always_inline)) {
-            constexpr bool masked = decltype(masked_tag)::value;
-#pragma unroll
-            for (int nb = 0; nb < NB; ++nb) {
-                float v[4];
-                bool valid[4];
-                float m = -INFINITY;
-#pragma unroll
-                for (int r = 0; r < 4; ++r) {
-                    const uint32_t token = tile * kTileTokens + mc * 4 + r;
-                    valid[r] = !masked || (token >= kv_begin && token < lim[nb]);
-                    v[r] = valid[r] ? s[nb][r] * a.scale_log2 : -INFINITY;
-                    m = fmaxf(m, v[r]);
-                }
-                m = quarter_wave_max(m);
-                const float next_max = m > run_max[nb] + kMaxSlack ? m : run_max[nb];
-                alpha[nb] = run_max[nb] > -INFINITY ? __builtin_amdgcn_exp2f(run_max[nb] - next_max) : 0.0f;
-                moved = moved || next_max != run_max[nb];
-                run_max[nb] = next_max;
-                float p[4], tile_sum = 0.0f;
-#pragma unroll
-                for (int r = 0; r < 4; ++r) {
-                    p[r] = valid[r] ? __builtin_amdgcn_exp2f(v[r] - next_max) : 0.0f;
-                    tile_sum += p[r];
-                }
-                lane_sum[nb] = lane_sum[nb] * alpha[nb] + tile_sum;
-                pa[nb].set(p);
-            }
-        };
-        if (tile * kTileTokens >= kv_begin && (tile + 1) * kTileTokens <= open_until) softmax(std::false_type());
-        else softmax(std::true_type());
-        const bool rescale = __any(moved);
-        if (rescale) {
-            // rare (a column's reference maximum moved): through the vector registers and back, inside the branch
-#pragma unroll
-            for (int nb = 0; nb < NB; ++nb) {
-                float al[4];
-#pragma unroll
-                for (int r = 0; r < 4; ++r) al[r] = __shfl(alpha[nb], mc * 4 + r, 64);
-#pragma unroll
-                for (int db = 0; db < kDimBlocks; ++db) {
-                    f32x4_t t = o[nb][db];
-                    asm volatile("" : "+v"(t));
-#pragma unroll
-                    for (int r = 0; r < 4; ++r) t[r] *= al[r];
-                    asm volatile("" : "+a"(t));
-                    o[nb][db] = t;
-                }
-            }
+            for (int ks = 0; ks < kKSteps; ++ks) q_reg[ks] = qb_lds[(kBlock0 * kKSteps + ks) * 64 + lane];
         }
-        anchor_accumulators();
-
-        // ---- O[column][dim] += P^T V: V(i) has landed once only K(i+1), V(i+1), K(i+2) are outstanding
-        wait_load_groups<kTileLoads>((has1 ? 2u : 0u) + (has2 ? 1u : 0u));
-        if (is_partial(tile)) {
-            // rows outside the split have probability 0, but their bytes may be NaN or Inf: zero them in LDS
-            for (uint32_t idx = lane; idx < kTileTokens * kDQ * 8; idx += 64) {
-                const uint32_t slot = idx & 63, block = idx >> 6;  // block = half * kDQ + line
-                const uint32_t vtoken = tile * kTileTokens + (block / kDQ) * 8 + (slot & 7);
-                if (vtoken < kv_begin || vtoken >= kv_end)
-                    *reinterpret_cast<uint4*>(v_tile + idx * 16) = make_uint4(0, 0, 0, 0);
-            }
-            wave_lds_fence();
+        float run_max[kB], lane_sum[kB];
+        f32x4_t o[kB][kDimBlocks];
+#pragma unroll
+        for (int nb = 0; nb < kB; ++nb) {
+            run_max[nb] = -INFINITY;
+            lane_sum[nb] = 0.0f;
+#pragma unroll
+            for (int db = 0; db < kDimBlocks; ++db) o[nb][db] = f32x4_t{0.0f, 0.0f, 0.0f, 0.0f};
         }
-        static_for<kDQ>([&](auto line_tag) __attribute__((always_inline)) {
-            constexpr int line = decltype(line_tag)::value;
-#pragma unroll
-            for (int db = 4 * line; db < 4 * line + 4; ++db) {
-                const uint2 b = lds_read_tr16_b64(v_tile + v_read + db * 256);
-#pragma unroll
-                for (int nb = 0; nb < NB; ++nb) {
-#pragma unroll
-                    for (int t = 0; t < ProbOperand<Tag>::kTerms; ++t)
-                        o[nb][db] = mfma_16x16x16<Tag>(pa[nb].term[t], b, o[nb][db]);
-                }
-            }
-            if (has2)
-                dma_tile_line<line, kHalfBytes>(my_stages_lds + (2 + stage) * kTileBytes, next_rows0 + v_region,
-                                                next_rows1 + v_region, o[NB - 1][4 * line + 3]);
-        });
-    }
 
-    // ---- merge the four wave states.  Column statistics live in the S layout (lane <-> column mt), the
-    // accumulators in the MFMA output layout (lane <-> columns 4*mc + r, dim mt).
+        TilePages pid_ahead = cur.page[2];  // of tile i + 2
+        for (uint32_t i = 0; i < my_tiles; ++i) {
+            const uint32_t tile = first_tile + i * kPairs;
+            const uint32_t stage = i & 1;
+            const bool has1 = i + 1 < my_tiles, has2 = i + 2 < my_tiles;
+            const TilePages pid2 = pid_ahead;
+            if (kLoads) pid_ahead = load_page_id(tile + 3 * kPairs);
+            const unsigned char* k_tile = my_stages + stage * kTileBytes;
+            unsigned char* v_tile = my_stages + (2 + stage) * kTileBytes;
+
+            // ---- K(i) is there: the loading wave sees its own loads return (they complete in order: K(i) has
+            // landed once only V(i), K(i+1), V(i+1) are outstanding) and says so; the other wave reads that.
+            if (kLoads) {
+                wait_load_groups<kTileLoads>(has1 ? 3u : 1u);
+                *landed_k = i + 1;
+            } else {
+                wait_until_above(landed_k, i);
+            }
+            // ---- logits S[token][column]
+            f32x4_t s[kB];
+            if constexpr (kBlocks > 0) {
 #pragma unroll
-    for (int nb = 0; nb < NB; ++nb) {
-        lane_sum[nb] += __shfl_xor(lane_sum[nb], 16, 64);
-        lane_sum[nb] += __shfl_xor(lane_sum[nb], 32, 64);
-        if (mc == 0) wave_max_lds[wave][nb * 16 + mt] = run_max[nb];
-    }
-    __syncthreads();  // every wave has left the main loop: the tile stages may now be reused
+                for (int nb = 0; nb < kBlocks; ++nb) s[nb] = f32x4_t{0.0f, 0.0f, 0.0f, 0.0f};
 #pragma unroll
-    for (int nb = 0; nb < NB; ++nb) {
-        const uint32_t c = nb * 16 + mt;
-        float gm = wave_max_lds[0][c];
+                for (int ks = 0; ks < kKSteps; ++ks) {
+                    const uint4 ka = *reinterpret_cast<const uint4*>(k_tile + k_read + ks * 512);
 #pragma unroll
-        for (int w = 1; w < kWaves; ++w) gm = fmaxf(gm, wave_max_lds[w][c]);
-        const float f = run_max[nb] > -INFINITY ? __builtin_amdgcn_exp2f(run_max[nb] - gm) : 0.0f;
-        lane_sum[nb] *= f;
-        if (wave == 0 && mc == 0) col_max_lds[c] = gm;
-        float fr[4];
-#pragma unroll
-        for (int r = 0; r < 4; ++r) fr[r] = __shfl(f, mc * 4 + r, 64);
-#pragma unroll
-        for (int db = 0; db < kDimBlocks; ++db)
-#pragma unroll
-            for (int r = 0; r < 4; ++r) o[nb][db][r] *= fr[r];
-    }
-    for (uint32_t w = 0; w < (uint32_t)kWaves; ++w) {
-        if (wave == w) {
-#pragma unroll
-            for (int nb = 0; nb < NB; ++nb) {
-                if ((uint32_t)nb < nb_active) {
-                    if (mc == 0) {
-                        const uint32_t c = nb * 16 + mt;
-                        col_sum_lds[c] = (w == 0 ? 0.0f : col_sum_lds[c]) + lane_sum[nb];
+                    for (int nb = 0; nb < kBlocks; ++nb)
+                        s[nb] = mfma_16x16x32<Tag>(ka, kQInRegs ? q_reg[kQInRegs ? ks : 0]
+                                                                : qb_lds[((kBlock0 + nb) * kKSteps + ks) * 64 + lane],
+                                                   s[nb]);
+                }
+                wave_lds_fence();  // this wave has read the K stage
+            }
+            if (kLoads) {
+                if (has2) {
+                    wait_until_above(read_k, i);  // and so has the other
+                    issue_k(tile + 2 * kPairs, pid2, stage);
+                }
+                // V(i) has landed once only K(i+1), V(i+1), K(i+2) are outstanding.  Rows outside the split have
+                // probability 0, but their bytes may be NaN or Inf: they are zeroed before anyone multiplies.
+                wait_load_groups<kTileLoads>((has1 ? 2u : 0u) + (has2 ? 1u : 0u));
+                if (is_partial(tile)) {
+                    for (uint32_t idx = lane; idx < kTileTokens * kDQ * 8; idx += 64) {
+                        const uint32_t slot = idx & 63, block = idx >> 6;  // block = half * kDQ + line
+                        const uint32_t vtoken = tile * kTileTokens + (block / kDQ) * 8 + (slot & 7);
+                        if (vtoken < kv_begin || vtoken >= kv_end)
+                            *reinterpret_cast<uint4*>(v_tile + idx * 16) = make_uint4(0, 0, 0, 0);
                     }
+                    wave_lds_fence();
+                }
+                *landed_v = i + 1;
+            } else {
+                *read_k = i + 1;
+            }
+
+            if constexpr (kBlocks > 0) {
+                // ---- online softmax per column over this lane's tokens 4*mc + r (see split_kv_tiled_map); nearly
+                // every tile lies inside the range of every column and needs no mask
+                ProbOperand<Tag> pa[kB];
+                float alpha[kB];
+                bool moved = false;
+                auto softmax = [&](auto masked_tag) __attribute__((always_inline)) {
+                    constexpr bool masked = decltype(masked_tag)::value;
 #pragma unroll
-                    for (int db = 0; db < kDimBlocks; ++db)
+                    for (int nb = 0; nb < kBlocks; ++nb) {
+                        float v[4];
+                        bool valid[4];
+                        float m = -INFINITY;
 #pragma unroll
                         for (int r = 0; r < 4; ++r) {
-                            float* dst = merge + (nb * 16 + mc * 4 + r) * kMergeStride + db * 16 + mt;
-                            *dst = (w == 0 ? 0.0f : *dst) + o[nb][db][r];
+                            const uint32_t token = tile * kTileTokens + mc * 4 + r;
+                            valid[r] = !masked || (token >= kv_begin && token < lim[nb]);
+                            v[r] = valid[r] ? s[nb][r] * a.scale_log2 : -INFINITY;
+                            m = fmaxf(m, v[r]);
                         }
+                        m = quarter_wave_max(m);
+                        const float next_max = m > run_max[nb] + kMaxSlack ? m : run_max[nb];
+                        alpha[nb] = run_max[nb] > -INFINITY ? __builtin_amdgcn_exp2f(run_max[nb] - next_max) : 0.0f;
+                        moved = moved || next_max != run_max[nb];
+                        run_max[nb] = next_max;
+                        float p[4], tile_sum = 0.0f;
+#pragma unroll
+                        for (int r = 0; r < 4; ++r) {
+                            p[r] = valid[r] ? __builtin_amdgcn_exp2f(v[r] - next_max) : 0.0f;
+                            tile_sum += p[r];
+                        }
+                        lane_sum[nb] = lane_sum[nb] * alpha[nb] + tile_sum;
+                        pa[nb].set(p);
+                    }
+                };
+                if (tile * kTileTokens >= kv_begin && (tile + 1) * kTileTokens <= open_until) softmax(std::false_type());
+                else softmax(std::true_type());
+                if (__any(moved)) {
+#pragma unroll
+                    for (int nb = 0; nb < kBlocks; ++nb) {
+                        float al[4];
+#pragma unroll
+                        for (int r = 0; r < 4; ++r) al[r] = __shfl(alpha[nb], mc * 4 + r, 64);
+#pragma unroll
+                        for (int db = 0; db < kDimBlocks; ++db)
+#pragma unroll
+                            for (int r = 0; r < 4; ++r) o[nb][db][r] *= al[r];
+                    }
                 }
+
+                // ---- O[column][dim] += P^T V
+                if (!kLoads) wait_until_above(landed_v, i);
+#pragma unroll
+                for (int db = 0; db < kDimBlocks; ++db) {
+                    const uint2 b = lds_read_tr16_b64(v_tile + v_read + db * 256);
+#pragma unroll
+                    for (int nb = 0; nb < kBlocks; ++nb) {
+#pragma unroll
+                        for (int t = 0; t < ProbOperand<Tag>::kTerms; ++t)
+                            o[nb][db] = mfma_16x16x16<Tag>(pa[nb].term[t], b, o[nb][db]);
+                    }
+                }
+                wave_lds_fence();  // this wave has read the V stage
+            } else if (!kLoads) {
+                wait_until_above(landed_v, i);
+            }
+            if (kLoads) {
+                if (has2) {
+                    wait_until_above(read_v, i);
+                    issue_v(tile + 2 * kPairs, pid2, stage);
+                }
+            } else {
+                *read_v = i + 1;
             }
         }
-        __syncthreads();
-    }
+
+        // ---- merge the states of the four waves that share these columns.  Column statistics live in the S layout
+        // (lane <-> column mt), the accumulators in the MFMA output layout (lane <-> columns 4*mc + r, dim mt).
+#pragma unroll
+        for (int nb = 0; nb < kBlocks; ++nb) {
+            lane_sum[nb] += __shfl_xor(lane_sum[nb], 16, 64);
+            lane_sum[nb] += __shfl_xor(lane_sum[nb], 32, 64);
+            if (mc == 0) wave_max_lds[pair][(kBlock0 + nb) * 16 + mt] = run_max[nb];
+        }
+        __syncthreads();  // every wave has left the tile loop: the stages may now be reused
+#pragma unroll
+        for (int nb = 0; nb < kBlocks; ++nb) {
+            const uint32_t c = (kBlock0 + nb) * 16 + mt;
+            float gm = wave_max_lds[0][c];
+#pragma unroll
+            for (int w = 1; w < kPairs; ++w) gm = fmaxf(gm, wave_max_lds[w][c]);
+            const float f = run_max[nb] > -INFINITY ? __builtin_amdgcn_exp2f(run_max[nb] - gm) : 0.0f;
+            lane_sum[nb] *= f;
+            if (pair == 0 && mc == 0) col_max_lds[c] = gm;
+            float fr[4];
+#pragma unroll
+            for (int r = 0; r < 4; ++r) fr[r] = __shfl(f, mc * 4 + r, 64);
+#pragma unroll
+            for (int db = 0; db < kDimBlocks; ++db)
+#pragma unroll
+                for (int r = 0; r < 4; ++r) o[nb][db][r] *= fr[r];
+        }
+        for (uint32_t w = 0; w < (uint32_t)kPairs; ++w) {
+            if (pair == w) {
+#pragma unroll
+                for (int nb = 0; nb < kBlocks; ++nb) {
+                    if ((uint32_t)(kBlock0 + nb) * 16 < ncols) {
+                        if (mc == 0) {
+                            const uint32_t c = (kBlock0 + nb) * 16 + mt;
+                            col_sum_lds[c] = (w == 0 ? 0.0f : col_sum_lds[c]) + lane_sum[nb];
+                        }
+#pragma unroll
+                        for (int db = 0; db < kDimBlocks; ++db)
+#pragma unroll
+                            for (int r = 0; r < 4; ++r) {
+                                float* dst =
+                                    merge + ((kBlock0 + nb) * 16 + mc * 4 + r) * kMergeStride + db * 16 + mt;
+                                *dst = (w == 0 ? 0.0f : *dst) + o[nb][db][r];
+                            }
+                    }
+                }
+            }
+            __syncthreads();
+        }
+    };
+    if (second) walk_row(std::integral_constant<int, kBlocksSecond>(), std::integral_constant<int, kBlocksFirst>(), std::true_type());
+    else walk_row(std::integral_constant<int, kBlocksFirst>(), std::integral_constant<int, 0>(), std::false_type());
 
     // ---- emit: partial row of (split, q_head, token_in_tile); 1 KiB of contiguous f32 per wave store
     const uint32_t rows = a.rows_per_split_head;
@@ -967,24 +1018,24 @@ inline int launch_tiled_map_typed(psi_hip_ctx* ctx, const Geometry& g, const Map
                                ctx->stream, a, a.walk.page_ids, a.kv_splits, a.req_slots, q, pages, a.q_token_tiles,   \
                                a.flat_token_indices, a.worker_cu);                                                     \
     } while (0)
-#define PSI_TILED_STREAM_LAUNCH(NB)                                                                                    \
+#define PSI_TILED_PAIRED_LAUNCH(NB)                                                                                    \
     do {                                                                                                               \
         if (g.tokens_per_page == 8)                                                                                    \
-            hipLaunchKernelGGL((split_kv_tiled_stream_map<Tag, D, NB, true>), grid, dim3(64 * kTiledTileWaves), 0,      \
+            hipLaunchKernelGGL((split_kv_tiled_paired_map<Tag, D, NB, true>), grid, dim3(128 * kTiledTileWaves), 0,      \
                                ctx->stream, a, a.walk.page_ids, a.kv_splits, a.req_slots, q, pages, a.q_token_tiles,   \
                                a.flat_token_indices, a.worker_cu);                                                     \
         else                                                                                                           \
-            hipLaunchKernelGGL((split_kv_tiled_stream_map<Tag, D, NB, false>), grid, dim3(64 * kTiledTileWaves), 0,     \
+            hipLaunchKernelGGL((split_kv_tiled_paired_map<Tag, D, NB, false>), grid, dim3(128 * kTiledTileWaves), 0,     \
                                ctx->stream, a, a.walk.page_ids, a.kv_splits, a.req_slots, q, pages, a.q_token_tiles,   \
                                a.flat_token_indices, a.worker_cu);                                                     \
     } while (0)
-    if (nb == 1) PSI_TILED_STREAM_LAUNCH(1);
-    else if (nb == 2) PSI_TILED_STREAM_LAUNCH(2);
-    else if (nb == 3) PSI_TILED_STREAM_LAUNCH(3);
+    if (nb == 1) PSI_TILED_PAIRED_LAUNCH(1);
+    else if (nb == 2) PSI_TILED_PAIRED_LAUNCH(2);
+    else if (nb == 3) PSI_TILED_PAIRED_LAUNCH(3);
     else if (nb <= 4) PSI_TILED_LAUNCH(2, 2);
     else return PSI_HIP_ERR_UNSUPPORTED;
 #undef PSI_TILED_LAUNCH
-#undef PSI_TILED_STREAM_LAUNCH
+#undef PSI_TILED_PAIRED_LAUNCH
     return PSI_HIP_OK;
 }
 
