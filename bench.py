@@ -34,7 +34,7 @@ sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBPS = 8000.0
 MFMA_BF16_PEAK_TFLOPS = 2500.0
-CONFIG_NAMES = ["C1", "C3", "C4_q2", "C4_q4", "C5_decode", "C5_prefill", "C5_mixed"]
+CONFIG_NAMES = ["C1", "C3", "C4_q2", "C4_q4", "C4_q8", "C5_decode", "C5_prefill", "C5_mixed"]
 
 
 def parse_args():
@@ -161,8 +161,8 @@ def build_case(psi, wl, device, name, args):
     if name == "C3":
         key = "decode_b4_ctx131072_16q2kv_d256_bf16_p16_part512_outliers1e-4_seed33"
         return decode_case(key, [131072] * 4, 16, 2, bf16, 512, args.arenas or 1, 33, outlier_rate=1e-4, outlier_sigma=8.0)
-    if name in ("C4_q2", "C4_q4"):
-        q_len = 2 if name == "C4_q2" else 4
+    if name in ("C4_q2", "C4_q4", "C4_q8"):
+        q_len = int(name[-1])  # one draft, three drafts, or the reference's full eight-token query tile
         ctx = wl.config_c2_context_lens(4, 64, 2048, 16384) + q_len
         return verify_case(f"verify_q{q_len}_b64_ctx2048-16384_24q4kv_d256_bf16_p16_part512_seed4", ctx, q_len, 512,
                            args.arenas or 1, 4)
