@@ -67,6 +67,9 @@ def parse_args():
     p.add_argument("--row-per-workgroup", action="store_true", help="one workgroup per partition row, no worker plan")
     p.add_argument("--graph", action="store_true",
                    help="submit every step through the per-bucket program cache (HIP graph replay) instead of launching")
+    p.add_argument("--graph-cache-counts", action="store_true",
+                   help="with --graph: the cache sets the active counts with a launch of its own ahead of each program "
+                        "(default: they travel with the metadata upload)")
     p.add_argument("--calibrate-copy", action="store_true",
                    help="run only the plain copy / read probes of known size (counter calibration, practical ceiling)")
     p.add_argument("--probe-mib", type=int, default=1024)
@@ -225,7 +228,9 @@ def time_case(psi, wl, device, case, args, with_spread=True):
         for i in range(first, first + n):
             a = arenas[i % len(arenas)]
             if graph_cache is not None:
-                graph_cache.submit(a.layer_input())
+                inp = a.layer_input()
+                inp.counts_uploaded = not args.graph_cache_counts
+                graph_cache.submit(inp)
             else:
                 a.step()
 

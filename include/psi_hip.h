@@ -521,6 +521,10 @@ typedef struct psi_hip_gqa_batch_metadata {
     uint32_t group_tiles;
     uint32_t num_row_groups;
     uint32_t max_active_q_tile_tokens;  /* TiledQ: bound on the tokens of any tile (0 = q_token_tile_size) */
+    /* null, or device u32[4] = {tokens, q-token tiles, KV splits, layer + 1 or 0} that the caller has already filled
+     * for this batch, e.g. as four more words of the copy that brings the arrays above to the device: the replay
+     * cache then reads its programs' counts there and a submit is the program's launch alone. */
+    const uint32_t* replay_counts;
 } psi_hip_gqa_batch_metadata;
 
 /* `GQACore` + `GQAMetalConfig` (backend.rs:114-146) as far as the attention needs them. */
@@ -647,8 +651,10 @@ int psi_hip_gqa_replay_cache_destroy(psi_hip_gqa_replay_cache* cache);
  * the three capacities of input->batch_metadata->shape, the layer index (when by value), and every buffer address
  * of the input (a program holds addresses).  The active counts of the shape go to the counts block, stream-ordered
  * ahead of the program; gqa_layer_parameter > 0 binds the page-table layer gqa_layer_parameter - 1 the same way
- * (`ReplayU32::Parameter`) instead of the input's gqa_layer_index.  *out_recorded (may be null): 1 if this call
- * recorded. */
+ * (`ReplayU32::Parameter`) instead of the input's gqa_layer_index.  When input->batch_metadata->replay_counts is
+ * set, the caller has placed the four words itself (the fourth as gqa_layer_parameter says): the program reads them
+ * there, nothing is launched ahead of it, and the address is part of the key.  *out_recorded (may be null): 1 if
+ * this call recorded. */
 int psi_hip_gqa_replay_cache_submit(psi_hip_gqa_replay_cache* cache, const psi_hip_gqa_layer_input* input,
                                     uint32_t gqa_layer_parameter, int* out_recorded);
 /* Programs held, recordings and replays so far; any out pointer may be null. */

@@ -122,6 +122,7 @@ class BatchMetadataStruct(ctypes.Structure):
         ("group_tiles", c_uint32),
         ("num_row_groups", c_uint32),
         ("max_active_q_tile_tokens", c_uint32),
+        ("replay_counts", c_void_p),
     ]
 
 

@@ -230,7 +230,7 @@ struct ProgramKey {
     uint32_t layer, replay_mode, layer_is_parameter;
     uint32_t num_workers, group_tiles, num_row_groups, max_active_q_tile_tokens;
     uint64_t kv_pages_bytes, partial_scratch_bytes;
-    const void* pointers[20];
+    const void* pointers[21];
 };
 
 ProgramKey make_key(const psi_hip_gqa_layer_input& in, bool layer_is_parameter) {
@@ -251,10 +251,10 @@ ProgramKey make_key(const psi_hip_gqa_layer_input& in, bool layer_is_parameter) 
     k.max_active_q_tile_tokens = md.max_active_q_tile_tokens;
     k.kv_pages_bytes = in.kv_pages_bytes;
     k.partial_scratch_bytes = in.partial_scratch_bytes;
-    const void* p[20] = {in.qgkv, in.q, in.k, in.v, in.g, in.kv_pages, in.page_ids, in.q_norm_weight,
+    const void* p[21] = {in.qgkv, in.q, in.k, in.v, in.g, in.kv_pages, in.page_ids, in.q_norm_weight,
                          in.k_norm_weight, in.q_norm_rope, in.partial_scratch, in.output, md.req_slots,
                          md.flat_token_indices, md.q_token_tiles, md.kv_splits, md.cu_kv_splits,
-                         md.partial_row_index, md.worker_cu, md.row_groups};
+                         md.partial_row_index, md.worker_cu, md.row_groups, md.replay_counts};
     std::memcpy(k.pointers, p, sizeof(p));
     return k;
 }
@@ -469,7 +469,7 @@ static int record_program(psi_hip_gqa_replay_cache* cache, const psi_hip_gqa_lay
 
     const uint32_t* bound_before = ctx->replay_counts;
     const bool timing_before = ctx->timing;
-    ctx->replay_counts = cache->device_counts;
+    ctx->replay_counts = md.replay_counts != nullptr ? md.replay_counts : cache->device_counts;
     ctx->timing = false;  // event records would become nodes of the program
     hipGraph_t graph = nullptr;
     hipError_t e = hipStreamBeginCapture(ctx->stream, hipStreamCaptureModeThreadLocal);
@@ -523,10 +523,13 @@ extern "C" int psi_hip_gqa_replay_cache_submit(psi_hip_gqa_replay_cache* cache, 
     } else if (it != cache->programs.begin()) {
         cache->programs.splice(cache->programs.begin(), cache->programs, it);
     }
-    const psi_hip_gqa_replay_shape& s = input->batch_metadata->shape;
-    hipLaunchKernelGGL(set_replay_counts_kernel, dim3(1), dim3(64), 0, ctx->stream, cache->device_counts, s.num_tokens,
-                       s.num_q_token_tiles, s.num_kv_splits, gqa_layer_parameter);
-    PSI_HIP_CHECK(hipGetLastError());
+    if (input->batch_metadata->replay_counts == nullptr) {
+        // the counts the program reads: one small launch ahead of it (a caller that places them itself saves it)
+        const psi_hip_gqa_replay_shape& s = input->batch_metadata->shape;
+        hipLaunchKernelGGL(set_replay_counts_kernel, dim3(1), dim3(64), 0, ctx->stream, cache->device_counts,
+                           s.num_tokens, s.num_q_token_tiles, s.num_kv_splits, gqa_layer_parameter);
+        PSI_HIP_CHECK(hipGetLastError());
+    }
     PSI_HIP_CHECK(hipGraphLaunch(cache->programs.front().exec, ctx->stream));
     cache->replays += 1;
     return PSI_HIP_OK;

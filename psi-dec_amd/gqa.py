@@ -531,7 +531,9 @@ class GQAMetadataBuffers:
         self._max_kv_splits = max_kv_splits if max_kv_splits is not None else max_tokens
         self._max_workers = max_workers
         rows = self._max_kv_splits + max_workers
-        sizes = (("req_slots", max_tokens), ("flat_token_indices", max_tokens), ("q_token_tiles", 2 * max_tokens),
+        # replay_counts: the four words a recorded program reads its active counts from; they travel with the arrays
+        sizes = (("replay_counts", 4), ("req_slots", max_tokens), ("flat_token_indices", max_tokens),
+                 ("q_token_tiles", 2 * max_tokens),
                  ("cu_kv_splits", max_tokens + 1), ("worker_cu", max_workers + 1), ("kv_splits", 3 * rows),
                  ("partial_row_index", rows))
         self._offsets, total = {}, 0
@@ -559,6 +561,7 @@ class GQAMetadataBuffers:
             off, n = self._offsets[name]
             return self._d_all[off:off + n]
 
+        self.h_replay_counts, self.d_replay_counts = host("replay_counts"), dev("replay_counts")
         self.h_req_slots, self.d_req_slots = host("req_slots"), dev("req_slots")
         self.h_flat_token_indices, self.d_flat_token_indices = host("flat_token_indices"), dev("flat_token_indices")
         self.h_q_token_tiles, self.d_q_token_tiles = host("q_token_tiles"), dev("q_token_tiles")
@@ -627,6 +630,9 @@ class GQAMetadataBuffers:
         import torch
 
         rows = self._shape.num_total_sdpa_map_task_templates if self._shape is not None else 0
+        if self._shape is not None:  # the layer word stays 0: programs that read these counts hold their layer
+            self.h_replay_counts[:] = (self._shape.num_tokens, self._shape.num_q_token_tiles,
+                                       self._shape.num_sdpa_map_task_templates, 0)
         off, _ = self._offsets["kv_splits"]
         end = off + 3 * rows
         with torch.cuda.stream(self.device.stream):
@@ -824,9 +830,11 @@ class GQAMetadataBuffers:
         assert self._variant is not None, "GQA batch metadata must be updated before recording"
         return self._variant
 
-    def struct(self, shape: Optional[GQAReplayShape] = None):
+    def struct(self, shape: Optional[GQAReplayShape] = None, counts_uploaded: bool = False):
         """The batch as the layer entry points take it (psi_hip_gqa_batch_metadata): device addresses of the
-        arrays, the shape (`shape` overrides the capacities, e.g. a replay bucket) and the launch plans."""
+        arrays, the shape (`shape` overrides the capacities, e.g. a replay bucket) and the launch plans.
+        `counts_uploaded`: name the count words that `upload()` brought along, so that a replay cache launches its
+        program without a launch of its own ahead of it (the layer is then the input's, not a parameter)."""
         assert self.device is not None and self._shape is not None
         s = shape or self._shape
         return L.BatchMetadataStruct(
@@ -836,7 +844,8 @@ class GQAMetadataBuffers:
             self._variant.struct(), _ptr(self.d_req_slots), _ptr(self.d_flat_token_indices),
             _ptr(self.d_q_token_tiles), _ptr(self.d_kv_splits), _ptr(self.d_cu_kv_splits),
             _ptr(self.d_partial_row_index), _ptr(self.d_worker_cu), self.num_workers, _ptr(self.d_row_groups),
-            self.group_tiles, self.num_row_groups, self.max_active_q_tile_tokens)
+            self.group_tiles, self.num_row_groups, self.max_active_q_tile_tokens,
+            _ptr(self.d_replay_counts) if counts_uploaded else None)
 
 
 # ------------------------------------------------------------------ request page table
@@ -1230,6 +1239,7 @@ class GQAInput:
     g: object = None
     output: object = None
     shape: Optional[GQAReplayShape] = None  # overrides batch_metadata.replay_shape() (e.g. wider capacities)
+    counts_uploaded: bool = False  # a replay cache reads the count words the metadata upload brought along
 
 
 class GQA:
@@ -1292,7 +1302,7 @@ class GQA:
 
     def input_struct(self, inp: GQAInput):
         """(psi_hip_gqa_layer_input, keep-alive objects) for an input."""
-        md = inp.batch_metadata.struct(inp.shape)
+        md = inp.batch_metadata.struct(inp.shape, counts_uploaded=inp.counts_uploaded)
         sc = inp.scratch
         qgkv = inp.qgkv if (inp.qgkv is not None or inp.q is not None) else sc.qgkv
         out = inp.output if inp.output is not None else sc.attention_output

@@ -212,13 +212,14 @@ def test_layer_input_validation(psi, device):
     assert "split q / k / v rows" in str(err.value)
 
 
-@pytest.mark.parametrize("q_len", [1, 2])
-def test_replay_cache_serves_buckets_and_matches_oracle(psi, oracle, device, q_len):
+@pytest.mark.parametrize("q_len,counts_uploaded", [(1, False), (2, False), (1, True), (2, True)])
+def test_replay_cache_serves_buckets_and_matches_oracle(psi, oracle, device, q_len, counts_uploaded):
     """One recorded program per (variant, token / tile / split capacities): batches of 5, 3, 1 and 4 of five
     requests are submitted twice through the cache with the capacities `ReplayBucketPolicy` gives them.  Every
     submission matches the CPU oracle on that batch (pages bit-exact, outputs within the bar), rows beyond the
     active tokens keep their canary, the second round records nothing, and the number of programs equals the
-    number of distinct capacity keys.  q_len 2: the multi-query kernels."""
+    number of distinct capacity keys.  q_len 2: the multi-query kernels.  counts_uploaded: the active counts reach
+    the device with the metadata upload and a submission is the program's launch alone."""
     import torch
 
     wl = importlib_workloads(psi)
@@ -269,7 +270,7 @@ def test_replay_cache_serves_buckets_and_matches_oracle(psi, oracle, device, q_l
                     pages.copy_(pristine)
                     out.fill_(-768.0)
                     inp = psi.GQAInput(w.layout, w.layer, meta, psi.GQAKVCacheBindings(pages, page_ids), scratch,
-                                       q=q, k=k, v=v, output=out, shape=caps)
+                                       q=q, k=k, v=v, output=out, shape=caps, counts_uploaded=counts_uploaded)
                     recorded = cache.submit(inp)
                     side.synchronize()
                 assert recorded == new_key and (round_ == 0 or not recorded), (round_, picks)
