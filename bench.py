@@ -429,6 +429,26 @@ def calibrate_copy(device, args):
         us = start.elapsed_time(stop) * 1e3 / args.steps
         moved = nbytes if read_only else 2 * nbytes
         out[name] = {"avg_launch_us": us, "bytes_moved_per_launch": moved, "GB/s": moved / (us / 1e6) / 1e9}
+    # the ceiling of the attention kernels' access pattern: scattered 64 KiB pages, 1 KiB per load, through LDS
+    probe.psi_probe_page_stream.restype = ctypes.c_int
+    probe.psi_probe_page_stream.argtypes = [ctypes.c_void_p, ctypes.c_void_p, ctypes.c_uint64, ctypes.c_int]
+    stream_bytes = nbytes - nbytes % (1024 * 16384)
+    out["page_stream_probe"] = {"bytes_read_per_launch": stream_bytes, "GB/s_by_loads_in_flight_per_wave": {}}
+    for outstanding in (1, 2, 4, 8, 32):
+        def launch_stream():
+            rc = probe.psi_probe_page_stream(stream, src.data_ptr(), stream_bytes, outstanding)
+            if rc != 0:
+                raise RuntimeError(f"psi_probe_page_stream failed: {rc}")
+        for _ in range(args.warmup):
+            launch_stream()
+        start, stop = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        start.record(device.stream)
+        for _ in range(args.steps):
+            launch_stream()
+        stop.record(device.stream)
+        stop.synchronize()
+        us = start.elapsed_time(stop) * 1e3 / args.steps
+        out["page_stream_probe"]["GB/s_by_loads_in_flight_per_wave"][str(outstanding)] = stream_bytes / (us / 1e6) / 1e9
     print(json.dumps(out))
 
 
