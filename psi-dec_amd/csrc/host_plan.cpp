@@ -442,6 +442,10 @@ extern "C" int psi_hip_gqa_metadata_update(uint32_t max_tokens, const uint32_t* 
     std::vector<uint32_t> splits, cu;
     if (fixed) {
         // Fixed partitions cut on partition boundaries rather than on even tile shares.
+        uint64_t rows = 0;
+        for (const auto& t : tiles) rows += t.num_splits;
+        splits.reserve((size_t)rows * 3);
+        cu.reserve(tiles.size() + 1);
         cu.assign(1, 0u);
         for (uint32_t i = 0; i < tiles.size(); ++i) {
             for (uint64_t s = 0; s < tiles[i].num_splits; ++s) {
@@ -524,15 +528,28 @@ extern "C" int psi_hip_split_kv_balance_plan(const uint32_t* kv_splits_in, uint3
     PSI_REQUIRE(num_workers > 0 && num_tokens > 0, "balanced plan needs workers and tokens");
     PSI_REQUIRE(cu_in[0] == 0 && cu_in[num_tokens] == num_rows_in, "cu_kv_splits must cover every input row");
     constexpr uint32_t kTile = 16;
-    auto tiles_of = [&](uint32_t r) -> uint64_t {
-        const uint32_t b = kv_splits_in[3 * r + 1], e = kv_splits_in[3 * r + 2];
-        return e > b ? (uint64_t)(e + kTile - 1) / kTile - b / kTile : 0;
+    // The cut depends on the tiles alone, and adjacent rows of one token that meet on a tile boundary are cut as if
+    // they were one row (a piece runs on across such a boundary at no cost): they are merged first, so that the
+    // passes below walk a batch's tokens rather than its partitions.
+    struct Run {
+        uint32_t token, begin, end;
+    };
+    std::vector<Run> runs;
+    runs.reserve(num_rows_in);
+    for (uint32_t r = 0; r < num_rows_in; ++r) {
+        const uint32_t token = kv_splits_in[3 * r], b = kv_splits_in[3 * r + 1], e = kv_splits_in[3 * r + 2];
+        PSI_REQUIRE(token < num_tokens, "balanced plan input must not hold padding rows");
+        if (!runs.empty() && e > b && runs.back().token == token && runs.back().end == b && b % kTile == 0 &&
+            runs.back().end > runs.back().begin)
+            runs.back().end = e;
+        else
+            runs.push_back(Run{token, b, e});
+    }
+    auto tiles_of = [&](const Run& run) -> uint64_t {
+        return run.end > run.begin ? (uint64_t)(run.end + kTile - 1) / kTile - run.begin / kTile : 0;
     };
     uint64_t total = 0;
-    for (uint32_t r = 0; r < num_rows_in; ++r) {
-        PSI_REQUIRE(kv_splits_in[3 * r] < num_tokens, "balanced plan input must not hold padding rows");
-        total += tiles_of(r);
-    }
+    for (const Run& run : runs) total += tiles_of(run);
     // A worker's cost is its tiles plus kRowStartTiles per row it starts (split record -> slot -> page ID ->
     // first keys, and the partial state written at the end: about 3.4 us against 0.62 us per tile on MI355X).
     // Workers are filled in order up to a common budget; the budget is the smallest one that leaves the last
@@ -542,24 +559,33 @@ extern "C" int psi_hip_split_kv_balance_plan(const uint32_t* kv_splits_in, uint3
         uint32_t token, begin, end, worker;
     };
     std::vector<Piece> pieces;
-    auto fill = [&](uint64_t budget) -> uint64_t {  // returns the cost that lands on the last worker
-        pieces.clear();
+    // One pass over the rows for a budget.  The search for the budget only needs the cost that lands on the last
+    // worker, so it runs with `emit` off and keeps the last piece alone; the pass that follows it writes the pieces.
+    auto fill = [&](uint64_t budget, bool emit) -> uint64_t {
+        if (emit) {
+            pieces.clear();
+            pieces.reserve((size_t)num_tokens + num_workers);
+        }
+        Piece last{0u, 0u, 0u, 0u};
+        bool have_last = false;
         uint32_t w = 0;
         uint64_t used = 0;
         bool open_row = false;  // the worker's last piece can still be extended (same token, adjacent keys)
-        for (uint32_t r = 0; r < num_rows_in; ++r) {
-            const uint32_t b = kv_splits_in[3 * r + 1], e = kv_splits_in[3 * r + 2];
-            uint64_t remaining = tiles_of(r);
+        for (const Run& run : runs) {
+            const uint32_t row_token = run.token, b = run.begin, e = run.end;
+            uint64_t remaining = tiles_of(run);
             uint32_t tile_cursor = b / kTile;
             if (remaining == 0) {  // degenerate row: keep it so that row counts per token stay positive
-                pieces.push_back({kv_splits_in[3 * r], b, e, w});
+                last = Piece{row_token, b, e, w};
+                have_last = true;
+                if (emit) pieces.push_back(last);
                 open_row = false;
                 continue;
             }
             while (remaining > 0) {
-                const bool extends = open_row && !pieces.empty() && pieces.back().worker == w &&
-                                     pieces.back().token == kv_splits_in[3 * r] &&
-                                     pieces.back().end == std::max<uint32_t>(b, tile_cursor * kTile);
+                const uint32_t piece_begin = std::max<uint32_t>(b, tile_cursor * kTile);
+                const bool extends =
+                    open_row && have_last && last.worker == w && last.token == row_token && last.end == piece_begin;
                 const uint64_t start_cost = extends ? 0 : kRowStartTiles;
                 if (w + 1 < num_workers && used + start_cost >= budget) {  // no room for even one tile: next worker
                     ++w;
@@ -569,12 +595,15 @@ extern "C" int psi_hip_split_kv_balance_plan(const uint32_t* kv_splits_in, uint3
                 }
                 const uint64_t room = w + 1 < num_workers ? budget - used - start_cost : remaining;
                 const uint64_t take = std::min<uint64_t>(remaining, std::max<uint64_t>(room, 1));
-                const uint32_t piece_begin = std::max<uint32_t>(b, tile_cursor * kTile);
                 const uint32_t piece_end = (uint32_t)std::min<uint64_t>(e, (uint64_t)(tile_cursor + take) * kTile);
-                if (extends)
-                    pieces.back().end = piece_end;  // same worker, same token, adjacent keys: one row, one partial state
-                else
-                    pieces.push_back({kv_splits_in[3 * r], piece_begin, piece_end, w});
+                if (extends) {
+                    last.end = piece_end;  // same worker, same token, adjacent keys: one row, one partial state
+                    if (emit) pieces.back().end = piece_end;
+                } else {
+                    last = Piece{row_token, piece_begin, piece_end, w};
+                    have_last = true;
+                    if (emit) pieces.push_back(last);
+                }
                 open_row = true;
                 tile_cursor += (uint32_t)take;
                 remaining -= take;
@@ -585,7 +614,8 @@ extern "C" int psi_hip_split_kv_balance_plan(const uint32_t* kv_splits_in, uint3
     };
     uint64_t budget = std::max<uint64_t>((total + kRowStartTiles * ((uint64_t)num_tokens + num_workers)) / num_workers,
                                         kRowStartTiles + 1);  // room for at least one tile
-    while (fill(budget) > budget) budget += std::max<uint64_t>(budget / 64, 1);
+    while (fill(budget, false) > budget) budget += std::max<uint64_t>(budget / 64, 1);
+    fill(budget, true);
 
     uint32_t out_rows = 0, worker = 0;
     worker_cu_out[0] = 0;

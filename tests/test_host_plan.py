@@ -452,6 +452,28 @@ def test_balance_plan_covers_the_same_ranges(psi):
         assert len(set(tokens)) == len(tokens), "adjacent pieces of a token inside a worker must be one row"
 
 
+def test_balance_plan_does_not_depend_on_the_partition_length(psi):
+    """The balanced cut depends on a batch's 16-token tiles alone: the same contexts planned with partitions of 16,
+    512, 2048 tokens or unsplit (every one a multiple of the tile) give the same rows, offsets and worker table."""
+    single = psi.GQASplitKVVariant.SingleQ(16, 256, 6)
+    rng = np.random.default_rng(11)
+    for trial in range(6):
+        n = int(rng.integers(1, 24))
+        ctx = rng.integers(1, 9000, n).tolist()
+        plans = []
+        for partition in (16, 512, 2048, 1 << 20):
+            md = psi.GQAMetadataBuffers(None, n, max_kv_splits=sum(-(-c // partition) for c in ctx) + 1, max_workers=32)
+            md.update_fixed_partition(list(range(n)), [c - 1 for c in ctx], list(range(n + 1)), single, partition)
+            s = md.balance(32)
+            rows = s.num_sdpa_map_task_templates
+            plans.append((rows, md.h_kv_splits[:3 * rows].copy(), md.h_cu_kv_splits[:n + 1].copy(),
+                          np.array(md.h_worker_cu).copy()))
+        for other in plans[1:]:
+            assert other[0] == plans[0][0]
+            for a, b in zip(other[1:], plans[0][1:]):
+                assert np.array_equal(a, b)
+
+
 def test_balance_plan_with_more_workers_than_tiles(psi):
     """Tiny batches: workers without work get empty row ranges, nothing is lost."""
     md = psi.GQAMetadataBuffers(None, 4, max_kv_splits=16)
