@@ -44,6 +44,8 @@ def test_prefill_chunk_on_prefix(psi, oracle, device, partition):
     ("Float32", 4, 2, 64, 4, 3),
     ("Bfloat16", 24, 4, 256, 8, 8),  # the reference's (256, 8) profile, full tiles
     ("Float16", 8, 1, 128, 8, 3),
+    ("Float16", 16, 2, 256, 16, 8),   # 8 heads per KV head, full tiles: 64 columns, the two-group kernel
+    ("Bfloat16", 16, 2, 256, 16, 7),  # 56 columns
 ])
 def test_tiled_geometries(psi, oracle, device, dtype_name, hq, hkv, d, p, q_len):
     wl = importlib_workloads(psi)
@@ -300,7 +302,8 @@ def test_grouped_and_plain_maps_agree(psi, oracle, device):
 @pytest.mark.parametrize("dtype_name,hq,hkv,d,p,q_lens", [
     ("Bfloat16", 24, 4, 256, 16, 2),                        # one-draft verify: one column block
     ("Bfloat16", 24, 4, 256, 16, 4),                        # three drafts: two column blocks
-    ("Bfloat16", 24, 4, 256, 16, [8, 3, 1, 8, 5, 2, 7]),    # full tiles: four column blocks on eight waves
+    ("Bfloat16", 24, 4, 256, 16, [8, 3, 1, 8, 5, 2, 7]),    # full tiles: three column blocks, the loading wave takes one
+    ("Bfloat16", 16, 2, 256, 16, [8, 2, 8, 1, 8, 3, 8]),    # 64 columns: the two-group kernel
     ("Float16", 16, 2, 256, 8, 3),                          # 8-token pages
     ("Bfloat16", 32, 8, 128, 16, [20, 1, 9, 2, 1, 1, 12]),  # several Q-token tiles per request
     ("Float32", 6, 2, 64, 8, 2),                            # generic kernels: one workgroup per row
