@@ -613,6 +613,16 @@ int psi_hip_gqa_layer_prepare(const psi_hip_gqa_layer_config* cfg, const psi_hip
                               const psi_hip_gqa_host_metadata* host, psi_hip_gqa_batch_metadata* out_plan,
                               uint32_t* out_uses);
 
+/* The next decode step of the batch psi_hip_gqa_layer_prepare planned last into `host` -- the same requests in the
+ * same order, one new token each at the next position -- without planning again: positions and the end of every
+ * token's last row move on by one, in place.  That equals a fresh preparation bit for bit as long as no sequence
+ * starts a new 16-token tile (a plan with fixed partitions, in plan order or balanced, depends on the tile counts
+ * alone); when one does, or when the plan is of another kind (greedy capacities, a row index, TiledQ), nothing is
+ * touched and *out_advanced is 0: prepare again.  `plan` is the preparation's output; its shape stays as it is.
+ * No counterpart in the reference, which plans every batch anew (batch_metadata.rs:128-317). */
+int psi_hip_gqa_layer_advance_decode(const psi_hip_gqa_plan_options* options, const psi_hip_gqa_host_metadata* host,
+                                     const psi_hip_gqa_batch_metadata* plan, uint32_t plan_uses, int* out_advanced);
+
 /* Bytes of `partial_scratch` for a variant and split capacity (`GQAScratch::new`, scratch.rs:48-92). */
 int psi_hip_gqa_layer_scratch_bytes(const psi_hip_gqa_layer_config* cfg, const psi_hip_split_kv_variant* variant,
                                     uint32_t num_total_kv_splits, uint64_t* out_bytes);

@@ -338,6 +338,9 @@ PROTOTYPES = {
     "psi_hip_gqa_layer_prepare": (
         c_int, [POINTER(LayerConfigStruct), POINTER(PlanOptionsStruct), c_void_p, c_void_p, c_void_p, c_uint32,
                 _VARIANT, POINTER(HostMetadataStruct), POINTER(BatchMetadataStruct), _U32P]),
+    "psi_hip_gqa_layer_advance_decode": (
+        c_int, [POINTER(PlanOptionsStruct), POINTER(HostMetadataStruct), POINTER(BatchMetadataStruct), c_uint32,
+                POINTER(ctypes.c_int)]),
     "psi_hip_gqa_layer_record": (c_int, [c_void_p, POINTER(LayerConfigStruct), POINTER(LayerInputStruct)]),
     "psi_hip_gqa_layer_record_static_scratch": (
         c_int, [c_void_p, POINTER(LayerConfigStruct), POINTER(LayerInputStruct)]),

@@ -391,6 +391,41 @@ extern "C" int psi_hip_gqa_layer_prepare(const psi_hip_gqa_layer_config* cfg, co
     return PSI_HIP_OK;
 }
 
+extern "C" int psi_hip_gqa_layer_advance_decode(const psi_hip_gqa_plan_options* options,
+                                                const psi_hip_gqa_host_metadata* host,
+                                                const psi_hip_gqa_batch_metadata* plan, uint32_t plan_uses,
+                                                int* out_advanced) {
+    PSI_REQUIRE(options && host && plan && out_advanced, "GQA advance: options, host arrays, plan and out_advanced must not be null");
+    PSI_REQUIRE(host->req_slots_by_token && host->flat_token_indices && host->kv_splits && host->cu_kv_splits,
+                "GQA advance: the metadata arrays must not be null");
+    *out_advanced = 0;
+    const uint32_t tokens = plan->shape.num_tokens;
+    PSI_REQUIRE(tokens > 0 && tokens <= host->max_tokens, "GQA advance: the plan's token count does not fit the arrays");
+    constexpr uint32_t kTile = 16;
+    // Only plans whose rows follow from the tile counts alone, in an order that does not depend on the lengths.
+    if (plan->variant.kind != PSI_HIP_VARIANT_SINGLE_Q || options->capacity_mode != PSI_HIP_CAPACITY_FIXED_PARTITION ||
+        options->partition_tokens % kTile != 0 || (plan_uses & (1u | 4u)) != 0)
+        return PSI_HIP_OK;
+    const uint32_t* slots = host->req_slots_by_token;
+    uint32_t* positions = host->flat_token_indices;
+    uint32_t* rows = host->kv_splits;
+    const uint32_t* cu = host->cu_kv_splits;
+    for (uint32_t t = 0; t < tokens; ++t) {
+        if (t > 0 && slots[t] == slots[t - 1]) return PSI_HIP_OK;  // several tokens of one request: not a decode batch
+        const uint64_t context = (uint64_t)positions[t] + 1;
+        if (context % kTile == 0 || context + 1 > 0xffffffffull) return PSI_HIP_OK;  // the next token starts a tile
+        if (cu[t + 1] <= cu[t] || cu[t + 1] > host->kv_splits_capacity) return PSI_HIP_OK;
+        const uint32_t* last = rows + (size_t)(cu[t + 1] - 1) * 3;
+        if (last[0] != t || last[2] != context) return PSI_HIP_OK;  // not the table a preparation left here
+    }
+    for (uint32_t t = 0; t < tokens; ++t) {
+        positions[t] += 1;
+        rows[(size_t)(cu[t + 1] - 1) * 3 + 2] += 1;
+    }
+    *out_advanced = 1;
+    return PSI_HIP_OK;
+}
+
 extern "C" int psi_hip_gqa_layer_record(psi_hip_ctx* ctx, const psi_hip_gqa_layer_config* cfg,
                                         const psi_hip_gqa_layer_input* input) {
     return record_layer(ctx, cfg, input);

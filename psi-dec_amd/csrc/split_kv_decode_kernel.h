@@ -65,6 +65,28 @@ __device__ __forceinline__ void unpack2<F16Tag>(uint32_t packed, float& lo, floa
 
 // Orders this wave's LDS traffic: earlier LDS operations have completed and the compiler keeps
 // later ones after this point.  A wave's LDS operations execute in issue order.
+// Maximum over the four lanes l % 16 == const of a wave, in every one of them, on the vector ALU: the two swaps
+// exchange the odd 16-lane (32-lane) rows of one operand with the even rows of the other.
+__device__ __forceinline__ float quarter_wave_max(float x) {
+    const uint32_t u = __float_as_uint(x);
+    const auto h = __builtin_amdgcn_permlane32_swap(u, u, false, false);
+    const uint32_t m = __float_as_uint(fmaxf(__uint_as_float(h[0]), __uint_as_float(h[1])));
+    const auto q = __builtin_amdgcn_permlane16_swap(m, m, false, false);
+    return fmaxf(__uint_as_float(q[0]), __uint_as_float(q[1]));
+}
+
+// The same for a sum: x + (the lane 32 on), and x + (the lanes 16, 32, 48 on).
+__device__ __forceinline__ float half_wave_sum(float x) {
+    const uint32_t u = __float_as_uint(x);
+    const auto h = __builtin_amdgcn_permlane32_swap(u, u, false, false);
+    return __uint_as_float(h[0]) + __uint_as_float(h[1]);
+}
+__device__ __forceinline__ float quarter_wave_sum(float x) {
+    const uint32_t m = __float_as_uint(half_wave_sum(x));
+    const auto q = __builtin_amdgcn_permlane16_swap(m, m, false, false);
+    return __uint_as_float(q[0]) + __uint_as_float(q[1]);
+}
+
 __device__ __forceinline__ void wave_lds_fence() { asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory"); }
 
 #ifndef PSI_DECODE_WAVES_PER_SIMD
@@ -265,8 +287,7 @@ __global__ __launch_bounds__(64 * kWaves, decode_waves_per_simd(G)) void split_k
             v[r] = valid ? (s0[r] + s1[r]) * a.scale_log2 : -INFINITY;
             m = fmaxf(m, v[r]);
         }
-        m = fmaxf(m, __shfl_xor(m, 16, 64));
-        m = fmaxf(m, __shfl_xor(m, 32, 64));
+        m = quarter_wave_max(m);
         const float next_max = fmaxf(run_max, m);
         const float alpha = __builtin_amdgcn_exp2f(run_max - next_max);  // 0 on the first tile
         const bool rescale = __any(mt < (uint32_t)G && next_max != run_max);
@@ -382,13 +403,9 @@ __global__ __launch_bounds__(64 * kWaves, decode_waves_per_simd(G)) void split_k
     for (int h = 0; h < G; ++h)
 #pragma unroll
         for (int e = 0; e < 8; ++e) {
-            float v = acc[h][e];
-            v += __shfl_xor(v, 32, 64);
-            if (kVTokensPerLoad == 4) v += __shfl_xor(v, 16, 64);
-            acc[h][e] = v;
+            acc[h][e] = kVTokensPerLoad == 4 ? quarter_wave_sum(acc[h][e]) : half_wave_sum(acc[h][e]);
         }
-    lane_sum += __shfl_xor(lane_sum, 16, 64);
-    lane_sum += __shfl_xor(lane_sum, 32, 64);
+    lane_sum = quarter_wave_sum(lane_sum);
     if (lane < (uint32_t)kVLanesPerToken) {
 #pragma unroll
         for (int h = 0; h < G; ++h) {

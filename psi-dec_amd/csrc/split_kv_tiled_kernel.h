@@ -495,16 +495,6 @@ __global__ __launch_bounds__(64 * kTiledTileWaves * CG, (TiledOccupancy<NB, CG>:
 // where it does (the builtin) it waits for every outstanding one before any LDS read, which would undo the prefetch.
 // ---------------------------------------------------------------------------------------------------------------
 
-// Maximum over the four lanes l % 16 == const of a wave, in every one of them, on the vector ALU: the two swaps
-// exchange the odd 16-lane (32-lane) rows of one operand with the even rows of the other.
-__device__ __forceinline__ float quarter_wave_max(float x) {
-    const uint32_t u = __float_as_uint(x);
-    const auto h = __builtin_amdgcn_permlane32_swap(u, u, false, false);
-    const uint32_t m = __float_as_uint(fmaxf(__uint_as_float(h[0]), __uint_as_float(h[1])));
-    const auto q = __builtin_amdgcn_permlane16_swap(m, m, false, false);
-    return fmaxf(__uint_as_float(q[0]), __uint_as_float(q[1]));
-}
-
 // Line `kLine` (64 elements) of the 8 + 8 rows of a tile: two loads of 1 KiB, one per half tile.  The instruction
 // offset is added to the global and to the LDS address alike, hence 1024 - 128 between the M0 values of consecutive
 // lines.

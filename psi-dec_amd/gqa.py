@@ -779,6 +779,7 @@ class GQAMetadataBuffers:
                 addr(self._h_worker_cu_all), addr(self._h_row_groups_all))
         plan, uses = L.BatchMetadataStruct(), ctypes.c_uint32()
         v = variant.struct() if variant is not None else None
+        self._last_prepare = (options, plan, uses, boundaries)  # what advance_decode() continues from
         L.check(L.load().psi_hip_gqa_layer_prepare(
             ctypes.byref(layer_struct), ctypes.byref(options), rs.ctypes.data, ti.ctypes.data, cu.ctypes.data, len(rs),
             ctypes.byref(v) if v is not None else None, ctypes.byref(self._host_struct), ctypes.byref(plan),
@@ -808,6 +809,20 @@ class GQAMetadataBuffers:
                     self._d_row_groups_all[:used].copy_(self._h_row_groups_t[:used], non_blocking=True)
             self.upload()
         return self._shape
+
+    def advance_decode(self) -> bool:
+        """The next decode step of the batch `prepare` planned last (same requests, one more token each) without
+        planning again (psi_hip_gqa_layer_advance_decode): True if the arrays were advanced in place and uploaded,
+        False if a sequence starts a new 16-token tile or the plan is of another kind: prepare again."""
+        assert getattr(self, "_last_prepare", None) is not None, "advance_decode() continues a prepare()"
+        options, plan, uses, _keep = self._last_prepare
+        self._staging_free()
+        advanced = ctypes.c_int()
+        L.check(L.load().psi_hip_gqa_layer_advance_decode(ctypes.byref(options), ctypes.byref(self._host_struct),
+                                                          ctypes.byref(plan), uses.value, ctypes.byref(advanced)))
+        if advanced.value and self.device is not None:
+            self.upload()
+        return bool(advanced.value)
 
     def _row_groups_words(self) -> int:
         return 0 if self._h_row_groups_all is None else len(self._h_row_groups_all)

@@ -662,3 +662,62 @@ def test_single_call_prepare_equals_the_step_by_step_plan(psi, seed):
         assert arrays(a) == arrays(b), dispatch
         if variant.is_tiled():
             assert b.max_active_q_tile_tokens == min(int(q_lens.max()), variant.q_token_tile_size)
+
+
+@pytest.mark.parametrize("balanced", [False, True])
+def test_advance_decode_equals_a_fresh_preparation(psi, balanced):
+    """psi_hip_gqa_layer_advance_decode moves a decode batch's plan on by one token per sequence in place.  Over 60
+    decode steps of six sequences: whenever it says it advanced, every array equals what a fresh preparation of
+    the grown contexts writes; it declines exactly when some sequence starts a new 16-token tile; and it declines
+    for plans it is not meant for (a row index, several tokens per request, the reference's greedy capacities)."""
+    core = psi.GQACore(0, 24 * 256, 256, 24, 4, 0.0625)
+    gqa = psi.GQA(None, core, psi.GQAMetalConfig(65536, 64, 1e-6, 1e6))
+    variant = psi.GQASplitKVVariant.SingleQ(16, 256, 6)
+    rng = np.random.default_rng(77)
+    n, workers = 6, 8
+    ctx = rng.integers(1, 1500, size=n).astype(np.int64)
+    ctx[0] = 510  # crosses a 512-token partition on the way
+    slots = rng.permutation(16)[:n].astype(np.uint32)
+    cu = np.arange(n + 1, dtype=np.uint32)
+
+    def prepared(contexts):
+        md = psi.GQAMetadataBuffers(None, 8, max_kv_splits=64, max_workers=workers)
+        gqa.prepare_fixed_partition(md, slots, (contexts - 1).astype(np.uint32), cu, 512, balanced=balanced,
+                                    variant=variant, num_workers=workers)
+        return md
+
+    def arrays(md):
+        s = md.replay_shape()
+        return (s, md.h_req_slots[:n].tolist(), md.h_flat_token_indices[:n].tolist(),
+                md.h_kv_splits[:3 * s.num_total_sdpa_map_task_templates].tolist(), md.h_cu_kv_splits[:n + 1].tolist(),
+                None if md.h_worker_cu is None else np.array(md.h_worker_cu).tolist())
+
+    md = prepared(ctx)
+    advanced = declined = 0
+    for step in range(60):
+        starts_a_tile = bool((ctx % 16 == 0).any())
+        ok = md.advance_decode()
+        ctx = ctx + 1
+        assert ok != starts_a_tile, (step, ctx.tolist())
+        if ok:
+            advanced += 1
+            assert arrays(md) == arrays(prepared(ctx)), step
+        else:
+            declined += 1
+            md = prepared(ctx)
+    assert advanced > 10 and declined > 10
+
+    # plans it leaves alone
+    md = psi.GQAMetadataBuffers(None, 8, max_kv_splits=64, max_workers=workers)
+    gqa.prepare_fixed_partition(md, slots, (ctx - 1).astype(np.uint32), cu, 512, balanced=False, variant=variant)
+    md.order_longest_first()
+    md._last_prepare[2].value |= 1  # the row index is now in use
+    assert not md.advance_decode()
+    md = psi.GQAMetadataBuffers(None, 16, max_kv_splits=64, max_workers=workers)
+    gqa.prepare_fixed_partition(md, slots[:2], np.array([100, 200], np.uint32), np.array([0, 2, 3], np.uint32), 512,
+                                balanced=balanced, variant=variant, num_workers=workers)   # two tokens of one request
+    assert not md.advance_decode()
+    md = psi.GQAMetadataBuffers(None, 8)
+    gqa.prepare(md, slots, (ctx - 1).astype(np.uint32), cu)  # the reference's greedy plan
+    kept = arrays(md)
+    assert not md.advance_decode() and arrays(md) == kept
