@@ -529,28 +529,40 @@ __device__ __forceinline__ void wait_load_groups(uint32_t groups) {
 }
 
 // ---------------------------------------------------------------------------------------------------------------
-// The multi-query map for tiles of up to 48 query columns: two waves per SIMD on each stream of KV tiles.
+// The multi-query map for tiles of up to 48 query columns: a loading wave and multiplying waves on each stream of
+// KV tiles, all on one SIMD.
 //
 // A wave stands at a load until the memory pipeline takes it, and at a product until the matrix cores take it: one
 // wave alone does the one or the other, and its time per tile is the sum (by the cycle counter, the K * Q^T phase of
-// one column block took 1800 cycles with the tile's eight K loads in it and 200 without).  Here eight waves form
-// four pairs; the waves p and p + 4 of a pair
-// (on one SIMD) walk the tiles p, p + 4, ... of the row together through one set of LDS stages.  The second wave of
-// the pair issues every load, announces each tile of K and of V in LDS as it lands and takes the smaller share of
-// the query columns (none of one block, one of two or three); the first wave takes the larger share and says in LDS
-// when it has read a stage, so that the second may refill it.  While one of them stands at a load the other
-// multiplies.  All of it is bounded: a wait on the other wave's progress gives up after 2^16 polls (the row's
-// results are then wrong, which the parity tests see, but no wave stays behind).
+// one column block took 1800 cycles with the tile's eight K loads in it and 200 without).  Here the waves p, p + 4,
+// p + 8 of a workgroup (they share a SIMD) walk the tiles p, p + 4, ... of the row together through one set of LDS
+// stages.  The last of them issues every load, announces each tile of K and of V in LDS as it lands and, in the
+// one- and two-block forms, does nothing else; the others multiply, one column block each, and say in LDS when they
+// have read a stage, so that it may be refilled.  While the loading wave stands at a load the others multiply.
+// With three column blocks a fourth wave per SIMD would leave each 128 registers, less than a block's accumulators
+// and operands take, so one wave multiplies two blocks and the loading wave takes the third (which costs: the same
+// split at two blocks runs 10 % slower than the pure loader).  All of it is bounded: a wait on another wave's
+// progress gives up after 2^16 polls (the row's results are then wrong, which the parity tests see, but no wave
+// stays behind).
 // ---------------------------------------------------------------------------------------------------------------
+// Waves per stream of tiles: one that loads, and one that multiplies per column block; with three blocks (four waves
+// of a SIMD would have 128 registers each, which a column block's 64 accumulators and its operands do not fit
+// into) one multiplying wave takes two blocks and the loading wave the third.
+constexpr int tiled_multiplying_waves(int column_blocks) { return column_blocks <= 2 ? column_blocks : 1; }
+constexpr int tiled_paired_waves(int column_blocks) { return (tiled_multiplying_waves(column_blocks) + 1) * kTiledTileWaves; }
+
 template <typename Tag, int D, int NB, bool kHalfPage>
-__global__ __launch_bounds__(128 * kTiledTileWaves, 1) void split_kv_tiled_paired_map(
+__global__ __launch_bounds__(64 * tiled_paired_waves(NB), 1) void split_kv_tiled_paired_map(
     MapArgs a, const uint32_t* __restrict__ page_ids, const uint32_t* __restrict__ kv_splits,
     const uint32_t* __restrict__ req_slots, const uint16_t* __restrict__ q, const uint16_t* __restrict__ pages,
     const uint32_t* __restrict__ q_token_tiles, const uint32_t* __restrict__ flat_token_indices,
     const uint32_t* __restrict__ worker_cu) {
     resolve_active(a);
     constexpr int kPairs = kTiledTileWaves;
-    constexpr int kWaves = 2 * kPairs;
+    constexpr int kWaves = tiled_paired_waves(NB);
+    constexpr int kMultipliers = tiled_multiplying_waves(NB);   // multiplying waves per stream
+    constexpr int kBlocksEach = NB <= 2 ? 1 : 2;                // column blocks of a multiplying wave
+    constexpr int kBlocksLoader = NB - kMultipliers * kBlocksEach;  // and of the loading wave (0, or 1 of 3)
     constexpr int kKSteps = D / 32;             // MFMA k-steps of QK^T
     constexpr int kDimBlocks = D / 16;          // 16-dim output blocks of PV
     constexpr int kDQ = D / 64;                 // 128-byte lines per row
@@ -562,8 +574,6 @@ __global__ __launch_bounds__(128 * kTiledTileWaves, 1) void split_kv_tiled_paire
     constexpr int kMergeStride = D + 4;         // floats per column row of the merge buffer
     constexpr int kStageBytes = kPairs * kPairBytes;
     constexpr int kQBytes = NB * kKSteps * 64 * 16;
-    constexpr int kBlocksSecond = NB > 2 ? NB - 2 : 0;  // column blocks of the loading wave
-    constexpr int kBlocksFirst = NB - kBlocksSecond;
     static_assert(kCols * kMergeStride * 4 <= kStageBytes, "the merge buffer reuses the tile stages");
 
     __shared__ __attribute__((aligned(1024))) unsigned char lds_union[kStageBytes + kQBytes];
@@ -571,7 +581,7 @@ __global__ __launch_bounds__(128 * kTiledTileWaves, 1) void split_kv_tiled_paire
     __shared__ float col_max_lds[kCols];
     __shared__ float col_sum_lds[kCols];
     // tiles of the row so far, per pair: [K landed, V landed, K read by the first wave, V read by the first wave]
-    __shared__ uint32_t progress[4][kPairs];
+    __shared__ uint32_t progress[2 + 2 * kMultipliers][kPairs];
     uint4* qb_lds = reinterpret_cast<uint4*>(lds_union + kStageBytes);  // [NB][kKSteps][64]
     float* merge = reinterpret_cast<float*>(lds_union);
 
@@ -579,14 +589,16 @@ __global__ __launch_bounds__(128 * kTiledTileWaves, 1) void split_kv_tiled_paire
     const uint32_t kv_head = blockIdx.x % a.walk.hkv;
     const uint32_t wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const uint32_t pair = wave % kPairs;
-    const bool second = wave >= (uint32_t)kPairs;
+    const uint32_t role = wave / kPairs;  // 0 .. kMultipliers - 1: a multiplying wave; kMultipliers: the loading wave
+    const bool second = role == (uint32_t)kMultipliers;
     unsigned char* my_stages = lds_union + pair * kPairBytes;
     const uint32_t my_stages_lds =
         (uint32_t)(size_t)(__attribute__((address_space(3))) unsigned char*)(lds_union) + pair * kPairBytes;
     volatile uint32_t* landed_k = &progress[0][pair];
     volatile uint32_t* landed_v = &progress[1][pair];
-    volatile uint32_t* read_k = &progress[2][pair];
-    volatile uint32_t* read_v = &progress[3][pair];
+    // what a multiplying wave reports; the loading wave waits for all of them
+    volatile uint32_t* read_k = &progress[2 + 2 * (second ? 0u : role)][pair];
+    volatile uint32_t* read_v = &progress[3 + 2 * (second ? 0u : role)][pair];
     auto wait_until_above = [&](volatile uint32_t* counter, uint32_t value) __attribute__((always_inline)) {
         for (uint32_t polls = 0; *counter <= value && polls < (1u << 16); ++polls) __builtin_amdgcn_s_sleep(1);
         asm volatile("" ::: "memory");
@@ -744,7 +756,7 @@ __global__ __launch_bounds__(128 * kTiledTileWaves, 1) void split_kv_tiled_paire
             qb_lds[(nb * kKSteps + i) * 64 + lane] = used ? v : make_uint4(0, 0, 0, 0);
         }
     }
-    if (tid < 4 * kPairs) (&progress[0][0])[tid] = 0;
+    if (tid < (2 + 2 * kMultipliers) * kPairs) (&progress[0][0])[tid] = 0;
     __syncthreads();
 
     // A operand of QK^T, k-step i: row mt, elements 32 * i + 8 * mc .. + 7 -> half mt / 8, line i / 2, chunk
@@ -757,21 +769,35 @@ __global__ __launch_bounds__(128 * kTiledTileWaves, 1) void split_kv_tiled_paire
         (mc >> 1) * kHalfBytes + (((mt & 3) >> 1) * 8 + (mc & 1) * 4 + (mt >> 2)) * 16 + (mt & 1) * 8;
     auto is_partial = [&](uint32_t t) { return t * kTileTokens < kv_begin || (t + 1) * kTileTokens > kv_end; };
 
+    // The position of this lane's query token in column block `block` (values, not an indexed array: the block of
+    // a wave is only known at run time, and an indexed array would live in memory).
+    uint32_t position_of_block[NB];
+#pragma unroll
+    for (int b = 0; b < NB; ++b) {
+        position_of_block[b] = cur.position[b];
+        asm volatile("" : "+v"(position_of_block[b]));
+    }
+    auto column_position = [&](uint32_t block) {
+        uint32_t p = position_of_block[0];
+#pragma unroll
+        for (int b = 1; b < NB; ++b) p = block == (uint32_t)b ? position_of_block[b] : p;
+        return p;
+    };
     // One wave's part of the row: the column blocks kBlock0 .. + kBlocks - 1, and the loads if it is the second
     // wave of its pair.  Both instances pass the same workgroup barriers.
-    auto walk_row = [&](auto blocks_tag, auto block0_tag, auto loads_tag) __attribute__((always_inline)) {
+    auto walk_row = [&](auto blocks_tag, auto block0, auto loads_tag) __attribute__((always_inline)) {
+        const uint32_t kBlock0 = block0;  // a constant where the wave's first column block is known at compile time
         constexpr int kBlocks = decltype(blocks_tag)::value;
-        constexpr int kBlock0 = decltype(block0_tag)::value;
         constexpr bool kLoads = decltype(loads_tag)::value;
         constexpr int kB = kBlocks > 0 ? kBlocks : 1;  // array extents
 
         uint32_t lim[kB];  // keys [kv_begin, lim) are visible to the column (0: column unused)
 #pragma unroll
         for (int nb = 0; nb < kBlocks; ++nb) {
-            const uint32_t position = cur.position[kBlock0 + nb];
+            const uint32_t position = column_position(kBlock0 + nb);
             lim[nb] = position != 0xffffffffu ? min(kv_end, position + 1) : 0u;
         }
-        // One column block per wave keeps its query operands in registers for the whole row.
+        // A wave with one column block keeps its query operands in registers for the whole row.
         constexpr bool kQInRegs = kBlocks == 1;
         uint4 q_reg[kQInRegs ? kKSteps : 1];
         if (kQInRegs) {
@@ -824,7 +850,8 @@ __global__ __launch_bounds__(128 * kTiledTileWaves, 1) void split_kv_tiled_paire
             }
             if (kLoads) {
                 if (has2) {
-                    wait_until_above(read_k, i);  // and so has the other
+#pragma unroll
+                    for (int r = 0; r < kMultipliers; ++r) wait_until_above(&progress[2 + 2 * r][pair], i);  // and so have the others
                     issue_k(tile + 2 * kPairs, pid2, stage);
                 }
                 // V(i) has landed once only K(i+1), V(i+1), K(i+2) are outstanding.  Rows outside the split have
@@ -912,7 +939,8 @@ __global__ __launch_bounds__(128 * kTiledTileWaves, 1) void split_kv_tiled_paire
             }
             if (kLoads) {
                 if (has2) {
-                    wait_until_above(read_v, i);
+#pragma unroll
+                    for (int r = 0; r < kMultipliers; ++r) wait_until_above(&progress[3 + 2 * r][pair], i);
                     issue_v(tile + 2 * kPairs, pid2, stage);
                 }
             } else {
@@ -969,8 +997,13 @@ __global__ __launch_bounds__(128 * kTiledTileWaves, 1) void split_kv_tiled_paire
             __syncthreads();
         }
     };
-    if (second) walk_row(std::integral_constant<int, kBlocksSecond>(), std::integral_constant<int, kBlocksFirst>(), std::true_type());
-    else walk_row(std::integral_constant<int, kBlocksFirst>(), std::integral_constant<int, 0>(), std::false_type());
+    if (second)
+        walk_row(std::integral_constant<int, kBlocksLoader>(), std::integral_constant<uint32_t, kMultipliers * kBlocksEach>(),
+                 std::true_type());
+    else if constexpr (kMultipliers == 1)
+        walk_row(std::integral_constant<int, kBlocksEach>(), std::integral_constant<uint32_t, 0>(), std::false_type());
+    else
+        walk_row(std::integral_constant<int, kBlocksEach>(), role * kBlocksEach, std::false_type());
 
     // ---- emit: partial row of (split, q_head, token_in_tile); 1 KiB of contiguous f32 per wave store
     const uint32_t rows = a.rows_per_split_head;
@@ -1011,11 +1044,11 @@ inline int launch_tiled_map_typed(psi_hip_ctx* ctx, const Geometry& g, const Map
 #define PSI_TILED_PAIRED_LAUNCH(NB)                                                                                    \
     do {                                                                                                               \
         if (g.tokens_per_page == 8)                                                                                    \
-            hipLaunchKernelGGL((split_kv_tiled_paired_map<Tag, D, NB, true>), grid, dim3(128 * kTiledTileWaves), 0,      \
+            hipLaunchKernelGGL((split_kv_tiled_paired_map<Tag, D, NB, true>), grid, dim3(64 * tiled_paired_waves(NB)), 0, \
                                ctx->stream, a, a.walk.page_ids, a.kv_splits, a.req_slots, q, pages, a.q_token_tiles,   \
                                a.flat_token_indices, a.worker_cu);                                                     \
         else                                                                                                           \
-            hipLaunchKernelGGL((split_kv_tiled_paired_map<Tag, D, NB, false>), grid, dim3(128 * kTiledTileWaves), 0,     \
+            hipLaunchKernelGGL((split_kv_tiled_paired_map<Tag, D, NB, false>), grid, dim3(64 * tiled_paired_waves(NB)), 0, \
                                ctx->stream, a, a.walk.page_ids, a.kv_splits, a.req_slots, q, pages, a.q_token_tiles,   \
                                a.flat_token_indices, a.worker_cu);                                                     \
     } while (0)
