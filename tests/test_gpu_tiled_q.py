@@ -93,6 +93,38 @@ def test_sentinel_split_rows_are_skipped(psi, oracle, device):
     assert (raw == 0x5A5A5A5A).sum() > 0, "padded rows of the scratch were overwritten"
 
 
+@pytest.mark.parametrize("balanced", [False, True])
+def test_tile_wider_than_the_launch_was_sized_for(psi, oracle, device, balanced):
+    """`max_active_q_tile_tokens` is a contract: a launch sized for two-token tiles (one column block) that meets a
+    four-token tile cannot compute its rows.  It must enter them as empty states over whatever the scratch held,
+    so that the combine merges nothing stale and the tile's output is visibly wrong (zeros), while every tile
+    within the bound is computed as usual."""
+    import torch
+
+    wl = importlib_workloads(psi)
+    w = wl.make_workload(73, [300, 90, 1200], 24, 4, 256, psi.Dtype.Bfloat16, 16, q_lens=[2, 4, 2])
+    dw = wl.DeviceWorkload(device, w, partition_tokens=512, max_tokens=32, f32_output=True, balanced=balanced,
+                           variant=psi.GQASplitKVVariant.TiledQ(8, 16, 6))
+    dw.scratch.buffer.view(torch.float32).fill_(7.0)   # stale partial states: finite, plausible
+    dw.append()
+    m, s = dw.meta, dw.shape
+    if balanced:
+        dw.kernels.invoke_map_balanced(dw.q, dw.pages, m.d_req_slots, dw.page_ids, m.d_flat_token_indices,
+                                       m.d_q_token_tiles, m.d_kv_splits, m.d_worker_cu, m.num_workers, dw.scratch,
+                                       w.layer, s.num_tokens, s.num_q_token_tiles, s.num_sdpa_map_task_templates, 2)
+    else:
+        dw.kernels.invoke_map_bucketed(dw.q, dw.pages, m.d_req_slots, dw.page_ids, m.d_flat_token_indices,
+                                       m.d_q_token_tiles, m.d_kv_splits, dw.scratch, w.layer, s.num_tokens,
+                                       s.num_q_token_tiles, s.num_sdpa_map_task_templates, 2)
+    dw.reduce()
+    got = dw.output_f32().reshape(w.num_tokens, -1)
+    _, exp = oracle_step(oracle, w)
+    exp = exp.reshape(w.num_tokens, -1)
+    assert_outputs_close(got[:2], exp[:2], "tile within the bound, before the wide one")
+    assert_outputs_close(got[6:], exp[6:], "tile within the bound, after the wide one")
+    assert (got[2:6] == 0.0).all(), "the wide tile's rows must come out as zeros, not as stale or partial sums"
+
+
 def test_verify_accept_rollback_cycle(psi, oracle, device):
     """Two verify steps with drafts: step 1 writes K/V for [token, d1, d2, d3]; the host accepts a
     prefix; step 2 starts at the first rejected position and overwrites it.  Attention of step 2
