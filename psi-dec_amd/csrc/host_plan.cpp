@@ -551,10 +551,12 @@ extern "C" int psi_hip_split_kv_balance_plan(const uint32_t* kv_splits_in, uint3
     uint64_t total = 0;
     for (const Run& run : runs) total += tiles_of(run);
     // A worker's cost is its tiles plus kRowStartTiles per row it starts (split record -> slot -> page ID ->
-    // first keys, and the partial state written at the end: about 3.4 us against 0.62 us per tile on MI355X).
+    // first keys, the pipeline running empty and filling again, and the partial state written at the end: about
+    // 6 us against 0.62 us per tile on MI355X; with a weight of five tiles the workgroups of C2's decode map that
+    // serve two rows ended 3 us after those that serve one).
     // Workers are filled in order up to a common budget; the budget is the smallest one that leaves the last
     // worker no more than the others.
-    constexpr uint64_t kRowStartTiles = 5;
+    constexpr uint64_t kRowStartTiles = 10;
     struct Piece {
         uint32_t token, begin, end, worker;
     };

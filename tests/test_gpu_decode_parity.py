@@ -90,9 +90,9 @@ def test_balanced_plan_matches_oracle(psi, oracle, device):
     tiles = (rows[:, 2] + 15) // 16 - rows[:, 1] // 16
     per_worker = [int(tiles[m.h_worker_cu[i]:m.h_worker_cu[i + 1]].sum()) for i in range(m.num_workers)]
     assert sum(per_worker) == sum(-(-c // 16) for c in ctx)
-    cost = [t + 5 * int(m.h_worker_cu[i + 1] - m.h_worker_cu[i]) for i, t in enumerate(per_worker)]
+    cost = [t + 10 * int(m.h_worker_cu[i + 1] - m.h_worker_cu[i]) for i, t in enumerate(per_worker)]
     busy = [c for c in cost if c]  # the last busy worker takes what is left
-    assert max(busy[:-1]) - min(busy[:-1]) <= 5 and busy[-1] <= max(busy[:-1])
+    assert max(busy[:-1]) - min(busy[:-1]) <= 10 and busy[-1] <= max(busy[:-1])
 
 
 @pytest.mark.parametrize("q_len", [1, 3])

@@ -439,13 +439,13 @@ def test_balance_plan_covers_the_same_ranges(psi):
         assert (part[:, 0] == row).all()
     w = md.h_worker_cu
     assert w[0] == 0 and w[-1] == s.num_sdpa_map_task_templates and (np.diff(w.astype(np.int64)) >= 0).all()
-    # equal shares of the cost (16-token tiles plus 5 per row started; the last worker takes what is left), and
+    # equal shares of the cost (16-token tiles plus 10 per row started; the last worker takes what is left), and
     # inside a worker one row per token: at most workers + tokens rows
     tiles = (-(-ks[:, 2].astype(np.int64) // 16)) - ks[:, 1].astype(np.int64) // 16
     per_worker = [int(tiles[w[i]:w[i + 1]].sum()) for i in range(24)]
     assert sum(per_worker) == sum(-(-c // 16) for c in ctx)
-    cost = [t + 5 * int(w[i + 1] - w[i]) for i, t in enumerate(per_worker)]
-    assert max(cost[:-1]) - min(cost[:-1]) <= 5 and 0 < cost[-1] <= max(cost[:-1])
+    cost = [t + 10 * int(w[i + 1] - w[i]) for i, t in enumerate(per_worker)]
+    assert max(cost[:-1]) - min(cost[:-1]) <= 10 and 0 < cost[-1] <= max(cost[:-1])
     assert s.num_sdpa_map_task_templates <= 24 + len(ctx)
     for i in range(24):
         tokens = ks[w[i]:w[i + 1], 0].tolist()
