@@ -5,14 +5,21 @@
 // decomposition: here the matrix cores and the LDS are the bound, not HBM.
 //
 // Work decomposition
-//   one workgroup (8 waves) = one (row group, kv_head [, half of the query heads]).  A row group is
-//   a run of consecutive Q-token tiles of one request whose kv_split rows start at the same key
-//   (the rows of one KV partition).  With more than 5 query heads per KV head the heads are dealt
-//   to two workgroups.  The workgroup's query columns, column c = token_in_group * heads + head,
-//   are dealt out 16 per wave: a wave keeps the online-softmax state and the accumulators of its
-//   columns for the whole KV range, so wave states never merge.  The eight waves walk the KV range
-//   together in tiles of 32 keys which they load once, together, into LDS (two buffers, one
-//   barrier per tile; global loads run two tiles ahead in two register sets).
+//   one workgroup = one (row group, kv_head [, part of the query heads]).  A row group is a run of consecutive
+//   Q-token tiles of one request whose kv_split rows start at the same key (the rows of one KV partition).  With
+//   more than 5 query heads per KV head the heads are dealt to two or three workgroups.  The workgroup's query
+//   columns, column c = token_in_group * heads + head, are dealt out 16 per multiplying wave: a wave keeps the
+//   online-softmax state and the accumulators of its columns for the whole KV range, so wave states never merge.
+//
+//   Twelve waves: eight that multiply (two per SIMD) and four that load (one per SIMD), around four LDS stages of
+//   32 keys.  A loading wave fetches its quarter of a tile into registers four tiles ahead (the tiles come from
+//   other compute units' L2 slices or from HBM, two microseconds away under load), stores it into the stage once
+//   every multiplying wave has said that it is through with the stage's previous tile, and announces it; a
+//   multiplying wave waits for the four announcements of its next tile, multiplies, and says so.  No barrier
+//   inside the range: the multiplying waves drift apart, and one wave's matrix work runs beside another's softmax
+//   and operand reads.  Every wait on another wave's word gives up after 2^16 polls (results are then wrong,
+//   which the parity tests see; no wave stays behind).  Three waves per SIMD leave each 168 registers, which is
+//   what a multiplying wave takes (64 accumulators, 32 of query operands, 32 of K operands in flight, 16 of V).
 //
 // Per 32-key tile and wave (16 columns)
 //   QK^T  S[key][column] on v_mfma_f32_16x16x32 of the storage type: A = K rows from LDS (key 16 * b + i in row i of
@@ -35,19 +42,21 @@
 //         tolerance for values that do).  The accumulators keep a column per lane, so rescaling needs no
 //         cross-lane traffic.
 //
-// LDS layout per buffer
+// LDS layout per stage
 //   K    [32 keys][D] elements, 16-byte chunk index XOR (key % 16): the 16 lanes of an operand read (16 rows, one
 //        chunk) then hit 16 different bank groups, and a row-wise store stays a permutation of its row.
 //   V    [32 keys][D] f16, rows padded to D * 2 + 32 bytes: the four keys of a quarter wave's transposing read
 //        (32 bytes each, 16 dims) then fall into different bank groups, and so do the eight keys of two quarters.
-//   page IDs of up to 4096 pages of the range, refilled for longer ranges.
+//   and twelve progress words: tiles stored, per loading wave; tiles read, per multiplying wave.
 #pragma once
 #include "split_kv_tiled_kernel.h"
 
 namespace psi {
 
 constexpr int kChunkKeys = 32;         // keys per KV tile
-constexpr int kChunkWaves = 8;
+constexpr int kChunkWaves = 8;          // multiplying waves
+constexpr int kChunkLoaders = 4;        // loading waves
+constexpr int kChunkStages = 4;         // KV tiles in LDS
 constexpr int kChunkColBlocks = 1;     // 16-column blocks per wave
 constexpr int kChunkWaveCols = 16 * kChunkColBlocks;
 static_assert(kChunkWaves * kChunkWaveCols == kChunkCols, "128 query columns per workgroup");
@@ -94,36 +103,36 @@ struct ChunkLds {
     static constexpr int kKBytes = kChunkKeys * D * 2;
     static constexpr int kVStride = D * 2 + 32;  // bytes per key row of the V tile
     static constexpr int kVtBytes = kChunkKeys * kVStride;
-    static constexpr int kIdCap = 4096;  // page IDs of a stretch of the KV range kept in LDS (+8: two tiles of look-ahead)
-    static constexpr int bytes = 2 * (kKBytes + kVtBytes) + (kIdCap + 8) * 4;
+    static constexpr int kStageBytes = kKBytes + kVtBytes;
+    static constexpr int kFlagsOffset = kChunkStages * kStageBytes;
+    static constexpr int bytes = kFlagsOffset + 64;  // tiles stored per loading wave [4], tiles read per multiplying wave [8]
 };
 
 template <typename Tag, int D>
-__global__ __launch_bounds__(64 * kChunkWaves, 2) void split_kv_chunk_map(
+__global__ __launch_bounds__(64 * (kChunkWaves + kChunkLoaders), 1) void split_kv_chunk_map(
     MapArgs a, const uint32_t* __restrict__ page_ids, const uint32_t* __restrict__ kv_splits,
     const uint32_t* __restrict__ req_slots, const uint16_t* __restrict__ q, const uint16_t* __restrict__ pages,
     const uint32_t* __restrict__ q_token_tiles, const uint32_t* __restrict__ flat_token_indices,
     const uint32_t* __restrict__ row_groups, uint32_t group_tiles, uint32_t num_groups, uint32_t head_subsets) {
     resolve_active(a);
     static_assert(D == 256, "the tile loaders are laid out for head_dim 256");
-    constexpr int kKSteps = D / 32;              // MFMA k-steps of QK^T
-    constexpr int kDimBlocks = D / 16;           // 16-dim output blocks of PV
-    constexpr int kRowChunks = D / 8;            // 16-byte chunks per K row
-    constexpr int kLoads = kChunkKeys * kRowChunks / (64 * kChunkWaves);  // 128-bit loads per thread and operand (2)
+    constexpr int kKSteps = D / 32;
+    constexpr int kDimBlocks = D / 16;
+    constexpr int kRowChunks = D / 8;
+    constexpr int kLoads = kChunkKeys * kRowChunks / (64 * kChunkLoaders);  // 128-bit loads per loading thread and operand (4)
     constexpr int kKBytes = ChunkLds<D>::kKBytes;
-    constexpr int kVtBytes = ChunkLds<D>::kVtBytes;
     constexpr int kVStride = ChunkLds<D>::kVStride;
-    constexpr int kBufBytes = kKBytes + kVtBytes;
-    constexpr int CB = kChunkColBlocks;
+    constexpr int kStageBytes = ChunkLds<D>::kStageBytes;
     constexpr float kSlack = 8.0f;
-    constexpr int kIdCap = ChunkLds<D>::kIdCap;
-    static_assert(kLoads == 2 && CB == 1, "loader and softmax are written for 8 waves of 16 columns");
-    // Dynamic LDS (the launcher passes ChunkLds<D>::bytes): with a static size the compiler sees
-    // that one workgroup fills the CU and lifts the register cap.
+    static_assert(kLoads == 4, "a loading thread takes keys s, s + 8, s + 16, s + 24 of one 16-byte chunk");
     extern __shared__ __attribute__((aligned(16))) unsigned char lds[];
+    // Progress words, addressed as LDS: through a generic pointer a volatile access becomes a flat one, which
+    // counts as a global load too, and waiting for its value would wait for every tile load in flight.
+    typedef volatile __attribute__((address_space(3))) uint32_t* LdsWords;
+    const LdsWords landed = (LdsWords)(lds + ChunkLds<D>::kFlagsOffset);  // tiles stored, per loading wave
+    const LdsWords done = landed + kChunkLoaders;                          // tiles read, per multiplying wave
 
-    const uint32_t TS = a.rows_per_split_head;  // Q tokens per tile
-    // heads of the KV head served here: head_first + [0, G)
+    const uint32_t TS = a.rows_per_split_head;
     const uint32_t subset = blockIdx.x % head_subsets;
     const uint32_t kv_head = (blockIdx.x / head_subsets) % a.walk.hkv;
     const uint32_t group = blockIdx.x / (head_subsets * a.walk.hkv);
@@ -136,7 +145,6 @@ __global__ __launch_bounds__(64 * kChunkWaves, 2) void split_kv_chunk_map(
     const uint32_t mt = lane & 15, mc = lane >> 4;
     if (group >= num_groups) return;
 
-    // ---- the group: rows[m] is the kv_split row of its m-th Q-token tile
     const uint32_t* rows = row_groups + (uint64_t)group * group_tiles;
     const uint32_t my_row = lane < group_tiles ? rows[lane] : kNoRow;
     const bool my_row_ok = my_row != kNoRow && my_row < a.num_active_kv_splits;
@@ -147,22 +155,132 @@ __global__ __launch_bounds__(64 * kChunkWaves, 2) void split_kv_chunk_map(
     const uint32_t q_tile0 = kv_splits[row0 * 3];
     if (q_tile0 >= a.num_active_q_token_tiles || q_tile0 + num_tiles > a.num_active_q_token_tiles) return;
     const uint32_t kv_begin = kv_splits[row0 * 3 + 1];
-    // wave-uniform by construction; said explicitly so that everything derived from it stays scalar
     const uint32_t kv_end_max = __builtin_amdgcn_readfirstlane(
         wave_max_u32(my_row_ok && lane < num_tiles ? kv_splits[my_row * 3 + 2] : 0u));
     const uint32_t flat_begin = q_token_tiles[q_tile0 * 2];
     const uint32_t flat_end = q_token_tiles[(q_tile0 + num_tiles - 1) * 2 + 1];
     if (flat_end <= flat_begin || flat_end > a.num_active_tokens || kv_end_max <= kv_begin) return;
     const uint32_t ncols = (flat_end - flat_begin) * G;
-    if (ncols > (uint32_t)kChunkCols || flat_end - flat_begin > num_tiles * TS) return;  // the planner never builds such a group
+    if (ncols > (uint32_t)kChunkCols || flat_end - flat_begin > num_tiles * TS) return;
     const uint32_t req_slot = req_slots[flat_begin];
+    const uint32_t key_base0 = kv_begin & ~(uint32_t)(kChunkKeys - 1);
+    const uint32_t num_kv_tiles = (kv_end_max - key_base0 + kChunkKeys - 1) / kChunkKeys;
 
-    // ---- this lane's column c = 16 * wave + mt: visible range, partial-state row, query row as B
-    // operands (dims 32 * ks + 8 * mc .. +8; zero for an unused column)
+    if (tid < kChunkLoaders + kChunkWaves) landed[tid] = 0u;
+    __syncthreads();
+    // Both roles poll with the word of wave (lane % count) in each lane and a wave-wide vote.
+    auto wait_all_above = [&](LdsWords words, uint32_t count_mask, uint32_t value) __attribute__((always_inline)) {
+        for (uint32_t polls = 0; polls < (1u << 16); ++polls) {
+            if (__all(words[lane & count_mask] > value)) break;
+            __builtin_amdgcn_s_sleep(1);
+        }
+        asm volatile("" ::: "memory");
+    };
+
+    if (wave >= (uint32_t)kChunkWaves) {
+        // =========================== a loading wave ===========================
+        const uint32_t log2p = 31 - __builtin_clz(a.walk.tokens_per_page);
+        const uint32_t page_mask = a.walk.tokens_per_page - 1;
+        const uint32_t* table_row = page_ids + ((uint64_t)req_slot * a.walk.num_layers + a.layer) *
+                                                          a.walk.num_blocks * a.walk.ids_per_block;
+        const uint32_t last_page = (kv_end_max - 1) >> log2p;
+        const uint64_t page_bytes = a.walk.page_elems * 2;
+        const unsigned char* base = reinterpret_cast<const unsigned char*>(pages);
+        struct TileBases {
+            const unsigned char* a;  // page of keys 0..15 of the tile, advanced to the tile's first token
+            const unsigned char* b;  // page of keys 16..31
+        };
+        // Page ids come through the scalar cache: a vector load would queue behind the tile loads in flight, and
+        // waiting for it would wait for all of them.  A tile's ids are fetched one step before its loads are issued.
+        // Tiles past the end of the range are clamped to the last one, so that loads stay unconditional.
+        typedef const __attribute__((address_space(4))) uint32_t* ConstantIds;
+        const ConstantIds ids_row = (ConstantIds)(uintptr_t)table_row;
+        struct TileIds {
+            uint32_t a, b;
+        };
+        auto fetch_ids = [&](uint32_t t) -> TileIds {
+            const uint32_t kb = key_base0 + min(t, num_kv_tiles - 1) * kChunkKeys;
+            return TileIds{ids_row[min(kb >> log2p, last_page)], ids_row[min((kb + 16) >> log2p, last_page)]};
+        };
+        auto tile_bases = [&](uint32_t t, TileIds ids) -> TileBases {
+            const uint32_t kb = key_base0 + min(t, num_kv_tiles - 1) * kChunkKeys;
+            const uint64_t in_page = (uint64_t)(kb & page_mask) * (D * 2);
+            return TileBases{base + ids.a * page_bytes + in_page, base + ids.b * page_bytes + in_page};
+        };
+        const uint32_t ltid = tid - 64 * kChunkWaves;
+        const uint32_t ld_chunk = ltid % kRowChunks;
+        const uint32_t ld_sub = ltid / kRowChunks;  // 0..7: keys ld_sub, +8 of either half of the tile
+        const uint32_t k_off = ((kv_head * a.walk.tokens_per_page + ld_sub) * D + ld_chunk * 8) * 2;
+        const uint32_t v_off = (((a.walk.hkv + kv_head) * a.walk.tokens_per_page + ld_sub) * D + ld_chunk * 8) * 2;
+        const uint32_t second_half = a.walk.tokens_per_page == 16 ? 0u : 16u * D * 2u;
+        constexpr uint32_t kEight = 8u * D * 2u;  // eight keys further on
+        struct Staging {
+            u32x4_t k[kLoads], v[kLoads];
+        };
+        auto issue_loads = [&](TileBases tb) __attribute__((always_inline)) -> Staging {
+            Staging st;
+            st.k[0] = *reinterpret_cast<const u32x4_t*>(tb.a + k_off);
+            st.k[1] = *reinterpret_cast<const u32x4_t*>(tb.a + k_off + kEight);
+            st.k[2] = *reinterpret_cast<const u32x4_t*>(tb.b + k_off + second_half);
+            st.k[3] = *reinterpret_cast<const u32x4_t*>(tb.b + k_off + second_half + kEight);
+            st.v[0] = *reinterpret_cast<const u32x4_t*>(tb.a + v_off);
+            st.v[1] = *reinterpret_cast<const u32x4_t*>(tb.a + v_off + kEight);
+            st.v[2] = *reinterpret_cast<const u32x4_t*>(tb.b + v_off + second_half);
+            st.v[3] = *reinterpret_cast<const u32x4_t*>(tb.b + v_off + second_half + kEight);
+            return st;
+        };
+        uint32_t k_store[kLoads], v_store[kLoads];
+#pragma unroll
+        for (int i = 0; i < kLoads; ++i) {
+            const uint32_t key = ld_sub + 8 * i;
+            k_store[i] = key * (D * 2) + ((ld_chunk ^ (key & 15)) * 16);
+            v_store[i] = kKBytes + key * kVStride + ld_chunk * 16;
+        }
+        auto store_tile = [&](uint32_t it, Staging& st) __attribute__((always_inline)) {
+            if (it >= (uint32_t)kChunkStages) wait_all_above(done, kChunkWaves - 1, it - kChunkStages);
+            unsigned char* stage = lds + (it % kChunkStages) * kStageBytes;
+            const uint32_t kb = key_base0 + it * kChunkKeys;
+            const bool edge = kb < kv_begin || kb + kChunkKeys > kv_end_max;  // first or last tile of the range
+            constexpr int kStores = kLoads;
+#pragma unroll
+            for (int i = 0; i < kStores; ++i) *reinterpret_cast<u32x4_t*>(stage + k_store[i]) = st.k[i];
+#pragma unroll
+            for (int i = 0; i < kStores; ++i) {
+                u32x4_t w = to_f16x8<Tag>(st.v[i]);
+                const uint32_t token = kb + ld_sub + 8 * i;
+                // V rows outside the range are zeroed: their probability is 0 but their bytes may be NaN / Inf
+                if (edge && (token < kv_begin || token >= kv_end_max)) w = u32x4_t{0u, 0u, 0u, 0u};
+                *reinterpret_cast<u32x4_t*>(stage + v_store[i]) = w;
+            }
+            if (lane == 0) landed[wave - kChunkWaves] = it + 1;  // behind the stores in the LDS queue
+        };
+        // Four tiles of loads in flight per wave (one register set per stage): the tiles come from the other
+        // compute units' L2 slices or from HBM, two microseconds away under load, and a tile is used up in less
+        // than one.
+        Staging st_a = issue_loads(tile_bases(0, fetch_ids(0)));
+        Staging st_b = issue_loads(tile_bases(1, fetch_ids(1)));
+        Staging st_c = issue_loads(tile_bases(2, fetch_ids(2)));
+        Staging st_d = issue_loads(tile_bases(3, fetch_ids(3)));
+        TileIds ids = fetch_ids(4);
+        auto step = [&](uint32_t it, Staging& st) __attribute__((always_inline)) {
+            if (it < num_kv_tiles) store_tile(it, st);
+            st = issue_loads(tile_bases(it + kChunkStages, ids));
+            ids = fetch_ids(it + kChunkStages + 1);
+        };
+        for (uint32_t it = 0; it < num_kv_tiles; it += 4) {
+            step(it, st_a);
+            step(it + 1, st_b);
+            step(it + 2, st_c);
+            step(it + 3, st_d);
+        }
+        return;
+    }
+
+    // =========================== a multiplying wave ===========================
     const uint32_t c = wave * kChunkWaveCols + mt;
     const bool used = c < ncols;
-    uint32_t lim = 0;        // keys [kv_begin, lim) are visible to the column; 0: column unused
-    uint64_t part_row = 0;   // partial-state row of the column
+    uint32_t lim = 0;
+    uint64_t part_row = 0;
     uint4 qreg[kKSteps];
     {
         const uint32_t t = used ? c / G : 0u, h = used ? c % G : 0u;
@@ -177,120 +295,26 @@ __global__ __launch_bounds__(64 * kChunkWaves, 2) void split_kv_chunk_map(
         for (int ks = 0; ks < kKSteps; ++ks)
             qreg[ks] = used ? *reinterpret_cast<const uint4*>(q_row + ks * 32) : make_uint4(0, 0, 0, 0);
     }
-    // Tiles at or beyond wave_hi hold no visible key for this wave; tiles inside [kv_begin, wave_lo)
-    // need no mask.
     const uint32_t wave_lo = __builtin_amdgcn_readfirstlane(wave_min_u32(used ? lim : 0xffffffffu));
     const uint32_t wave_hi = __builtin_amdgcn_readfirstlane(wave_max_u32(lim));
+    // tiles that hold a visible key of this wave
+    const uint32_t my_tiles = wave_hi > key_base0 ? min(num_kv_tiles, (wave_hi - key_base0 + kChunkKeys - 1) / kChunkKeys) : 0u;
 
-    // ---- page walk.  The page IDs of a stretch of the KV range (kIdCap pages) sit in LDS, so the
-    // per-tile path has no dependent global access; a tile's two IDs are read one step before they
-    // are needed.
-    const uint32_t log2p = 31 - __builtin_clz(a.walk.tokens_per_page);
-    const uint32_t page_mask = a.walk.tokens_per_page - 1;
-    const uint32_t* table_row = page_ids + ((uint64_t)req_slot * a.walk.num_layers + a.layer) *
-                                                      a.walk.num_blocks * a.walk.ids_per_block;
-    const uint32_t last_page = (kv_end_max - 1) >> log2p;
-    const uint32_t key_base0 = kv_begin & ~(uint32_t)(kChunkKeys - 1);
-    const uint32_t num_kv_tiles = (kv_end_max - key_base0 + kChunkKeys - 1) / kChunkKeys;
-    const uint32_t stretch_tiles = ((uint32_t)kIdCap << log2p) / kChunkKeys;  // tiles per refill of the ID table
-    uint32_t* id_lds = reinterpret_cast<uint32_t*>(lds + 2 * kBufBytes);
-    uint32_t id_page0 = 0;  // page behind id_lds[0]
-    auto refill_ids = [&](uint32_t first_tile) {
-        id_page0 = (key_base0 + first_tile * kChunkKeys) >> log2p;
-        // only the pages the range still has: every later lookup is clamped to last_page
-        const uint32_t count = min((uint32_t)kIdCap + 8, last_page - id_page0 + 1);
-        for (uint32_t i = tid; i < count; i += 64 * kChunkWaves) id_lds[i] = table_row[id_page0 + i];
-    };
-    struct TileIds {
-        uint32_t a, b;  // page of keys 0..15 and of keys 16..31 of a tile (the same value in every lane)
-    };
-    // Tiles past the end of the range are clamped to the last one: loads and stores stay
-    // unconditional, which keeps the compiler's count of outstanding loads exact.
-    auto read_ids = [&](uint32_t t) -> TileIds {
-        const uint32_t kb = key_base0 + min(t, num_kv_tiles - 1) * kChunkKeys;
-        return TileIds{id_lds[min(kb >> log2p, last_page) - id_page0], id_lds[min((kb + 16) >> log2p, last_page) - id_page0]};
-    };
-    struct TileBases {
-        const unsigned char* a;  // page of keys 0..15 of the tile, advanced to the tile's first token
-        const unsigned char* b;  // page of keys 16..31
-    };
-    const uint64_t page_bytes = a.walk.page_elems * 2;
-    auto tile_bases = [&](uint32_t t, TileIds ids) -> TileBases {
-        const uint32_t kb = key_base0 + min(t, num_kv_tiles - 1) * kChunkKeys;
-        const uint64_t in_page = (uint64_t)(kb & page_mask) * (D * 2);
-        const unsigned char* base = reinterpret_cast<const unsigned char*>(pages);
-        return TileBases{base + __builtin_amdgcn_readfirstlane(ids.a) * page_bytes + in_page,
-                         base + __builtin_amdgcn_readfirstlane(ids.b) * page_bytes + in_page};
-    };
-
-    // ---- cooperative tile loaders: per-thread byte offsets inside a page are fixed for the kernel.  Thread
-    // (ld_sub, ld_chunk) takes the 16-byte chunk ld_chunk of keys ld_sub and 16 + ld_sub, of K and of V.
-    constexpr int kSubs = 64 * kChunkWaves / kRowChunks;  // 16
-    const uint32_t ld_chunk = tid % kRowChunks;
-    const uint32_t ld_sub = tid / kRowChunks;
-    const uint32_t k_off = ((kv_head * a.walk.tokens_per_page + ld_sub) * D + ld_chunk * 8) * 2;
-    const uint32_t v_off = (((a.walk.hkv + kv_head) * a.walk.tokens_per_page + ld_sub) * D + ld_chunk * 8) * 2;
-    // keys 16..31 sit 16 rows further on in a page that holds the whole tile, and at the same offset of the next
-    // page otherwise (tile_bases then points at that page)
-    const uint32_t second_half = a.walk.tokens_per_page == 16 ? 0u : 16u * D * 2u;
-    struct Staging {
-        u32x4_t k[kLoads], v[kLoads];
-    };
-    auto issue_loads = [&](TileBases tb) __attribute__((always_inline)) -> Staging {
-        Staging st;
-        st.k[0] = *reinterpret_cast<const u32x4_t*>(tb.a + k_off);                // keys 0..15
-        st.k[1] = *reinterpret_cast<const u32x4_t*>(tb.b + k_off + second_half);  // keys 16..31
-        st.v[0] = *reinterpret_cast<const u32x4_t*>(tb.a + v_off);
-        st.v[1] = *reinterpret_cast<const u32x4_t*>(tb.b + v_off + second_half);
-        return st;
-    };
-    // Registers -> LDS buffer `buf`.  V rows outside [kv_begin, kv_end_max) are zeroed: their
-    // probability is 0 but their bytes may be NaN / Inf.
-    const uint32_t k_store0 = ld_sub * (D * 2) + ((ld_chunk ^ ld_sub) * 16);
-    const uint32_t k_store1 = k_store0 + kSubs * (D * 2);
-    const uint32_t v_store0 = ld_sub * kVStride + ld_chunk * 16;
-    const uint32_t v_store1 = v_store0 + kSubs * kVStride;
-    auto store_tile = [&](uint32_t it, uint32_t buf, const Staging& st) __attribute__((always_inline)) {
-        unsigned char* kbuf = lds + buf * kBufBytes;
-        unsigned char* vbuf = kbuf + kKBytes;
-        const uint32_t kb = key_base0 + min(it, num_kv_tiles - 1) * kChunkKeys;
-        *reinterpret_cast<u32x4_t*>(kbuf + k_store0) = st.k[0];
-        *reinterpret_cast<u32x4_t*>(kbuf + k_store1) = st.k[1];
-        u32x4_t w0 = to_f16x8<Tag>(st.v[0]), w1 = to_f16x8<Tag>(st.v[1]);
-        if (kb < kv_begin || kb + kChunkKeys > kv_end_max) {  // first or last tile of the range
-            const uint32_t token = kb + ld_sub;
-            if (token < kv_begin || token >= kv_end_max) w0 = u32x4_t{0u, 0u, 0u, 0u};
-            if (token + kSubs < kv_begin || token + kSubs >= kv_end_max) w1 = u32x4_t{0u, 0u, 0u, 0u};
-        }
-        *reinterpret_cast<u32x4_t*>(vbuf + v_store0) = w0;
-        *reinterpret_cast<u32x4_t*>(vbuf + v_store1) = w1;
-    };
-
-    // ---- operand read addresses of this lane
-    // K row of (block b, lane row mt): key 16 * b + mt, chunk (4 * ks + mc) ^ mt
     const uint32_t k_row0 = mt * (D * 2);
-    // V^T operand of (dim block db, key block b): the lane hands in the address of key 16 * b + 4 * mc + mt / 4,
-    // dims 16 * db + 4 * (mt % 4) .. + 3, and receives keys 16 * b + 4 * mc + 0..3 of dim 16 * db + mt
     const uint32_t vt_base = (4 * mc + (mt >> 2)) * kVStride + (mt & 3) * 8;
-
     float run_max = -INFINITY, lane_sum = 0.0f;
     f32x4_t o[kDimBlocks];
 #pragma unroll
     for (int db = 0; db < kDimBlocks; ++db) o[db] = f32x4_t{0.0f, 0.0f, 0.0f, 0.0f};
-    const bool wave_has_cols = wave * kChunkWaveCols < ncols;
 
-    // `masked`: the tile touches the start of the range or a causal limit of this wave (wave-uniform).
-    auto compute_tile = [&](uint32_t it, uint32_t buf, bool masked) __attribute__((always_inline)) {
-        const unsigned char* kbuf = lds + buf * kBufBytes;
+    constexpr int kAhead = 4;  // k-steps between an operand's read and its product
+    for (uint32_t it = 0; it < my_tiles; ++it) {
+        wait_all_above(landed, kChunkLoaders - 1, it);
+        const unsigned char* kbuf = lds + (it % kChunkStages) * kStageBytes;
         const unsigned char* vbuf = kbuf + kKBytes;
         const uint32_t kb = key_base0 + it * kChunkKeys;
-        // ---- logits S[key][column]: two key blocks
-        // The K operands are read kAhead k-steps before the products that take them, and the order is pinned: left
-        // to itself the compiler keeps two operands in flight, and every product then waits out the LDS latency
-        // (450 -> 441 us on the 2048-on-4096 chunk, side by side).  The same treatment of the V^T operands measures
-        // slower than the compiler's own order (+3 %; +4 % with the first reads issued ahead of the softmax).
+        const bool masked = !(kb >= kv_begin && kb + kChunkKeys <= wave_lo);
         f32x4_t s0 = f32x4_t{0.0f, 0.0f, 0.0f, 0.0f}, s1 = s0;
-        constexpr int kAhead = 4;
         uint4 k0[kKSteps], k1[kKSteps];
         auto read_k = [&](int ks) __attribute__((always_inline)) {
             const uint32_t off = k_row0 + (((4 * ks + mc) ^ mt) * 16);
@@ -314,9 +338,7 @@ __global__ __launch_bounds__(64 * kChunkWaves, 2) void split_kv_chunk_map(
         }
         __builtin_amdgcn_sched_group_barrier(0x008, 2 * kAhead, 0);
         __builtin_amdgcn_sched_barrier(0);
-        // ---- online softmax; this lane holds keys kb + 16 * b + 4 * mc + r, j = 4 * b + r, of column mt.
-        // Logits relative to the column's reference maximum; masked keys at -inf.
-        float v[8];  // raw logits; masked keys at -inf
+        float v[8];
 #pragma unroll
         for (int j = 0; j < 8; ++j) v[j] = j < 4 ? s0[j] : s1[j - 4];
         if (masked) {
@@ -326,11 +348,7 @@ __global__ __launch_bounds__(64 * kChunkWaves, 2) void split_kv_chunk_map(
                 if (token < kv_begin || token >= lim) v[j] = -INFINITY;
             }
         }
-        // scale > 0: the maximum of the scaled logits is the scaled maximum
         float m = fmaxf(fmaxf(fmaxf(v[0], v[1]), fmaxf(v[2], v[3])), fmaxf(fmaxf(v[4], v[5]), fmaxf(v[6], v[7]))) * a.scale_log2;
-        // The reference maximum moves only when some key exceeds it by more than kSlack (log2 domain):
-        // rare after the first tiles, so the cross-lane maximum and the rescaling sit behind a
-        // wave-wide test.  A column with no visible key so far keeps max = -inf, sum = 0, O = 0.
         if (__any(m > run_max + kSlack)) {
             m = fmaxf(m, __shfl_xor(m, 16, 64));
             m = fmaxf(m, __shfl_xor(m, 32, 64));
@@ -344,8 +362,6 @@ __global__ __launch_bounds__(64 * kChunkWaves, 2) void split_kv_chunk_map(
                     for (int r = 0; r < 4; ++r) o[db][r] *= alpha;
             }
         }
-        // exp2(logit * scale - reference); a column that has seen no key at all (reference -inf) has
-        // only masked keys here: -inf - 0 keeps them at probability 0
         const float neg_ref = run_max > -INFINITY ? -run_max : 0.0f;
         float p[8], tile_sum = 0.0f;
 #pragma unroll
@@ -354,8 +370,7 @@ __global__ __launch_bounds__(64 * kChunkWaves, 2) void split_kv_chunk_map(
             tile_sum += p[j];
         }
         lane_sum += tile_sum;
-        const uint4 pb = prob_operand_f16(p);
-        // ---- O^T[dim][column] += V^T * P^T, four dim blocks at a time
+        uint4 pb = prob_operand_f16(p);
 #pragma unroll
         for (int g = 0; g < kDimBlocks; g += 4) {
             uint4 vt[4];
@@ -368,40 +383,10 @@ __global__ __launch_bounds__(64 * kChunkWaves, 2) void split_kv_chunk_map(
 #pragma unroll
             for (int i = 0; i < 4; ++i) o[g + i] = mfma_16x16x32<F16Tag>(vt[i], pb, o[g + i]);
         }
-    };
-
-    // ---- main loop: tile `it` lives in LDS buffer it % 2.  Its global loads are issued two tiles
-    // earlier into one of two register sets and parked in LDS one tile earlier, so a load has two
-    // tile times to arrive.  The loop body is written twice so that the register sets keep their names.
-    auto step = [&](uint32_t it, Staging& incoming, const Staging& parked, TileIds& ids) __attribute__((always_inline)) {
-        incoming = issue_loads(tile_bases(it + 2, ids));
-        ids = read_ids(it + 3);
-        const uint32_t kb = key_base0 + it * kChunkKeys;
-        if (it < num_kv_tiles && wave_has_cols && kb < wave_hi)
-            compute_tile(it, it & 1, !(kb >= kv_begin && kb + kChunkKeys <= wave_lo));
-        store_tile(it + 1, (it + 1) & 1, parked);
-        __syncthreads();
-    };
-    refill_ids(0);
-    __syncthreads();
-    Staging st_a, st_b;
-    st_a = issue_loads(tile_bases(0, read_ids(0)));
-    store_tile(0, 0, st_a);
-    st_a = issue_loads(tile_bases(1, read_ids(1)));
-    TileIds ids = read_ids(2);
-    uint32_t next_refill = stretch_tiles;
-    __syncthreads();
-    for (uint32_t it = 0; it < num_kv_tiles; it += 2) {
-        if (it >= next_refill) {  // rare: the range is longer than the ID table
-            refill_ids(it);
-            next_refill += stretch_tiles;
-            __syncthreads();
-        }
-        step(it, st_b, st_a, ids);
-        step(it + 1, st_a, st_b, ids);
+        if (lane == 0) done[wave] = it + 1;  // behind this tile's reads in the LDS queue
     }
+    if (lane == 0) done[wave] = 0xffffffffu;
 
-    // ---- emit this wave's columns: un-normalised accumulators, log2-domain maximum, sum
     lane_sum += __shfl_xor(lane_sum, 16, 64);
     lane_sum += __shfl_xor(lane_sum, 32, 64);
     if (lim != 0) {
@@ -424,8 +409,8 @@ inline int launch_chunk_map_typed(psi_hip_ctx* ctx, const Geometry& g, const Map
     static const hipError_t lds_ok = hipFuncSetAttribute(reinterpret_cast<const void*>(&split_kv_chunk_map<Tag, D>),
                                                          hipFuncAttributeMaxDynamicSharedMemorySize, ChunkLds<D>::bytes);
     if (lds_ok != hipSuccess) return PSI_HIP_ERR_UNSUPPORTED;
-    hipLaunchKernelGGL((split_kv_chunk_map<Tag, D>), grid, dim3(64 * kChunkWaves), ChunkLds<D>::bytes, ctx->stream, a, a.walk.page_ids,
-                       a.kv_splits, a.req_slots, reinterpret_cast<const uint16_t*>(a.q),
+    hipLaunchKernelGGL((split_kv_chunk_map<Tag, D>), grid, dim3(64 * (kChunkWaves + kChunkLoaders)), ChunkLds<D>::bytes,
+                       ctx->stream, a, a.walk.page_ids, a.kv_splits, a.req_slots, reinterpret_cast<const uint16_t*>(a.q),
                        reinterpret_cast<const uint16_t*>(a.kv_pages), a.q_token_tiles, a.flat_token_indices, row_groups,
                        group_tiles, num_groups, subsets);
     return PSI_HIP_OK;

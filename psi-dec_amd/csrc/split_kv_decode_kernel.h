@@ -194,11 +194,12 @@ __global__ __launch_bounds__(64 * kWaves, decode_waves_per_simd(G)) void split_k
             // this workgroup owns the token's append for its KV head: one 16-byte chunk per lane, K line then V line
             const uint32_t page_id = table_row[own >> log2p];
             constexpr uint32_t kChunks = D / 8;
-            const uint16_t* flat[2] = {reinterpret_cast<const uint16_t*>(a.flat_k),
-                                       reinterpret_cast<const uint16_t*>(a.flat_v)};
+            const uint16_t* flat_k = reinterpret_cast<const uint16_t*>(a.flat_k);
+            const uint16_t* flat_v = reinterpret_cast<const uint16_t*>(a.flat_v);
             for (uint32_t c = lane; c < 2 * kChunks; c += 64) {
                 const uint32_t kind = c / kChunks, chunk = c % kChunks;
-                const uint16_t* src = flat[kind] + ((uint64_t)q_token * a.walk.hkv + kv_head) * D + chunk * 8;
+                // a choice of two pointers, not an index into an array of them: the load stays a global one
+                const uint16_t* src = (kind ? flat_v : flat_k) + ((uint64_t)q_token * a.walk.hkv + kv_head) * D + chunk * 8;
                 uint16_t* dst = const_cast<uint16_t*>(pages) + (uint64_t)page_id * a.walk.page_elems + kind * v_region +
                                 ((uint64_t)kv_head * a.walk.tokens_per_page + (own & page_mask)) * D + chunk * 8;
                 *reinterpret_cast<uint4*>(dst) = *reinterpret_cast<const uint4*>(src);

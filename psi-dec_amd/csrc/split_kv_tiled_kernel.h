@@ -594,12 +594,20 @@ __global__ __launch_bounds__(64 * tiled_paired_waves(NB), 1) void split_kv_tiled
     unsigned char* my_stages = lds_union + pair * kPairBytes;
     const uint32_t my_stages_lds =
         (uint32_t)(size_t)(__attribute__((address_space(3))) unsigned char*)(lds_union) + pair * kPairBytes;
-    volatile uint32_t* landed_k = &progress[0][pair];
-    volatile uint32_t* landed_v = &progress[1][pair];
+    // With three column blocks the words are addressed as LDS.  Through a generic pointer a volatile access becomes a
+    // flat one, which counts as a global load too: waiting for its value then waits for every tile load the wave has
+    // in flight, so that the loading wave drains its loads at each poll (449 against 482 us on the batch of 64 with
+    // 8 new tokens).  With one and two blocks the generic form is kept on purpose: it measures 2.5 % faster there
+    // (399 against 409 us and 414 against 425 us with 2 and 4 new tokens), and draining the loads by hand before each
+    // new tile's loads recovers less than half of that.  Measured, not explained.
+    typedef std::conditional_t<(NB <= 2), volatile uint32_t*, volatile __attribute__((address_space(3))) uint32_t*> LdsWord;
+    auto word = [&](uint32_t which) { return (LdsWord)(&progress[which][pair]); };
+    const LdsWord landed_k = word(0);
+    const LdsWord landed_v = word(1);
     // what a multiplying wave reports; the loading wave waits for all of them
-    volatile uint32_t* read_k = &progress[2 + 2 * (second ? 0u : role)][pair];
-    volatile uint32_t* read_v = &progress[3 + 2 * (second ? 0u : role)][pair];
-    auto wait_until_above = [&](volatile uint32_t* counter, uint32_t value) __attribute__((always_inline)) {
+    const LdsWord read_k = word(2 + 2 * (second ? 0u : role));
+    const LdsWord read_v = word(3 + 2 * (second ? 0u : role));
+    auto wait_until_above = [&](LdsWord counter, uint32_t value) __attribute__((always_inline)) {
         for (uint32_t polls = 0; *counter <= value && polls < (1u << 16); ++polls) __builtin_amdgcn_s_sleep(1);
         asm volatile("" ::: "memory");
     };
@@ -851,7 +859,7 @@ __global__ __launch_bounds__(64 * tiled_paired_waves(NB), 1) void split_kv_tiled
             if (kLoads) {
                 if (has2) {
 #pragma unroll
-                    for (int r = 0; r < kMultipliers; ++r) wait_until_above(&progress[2 + 2 * r][pair], i);  // and so have the others
+                    for (int r = 0; r < kMultipliers; ++r) wait_until_above(word(2 + 2 * r), i);  // and so have the others
                     issue_k(tile + 2 * kPairs, pid2, stage);
                 }
                 // V(i) has landed once only K(i+1), V(i+1), K(i+2) are outstanding.  Rows outside the split have
@@ -940,7 +948,7 @@ __global__ __launch_bounds__(64 * tiled_paired_waves(NB), 1) void split_kv_tiled
             if (kLoads) {
                 if (has2) {
 #pragma unroll
-                    for (int r = 0; r < kMultipliers; ++r) wait_until_above(&progress[3 + 2 * r][pair], i);
+                    for (int r = 0; r < kMultipliers; ++r) wait_until_above(word(3 + 2 * r), i);
                     issue_v(tile + 2 * kPairs, pid2, stage);
                 }
             } else {
