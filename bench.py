@@ -19,7 +19,7 @@ after every single step of a further run; the event between two steps keeps the 
 starting under the previous step's tail, so these read a few microseconds higher than the back-to-back figure.
 `host_plan_us`: what the host does per step before it can launch -- metadata update, worker plan, upload -- and is
 not part of the step time (the launches of step n overlap the planning of step n + 1 only if the caller
-pipelines them).  Before the W warm-up steps every workload runs untimed for about 30 ms (`settle_steps_before_warmup`):
+pipelines them).  Before the W warm-up steps every workload runs untimed for about 100 ms (`settle_steps_before_warmup`):
 set-up, so that the clocks have settled after the arena was generated.
 """
 import argparse
@@ -242,10 +242,11 @@ def time_case(psi, wl, device, case, args, with_spread=True):
     body = run_maps if kernel_only else run_steps
     # Set-up, not measurement: generating a workload's arena leaves the GPU's clocks unsettled for some 20 ms of
     # attention work (step times drift by 5-10 % over the first 40 steps), and an arena's first step pays for the
-    # first touch of its buffers.  Every arena is run once and the workload for at least 30 ms before the W
-    # warm-up steps and the K timed ones.
+    # first touch of its buffers; steps of a millisecond keep speeding up for longer (C5's decode side: 1313 us per
+    # step after 30 ms against 1262 us later).  Every arena is run once and the workload for at least 100 ms before
+    # the W warm-up steps and the K timed ones.
     settle_steps, t_settle = 0, time.perf_counter()
-    while settle_steps < len(arenas) or (time.perf_counter() - t_settle < 0.03 and settle_steps < 2000):
+    while settle_steps < len(arenas) or (time.perf_counter() - t_settle < 0.1 and settle_steps < 4000):
         body(1, first=settle_steps)
         settle_steps += 1
         if settle_steps % 8 == 0:
