@@ -294,6 +294,18 @@ def test_grouped_prefill_chunk(psi, oracle, device, partition, prefix, chunk):
     print("grouped chunk max_abs %.3e rel_rms %.3e" % stats, dw.shape, dw.meta.num_row_groups)
 
 
+def test_grouped_long_unsplit_range(psi, oracle, device):
+    """A chunk against 20000 cached tokens in a single partition: 627 KV tiles go round the row-group map's four LDS
+    stages, with its loading waves several tiles ahead of the multiplying ones all the way, and the range neither
+    begins nor ends on a tile."""
+    wl = importlib_workloads(psi)
+    w = wl.make_workload(97, [20000 + 57, 9], 4, 2, 256, psi.Dtype.Bfloat16, 16, q_lens=[57, 9])
+    stats, dw = run_and_check(psi, oracle, device, w, "grouped chunk 57 on 20000, one partition", max_tokens=128,
+                              variant=psi.GQASplitKVVariant.TiledQ(8, 16, 2), partition_tokens=32768, grouped=True)
+    assert dw.meta.num_row_groups > 0
+    print("long range max_abs %.3e rel_rms %.3e" % stats, dw.shape, dw.meta.num_row_groups)
+
+
 @pytest.mark.parametrize("dtype_name,hq,hkv,p,q_len", [
     ("Float16", 16, 2, 16, 50),    # 8 heads per KV head: two head subsets of 4, f16 single-term P
     ("Bfloat16", 4, 4, 32, 130),   # one head per KV head: 16 tiles per group, 32-token pages
