@@ -49,6 +49,8 @@
 //        (32 bytes each, 16 dims) then fall into different bank groups, and so do the eight keys of two quarters.
 //   and twelve progress words: tiles stored, per loading wave; tiles read, per multiplying wave.
 #pragma once
+#include <atomic>
+
 #include "split_kv_tiled_kernel.h"
 
 namespace psi {
@@ -406,9 +408,16 @@ inline int launch_chunk_map_typed(psi_hip_ctx* ctx, const Geometry& g, const Map
                                   uint32_t group_tiles, uint32_t num_groups) {
     const uint32_t subsets = chunk_head_subsets(g.group);
     const dim3 grid(num_groups * g.hkv * subsets);
-    static const hipError_t lds_ok = hipFuncSetAttribute(reinterpret_cast<const void*>(&split_kv_chunk_map<Tag, D>),
-                                                         hipFuncAttributeMaxDynamicSharedMemorySize, ChunkLds<D>::bytes);
-    if (lds_ok != hipSuccess) return PSI_HIP_ERR_UNSUPPORTED;
+    // The kernel's LDS is above the default limit of a launch; the limit is raised once per GPU (a function's
+    // attributes belong to the device it is loaded on).
+    static std::atomic<uint64_t> raised_on{0};
+    const uint64_t device_bit = 1ull << (ctx->device & 63);
+    if ((raised_on.load(std::memory_order_relaxed) & device_bit) == 0) {
+        if (hipFuncSetAttribute(reinterpret_cast<const void*>(&split_kv_chunk_map<Tag, D>),
+                                hipFuncAttributeMaxDynamicSharedMemorySize, ChunkLds<D>::bytes) != hipSuccess)
+            return PSI_HIP_ERR_UNSUPPORTED;
+        raised_on.fetch_or(device_bit, std::memory_order_relaxed);
+    }
     hipLaunchKernelGGL((split_kv_chunk_map<Tag, D>), grid, dim3(64 * (kChunkWaves + kChunkLoaders)), ChunkLds<D>::bytes,
                        ctx->stream, a, a.walk.page_ids, a.kv_splits, a.req_slots, reinterpret_cast<const uint16_t*>(a.q),
                        reinterpret_cast<const uint16_t*>(a.kv_pages), a.q_token_tiles, a.flat_token_indices, row_groups,
