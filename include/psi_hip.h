@@ -114,7 +114,26 @@ int psi_hip_ctx_reset_timing(psi_hip_ctx* ctx);
 /* F32_OUTPUT makes the combine kernels store the attention output as f32 [tokens, Hq, D] instead of
  * the io dtype, so a harness can check the f32-accumulated result before output rounding. */
 #define PSI_HIP_FLAG_F32_OUTPUT 2u
+/* WAIT_POLL_LIMIT bounds every wait of one wave on another wave's progress inside the multi-query and
+ * prefill-chunk maps: `value` polls (0 restores the default, 65536).  A wait that runs out sets
+ * PSI_HIP_DEVICE_ERR_WAIT_GAVE_UP below.  A harness sets a limit of 1 to see that path taken. */
+#define PSI_HIP_FLAG_WAIT_POLL_LIMIT 3u
 int psi_hip_ctx_set_flag(psi_hip_ctx* ctx, uint32_t flag, uint32_t value);
+
+/* Errors a kernel found while it ran.  The reference has no counterpart: its Metal kernels have no
+ * waits between simdgroups and multiply K and V in the storage type.  Here a kernel that could not
+ * compute a row reports it in a word of pinned host memory that belongs to the context (written by the
+ * GPU, read by the host after a synchronisation), and stores the affected partial rows as empty states
+ * (maximum -inf, sum 0), so that no stale or half-computed row is merged.
+ *   WAIT_GAVE_UP  a wave's bounded wait for another wave of its workgroup ran out;
+ *   V_RANGE       the prefill-chunk map met a V element of a bf16 cache that f16 cannot hold (finite
+ *                 |v| > 65504, Inf or NaN): that map multiplies V as f16.  Run the batch through
+ *                 psi_hip_split_kv_tiled_q_map instead, which keeps V in the storage type.
+ * psi_hip_sync returns PSI_HIP_ERR_RUNTIME while a bit is set; psi_hip_ctx_take_device_error
+ * synchronises the context's stream, returns the bits and clears them. */
+#define PSI_HIP_DEVICE_ERR_WAIT_GAVE_UP 1u
+#define PSI_HIP_DEVICE_ERR_V_RANGE 2u
+int psi_hip_ctx_take_device_error(psi_hip_ctx* ctx, uint32_t* out_bits);
 
 /* Device-side active counts for captured launches: the counterpart of `ReplayU32::Parameter`
  * (crates/inference-backend-metal/src/metal/replay.rs; bound at submit by `ReplayArguments::with_u32`).
@@ -580,6 +599,13 @@ typedef struct psi_hip_gqa_plan_options {
     uint32_t bucket_max_tokens;       /* variant selection: `GQAReplayBucketPolicy::max_tokens`, 0 = none */
     const uint32_t* topology_boundaries;
     uint32_t num_boundaries;
+    uint32_t bucket_capacities;       /* FIXED_PARTITION only: 1 = the recorded capacities of the shape (tokens, Q-token
+                                         tiles, KV splits -- the re-cut rows of a balanced plan included -- and the
+                                         number of row groups) are rounded up to `ReplayBucketPolicy` buckets of
+                                         host->max_tokens (with the topology boundaries), host->max_tokens,
+                                         host->kv_splits_capacity and the row-group table's capacity, and the arrays
+                                         are padded with PSI_HIP_SENTINEL up to them: a replay cache then sees one key
+                                         per bucket instead of one per batch */
 } psi_hip_gqa_plan_options;
 
 /* Host arrays of one batch's metadata with their capacities (e.g. views of one pinned staging block that is then

@@ -22,6 +22,9 @@ VARIANT_SINGLE_Q, VARIANT_TILED_Q = 0, 1
 CAPACITY_EXACT, CAPACITY_BUCKETED, CAPACITY_CALLER_TOKENS, CAPACITY_FIXED_PARTITION = 0, 1, 2, 3
 FLAG_FORCE_GENERIC = 1
 FLAG_F32_OUTPUT = 2
+FLAG_WAIT_POLL_LIMIT = 3
+DEVICE_ERR_WAIT_GAVE_UP = 1
+DEVICE_ERR_V_RANGE = 2
 REPLAY_EXACT, REPLAY_BUCKETED = 0, 1
 DISPATCH_PLAN_ORDER, DISPATCH_LONGEST_FIRST, DISPATCH_BALANCED, DISPATCH_ROW_GROUPS = 0, 1, 2, 3
 STATIC_SCRATCH_BYTES = 16 << 20
@@ -147,6 +150,7 @@ class PlanOptionsStruct(ctypes.Structure):
         ("bucket_max_tokens", c_uint32),
         ("topology_boundaries", POINTER(c_uint32)),
         ("num_boundaries", c_uint32),
+        ("bucket_capacities", c_uint32),
     ]
 
 
@@ -241,6 +245,7 @@ PROTOTYPES = {
     "psi_hip_ctx_reset_timing": (c_int, [c_void_p]),
     "psi_hip_ctx_bind_replay_counts": (c_int, [c_void_p, c_void_p]),
     "psi_hip_ctx_set_flag": (c_int, [c_void_p, c_uint32, c_uint32]),
+    "psi_hip_ctx_take_device_error": (c_int, [c_void_p, POINTER(c_uint32)]),
     "psi_hip_gqa_tokens_per_page": (c_int, [_CFG, _U32P]),
     "psi_hip_split_kv_select": (c_int, [_CFG, c_int, c_uint32, c_uint32, _VARIANT]),
     "psi_hip_split_kv_max_q_tokens_per_partial_output": (c_int, [_CFG, c_int, _U32P]),

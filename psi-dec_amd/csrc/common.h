@@ -45,6 +45,9 @@ int make_geometry(const psi_hip_gqa_config* cfg, Geometry* g);
 int resolve_static_scratch(int device);
 int check_layout(const psi_hip_page_table_layout* layout);
 
+constexpr uint32_t kDeviceStatusWords = 2;
+constexpr uint32_t kDefaultWaitPolls = 1u << 16;
+
 struct KernelTimer {
     double total_ms = 0;
     uint64_t launches = 0;
@@ -62,6 +65,12 @@ struct psi_hip_ctx {
     // Device u32[4] = {active tokens, active Q-token tiles, active KV splits, reserved} read by every
     // kernel when it runs (graph replay); null: the counts passed by value apply.
     const uint32_t* replay_counts = nullptr;
+    // Errors found by running kernels: kDeviceStatusWords words of pinned host memory mapped into the GPU's address
+    // space (word i set to 1 by a kernel = bit i of the PSI_HIP_DEVICE_ERR_* mask).  One word per kind, written
+    // with plain stores: nothing on the GPU reads or clears them.
+    volatile uint32_t* status_host = nullptr;
+    uint32_t* status_device = nullptr;
+    uint32_t wait_polls = 0;  // bound of the cross-wave waits (0: the default)
     std::map<std::string, psi::KernelTimer> timers;
     std::vector<hipEvent_t> event_pool;
 };

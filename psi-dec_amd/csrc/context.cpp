@@ -102,7 +102,19 @@ int psi_hip_ctx_create(int device, void* stream, psi_hip_ctx** out_ctx) {
     // with this GPU current, so that the entry point itself only launches
     int rc = psi::resolve_static_scratch(device);
     if (rc != PSI_HIP_OK) return rc;
+    // the words in which kernels report what they could not compute: pinned host memory, so that reading them
+    // after a synchronisation costs no copy
+    void* status_host = nullptr;
+    void* status_device = nullptr;
+    PSI_HIP_CHECK(hipHostMalloc(&status_host, 64, hipHostMallocMapped));
+    if (hipHostGetDevicePointer(&status_device, status_host, 0) != hipSuccess) {
+        (void)hipHostFree(status_host);
+        return psi::fail(PSI_HIP_ERR_RUNTIME, "the device status words cannot be mapped into device %d", device);
+    }
+    memset(status_host, 0, 64);
     auto* ctx = new psi_hip_ctx();
+    ctx->status_host = static_cast<volatile uint32_t*>(status_host);
+    ctx->status_device = static_cast<uint32_t*>(status_device);
     ctx->device = device;
     ctx->stream = (hipStream_t)stream;
     *out_ctx = ctx;
@@ -117,6 +129,7 @@ int psi_hip_ctx_destroy(psi_hip_ctx* ctx) {
             (void)hipEventDestroy(p.second);
         }
     for (auto ev : ctx->event_pool) (void)hipEventDestroy(ev);
+    if (ctx->status_host != nullptr) (void)hipHostFree(const_cast<uint32_t*>(ctx->status_host));
     delete ctx;
     return PSI_HIP_OK;
 }
@@ -127,9 +140,31 @@ int psi_hip_ctx_set_stream(psi_hip_ctx* ctx, void* stream) {
     return PSI_HIP_OK;
 }
 
+static uint32_t device_error_bits(const psi_hip_ctx* ctx) {
+    uint32_t bits = 0;
+    for (uint32_t i = 0; i < psi::kDeviceStatusWords; ++i)
+        if (ctx->status_host[i] != 0) bits |= 1u << i;
+    return bits;
+}
+
+static int report_device_error(uint32_t bits) {
+    if (bits == 0) return PSI_HIP_OK;
+    return psi::fail(PSI_HIP_ERR_RUNTIME, "a kernel reported an error (bits 0x%x):%s%s; the affected partial rows are empty states",
+                     bits, (bits & PSI_HIP_DEVICE_ERR_WAIT_GAVE_UP) ? " a bounded wait between waves ran out" : "",
+                     (bits & PSI_HIP_DEVICE_ERR_V_RANGE) ? " the prefill-chunk map met V values outside the f16 range" : "");
+}
+
 int psi_hip_sync(psi_hip_ctx* ctx) {
     PSI_REQUIRE(ctx != nullptr, "ctx must not be null");
     PSI_HIP_CHECK(hipStreamSynchronize(ctx->stream));
+    return report_device_error(device_error_bits(ctx));
+}
+
+int psi_hip_ctx_take_device_error(psi_hip_ctx* ctx, uint32_t* out_bits) {
+    PSI_REQUIRE(ctx != nullptr && out_bits != nullptr, "ctx and out_bits must not be null");
+    PSI_HIP_CHECK(hipStreamSynchronize(ctx->stream));
+    *out_bits = device_error_bits(ctx);
+    for (uint32_t i = 0; i < psi::kDeviceStatusWords; ++i) ctx->status_host[i] = 0;
     return PSI_HIP_OK;
 }
 
@@ -144,6 +179,7 @@ int psi_hip_ctx_set_flag(psi_hip_ctx* ctx, uint32_t flag, uint32_t value) {
     switch (flag) {
         case PSI_HIP_FLAG_FORCE_GENERIC: ctx->force_generic = value != 0; break;
         case PSI_HIP_FLAG_F32_OUTPUT: ctx->f32_output = value != 0; break;
+        case PSI_HIP_FLAG_WAIT_POLL_LIMIT: ctx->wait_polls = value; break;
         default: return psi::fail(PSI_HIP_ERR_INVALID_ARGUMENT, "unknown context flag %u", flag);
     }
     return PSI_HIP_OK;

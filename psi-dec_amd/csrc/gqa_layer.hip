@@ -10,6 +10,7 @@
 // splits)` key, captured from that call with the device-side count block bound, as the reference keeps one
 // recorded program per key and binds `gqa.num_active_*` at submission
 // (crates/inference-executor-core/src/replay.rs:4-87, backend.rs:55-57).
+#include <algorithm>
 #include <cstring>
 #include <list>
 #include <vector>
@@ -229,11 +230,13 @@ struct ProgramKey {
     psi_hip_page_table_layout layout;
     uint32_t layer, replay_mode, layer_is_parameter;
     uint32_t num_workers, group_tiles, num_row_groups, max_active_q_tile_tokens;
+    // context state that ends up in kernel arguments or decides which kernel runs
+    uint32_t f32_output, force_generic, wait_polls;
     uint64_t kv_pages_bytes, partial_scratch_bytes;
     const void* pointers[21];
 };
 
-ProgramKey make_key(const psi_hip_gqa_layer_input& in, bool layer_is_parameter) {
+ProgramKey make_key(const psi_hip_ctx& ctx, const psi_hip_gqa_layer_input& in, bool layer_is_parameter) {
     ProgramKey k;
     std::memset(&k, 0, sizeof(k));  // padding bytes take part in the comparison
     const psi_hip_gqa_batch_metadata& md = *in.batch_metadata;
@@ -249,6 +252,9 @@ ProgramKey make_key(const psi_hip_gqa_layer_input& in, bool layer_is_parameter) 
     k.group_tiles = md.row_groups ? md.group_tiles : 0;
     k.num_row_groups = md.row_groups ? md.num_row_groups : 0;
     k.max_active_q_tile_tokens = md.max_active_q_tile_tokens;
+    k.f32_output = ctx.f32_output;
+    k.force_generic = ctx.force_generic;
+    k.wait_polls = ctx.wait_polls;
     k.kv_pages_bytes = in.kv_pages_bytes;
     k.partial_scratch_bytes = in.partial_scratch_bytes;
     const void* p[21] = {in.qgkv, in.q, in.k, in.v, in.g, in.kv_pages, in.page_ids, in.q_norm_weight,
@@ -372,6 +378,33 @@ extern "C" int psi_hip_gqa_layer_prepare(const psi_hip_gqa_layer_config* cfg, co
         rc = psi_hip_split_kv_order_longest_first(host->kv_splits, shape.num_kv_splits, host->partial_row_index);
         if (rc != PSI_HIP_OK) return rc;
         uses |= 1u;
+    }
+    if (options->bucket_capacities != 0 && options->capacity_mode == PSI_HIP_CAPACITY_FIXED_PARTITION) {
+        // `ReplayBucketPolicy` capacities for the shape a replay cache keys its programs by (replay.rs:4-87): the
+        // reference buckets its greedy plan the same way (batch_metadata.rs:277-294); here the row count being
+        // bucketed is the dispatch plan's.
+        uint32_t cap = 0;
+        rc = psi_hip_replay_bucket_capacity(host->max_tokens, options->topology_boundaries, options->num_boundaries,
+                                            shape.num_tokens, &cap);
+        if (rc != PSI_HIP_OK) return rc;
+        shape.num_total_tokens = cap;
+        rc = psi_hip_replay_bucket_capacity(host->max_tokens, nullptr, 0, shape.num_q_token_tiles, &cap);
+        if (rc != PSI_HIP_OK) return rc;
+        shape.num_total_q_token_tiles = cap;
+        rc = psi_hip_replay_bucket_capacity(host->kv_splits_capacity, nullptr, 0, shape.num_kv_splits, &cap);
+        if (rc != PSI_HIP_OK) return rc;
+        for (uint64_t i = (uint64_t)shape.num_kv_splits * 3; i < (uint64_t)cap * 3; ++i)
+            host->kv_splits[i] = PSI_HIP_SENTINEL;
+        shape.num_total_kv_splits = cap;
+        if (num_groups != 0) {
+            const uint64_t max_groups = host->row_groups_capacity / group_tiles;
+            rc = psi_hip_replay_bucket_capacity((uint32_t)std::min<uint64_t>(max_groups, 0x7fffffffu), nullptr, 0,
+                                                num_groups, &cap);
+            if (rc != PSI_HIP_OK) return rc;
+            for (uint64_t i = (uint64_t)num_groups * group_tiles; i < (uint64_t)cap * group_tiles; ++i)
+                host->row_groups[i] = PSI_HIP_SENTINEL;  // a group without rows: its workgroups return at once
+            num_groups = cap;
+        }
     }
     uint32_t max_tile_tokens = 0;
     if (tiled) {
@@ -537,7 +570,7 @@ extern "C" int psi_hip_gqa_replay_cache_submit(psi_hip_gqa_replay_cache* cache, 
     PSI_REQUIRE(gqa_layer_parameter <= input->page_table_layout.num_gqa_layers,
                 "GQA page-table index exceeds layer count");
     if (out_recorded) *out_recorded = 0;
-    const ProgramKey key = make_key(*input, gqa_layer_parameter != 0);
+    const ProgramKey key = make_key(*ctx, *input, gqa_layer_parameter != 0);
     auto it = cache->programs.begin();
     for (; it != cache->programs.end(); ++it)
         if (std::memcmp(&it->key, &key, sizeof(key)) == 0) break;

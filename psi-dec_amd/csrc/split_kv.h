@@ -59,7 +59,17 @@ struct MapArgs {
     // position appended in this step is read from these rows instead of the page.
     const void* flat_k = nullptr;
     const void* flat_v = nullptr;
+    // Where a kernel reports a row that it could not compute (word i = bit i of PSI_HIP_DEVICE_ERR_*), and the
+    // number of polls after which a wave stops waiting for another wave's progress.
+    uint32_t* status = nullptr;
+    uint32_t wait_polls = kDefaultWaitPolls;
 };
+
+// Fills the two fields above from the context.
+inline void set_device_status(MapArgs* a, const psi_hip_ctx* ctx) {
+    a->status = ctx->status_device;
+    a->wait_polls = ctx->wait_polls != 0 ? ctx->wait_polls : kDefaultWaitPolls;
+}
 
 // First statement of every map kernel.
 __device__ __forceinline__ void resolve_active(MapArgs& a) {

@@ -72,8 +72,8 @@ __device__ __forceinline__ uint4 prob_operand_f16(const float (&p)[8]) {
     return __builtin_bit_cast(uint4, h);
 }
 
-// 8 elements of the storage type -> 8 f16.  bf16: widening is exact, the narrowing truncates (exact inside the
-// f16 range, see the header).
+// 8 elements of the storage type -> 8 f16.  bf16: widening is exact, the narrowing is exact inside the range of
+// f16's normal numbers (see the header).
 template <typename Tag>
 __device__ __forceinline__ u32x4_t to_f16x8(u32x4_t w);
 template <>
@@ -84,7 +84,8 @@ __device__ __forceinline__ u32x4_t to_f16x8<BF16Tag>(u32x4_t w) {
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
         const float lo = __uint_as_float(w[i] << 16), hi = __uint_as_float(w[i] & 0xffff0000u);
-        out[i] = __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_pkrtz(lo, hi));
+        const f16x2_t h = {(_Float16)lo, (_Float16)hi};  // to nearest: what f16 cannot hold becomes Inf
+        out[i] = __builtin_bit_cast(uint32_t, h);
     }
     return out;
 }
@@ -171,12 +172,21 @@ __global__ __launch_bounds__(64 * (kChunkWaves + kChunkLoaders), 1) void split_k
     if (tid < kChunkLoaders + kChunkWaves) landed[tid] = 0u;
     __syncthreads();
     // Both roles poll with the word of wave (lane % count) in each lane and a wave-wide vote.
-    auto wait_all_above = [&](LdsWords words, uint32_t count_mask, uint32_t value) __attribute__((always_inline)) {
-        for (uint32_t polls = 0; polls < (1u << 16); ++polls) {
-            if (__all(words[lane & count_mask] > value)) break;
+    // False when the wait ran out: the wave then reports it to the host and stops (a loading wave stores no more
+    // tiles, so the multiplying waves run out in turn; a multiplying wave stores empty states for its columns).
+    auto wait_all_above = [&](LdsWords words, uint32_t count_mask, uint32_t value) __attribute__((always_inline)) -> bool {
+        uint32_t polls = 0;
+        bool there = true;
+        while (!__all(words[lane & count_mask] > value)) {
+            if (++polls > a.wait_polls) {
+                there = false;
+                if (lane == 0) __hip_atomic_store(a.status, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
+                break;
+            }
             __builtin_amdgcn_s_sleep(1);
         }
         asm volatile("" ::: "memory");
+        return there;
     };
 
     if (wave >= (uint32_t)kChunkWaves) {
@@ -238,8 +248,10 @@ __global__ __launch_bounds__(64 * (kChunkWaves + kChunkLoaders), 1) void split_k
             k_store[i] = key * (D * 2) + ((ld_chunk ^ (key & 15)) * 16);
             v_store[i] = kKBytes + key * kVStride + ld_chunk * 16;
         }
+        bool stage_free = true;
         auto store_tile = [&](uint32_t it, Staging& st) __attribute__((always_inline)) {
-            if (it >= (uint32_t)kChunkStages) wait_all_above(done, kChunkWaves - 1, it - kChunkStages);
+            if (it >= (uint32_t)kChunkStages) stage_free = wait_all_above(done, kChunkWaves - 1, it - kChunkStages);
+            if (!stage_free) return;
             unsigned char* stage = lds + (it % kChunkStages) * kStageBytes;
             const uint32_t kb = key_base0 + it * kChunkKeys;
             const bool edge = kb < kv_begin || kb + kChunkKeys > kv_end_max;  // first or last tile of the range
@@ -269,7 +281,7 @@ __global__ __launch_bounds__(64 * (kChunkWaves + kChunkLoaders), 1) void split_k
             st = issue_loads(tile_bases(it + kChunkStages, ids));
             ids = fetch_ids(it + kChunkStages + 1);
         };
-        for (uint32_t it = 0; it < num_kv_tiles; it += 4) {
+        for (uint32_t it = 0; it < num_kv_tiles && stage_free; it += 4) {
             step(it, st_a);
             step(it + 1, st_b);
             step(it + 2, st_c);
@@ -310,8 +322,12 @@ __global__ __launch_bounds__(64 * (kChunkWaves + kChunkLoaders), 1) void split_k
     for (int db = 0; db < kDimBlocks; ++db) o[db] = f32x4_t{0.0f, 0.0f, 0.0f, 0.0f};
 
     constexpr int kAhead = 4;  // k-steps between an operand's read and its product
+    bool complete = true;
     for (uint32_t it = 0; it < my_tiles; ++it) {
-        wait_all_above(landed, kChunkLoaders - 1, it);
+        if (!wait_all_above(landed, kChunkLoaders - 1, it)) {
+            complete = false;
+            break;
+        }
         const unsigned char* kbuf = lds + (it % kChunkStages) * kStageBytes;
         const unsigned char* vbuf = kbuf + kKBytes;
         const uint32_t kb = key_base0 + it * kChunkKeys;
@@ -391,6 +407,23 @@ __global__ __launch_bounds__(64 * (kChunkWaves + kChunkLoaders), 1) void split_k
 
     lane_sum += __shfl_xor(lane_sum, 16, 64);
     lane_sum += __shfl_xor(lane_sum, 32, 64);
+    // A V element that f16 cannot hold has reached the accumulators as Inf or NaN (the conversion rounds to nearest,
+    // so that it overflows instead of saturating): the host is told, and the rows stay as they are, visibly wrong.
+    {
+        float probe = 0.0f;
+#pragma unroll
+        for (int db = 0; db < kDimBlocks; ++db)
+#pragma unroll
+            for (int r = 0; r < 4; ++r) probe = __builtin_fmaf(o[db][r], 0.0f, probe);
+        if (__any(lim != 0 && probe != probe) && lane == 0)
+            __hip_atomic_store(a.status + 1, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
+    }
+    if (!complete) {  // a wait ran out: empty states
+        run_max = -INFINITY;
+        lane_sum = 0.0f;
+#pragma unroll
+        for (int db = 0; db < kDimBlocks; ++db) o[db] = f32x4_t{0.0f, 0.0f, 0.0f, 0.0f};
+    }
     if (lim != 0) {
         if (mc == 0) {
             a.part_max[part_row] = run_max;

@@ -542,8 +542,8 @@ __device__ __forceinline__ void wait_load_groups(uint32_t groups) {
 // With three column blocks a fourth wave per SIMD would leave each 128 registers, less than a block's accumulators
 // and operands take, so one wave multiplies two blocks and the loading wave takes the third (which costs: the same
 // split at two blocks runs 10 % slower than the pure loader).  All of it is bounded: a wait on another wave's
-// progress gives up after 2^16 polls (the row's results are then wrong, which the parity tests see, but no wave
-// stays behind).
+// progress gives up after MapArgs::wait_polls polls; the row is then stored as an empty state and the host is
+// told through MapArgs::status, and no wave stays behind.
 // ---------------------------------------------------------------------------------------------------------------
 // Waves per stream of tiles: one that loads, and one that multiplies per column block; with three blocks (four waves
 // of a SIMD would have 128 registers each, which a column block's 64 accumulators and its operands do not fit
@@ -582,6 +582,7 @@ __global__ __launch_bounds__(64 * tiled_paired_waves(NB), 1) void split_kv_tiled
     __shared__ float col_sum_lds[kCols];
     // tiles of the row so far, per pair: [K landed, V landed, K read by the first wave, V read by the first wave]
     __shared__ uint32_t progress[2 + 2 * kMultipliers][kPairs];
+    __shared__ uint32_t row_failed;  // a wait of some wave ran out on the current row
     uint4* qb_lds = reinterpret_cast<uint4*>(lds_union + kStageBytes);  // [NB][kKSteps][64]
     float* merge = reinterpret_cast<float*>(lds_union);
 
@@ -607,8 +608,24 @@ __global__ __launch_bounds__(64 * tiled_paired_waves(NB), 1) void split_kv_tiled
     // what a multiplying wave reports; the loading wave waits for all of them
     const LdsWord read_k = word(2 + 2 * (second ? 0u : role));
     const LdsWord read_v = word(3 + 2 * (second ? 0u : role));
+    // A wait that runs out marks the row as failed (it is then stored as an empty state), reports it to the host,
+    // and is this wave's last wait on the row: the wave walks on without waiting, so that the waves that wait for
+    // its progress get through as well.
+    bool gave_up = false;
     auto wait_until_above = [&](LdsWord counter, uint32_t value) __attribute__((always_inline)) {
-        for (uint32_t polls = 0; *counter <= value && polls < (1u << 16); ++polls) __builtin_amdgcn_s_sleep(1);
+        if (gave_up) return;
+        uint32_t polls = 0;
+        while (*counter <= value) {
+            if (++polls > a.wait_polls) {
+                gave_up = true;
+                if ((threadIdx.x & 63) == 0) {
+                    row_failed = 1u;
+                    __hip_atomic_store(a.status, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
+                }
+                break;
+            }
+            __builtin_amdgcn_s_sleep(1);
+        }
         asm volatile("" ::: "memory");
     };
 
@@ -765,6 +782,8 @@ __global__ __launch_bounds__(64 * tiled_paired_waves(NB), 1) void split_kv_tiled
         }
     }
     if (tid < (2 + 2 * kMultipliers) * kPairs) (&progress[0][0])[tid] = 0;
+    if (tid == 0) row_failed = 0u;
+    gave_up = false;
     __syncthreads();
 
     // A operand of QK^T, k-step i: row mt, elements 32 * i + 8 * mc .. + 7 -> half mt / 8, line i / 2, chunk
@@ -1013,18 +1032,21 @@ __global__ __launch_bounds__(64 * tiled_paired_waves(NB), 1) void split_kv_tiled
     else
         walk_row(std::integral_constant<int, kBlocksEach>(), role * kBlocksEach, std::false_type());
 
-    // ---- emit: partial row of (split, q_head, token_in_tile); 1 KiB of contiguous f32 per wave store
+    // ---- emit: partial row of (split, q_head, token_in_tile); 1 KiB of contiguous f32 per wave store.  A row on
+    // which a wait ran out is stored as an empty state.
+    const bool failed = row_failed != 0u;  // written before the barriers of the merge
     const uint32_t rows = a.rows_per_split_head;
     for (uint32_t idx = tid; idx < ncols * (D / 4); idx += 64 * kWaves) {
         const uint32_t c = idx / (D / 4), d4 = idx % (D / 4);
         const uint64_t row = ((uint64_t)split * a.hq + (uint64_t)kv_head * G + c % G) * rows + c / G;
-        const float4 val = *reinterpret_cast<const float4*>(merge + c * kMergeStride + d4 * 4);
+        float4 val = *reinterpret_cast<const float4*>(merge + c * kMergeStride + d4 * 4);
+        if (failed) val = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
         *reinterpret_cast<float4*>(&a.part_acc[row * D + d4 * 4]) = val;
     }
     if (tid < ncols) {
         const uint64_t row = ((uint64_t)split * a.hq + (uint64_t)kv_head * G + tid % G) * rows + tid / G;
-        a.part_max[row] = col_max_lds[tid];
-        a.part_sum[row] = col_sum_lds[tid];
+        a.part_max[row] = failed ? -INFINITY : col_max_lds[tid];
+        a.part_sum[row] = failed ? 0.0f : col_sum_lds[tid];
     }
     }  // rows of this workgroup
 }

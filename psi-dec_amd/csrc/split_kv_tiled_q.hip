@@ -89,6 +89,7 @@ static int tiled_q_map(psi_hip_ctx* ctx, const psi_hip_gqa_config* cfg, const ps
     a.num_active_tokens = num_active_tokens;
     a.num_active_kv_splits = num_active_kv_splits;
     a.replay_counts = ctx->replay_counts;
+    set_device_status(&a, ctx);
     a.scale_log2 = g.scale * kLog2eTiled;
     a.q_token_tiles = q_token_tiles;
     a.flat_token_indices = flat_token_indices;

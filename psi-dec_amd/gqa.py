@@ -105,6 +105,17 @@ class Device:
         """Combine kernels then store f32 outputs (for checking the result before output rounding)."""
         L.check(self.lib.psi_hip_ctx_set_flag(self.ctx, L.FLAG_F32_OUTPUT, int(on)))
 
+    def wait_poll_limit(self, polls: int):
+        """Bound of every wait of one wave on another inside the multi-query and prefill-chunk maps (0: default)."""
+        L.check(self.lib.psi_hip_ctx_set_flag(self.ctx, L.FLAG_WAIT_POLL_LIMIT, int(polls)))
+
+    def take_device_error(self) -> int:
+        """Synchronises, then returns and clears the errors that kernels reported (`L.DEVICE_ERR_*` bits);
+        `sync()` raises while one is set."""
+        bits = ctypes.c_uint32()
+        L.check(self.lib.psi_hip_ctx_take_device_error(self.ctx, ctypes.byref(bits)))
+        return bits.value
+
     def close(self):
         if self.ctx:
             self.lib.psi_hip_ctx_destroy(self.ctx)
@@ -754,7 +765,7 @@ class GQAMetadataBuffers:
     def prepare(self, layer_struct, req_slots, token_indices, cu_tokens, capacity_mode=L.CAPACITY_EXACT,
                 partition_tokens: int = 0, dispatch: int = L.DISPATCH_PLAN_ORDER, num_workers: int = 0,
                 variant: Optional[GQASplitKVVariant] = None, policy: Optional[GQAReplayBucketPolicy] = None,
-                caller_num_total_tokens: int = 0) -> GQAReplayShape:
+                caller_num_total_tokens: int = 0, bucket_capacities: bool = False) -> GQAReplayShape:
         """One host call for the whole of a step's planning (psi_hip_gqa_layer_prepare): variant selection when
         `variant` is None, metadata update, dispatch plan; then one upload.  `layer_struct`: `GQA.struct()`."""
         self._staging_free()
@@ -765,7 +776,8 @@ class GQAMetadataBuffers:
         boundaries = L.u32_array(policy.token_topology_boundaries) if policy is not None else None
         options = L.PlanOptionsStruct(capacity_mode, partition_tokens, caller_num_total_tokens, dispatch, num_workers,
                                       policy.max_tokens() if policy is not None else 0, boundaries,
-                                      len(policy.token_topology_boundaries) if policy is not None else 0)
+                                      len(policy.token_topology_boundaries) if policy is not None else 0,
+                                      int(bucket_capacities))
         if dispatch == L.DISPATCH_ROW_GROUPS and self._row_groups_words() == 0:
             self._alloc_row_groups((self._max_kv_splits + self._max_workers) * 32)
         if self._host_struct is None or self._host_struct.row_groups_capacity != self._row_groups_words():
@@ -1306,14 +1318,19 @@ class GQA:
 
     def prepare_fixed_partition(self, batch_metadata, req_slots, token_indices, cu_tokens, partition_tokens: int,
                                 balanced: bool = True, grouped: bool = False,
-                                variant: Optional[GQASplitKVVariant] = None, num_workers: int = 0) -> GQAReplayShape:
+                                variant: Optional[GQASplitKVVariant] = None, num_workers: int = 0,
+                                bucket_capacities: bool = False,
+                                policy: Optional[GQAReplayBucketPolicy] = None) -> GQAReplayShape:
         """Not in the reference: partitions of fixed length instead of the greedy budget, then (by default) the
         balanced worker plan that gives every compute unit an equal share of the batch's tiles; `grouped`
-        selects the row-group plan of the prefill-chunk map instead.  One host call and one upload."""
+        selects the row-group plan of the prefill-chunk map instead.  One host call and one upload.
+        `bucket_capacities`: the recorded capacities (the re-cut row count included) are rounded up to
+        `ReplayBucketPolicy` buckets, so that a `GQAReplayCache` keeps one program per bucket."""
         dispatch = (L.DISPATCH_ROW_GROUPS if grouped else L.DISPATCH_BALANCED if balanced else L.DISPATCH_PLAN_ORDER)
         return batch_metadata.prepare(self.struct(), req_slots, token_indices, cu_tokens,
                                       capacity_mode=L.CAPACITY_FIXED_PARTITION, partition_tokens=partition_tokens,
-                                      dispatch=dispatch, num_workers=num_workers, variant=variant)
+                                      dispatch=dispatch, num_workers=num_workers, variant=variant,
+                                      bucket_capacities=bucket_capacities, policy=policy)
 
     def input_struct(self, inp: GQAInput):
         """(psi_hip_gqa_layer_input, keep-alive objects) for an input."""

@@ -131,3 +131,22 @@ def test_product_sources_never_touch_the_oracle():
                 if re.search(r"\boracle\b", src):
                     offenders.append(os.path.join(dirpath, f))
     assert not offenders, offenders
+
+
+def test_device_error_constants_and_argument_checks(psi):
+    """The device error bits and the poll-limit flag as the header numbers them; the entry point rejects null
+    arguments before it touches a GPU."""
+    import importlib
+
+    L = importlib.import_module("psi-dec_amd._lib")
+    text = open(os.path.join(ROOT, "include", "psi_hip.h")).read()
+    for name, value in (("PSI_HIP_DEVICE_ERR_WAIT_GAVE_UP", L.DEVICE_ERR_WAIT_GAVE_UP),
+                        ("PSI_HIP_DEVICE_ERR_V_RANGE", L.DEVICE_ERR_V_RANGE),
+                        ("PSI_HIP_FLAG_WAIT_POLL_LIMIT", L.FLAG_WAIT_POLL_LIMIT)):
+        m = re.search(rf"#define {name}\s+(\d+)u", text)
+        assert m and int(m.group(1)) == value, name
+    lib = psi.load()
+    bits = ctypes.c_uint32(5)
+    assert lib.psi_hip_ctx_take_device_error(None, ctypes.byref(bits)) == L.ERR_INVALID_ARGUMENT
+    assert bits.value == 5
+    assert b"must not be null" in lib.psi_hip_last_error()

@@ -287,3 +287,114 @@ def test_replay_cache_serves_buckets_and_matches_oracle(psi, oracle, device, q_l
     finally:
         device.f32_output(False)
         device.use_stream(main)
+
+
+def test_prepare_with_bucketed_capacities_feeds_the_replay_cache(psi, oracle, device):
+    """The one-call preparation with `bucket_capacities` gives the balanced plan's re-cut rows a bucketed capacity,
+    so that decode batches of varying size and length share recorded programs: twelve different batches, far fewer
+    recordings, every replay equal to the CPU oracle on its batch."""
+    import torch
+
+    wl = importlib_workloads(psi)
+    rng = np.random.default_rng(7)
+    ctx = rng.integers(30, 2500, size=10).tolist()
+    w = wl.make_workload(171, ctx, 24, 4, 256, psi.Dtype.Bfloat16, 16)
+    hq, hkv, d = w.num_q_heads, w.num_kv_heads, w.head_dim
+    row, kv_row = hq * d, hkv * d
+    max_tokens, max_splits, workers = 16, 96, 8
+    gqa = _layer(psi, device, w, gated=False)
+    meta = psi.GQAMetadataBuffers(device, max_tokens, max_kv_splits=max_splits, max_workers=workers)
+    scratch = gqa.new_scratch(max_tokens, max_splits + workers)
+    bf = dict(dtype=torch.bfloat16, device=device.torch_device)
+    q, k, v = torch.zeros(max_tokens * row, **bf), torch.zeros(max_tokens * kv_row, **bf), torch.zeros(max_tokens * kv_row, **bf)
+    out = torch.zeros(max_tokens * row, dtype=torch.float32, device=device.torch_device)
+    pristine = device.from_numpy(w.pages.reshape(-1)).view(torch.bfloat16)
+    pages = pristine.clone()
+    page_ids = device.from_numpy(w.page_ids)
+    side, main = torch.cuda.Stream(), device.stream
+    device.use_stream(side)
+    device.f32_output(True)
+    batches = 12
+    try:
+        cache = psi.GQAReplayCache(device, gqa)
+        for b in range(batches):
+            picks = sorted(rng.choice(len(ctx), size=int(rng.integers(1, len(ctx) + 1)), replace=False).tolist())
+            n = len(picks)
+            sub = dataclasses.replace(w, req_slots=w.req_slots[picks], token_indices=w.token_indices[picks],
+                                      cu_tokens=np.arange(n + 1, dtype=np.uint32),
+                                      q=w.q.reshape(-1, row)[picks].reshape(-1),
+                                      flat_k=w.flat_k.reshape(-1, kv_row)[picks].reshape(-1),
+                                      flat_v=w.flat_v.reshape(-1, kv_row)[picks].reshape(-1))
+            with torch.cuda.stream(side):
+                shape = gqa.prepare_fixed_partition(meta, sub.req_slots, sub.token_indices, sub.cu_tokens, 512,
+                                                    balanced=True, num_workers=workers, bucket_capacities=True)
+                assert shape.num_total_sdpa_map_task_templates >= shape.num_sdpa_map_task_templates
+                for dst, src in ((q, sub.q), (k, sub.flat_k), (v, sub.flat_v)):
+                    dst.zero_()
+                    dst[:src.size].copy_(device.from_numpy(src).view(torch.bfloat16))
+                pages.copy_(pristine)
+                out.fill_(-768.0)
+                inp = psi.GQAInput(w.layout, w.layer, meta, psi.GQAKVCacheBindings(pages, page_ids), scratch,
+                                   q=q, k=k, v=v, output=out)
+                cache.submit(inp)
+                side.synchronize()
+            exp_pages, exp = oracle_step(oracle, sub)
+            got = out.cpu().numpy()
+            assert_outputs_close(got[:n * row], exp, f"bucketed batch {b} {picks}")
+            assert (got[n * row:] == -768.0).all(), "rows beyond the active tokens were written"
+            assert np.array_equal(pages.view(torch.int16).cpu().numpy().view(np.uint16).reshape(exp_pages.shape), exp_pages)
+        programs, recordings, replays = cache.stats()
+        assert replays == batches and recordings == programs and recordings <= batches // 2, (recordings, batches)
+        cache.close()
+    finally:
+        device.f32_output(False)
+        device.use_stream(main)
+
+
+def test_replay_cache_records_again_when_a_context_flag_changes(psi, oracle, device):
+    """The output type of the combine (context flag F32_OUTPUT) is baked into a recorded program's arguments: a
+    submission after the flag has changed must record a new program, not replay the old one into a buffer of the
+    other element size."""
+    import torch
+
+    wl = importlib_workloads(psi)
+    w = wl.make_workload(172, [700, 33, 1500], 24, 4, 256, psi.Dtype.Bfloat16, 16)
+    row = w.num_q_heads * w.head_dim
+    gqa = _layer(psi, device, w, gated=False)
+    meta = psi.GQAMetadataBuffers(device, 8, max_kv_splits=32, max_workers=8)
+    scratch = gqa.new_scratch(8, 40)
+    q, k, v = (device.from_numpy(a.reshape(-1)).view(torch.bfloat16) for a in (w.q, w.flat_k, w.flat_v))
+    pages = device.from_numpy(w.pages.reshape(-1)).view(torch.bfloat16)
+    page_ids = device.from_numpy(w.page_ids)
+    # one buffer for both element sizes: f32 rows fill it, bf16 rows fill its first half
+    out = torch.zeros(w.num_tokens * row, dtype=torch.float32, device=device.torch_device)
+    side, main = torch.cuda.Stream(), device.stream
+    device.use_stream(side)
+    try:
+        cache = psi.GQAReplayCache(device, gqa)
+        _, exp = oracle_step(oracle, w)
+        results = []
+        for f32 in (True, False, True):
+            device.f32_output(f32)
+            with torch.cuda.stream(side):
+                gqa.prepare_fixed_partition(meta, w.req_slots, w.token_indices, w.cu_tokens, 512, balanced=True,
+                                            num_workers=8)
+                out.fill_(-768.0)
+                inp = psi.GQAInput(w.layout, w.layer, meta, psi.GQAKVCacheBindings(pages, page_ids), scratch,
+                                   q=q, k=k, v=v, output=out)
+                results.append(cache.submit(inp))
+                side.synchronize()
+            if f32:
+                assert_outputs_close(out.cpu().numpy(), exp, "f32 output")
+            else:
+                half = out.view(torch.bfloat16)
+                got = half[:w.num_tokens * row].to(torch.float32).cpu().numpy()
+                assert np.abs(got - exp).max() <= 2e-2
+                assert (out[w.num_tokens * row // 2:] == -768.0).all(), "a bf16 program wrote beyond its rows"
+        assert results == [True, True, False]
+        programs, recordings, replays = cache.stats()
+        assert (programs, recordings, replays) == (2, 2, 3)
+        cache.close()
+    finally:
+        device.f32_output(False)
+        device.use_stream(main)

@@ -664,6 +664,59 @@ def test_single_call_prepare_equals_the_step_by_step_plan(psi, seed):
             assert b.max_active_q_tile_tokens == min(int(q_lens.max()), variant.q_token_tile_size)
 
 
+@pytest.mark.parametrize("dispatch_name", ["plan", "balanced", "groups"])
+def test_prepare_buckets_the_dispatch_plans_capacities(psi, dispatch_name):
+    """With `bucket_capacities` the one-call preparation rounds the recorded capacities - tokens, Q-token tiles,
+    KV splits (the re-cut rows of a balanced plan) and row groups - up to `ReplayBucketPolicy` buckets
+    (crates/inference-executor-core/src/replay.rs:4-87) and pads the tables with the sentinel up to them: many
+    different batches then share few (capacity) keys, and the active part of every array is what the unbucketed
+    preparation writes."""
+    import importlib
+
+    L = importlib.import_module("psi-dec_amd._lib")
+    MAX = 0xFFFFFFFF
+    core = psi.GQACore(0, 24 * 256, 256, 24, 4, 0.0625)
+    gqa = psi.GQA(None, core, psi.GQAMetalConfig(65536, 64, 1e-6, 1e6))
+    max_tokens, max_splits, workers = 256, 512, 8
+    dispatch = {"plan": L.DISPATCH_PLAN_ORDER, "balanced": L.DISPATCH_BALANCED, "groups": L.DISPATCH_ROW_GROUPS}[dispatch_name]
+    tiled = dispatch_name == "groups"
+    variant = psi.GQASplitKVVariant.TiledQ(8, 16, 6) if tiled else psi.GQASplitKVVariant.SingleQ(256, 256, 6)
+    token_policy, split_policy = psi.ReplayBucketPolicy(max_tokens), psi.ReplayBucketPolicy(max_splits + workers)
+    rng = np.random.default_rng(77)
+    keys, exact_keys = set(), set()
+    for _ in range(40):
+        n = int(rng.integers(1, 12))
+        q_lens = rng.integers(9, 20, size=n) if tiled else np.ones(n, dtype=np.int64)
+        starts = rng.integers(0, 3000, size=n).astype(np.uint32)
+        slots = rng.permutation(16)[:n].astype(np.uint32)
+        cu = np.concatenate([[0], np.cumsum(q_lens)]).astype(np.uint32)
+        plain = psi.GQAMetadataBuffers(None, max_tokens, max_kv_splits=max_splits, max_workers=workers)
+        plain.prepare(gqa.struct(), slots, starts, cu, capacity_mode=L.CAPACITY_FIXED_PARTITION, partition_tokens=256,
+                      dispatch=dispatch, num_workers=workers, variant=variant)
+        md = psi.GQAMetadataBuffers(None, max_tokens, max_kv_splits=max_splits, max_workers=workers)
+        md.h_kv_splits[:] = 0x5A5A5A5A
+        s = md.prepare(gqa.struct(), slots, starts, cu, capacity_mode=L.CAPACITY_FIXED_PARTITION, partition_tokens=256,
+                       dispatch=dispatch, num_workers=workers, variant=variant, bucket_capacities=True)
+        e = plain.replay_shape()
+        assert (s.num_tokens, s.num_q_token_tiles, s.num_sdpa_map_task_templates) == \
+               (e.num_tokens, e.num_q_token_tiles, e.num_sdpa_map_task_templates)
+        assert s.num_total_tokens == token_policy.capacity(s.num_tokens)
+        assert s.num_total_q_token_tiles == token_policy.capacity(s.num_q_token_tiles)
+        assert s.num_total_sdpa_map_task_templates == split_policy.capacity(s.num_sdpa_map_task_templates)
+        rows, total = s.num_sdpa_map_task_templates, s.num_total_sdpa_map_task_templates
+        assert md._h_kv_splits_all[:3 * rows].tolist() == plain._h_kv_splits_all[:3 * rows].tolist()
+        assert (md._h_kv_splits_all[3 * rows:3 * total] == MAX).all()
+        if tiled:
+            assert md.num_row_groups >= plain.num_row_groups > 0 and md.group_tiles == plain.group_tiles
+            used = plain.num_row_groups * plain.group_tiles
+            assert md.h_row_groups[:used].tolist() == plain.h_row_groups[:used].tolist()
+            assert (md.h_row_groups[used:md.num_row_groups * md.group_tiles] == MAX).all()
+        keys.add((s.num_total_tokens, s.num_total_q_token_tiles, total, md.num_row_groups))
+        exact_keys.add((e.num_total_tokens, e.num_total_q_token_tiles, e.num_total_sdpa_map_task_templates,
+                        plain.num_row_groups))
+    assert len(keys) < len(exact_keys) and (tiled or len(keys) <= 20), (len(keys), len(exact_keys))
+
+
 @pytest.mark.parametrize("balanced", [False, True])
 def test_advance_decode_equals_a_fresh_preparation(psi, balanced):
     """psi_hip_gqa_layer_advance_decode moves a decode batch's plan on by one token per sequence in place.  Over 60
