@@ -114,10 +114,10 @@ int psi_hip_ctx_reset_timing(psi_hip_ctx* ctx);
 /* F32_OUTPUT makes the combine kernels store the attention output as f32 [tokens, Hq, D] instead of
  * the io dtype, so a harness can check the f32-accumulated result before output rounding. */
 #define PSI_HIP_FLAG_F32_OUTPUT 2u
-/* WAIT_POLL_LIMIT bounds every wait of one wave on another wave's progress inside the multi-query and
- * prefill-chunk maps: `value` polls (0 restores the default, 65536).  A wait that runs out sets
- * PSI_HIP_DEVICE_ERR_WAIT_GAVE_UP below.  A harness sets a limit of 1 to see that path taken. */
-#define PSI_HIP_FLAG_WAIT_POLL_LIMIT 3u
+/* MUTE_LOADERS is for harnesses: while it is set, the loading waves of the multi-query and prefill-chunk maps never
+ * say that a tile has landed, so that the other waves' waits (bounded at 65536 polls) run out, which sets
+ * PSI_HIP_DEVICE_ERR_WAIT_GAVE_UP below while every kernel still runs to its end. */
+#define PSI_HIP_FLAG_MUTE_LOADERS 3u
 int psi_hip_ctx_set_flag(psi_hip_ctx* ctx, uint32_t flag, uint32_t value);
 
 /* Errors a kernel found while it ran.  The reference has no counterpart: its Metal kernels have no

@@ -22,7 +22,7 @@ VARIANT_SINGLE_Q, VARIANT_TILED_Q = 0, 1
 CAPACITY_EXACT, CAPACITY_BUCKETED, CAPACITY_CALLER_TOKENS, CAPACITY_FIXED_PARTITION = 0, 1, 2, 3
 FLAG_FORCE_GENERIC = 1
 FLAG_F32_OUTPUT = 2
-FLAG_WAIT_POLL_LIMIT = 3
+FLAG_MUTE_LOADERS = 3
 DEVICE_ERR_WAIT_GAVE_UP = 1
 DEVICE_ERR_V_RANGE = 2
 REPLAY_EXACT, REPLAY_BUCKETED = 0, 1

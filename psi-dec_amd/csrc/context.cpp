@@ -179,7 +179,7 @@ int psi_hip_ctx_set_flag(psi_hip_ctx* ctx, uint32_t flag, uint32_t value) {
     switch (flag) {
         case PSI_HIP_FLAG_FORCE_GENERIC: ctx->force_generic = value != 0; break;
         case PSI_HIP_FLAG_F32_OUTPUT: ctx->f32_output = value != 0; break;
-        case PSI_HIP_FLAG_WAIT_POLL_LIMIT: ctx->wait_polls = value; break;
+        case PSI_HIP_FLAG_MUTE_LOADERS: ctx->mute_loaders = value != 0; break;
         default: return psi::fail(PSI_HIP_ERR_INVALID_ARGUMENT, "unknown context flag %u", flag);
     }
     return PSI_HIP_OK;

@@ -231,7 +231,7 @@ struct ProgramKey {
     uint32_t layer, replay_mode, layer_is_parameter;
     uint32_t num_workers, group_tiles, num_row_groups, max_active_q_tile_tokens;
     // context state that ends up in kernel arguments or decides which kernel runs
-    uint32_t f32_output, force_generic, wait_polls;
+    uint32_t f32_output, force_generic, mute_loaders;
     uint64_t kv_pages_bytes, partial_scratch_bytes;
     const void* pointers[21];
 };
@@ -254,7 +254,7 @@ ProgramKey make_key(const psi_hip_ctx& ctx, const psi_hip_gqa_layer_input& in, b
     k.max_active_q_tile_tokens = md.max_active_q_tile_tokens;
     k.f32_output = ctx.f32_output;
     k.force_generic = ctx.force_generic;
-    k.wait_polls = ctx.wait_polls;
+    k.mute_loaders = ctx.mute_loaders;
     k.kv_pages_bytes = in.kv_pages_bytes;
     k.partial_scratch_bytes = in.partial_scratch_bytes;
     const void* p[21] = {in.qgkv, in.q, in.k, in.v, in.g, in.kv_pages, in.page_ids, in.q_norm_weight,

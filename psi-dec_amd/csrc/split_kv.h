@@ -59,16 +59,17 @@ struct MapArgs {
     // position appended in this step is read from these rows instead of the page.
     const void* flat_k = nullptr;
     const void* flat_v = nullptr;
-    // Where a kernel reports a row that it could not compute (word i = bit i of PSI_HIP_DEVICE_ERR_*), and the
-    // number of polls after which a wave stops waiting for another wave's progress.
+    // Where a kernel reports a row that it could not compute (word i = bit i of PSI_HIP_DEVICE_ERR_*); and, for
+    // harnesses, non-zero: the loading waves of the multi-query and prefill-chunk maps do not say that their tiles
+    // have landed, so that the other waves' waits run out.
     uint32_t* status = nullptr;
-    uint32_t wait_polls = kDefaultWaitPolls;
+    uint32_t mute_loaders = 0;
 };
 
 // Fills the two fields above from the context.
 inline void set_device_status(MapArgs* a, const psi_hip_ctx* ctx) {
     a->status = ctx->status_device;
-    a->wait_polls = ctx->wait_polls != 0 ? ctx->wait_polls : kDefaultWaitPolls;
+    a->mute_loaders = ctx->mute_loaders ? 1u : 0u;
 }
 
 // First statement of every map kernel.
@@ -147,11 +148,13 @@ inline uint32_t chunk_group_tiles(uint32_t group, uint32_t q_token_tile_size) {
     const uint32_t tiles = (uint32_t)kChunkCols / (heads * q_token_tile_size);
     return tiles > 32 ? 32u : tiles;
 }
-// True when the prefill-chunk map covers the geometry (2-byte elements, head_dim 256, pages of 16*2^k tokens).
+// True when the prefill-chunk map covers the geometry: 2-byte elements, head_dim 128 or 256, pages of 8 * 2^k tokens
+// (the reference's TiledQ profiles (128, 8), (256, 8), (256, 16) among them,
+// crates/inference-backend-metal/src/components/gqa_split_kv_tiled_q.rs:66-76).
 inline bool chunk_map_supported(const Geometry& g, uint32_t q_token_tile_size) {
     const uint32_t p = g.tokens_per_page;
-    return (g.dtype == PSI_HIP_BF16 || g.dtype == PSI_HIP_F16) && g.d == 256 && p >= 16 && (p & (p - 1)) == 0 &&
-           q_token_tile_size > 0 && chunk_group_tiles(g.group, q_token_tile_size) >= 1;
+    return (g.dtype == PSI_HIP_BF16 || g.dtype == PSI_HIP_F16) && (g.d == 256 || g.d == 128) && p >= 8 &&
+           (p & (p - 1)) == 0 && q_token_tile_size > 0 && chunk_group_tiles(g.group, q_token_tile_size) >= 1;
 }
 
 // Shape-generic kernels (any head_dim / page size / element type), SingleQ and TiledQ layouts.

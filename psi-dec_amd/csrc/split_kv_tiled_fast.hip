@@ -13,6 +13,10 @@ int launch_chunk_map_bf16_d256(psi_hip_ctx* ctx, const Geometry& g, const MapArg
                                uint32_t group_tiles, uint32_t num_groups);
 int launch_chunk_map_f16_d256(psi_hip_ctx* ctx, const Geometry& g, const MapArgs& a, const uint32_t* row_groups,
                               uint32_t group_tiles, uint32_t num_groups);
+int launch_chunk_map_bf16_d128(psi_hip_ctx* ctx, const Geometry& g, const MapArgs& a, const uint32_t* row_groups,
+                               uint32_t group_tiles, uint32_t num_groups);
+int launch_chunk_map_f16_d128(psi_hip_ctx* ctx, const Geometry& g, const MapArgs& a, const uint32_t* row_groups,
+                              uint32_t group_tiles, uint32_t num_groups);
 
 int launch_chunk_map(psi_hip_ctx* ctx, const Geometry& g, const MapArgs& a, const uint32_t* row_groups,
                      uint32_t group_tiles, uint32_t num_groups) {
@@ -20,6 +24,9 @@ int launch_chunk_map(psi_hip_ctx* ctx, const Geometry& g, const MapArgs& a, cons
     const bool aligned = reinterpret_cast<uintptr_t>(a.q) % 16 == 0 && reinterpret_cast<uintptr_t>(a.kv_pages) % 16 == 0;
     if (!aligned || group_tiles == 0 || group_tiles > chunk_group_tiles(g.group, a.rows_per_split_head)) return PSI_HIP_ERR_UNSUPPORTED;
     if ((uint64_t)num_groups * g.hkv * chunk_head_subsets(g.group) > 0x7fffffffull) return PSI_HIP_ERR_UNSUPPORTED;
+    if (g.d == 128)
+        return g.dtype == PSI_HIP_BF16 ? launch_chunk_map_bf16_d128(ctx, g, a, row_groups, group_tiles, num_groups)
+                                       : launch_chunk_map_f16_d128(ctx, g, a, row_groups, group_tiles, num_groups);
     return g.dtype == PSI_HIP_BF16 ? launch_chunk_map_bf16_d256(ctx, g, a, row_groups, group_tiles, num_groups)
                                    : launch_chunk_map_f16_d256(ctx, g, a, row_groups, group_tiles, num_groups);
 }

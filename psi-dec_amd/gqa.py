@@ -105,9 +105,11 @@ class Device:
         """Combine kernels then store f32 outputs (for checking the result before output rounding)."""
         L.check(self.lib.psi_hip_ctx_set_flag(self.ctx, L.FLAG_F32_OUTPUT, int(on)))
 
-    def wait_poll_limit(self, polls: int):
-        """Bound of every wait of one wave on another inside the multi-query and prefill-chunk maps (0: default)."""
-        L.check(self.lib.psi_hip_ctx_set_flag(self.ctx, L.FLAG_WAIT_POLL_LIMIT, int(polls)))
+    def mute_loaders(self, on: bool):
+        """For harnesses: the loading waves of the multi-query and prefill-chunk maps never say that a tile has
+        landed, so that the other waves' bounded waits run out and the device error path runs, while every kernel
+        still ends normally."""
+        L.check(self.lib.psi_hip_ctx_set_flag(self.ctx, L.FLAG_MUTE_LOADERS, int(on)))
 
     def take_device_error(self) -> int:
         """Synchronises, then returns and clears the errors that kernels reported (`L.DEVICE_ERR_*` bits);

@@ -142,7 +142,7 @@ def test_device_error_constants_and_argument_checks(psi):
     text = open(os.path.join(ROOT, "include", "psi_hip.h")).read()
     for name, value in (("PSI_HIP_DEVICE_ERR_WAIT_GAVE_UP", L.DEVICE_ERR_WAIT_GAVE_UP),
                         ("PSI_HIP_DEVICE_ERR_V_RANGE", L.DEVICE_ERR_V_RANGE),
-                        ("PSI_HIP_FLAG_WAIT_POLL_LIMIT", L.FLAG_WAIT_POLL_LIMIT)):
+                        ("PSI_HIP_FLAG_MUTE_LOADERS", L.FLAG_MUTE_LOADERS)):
         m = re.search(rf"#define {name}\s+(\d+)u", text)
         assert m and int(m.group(1)) == value, name
     lib = psi.load()

@@ -3,7 +3,7 @@
 Two conditions, neither of which the reference has (its Metal kernels have no waits between simdgroups, and they
 multiply V in the storage type):
   * a wave's bounded wait on another wave of its workgroup runs out (multi-query and prefill-chunk maps).  The
-    tests force it from the host with a poll limit of 1, so that every kernel still runs to its end;
+    tests force it from the host (the loading waves never say that a tile has landed), so that every kernel still runs to its end;
   * the prefill-chunk map multiplies V as f16 and meets a bf16 value that f16 cannot hold.
 Either way `sync()` must fail, `take_device_error()` must name the condition and clear it, no stale or half
 computed row may reach the output, and the same batch must then run clean."""
@@ -46,14 +46,14 @@ def test_a_wait_that_runs_out_is_reported(psi, oracle, device, kind):
     _, exp = oracle_step(oracle, w)
     assert device.take_device_error() == 0
     dw.scratch.buffer.view(torch.float32).fill_(7.0)  # stale partial states: finite, plausible
-    device.wait_poll_limit(1)
+    device.mute_loaders(True)
     try:
         dw.step()
         with pytest.raises(psi.PsiHipError, match="bounded wait"):
             device.sync()
         assert device.take_device_error() & L.DEVICE_ERR_WAIT_GAVE_UP
     finally:
-        device.wait_poll_limit(0)
+        device.mute_loaders(False)
     device.sync()  # taken: clean again
     got = dw.output_f32().reshape(w.num_tokens, -1)
     assert np.isfinite(got).all()

@@ -306,29 +306,35 @@ def test_grouped_long_unsplit_range(psi, oracle, device):
     print("long range max_abs %.3e rel_rms %.3e" % stats, dw.shape, dw.meta.num_row_groups)
 
 
-@pytest.mark.parametrize("dtype_name,hq,hkv,p,q_len", [
-    ("Float16", 16, 2, 16, 50),    # 8 heads per KV head: two head subsets of 4, f16 single-term P
-    ("Bfloat16", 4, 4, 32, 130),   # one head per KV head: 16 tiles per group, 32-token pages
-    ("Bfloat16", 10, 2, 64, 41),   # 5 heads per KV head: one subset, 3 tiles per group
-    ("Bfloat16", 14, 2, 16, 23),   # 7 heads: subsets of 4 and 3
+@pytest.mark.parametrize("dtype_name,hq,hkv,d,p,q_len", [
+    ("Float16", 16, 2, 256, 16, 50),    # 8 heads per KV head: two head subsets of 4, f16 single-term P
+    ("Bfloat16", 4, 4, 256, 32, 130),   # one head per KV head: 16 tiles per group, 32-token pages
+    ("Bfloat16", 10, 2, 256, 64, 41),   # 5 heads per KV head: one subset, 3 tiles per group
+    ("Bfloat16", 14, 2, 256, 16, 23),   # 7 heads: subsets of 4 and 3
+    # the reference's TiledQ profiles (crates/inference-backend-metal/src/components/gqa_split_kv_tiled_q.rs:66-76)
+    ("Bfloat16", 24, 4, 256, 8, 77),    # (256, 8): a 32-key tile spans four pages
+    ("Bfloat16", 32, 8, 128, 8, 90),    # (128, 8), the heads of the reference's Criterion bench
+    ("Bfloat16", 40, 8, 128, 8, 61),    # (128, 8), the heads of its published timing: 5 per KV head
+    ("Bfloat16", 32, 8, 128, 16, 130),  # head_dim 128 on 16-token pages
+    ("Float16", 16, 2, 128, 32, 35),    # head_dim 128, f16, 8 heads per KV head
 ])
-def test_grouped_geometries(psi, oracle, device, dtype_name, hq, hkv, p, q_len):
+def test_grouped_geometries(psi, oracle, device, dtype_name, hq, hkv, d, p, q_len):
     wl = importlib_workloads(psi)
     dtype = getattr(psi.Dtype, dtype_name)
-    w = wl.make_workload(93, [300, 31 + q_len, q_len], hq, hkv, 256, dtype, p, q_lens=[q_len, q_len, q_len],
+    w = wl.make_workload(93, [300, 31 + q_len, q_len], hq, hkv, d, dtype, p, q_lens=[q_len, q_len, q_len],
                          num_page_ids_per_block=2)
     variant = psi.GQASplitKVVariant.TiledQ(8, 16, min(hq // hkv, 8))
-    _, dw = run_and_check(psi, oracle, device, w, f"grouped {dtype_name} {hq}/{hkv} P={p} q={q_len}", max_tokens=512,
-                          variant=variant, partition_tokens=128, grouped=True)
+    _, dw = run_and_check(psi, oracle, device, w, f"grouped {dtype_name} {hq}/{hkv}/{d} P={p} q={q_len}",
+                          max_tokens=512, variant=variant, partition_tokens=128, grouped=True)
     assert dw.meta.num_row_groups > 0
 
 
 def test_grouped_and_plain_maps_agree(psi, oracle, device):
     """Same plan through both maps: the outputs differ only in rounding, the grouped table falls
-    back to the plain map where the geometry has no grouped kernel (8-token pages)."""
+    back to the plain map where the geometry has no grouped kernel (head_dim 64)."""
     wl = importlib_workloads(psi)
-    for p, expect_groups in [(16, True), (8, False)]:
-        w = wl.make_workload(95, [900, 450], 24, 4, 256, psi.Dtype.Bfloat16, p, q_lens=[300, 450])
+    for d, p, expect_groups in [(256, 16, True), (256, 8, True), (128, 8, True), (64, 16, False)]:
+        w = wl.make_workload(95, [900, 450], 24, 4, d, psi.Dtype.Bfloat16, p, q_lens=[300, 450])
         outs = []
         for grouped in (False, True):
             dw = wl.DeviceWorkload(device, w, partition_tokens=256, max_tokens=1024, f32_output=True, grouped=grouped,

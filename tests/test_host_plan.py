@@ -573,9 +573,12 @@ def test_row_groups_unsupported_geometry_and_greedy_plan(psi):
     meta = psi.GQAMetadataBuffers(None, 64)
     variant = psi.GQASplitKVVariant.TiledQ(8, 16, 4)
     shape = meta.update([0, 1], [100, 7], [0, 20, 24], variant)
-    # head_dim 128 and 8-token pages have no grouped kernel
-    assert meta.group_rows(tiled_config(psi, 8, 2, d=128)) == 0 and meta.group_tiles == 0
-    assert meta.group_rows(tiled_config(psi, 8, 2, p=8)) == 0
+    # head_dim 64, 4-token pages and f32 storage have no grouped kernel; the reference's TiledQ profiles
+    # (128, 8), (256, 8), (256, 16) (gqa_split_kv_tiled_q.rs:66-76) do
+    assert meta.group_rows(tiled_config(psi, 8, 2, d=64)) == 0 and meta.group_tiles == 0
+    assert meta.group_rows(tiled_config(psi, 8, 2, p=4)) == 0
+    assert meta.group_rows(tiled_config(psi, 8, 2, d=128, p=8)) > 0
+    assert meta.group_rows(tiled_config(psi, 8, 2, p=8)) > 0
     # the reference's greedy plan cuts every tile differently: groups degenerate but stay complete
     assert meta.group_rows(tiled_config(psi, 8, 2)) > 0
     check_groups(meta, shape, 8, 4)
