@@ -9,9 +9,13 @@ launch).  Headline workload (`C2`): batch 32, contexts uniform in [1024, 8192], 
 Prints ONE JSON line.  Top level = the headline workload: `value` is the achieved HBM bandwidth of the whole
 layer-step (algorithmic bytes / wall time), `us_per_layer_step` the time itself; `roofline` prices the dominant
 kernel (the split-KV map) against the 8 TB/s HBM3E peak from HIP events on the launch stream; `cpu_baseline` times
-the scalar CPU oracle on a bounded sample of the same workload on this box's host cores.  `configs` carries the
-same figures for the other benchmark configurations (C1, C3, C4 with one and three drafts, C5's decode side, its
-prefill chunk, and the mixed step), each timed in this run with the same step and warm-up counts.
+the scalar CPU oracle on a bounded sample of the same workload on this box's host cores (`cpu_baseline_openmp`: the
+same sample on all of them).  `configs` carries the same figures for the other benchmark configurations (C1, the
+headline batch with one workgroup per 512-token partition row, the headline's shape at batch 4 / 8 / 16, C3, C4 with
+one, three and seven drafts, C5's decode side, its prefill chunk, and the mixed step) and for the shapes the
+reference itself times (`REF_*`), each timed in this run with the same step and warm-up counts.  Every workload
+also carries a `cold` figure (the first steps after set-up), and every HBM roofline the read bandwidth of a bare
+page stream measured in the same run (`measured_stream_GBps`, `frac_of_measured_stream`).
 
 Clocks.  `ms_per_step` / `us_per_layer_step`: host wall clock around K queued steps, device synchronised on both
 sides -- steps run back to back, as the layers of a decoder do.  `us_per_layer_step_p10_median_p90`: a HIP event
@@ -34,7 +38,17 @@ sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBPS = 8000.0
 MFMA_BF16_PEAK_TFLOPS = 2500.0
-CONFIG_NAMES = ["C1", "C3", "C4_q2", "C4_q4", "C4_q8", "C5_decode", "C5_prefill", "C5_mixed"]
+CONFIG_NAMES = ["C1", "C2_rows512", "C2_b4", "C2_b8", "C2_b16", "C3", "C4_q2", "C4_q4", "C4_q8", "C5_decode", "C5_prefill",
+                "C5_mixed", "GENERIC_f32_b8"]
+# The shapes the reference itself times (the only figures it publishes for these kernels, on an Apple M3 Max):
+#   REF_tiled      "SplitKV TiledQ only", 40 Q / 8 KV heads, head_dim 128, 8-token pages, one request with 8 new tokens
+#                  on 128 cached ones: 0.319 ms median, map + reduce (docs/qwen3_dspark_design_draft.md:1453-1458, the
+#                  command at :1470-1477)
+#   REF_criterion  its Criterion bench of the decode kernels, map + reduce per iteration, no recorded result: 32 / 8
+#                  heads, head_dim 128, 16-token pages, contexts 128 / 1024 / 2048 / 4096 and the ragged batch
+#                  7 x 128 + 1 x 4096 (crates/inference-backend-metal/benches/gqa/split_kv.rs:19-27,44)
+REF_NAMES = ["REF_tiled", "REF_criterion_ctx128", "REF_criterion_ctx1024", "REF_criterion_ctx2048",
+             "REF_criterion_ctx4096", "REF_criterion_ragged"]
 
 
 def parse_args():
@@ -43,7 +57,8 @@ def parse_args():
     p.add_argument("--steps", type=int, default=200)
     p.add_argument("--warmup", type=int, default=20)
     p.add_argument("--only", default=None,
-                   help="time one workload only: C2 (the headline), " + ", ".join(CONFIG_NAMES) + ", or `custom`")
+                   help="time one workload only: C2 (the headline), " + ", ".join(CONFIG_NAMES + REF_NAMES) +
+                        ", or `custom`")
     p.add_argument("--no-configs", action="store_true", help="headline workload only")
     p.add_argument("--kernel-only", action="store_true", help="time only the map kernel (for profiling runs)")
     p.add_argument("--cpu-seconds", type=float, default=12.0, help="budget of the CPU baseline sample")
@@ -56,7 +71,10 @@ def parse_args():
     p.add_argument("--q-heads", type=int, default=24)
     p.add_argument("--kv-heads", type=int, default=4)
     p.add_argument("--q-len", type=int, default=1, help="custom workload: new tokens per sequence")
-    p.add_argument("--dtype", choices=["bf16", "f16"], default="bf16")
+    p.add_argument("--head-dim", type=int, default=256, help="custom workload: head_dim")
+    p.add_argument("--page-tokens", type=int, default=16, help="custom workload: tokens per page")
+    p.add_argument("--dtype", choices=["bf16", "f16", "f32"], default="bf16",
+                   help="custom workload: element type (f32 runs the shape-generic kernels)")
     p.add_argument("--partition", type=int, default=512)
     p.add_argument("--arenas", type=int, default=0, help="page arenas rotated between steps (0 = per workload)")
     p.add_argument("--identity-pages", action="store_true", help="unshuffled page pool (diagnostic)")
@@ -106,6 +124,7 @@ class Case:
         self.name, self.key, self.arenas, self.kind = name, key, arenas, kind
         self.map_kernel, self.roof_kernel, self.description = map_kernel, roof_kernel, description
         self.flops = None  # per map launch, for MFMA-priced workloads
+        self.submit_and_wait = False  # also time every step with a synchronisation after it
 
 
 def build_case(psi, wl, device, name, args):
@@ -117,44 +136,90 @@ def build_case(psi, wl, device, name, args):
     verify_how = dict(balanced=not args.row_per_workgroup, longest_first=not args.plan_order,
                       num_workers=args.workers or None)
 
-    def decode_case(key, ctxs, hq, hkv, dtype, partition, arenas, seed, kernel="split_kv_decode_map", **kw):
+    def decode_case(key, ctxs, hq, hkv, dtype, partition, arenas, seed, kernel="split_kv_decode_map", d=256, p=16,
+                    how=None, **kw):
         out = []
         for i in range(arenas):
-            w = wl.make_workload(seed, ctxs, hq, hkv, 256, dtype, 16, host_pages=False,
+            w = wl.make_workload(seed, ctxs, hq, hkv, d, dtype, p, host_pages=False,
                                  shuffle_pages=not args.identity_pages, **kw)
             w.seed = seed + 1000 * i  # same geometry, different page contents
-            out.append(wl.DeviceWorkload(device, w, partition_tokens=partition, **decode_how))
+            out.append(wl.DeviceWorkload(device, w, partition_tokens=partition, **(how or decode_how)))
         return Case(name, key, out, "decode", "split_kv_map", kernel, "kv append + split-KV map (one launch) -> LSE combine")
 
-    def verify_case(key, ctxs, q_len, partition, arenas, seed):
+    def verify_case(key, ctxs, q_len, partition, arenas, seed, hq=24, hkv=4, d=256, p=16, dtype=bf16, variant=None):
         out = []
         for i in range(arenas):
-            w = wl.make_workload(seed, ctxs, 24, 4, 256, bf16, 16, q_lens=q_len, host_pages=False,
+            w = wl.make_workload(seed, ctxs, hq, hkv, d, dtype, p, q_lens=q_len, host_pages=False,
                                  shuffle_pages=not args.identity_pages)
             w.seed = seed + 1000 * i
-            out.append(wl.DeviceWorkload(device, w, partition_tokens=partition, **verify_how))
+            out.append(wl.DeviceWorkload(device, w, partition_tokens=partition, variant=variant, **verify_how))
         return Case(name, key, out, "verify", "tiled_q_map", "split_kv_tiled_map",
                     "kv append -> multi-query split-KV map -> LSE combine")
+
+    def map_and_reduce_only(case):
+        """The reference's own benches time the map and the reduce of an attention whose K/V are already in the
+        pages: the step of such a case is those two launches."""
+        for dw in case.arenas:
+            dw.append()  # once, so that the pages hold the new tokens' K/V
+            dw.step = (lambda d: lambda: (d.map(), d.reduce()))(dw)
+        case.description = "split-KV map -> LSE combine (the new tokens' K/V already in their pages)"
+        case.submit_and_wait = True
+        return case
 
     if name == "C2":
         ctx = wl.config_c2_context_lens(args.seed, 32, 1024, 8192) + 1
         key = f"decode_b32_ctx1024-8192_24q4kv_d256_bf16_p16_part{args.partition}_seed{args.seed}"
         return decode_case(key, ctx, 24, 4, bf16, args.partition, args.arenas or 2, args.seed)
     if name == "custom":
-        elem = bf16 if args.dtype == "bf16" else psi.Dtype.Float16
+        elem = {"bf16": bf16, "f16": psi.Dtype.Float16, "f32": psi.Dtype.Float32}[args.dtype]
+        d, p = args.head_dim, args.page_tokens
         ctx = wl.config_c2_context_lens(args.seed, args.batch, args.ctx_lo, args.ctx_hi) + args.q_len
         key = (f"{'decode' if args.q_len == 1 else 'verify_q%d' % args.q_len}_b{args.batch}_ctx{args.ctx_lo}-{args.ctx_hi}"
-               f"_{args.q_heads}q{args.kv_heads}kv_d256_{args.dtype}_p16_part{args.partition}_seed{args.seed}")
+               f"_{args.q_heads}q{args.kv_heads}kv_d{d}_{args.dtype}_p{p}_part{args.partition}_seed{args.seed}")
+        fast = elem != psi.Dtype.Float32 and d in (128, 256) and p >= 8 and p & (p - 1) == 0 and \
+            args.q_heads // args.kv_heads <= 8
         if args.q_len == 1:
-            return decode_case(key, ctx, args.q_heads, args.kv_heads, elem, args.partition, args.arenas or 2, args.seed)
+            return decode_case(key, ctx, args.q_heads, args.kv_heads, elem, args.partition, args.arenas or 2, args.seed,
+                               kernel="split_kv_decode_map" if fast else "split_kv_map_generic", d=d, p=p)
+        group = min(args.q_heads // args.kv_heads, 8)
         if args.grouped:
-            w = wl.make_workload(args.seed, ctx, args.q_heads, args.kv_heads, 256, elem, 16, q_lens=args.q_len,
+            w = wl.make_workload(args.seed, ctx, args.q_heads, args.kv_heads, d, elem, p, q_lens=args.q_len,
                                  host_pages=False)
             dw = wl.DeviceWorkload(device, w, partition_tokens=args.partition, grouped=True,
-                                   variant=psi.GQASplitKVVariant.TiledQ(8, 16, args.q_heads // args.kv_heads))
+                                   variant=psi.GQASplitKVVariant.TiledQ(8, 16, group))
             return Case(name, key + "_grouped", [dw], "verify", "tiled_q_map", "split_kv_chunk_map",
                         "kv append -> row-group (prefill-chunk) map -> LSE combine")
-        return verify_case(key, ctx, args.q_len, args.partition, args.arenas or 1, args.seed)
+        return verify_case(key, ctx, args.q_len, args.partition, args.arenas or 1, args.seed, hq=args.q_heads,
+                           hkv=args.kv_heads, d=d, p=p, dtype=elem, variant=psi.GQASplitKVVariant.TiledQ(8, 16, group))
+    if name == "C2_rows512":
+        # the headline batch with its 512-token partitions launched as they are: one workgroup per partition row
+        ctx = wl.config_c2_context_lens(args.seed, 32, 1024, 8192) + 1
+        key = f"decode_b32_ctx1024-8192_24q4kv_d256_bf16_p16_part512_seed{args.seed}_row_per_workgroup"
+        return decode_case(key, ctx, 24, 4, bf16, 512, args.arenas or 2, args.seed,
+                           how=dict(balanced=False, longest_first=True, fused_append=not args.separate_append))
+    if name in ("C2_b4", "C2_b8", "C2_b16"):
+        # the headline's shape at the batch sizes of a lightly loaded server
+        b = int(name[4:])
+        ctx = wl.config_c2_context_lens(args.seed, b, 1024, 8192) + 1
+        return decode_case(f"decode_b{b}_ctx1024-8192_24q4kv_d256_bf16_p16_part512_seed{args.seed}", ctx, 24, 4, bf16, 512,
+                           args.arenas or max(2, 64 // b), args.seed)
+    if name == "GENERIC_f32_b8":
+        # what the shape-generic kernels cost (f32 storage, and every geometry outside the fast kernels' domain):
+        # the headline's shape at batch 8 with f32 K/V
+        ctx = wl.config_c2_context_lens(args.seed, 8, 1024, 8192) + 1
+        return decode_case(f"decode_b8_ctx1024-8192_24q4kv_d256_f32_p16_part512_seed{args.seed}", ctx, 24, 4,
+                           psi.Dtype.Float32, 512, args.arenas or 2, args.seed, kernel="split_kv_map_generic")
+    if name == "REF_tiled":
+        case = verify_case("ref_tiled_q8_b1_ctx128_40q8kv_d128_bf16_p8_seed7", [128 + 8], 8, 512, args.arenas or 64, 7,
+                           hq=40, hkv=8, d=128, p=8, variant=psi.GQASplitKVVariant.TiledQ(8, 16, 5))
+        return map_and_reduce_only(case)
+    if name.startswith("REF_criterion_"):
+        which = name[len("REF_criterion_"):]
+        ctxs = [128] * 7 + [4096] if which == "ragged" else [int(which[3:])]
+        case = decode_case(f"ref_criterion_{which}_32q8kv_d128_bf16_p16_part512_seed8", ctxs, 32, 8, bf16, 512,
+                           args.arenas or 64, 8, d=128, p=16,
+                           how=dict(balanced=True, longest_first=True, fused_append=False))
+        return map_and_reduce_only(case)
     if name == "C1":
         # 1 MB per arena: enough arenas that a page comes back only after 300 MB of other pages went through the
         # 256 MB last-level cache
@@ -240,6 +305,17 @@ def time_case(psi, wl, device, case, args, with_spread=True):
 
     kernel_only = args.kernel_only and case.kind != "mixed"
     body = run_maps if kernel_only else run_steps
+    # Cold: the very first step after the arenas were set up (code objects loaded on first use, clocks wherever the
+    # set-up left them), then the mean of the next K steps, before anything has settled.
+    device.sync()
+    t0 = time.perf_counter()
+    body(1)
+    device.sync()
+    first_step_us = (time.perf_counter() - t0) * 1e6
+    t0 = time.perf_counter()
+    body(args.steps, first=1)
+    device.sync()
+    cold_us = (time.perf_counter() - t0) * 1e6 / args.steps
     # Set-up, not measurement: generating a workload's arena leaves the GPU's clocks unsettled for some 20 ms of
     # attention work (step times drift by 5-10 % over the first 40 steps), and an arena's first step pays for the
     # first touch of its buffers; steps of a millisecond keep speeding up for longer (C5's decode side: 1313 us per
@@ -260,6 +336,8 @@ def time_case(psi, wl, device, case, args, with_spread=True):
     ms_per_step = (time.perf_counter() - t0) * 1e3 / args.steps
     out = {"workload": case.key, "step": "map kernel only" if kernel_only else case.description,
            "us_per_layer_step": ms_per_step * 1e3, "settle_steps_before_warmup": settle_steps,
+           "cold": {"first_step_us": first_step_us, "us_per_layer_step_first_k_steps": cold_us,
+                    "note": "wall clock, before the settle run: the first step alone, then the mean of the next K"},
            "algorithmic_bytes_per_step": step_bytes,
            "step_GBps": step_bytes / (ms_per_step / 1e3) / 1e9,
            "step_frac_of_hbm_peak": step_bytes / (ms_per_step / 1e3) / 1e9 / HBM_PEAK_GBPS}
@@ -274,6 +352,16 @@ def time_case(psi, wl, device, case, args, with_spread=True):
         ticks[-1].synchronize()
         step_us = sorted(ticks[i].elapsed_time(ticks[i + 1]) * 1e3 for i in range(n_spread))
         out["us_per_layer_step_p10_median_p90"] = [step_us[int(f * (len(step_us) - 1))] for f in (0.1, 0.5, 0.9)]
+    if case.submit_and_wait:
+        # what a bench that waits for every submission sees (the reference's Criterion bench and its `--iters`
+        # diagnostics do): launch latency and the host's wake-up included
+        n = min(args.steps, 100)
+        device.sync()
+        t0 = time.perf_counter()
+        for i in range(n):
+            body(1, first=i)
+            device.sync()
+        out["us_per_step_submit_and_wait"] = (time.perf_counter() - t0) * 1e6 / n
     if case.kind == "mixed":
         m = arenas[0]
         device.set_timing(True)
@@ -329,9 +417,13 @@ def time_case(psi, wl, device, case, args, with_spread=True):
     timing = {"avg_launch_us": map_us, "back_to_back_launch_us": map_b2b_us, "event_pair_per_launch_us": map_pair_us,
               "launches_timed": int(n_groups * group_launches if map_b2b_us <= map_pair_us else map_launches),
               "timing": "HIP events on the launch stream; the smaller of the back-to-back and per-launch figures"}
-    hbm = {"bound": "hbm", "kernel": case.roof_kernel, "achieved": map_bytes / (map_us / 1e6) / 1e9,
-           "peak": HBM_PEAK_GBPS, "unit": "GB/s", "frac": map_bytes / (map_us / 1e6) / 1e9 / HBM_PEAK_GBPS,
-           "traffic": read_profile_traffic(case.key), "algorithmic_bytes_per_launch": map_bytes, **timing}
+    achieved = map_bytes / (map_us / 1e6) / 1e9
+    stream_gbps = measured_stream_gbps(device)
+    hbm = {"bound": "hbm", "kernel": case.roof_kernel, "achieved": achieved,
+           "peak": HBM_PEAK_GBPS, "unit": "GB/s", "frac": achieved / HBM_PEAK_GBPS,
+           "traffic": read_profile_traffic(case.key), "algorithmic_bytes_per_launch": map_bytes,
+           "measured_stream_GBps": stream_gbps,
+           "frac_of_measured_stream": achieved / stream_gbps if stream_gbps else None, **timing}
     if case.flops:
         tflops = case.flops / (map_us / 1e6) / 1e12
         out["roofline"] = {"bound": "mfma", "kernel": case.roof_kernel, "achieved": tflops, "peak": MFMA_BF16_PEAK_TFLOPS,
@@ -393,6 +485,47 @@ def cpu_baseline(psi, wl, w, dw, budget_s):
         "us_per_layer_step_extrapolated": t * 1e6 * (w.algorithmic_bytes() / b),
         "openmp": {"value": bp / tp / 1e9, "unit": "GB/s", "cores": threads, "seconds": tp},
     }
+
+
+_STREAM_PROBE = {}
+
+
+def measured_stream_gbps(device):
+    """Read bandwidth of a bare stream in the attention's access pattern, measured in this run: the page-stream
+    probe of psi-dec_amd/lib/libpsi_hip_probe.so over 1 GiB of scattered 64 KiB pages, 1 KiB per load through LDS,
+    eight loads in flight per wave.  What the HBM-bound maps could reach at best on this box."""
+    import ctypes
+
+    import torch
+
+    if "gbps" in _STREAM_PROBE:
+        return _STREAM_PROBE["gbps"]
+    try:
+        probe = ctypes.CDLL(os.path.join(ROOT, "psi-dec_amd", "lib", "libpsi_hip_probe.so"))
+        probe.psi_probe_page_stream.restype = ctypes.c_int
+        probe.psi_probe_page_stream.argtypes = [ctypes.c_void_p, ctypes.c_void_p, ctypes.c_uint64, ctypes.c_int]
+        nbytes = 1 << 30
+        src = torch.empty(nbytes, dtype=torch.uint8, device="cuda").random_(0, 255)
+        stream = ctypes.c_void_p(device.stream.cuda_stream)
+        best = 0.0
+        for _ in range(2):
+            for _ in range(5):
+                if probe.psi_probe_page_stream(stream, src.data_ptr(), nbytes, 8) != 0:
+                    raise RuntimeError("psi_probe_page_stream failed")
+            start, stop = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            start.record(device.stream)
+            for _ in range(20):
+                probe.psi_probe_page_stream(stream, src.data_ptr(), nbytes, 8)
+            stop.record(device.stream)
+            stop.synchronize()
+            best = max(best, nbytes / (start.elapsed_time(stop) * 1e-3 / 20) / 1e9)
+        del src
+        torch.cuda.empty_cache()
+        _STREAM_PROBE["gbps"] = best
+    except (OSError, RuntimeError) as e:  # the probe library is a measurement aid: a figure less, not a failure
+        print(f"bench.py: stream probe unavailable ({e})", file=sys.stderr)
+        _STREAM_PROBE["gbps"] = None
+    return _STREAM_PROBE["gbps"]
 
 
 def calibrate_copy(device, args):
@@ -494,7 +627,7 @@ def main():
         "higher_is_better": True,
         "scaling": "weak",
         "vs_baseline": None,
-        "dtype": "f16" if headline_name == "C1" or (headline_name == "custom" and args.dtype == "f16") else "bf16",
+        "dtype": ("f16" if headline_name == "C1" else args.dtype if headline_name == "custom" else "bf16"),
         "data": "synthetic",
         "config": {k: v for k, v in head.items() if k not in ("roofline", "step_GBps", "step_frac_of_hbm_peak",
                                                               "us_per_layer_step", "us_per_layer_step_p10_median_p90",
@@ -511,11 +644,14 @@ def main():
         result["hbm"] = head["hbm_view"]
     if not args.no_cpu_baseline and case.kind != "mixed":
         result["cpu_baseline"] = cpu_baseline(psi, wl, case.arenas[0].w, case.arenas[0], args.cpu_seconds)
+        result["cpu_baseline_openmp"] = dict(result["cpu_baseline"]["openmp"], kind="port",
+                                             sample=result["cpu_baseline"]["sample"].split(", scalar")[0] +
+                                             ", the same oracle with OpenMP over (token, head) rows")
     del case, head
     torch.cuda.empty_cache()
     if not args.only and not args.no_configs and not args.kernel_only:
         configs = {}
-        for name in CONFIG_NAMES:
+        for name in CONFIG_NAMES + REF_NAMES:
             c = build_case(psi, wl, device, name, args)
             r = time_case(psi, wl, device, c, args)
             r["host_plan_us"] = host_plan_us(psi, wl, c)
