@@ -260,23 +260,19 @@ def build_case(psi, wl, device, name, args):
 
 def algorithmic_bytes(case):
     a = case.arenas[0]
-    if case.kind == "mixed":
-        return a.chunk.w.algorithmic_bytes() + a.decode.w.algorithmic_bytes()
     return a.w.algorithmic_bytes()
 
 
 def host_plan_us(psi, wl, case, repeats=15):
     """Median host time of one step's planning for the workload: metadata update (+ worker plan / dispatch order /
     row groups) and the upload of the arrays to their fixed device buffers, as the Python mirror issues it."""
-    parts = [case.arenas[0]] if case.kind != "mixed" else [case.arenas[0].chunk, case.arenas[0].decode]
+    dw = case.arenas[0]
     times = []
     for _ in range(repeats):
         t0 = time.perf_counter()
-        for dw in parts:
-            dw.plan()
+        dw.plan()
         times.append((time.perf_counter() - t0) * 1e6)
-    for dw in parts:
-        dw.device.sync()
+    dw.device.sync()
     return sorted(times)[len(times) // 2]
 
 
@@ -373,9 +369,24 @@ def time_case(psi, wl, device, case, args, with_spread=True):
             kernels[k] = ms / max(n, 1) * 1e3
         device.set_timing(False)
         out["kernel_us_in_step"] = kernels
-        out["roofline"] = None  # two dominant kernels with two bounds: see C5_prefill and C5_decode
-        out["chunk_rows"] = m.chunk.shape.num_sdpa_map_task_templates
-        out["decode_rows"] = m.decode.shape.num_sdpa_map_task_templates
+        # Two dominant kernels with two bounds, issued in turn: each priced against its own peak with its time
+        # inside the step, and the step against the time the two peaks would allow one after the other.
+        chunk_us, decode_us = kernels["tiled_q_map"], kernels["split_kv_map"]
+        flops, dbytes = m.chunk_flops(), m.decode_map_bytes()
+        tflops = flops / (chunk_us / 1e6) / 1e12
+        gbps = dbytes / (decode_us / 1e6) / 1e9
+        ideal_us = flops / (MFMA_BF16_PEAK_TFLOPS * 1e12) * 1e6 + dbytes / (HBM_PEAK_GBPS * 1e9) * 1e6
+        out["roofline"] = {
+            "bound": "hbm", "kernel": "split_kv_decode_map", "achieved": gbps, "peak": HBM_PEAK_GBPS, "unit": "GB/s",
+            "frac": gbps / HBM_PEAK_GBPS, "traffic": None, "algorithmic_bytes_per_launch": dbytes,
+            "avg_launch_us": decode_us, "timing": "HIP event pairs around every launch inside the step",
+            "second_kernel": {"bound": "mfma", "kernel": "split_kv_chunk_map", "achieved": tflops,
+                              "peak": MFMA_BF16_PEAK_TFLOPS, "unit": "TFLOP/s", "frac": tflops / MFMA_BF16_PEAK_TFLOPS,
+                              "flops_per_launch": flops, "avg_launch_us": chunk_us},
+            "step_frac_of_both_peaks_in_turn": ideal_us / (ms_per_step * 1e3)}
+        out["chunk_rows"] = m.chunk_meta.replay_shape().num_sdpa_map_task_templates
+        out["decode_rows"] = m.decode_meta.replay_shape().num_sdpa_map_task_templates
+        out["step"] = "one planning call and one layer call for the whole batch: " + case.description
         return out
 
     # Dominant kernel: HIP events on the launch stream around every map launch ...

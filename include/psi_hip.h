@@ -658,6 +658,42 @@ int psi_hip_gqa_layer_scratch_bytes(const psi_hip_gqa_layer_config* cfg, const p
 int psi_hip_gqa_layer_record(psi_hip_ctx* ctx, const psi_hip_gqa_layer_config* cfg,
                              const psi_hip_gqa_layer_input* input);
 
+/* A batch that holds prefill chunks and decode requests at once.  The reference runs such a batch through one
+ * SplitKV variant (`select_split_kv_variant`, crates/inference-executor-metal/src/attn/gqa/mod.rs:64-94, then
+ * `GQA::record`, backend.rs:394-658), and its server caps a request at 64 tokens per batch; here the requests with more
+ * than chunk_min_tokens new tokens go through the TiledQ kernels with the row-group plan (matrix-core bound) and the
+ * others through the variant psi_hip_split_kv_select_batch picks for them (HBM bound): two parts of one batch,
+ * planned by one call and recorded by one call.  The chunk requests must come first in the batch, so that either
+ * part's tokens are one run of the flat q / k / v / output rows; a batch with only one kind has one empty part.
+ *
+ * psi_hip_gqa_layer_prepare_mixed is psi_hip_gqa_layer_prepare for both parts (chunk_options / decode_options and
+ * chunk_host / decode_host as there; the chunk part's dispatch is ROW_GROUPS whatever chunk_options->dispatch says,
+ * its variant TiledQ with 8-token tiles).  out_plan->chunk and ->decode receive what psi_hip_gqa_layer_prepare writes
+ * to its out_plan (the pointer fields are left to the caller), ->chunk_uses and ->decode_uses its out_uses. */
+typedef struct psi_hip_gqa_mixed_plan {
+    uint32_t num_chunk_reqs;   /* the batch's first requests: the prefill chunks */
+    uint32_t num_chunk_tokens; /* their tokens: rows [0, num_chunk_tokens) of q / k / v / output */
+    uint32_t chunk_uses;
+    uint32_t decode_uses;
+    psi_hip_gqa_batch_metadata chunk;
+    psi_hip_gqa_batch_metadata decode;
+} psi_hip_gqa_mixed_plan;
+int psi_hip_gqa_layer_prepare_mixed(const psi_hip_gqa_layer_config* cfg, const psi_hip_gqa_plan_options* chunk_options,
+                                    const psi_hip_gqa_plan_options* decode_options, uint32_t chunk_min_tokens,
+                                    const uint32_t* req_slots, const uint32_t* token_indices, const uint32_t* cu_tokens,
+                                    uint32_t num_reqs, const psi_hip_gqa_host_metadata* chunk_host,
+                                    const psi_hip_gqa_host_metadata* decode_host, psi_hip_gqa_mixed_plan* out_plan);
+/* Bytes of `partial_scratch` for a mixed batch: the chunk part's partial states, then the decode part's. */
+int psi_hip_gqa_layer_mixed_scratch_bytes(const psi_hip_gqa_layer_config* cfg, const psi_hip_gqa_mixed_plan* plan,
+                                          uint64_t* out_bytes);
+/* `GQA::record` for a mixed batch: the chunk part, then the decode part, on the context's stream (input->
+ * batch_metadata is not used; the row pointers of the input name the whole batch and the decode part's rows start
+ * num_chunk_tokens rows in).  Both parts' kernels need a compute unit to themselves and scale with the compute
+ * units they get, so running them side by side on two streams gains nothing (measured: 1622 us at best against
+ * 1643 us one after the other on a 2048-token chunk next to 128 decode sequences); they are issued in turn. */
+int psi_hip_gqa_layer_record_mixed(psi_hip_ctx* ctx, const psi_hip_gqa_layer_config* cfg,
+                                   const psi_hip_gqa_layer_input* input, const psi_hip_gqa_mixed_plan* plan);
+
 /* psi_hip_gqa_layer_record with the partial states in a buffer built into the library instead of
  * input->partial_scratch (which is ignored, as is partial_scratch_bytes).  No counterpart in the reference.  It is
  * for callers that cannot allocate device memory: code under HIP graph capture, tight serving loops, harnesses

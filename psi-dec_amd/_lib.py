@@ -129,6 +129,17 @@ class BatchMetadataStruct(ctypes.Structure):
     ]
 
 
+class MixedPlanStruct(ctypes.Structure):
+    _fields_ = [
+        ("num_chunk_reqs", c_uint32),
+        ("num_chunk_tokens", c_uint32),
+        ("chunk_uses", c_uint32),
+        ("decode_uses", c_uint32),
+        ("chunk", BatchMetadataStruct),
+        ("decode", BatchMetadataStruct),
+    ]
+
+
 class LayerConfigStruct(ctypes.Structure):
     _fields_ = [
         ("attention", GQAConfigStruct),
@@ -347,6 +358,14 @@ PROTOTYPES = {
         c_int, [POINTER(PlanOptionsStruct), POINTER(HostMetadataStruct), POINTER(BatchMetadataStruct), c_uint32,
                 POINTER(ctypes.c_int)]),
     "psi_hip_gqa_layer_record": (c_int, [c_void_p, POINTER(LayerConfigStruct), POINTER(LayerInputStruct)]),
+    "psi_hip_gqa_layer_prepare_mixed": (
+        c_int, [POINTER(LayerConfigStruct), POINTER(PlanOptionsStruct), POINTER(PlanOptionsStruct), c_uint32, c_void_p,
+                c_void_p, c_void_p, c_uint32, POINTER(HostMetadataStruct), POINTER(HostMetadataStruct),
+                POINTER(MixedPlanStruct)]),
+    "psi_hip_gqa_layer_mixed_scratch_bytes": (
+        c_int, [POINTER(LayerConfigStruct), POINTER(MixedPlanStruct), POINTER(c_uint64)]),
+    "psi_hip_gqa_layer_record_mixed": (
+        c_int, [c_void_p, POINTER(LayerConfigStruct), POINTER(LayerInputStruct), POINTER(MixedPlanStruct)]),
     "psi_hip_gqa_layer_record_static_scratch": (
         c_int, [c_void_p, POINTER(LayerConfigStruct), POINTER(LayerInputStruct)]),
     "psi_hip_gqa_replay_cache_create": (

@@ -464,6 +464,124 @@ extern "C" int psi_hip_gqa_layer_record(psi_hip_ctx* ctx, const psi_hip_gqa_laye
     return record_layer(ctx, cfg, input);
 }
 
+extern "C" int psi_hip_gqa_layer_prepare_mixed(const psi_hip_gqa_layer_config* cfg,
+                                               const psi_hip_gqa_plan_options* chunk_options,
+                                               const psi_hip_gqa_plan_options* decode_options, uint32_t chunk_min_tokens,
+                                               const uint32_t* req_slots, const uint32_t* token_indices,
+                                               const uint32_t* cu_tokens, uint32_t num_reqs,
+                                               const psi_hip_gqa_host_metadata* chunk_host,
+                                               const psi_hip_gqa_host_metadata* decode_host,
+                                               psi_hip_gqa_mixed_plan* out_plan) {
+    PSI_REQUIRE(cfg && chunk_options && decode_options && out_plan, "GQA mixed prepare: config, options and out_plan must not be null");
+    PSI_REQUIRE(req_slots && token_indices && cu_tokens && num_reqs > 0, "GQA prepare needs a batch");
+    PSI_REQUIRE(cu_tokens[0] == 0, "GQA cu_tokens must start at zero");
+    uint32_t n_chunk = 0;
+    while (n_chunk < num_reqs && cu_tokens[n_chunk + 1] - cu_tokens[n_chunk] > chunk_min_tokens) ++n_chunk;
+    for (uint32_t r = n_chunk; r < num_reqs; ++r)
+        PSI_REQUIRE(cu_tokens[r + 1] >= cu_tokens[r] && cu_tokens[r + 1] - cu_tokens[r] <= chunk_min_tokens,
+                    "GQA mixed batch: the requests with more than %u new tokens must come first (request %u)",
+                    chunk_min_tokens, r);
+    std::memset(out_plan, 0, sizeof(*out_plan));
+    out_plan->num_chunk_reqs = n_chunk;
+    out_plan->num_chunk_tokens = cu_tokens[n_chunk];
+    int rc = PSI_HIP_OK;
+    if (n_chunk > 0) {
+        PSI_REQUIRE(chunk_host != nullptr, "GQA mixed prepare: the chunk part needs its host arrays");
+        Geometry g;
+        rc = make_geometry(&cfg->attention, &g);
+        if (rc != PSI_HIP_OK) return rc;
+        psi_hip_gqa_plan_options options = *chunk_options;
+        options.dispatch = PSI_HIP_DISPATCH_ROW_GROUPS;
+        const psi_hip_split_kv_variant tiled{PSI_HIP_VARIANT_TILED_Q, 8u, 16u, 0u, g.group < 8u ? g.group : 8u};
+        rc = psi_hip_gqa_layer_prepare(cfg, &options, req_slots, token_indices, cu_tokens, n_chunk, &tiled, chunk_host,
+                                       &out_plan->chunk, &out_plan->chunk_uses);
+        if (rc != PSI_HIP_OK) return rc;
+    }
+    if (n_chunk < num_reqs) {
+        PSI_REQUIRE(decode_host != nullptr, "GQA mixed prepare: the decode part needs its host arrays");
+        thread_local std::vector<uint32_t> cu;
+        cu.resize(num_reqs - n_chunk + 1);
+        for (uint32_t r = n_chunk; r <= num_reqs; ++r) cu[r - n_chunk] = cu_tokens[r] - cu_tokens[n_chunk];
+        rc = psi_hip_gqa_layer_prepare(cfg, decode_options, req_slots + n_chunk, token_indices + n_chunk, cu.data(),
+                                       num_reqs - n_chunk, nullptr, decode_host, &out_plan->decode,
+                                       &out_plan->decode_uses);
+        if (rc != PSI_HIP_OK) return rc;
+    }
+    return PSI_HIP_OK;
+}
+
+// Bytes of one part's partial states, rounded up so that the next part starts on a 256-byte boundary.
+static int mixed_part_bytes(const psi_hip_gqa_layer_config* cfg, const psi_hip_gqa_batch_metadata& md, uint64_t* out) {
+    *out = 0;
+    if (md.shape.num_tokens == 0) return PSI_HIP_OK;
+    int rc = psi_hip_gqa_layer_scratch_bytes(cfg, &md.variant, md.shape.num_total_kv_splits, out);
+    *out = (*out + 255) & ~uint64_t(255);
+    return rc;
+}
+
+extern "C" int psi_hip_gqa_layer_mixed_scratch_bytes(const psi_hip_gqa_layer_config* cfg,
+                                                     const psi_hip_gqa_mixed_plan* plan, uint64_t* out_bytes) {
+    PSI_REQUIRE(cfg && plan && out_bytes, "GQA mixed scratch: config, plan and out pointer must not be null");
+    uint64_t chunk = 0, decode = 0;
+    int rc = mixed_part_bytes(cfg, plan->chunk, &chunk);
+    if (rc != PSI_HIP_OK) return rc;
+    rc = mixed_part_bytes(cfg, plan->decode, &decode);
+    if (rc != PSI_HIP_OK) return rc;
+    *out_bytes = chunk + decode;
+    return PSI_HIP_OK;
+}
+
+extern "C" int psi_hip_gqa_layer_record_mixed(psi_hip_ctx* ctx, const psi_hip_gqa_layer_config* cfg,
+                                              const psi_hip_gqa_layer_input* input, const psi_hip_gqa_mixed_plan* plan) {
+    PSI_REQUIRE(ctx && cfg && input && plan, "ctx, config, input and plan must not be null");
+    LayerPlan lp;
+    int rc = make_layer_plan(cfg, &lp);
+    if (rc != PSI_HIP_OK) return rc;
+    const Geometry& g = lp.g;
+    const bool has_chunk = plan->chunk.shape.num_tokens != 0, has_decode = plan->decode.shape.num_tokens != 0;
+    PSI_REQUIRE(has_chunk || has_decode, "GQA mixed plan holds no tokens");
+    PSI_REQUIRE(!has_chunk || plan->chunk.shape.num_tokens == plan->num_chunk_tokens,
+                "GQA mixed plan: the chunk part's token count differs from num_chunk_tokens");
+    uint64_t chunk_bytes = 0, decode_bytes = 0;
+    rc = mixed_part_bytes(cfg, plan->chunk, &chunk_bytes);
+    if (rc != PSI_HIP_OK) return rc;
+    rc = mixed_part_bytes(cfg, plan->decode, &decode_bytes);
+    if (rc != PSI_HIP_OK) return rc;
+    PSI_REQUIRE(input->partial_scratch != nullptr && input->partial_scratch_bytes >= chunk_bytes + decode_bytes,
+                "GQA mixed scratch too small: %llu < %llu", (unsigned long long)input->partial_scratch_bytes,
+                (unsigned long long)(chunk_bytes + decode_bytes));
+    if (has_chunk) {
+        psi_hip_gqa_layer_input part = *input;
+        part.batch_metadata = &plan->chunk;
+        part.partial_scratch_bytes = chunk_bytes;
+        rc = record_layer(ctx, cfg, &part);
+        if (rc != PSI_HIP_OK) return rc;
+    }
+    if (has_decode) {
+        // the decode part's rows start behind the chunk part's: num_chunk_tokens rows of every per-token array
+        const uint64_t skip = has_chunk ? plan->num_chunk_tokens : 0;
+        const uint64_t q_row = (uint64_t)g.hq * g.d, kv_row = (uint64_t)g.hkv * g.d;
+        const uint32_t out_elem = ctx->f32_output ? 4u : g.elem;
+        auto rows_on = [&](const void* base, uint64_t row_elems, uint32_t elem) -> const void* {
+            return base == nullptr ? nullptr : static_cast<const char*>(base) + skip * row_elems * elem;
+        };
+        psi_hip_gqa_layer_input part = *input;
+        part.batch_metadata = &plan->decode;
+        part.qgkv = rows_on(input->qgkv, lp.token_width, g.elem);
+        part.q = rows_on(input->q, q_row, g.elem);
+        part.k = rows_on(input->k, kv_row, g.elem);
+        part.v = rows_on(input->v, kv_row, g.elem);
+        part.g = rows_on(input->g, q_row, g.elem);
+        part.q_norm_rope = const_cast<void*>(rows_on(input->q_norm_rope, q_row, g.elem));
+        part.output = const_cast<void*>(rows_on(input->output, q_row, out_elem));
+        part.partial_scratch = static_cast<char*>(input->partial_scratch) + chunk_bytes;
+        part.partial_scratch_bytes = decode_bytes;
+        rc = record_layer(ctx, cfg, &part);
+        if (rc != PSI_HIP_OK) return rc;
+    }
+    return PSI_HIP_OK;
+}
+
 extern "C" int psi_hip_gqa_layer_record_static_scratch(psi_hip_ctx* ctx, const psi_hip_gqa_layer_config* cfg,
                                                        const psi_hip_gqa_layer_input* input) {
     PSI_REQUIRE(ctx != nullptr && cfg != nullptr && input != nullptr && input->batch_metadata != nullptr,

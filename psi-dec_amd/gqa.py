@@ -780,6 +780,20 @@ class GQAMetadataBuffers:
                                       policy.max_tokens() if policy is not None else 0, boundaries,
                                       len(policy.token_topology_boundaries) if policy is not None else 0,
                                       int(bucket_capacities))
+        host = self._host_metadata(dispatch)
+        plan, uses = L.BatchMetadataStruct(), ctypes.c_uint32()
+        v = variant.struct() if variant is not None else None
+        self._last_prepare = (options, plan, uses, boundaries)  # what advance_decode() continues from
+        L.check(L.load().psi_hip_gqa_layer_prepare(
+            ctypes.byref(layer_struct), ctypes.byref(options), rs.ctypes.data, ti.ctypes.data, cu.ctypes.data, len(rs),
+            ctypes.byref(v) if v is not None else None, ctypes.byref(host), ctypes.byref(plan),
+            ctypes.byref(uses)))
+        return self._adopt(plan, uses.value)
+
+    def _host_metadata(self, dispatch: int):
+        """The host arrays as psi_hip_gqa_layer_prepare takes them (`psi_hip_gqa_host_metadata`); waits until the last
+        upload has left the staging block."""
+        self._staging_free()
         if dispatch == L.DISPATCH_ROW_GROUPS and self._row_groups_words() == 0:
             self._alloc_row_groups((self._max_kv_splits + self._max_workers) * 32)
         if self._host_struct is None or self._host_struct.row_groups_capacity != self._row_groups_words():
@@ -791,19 +805,17 @@ class GQAMetadataBuffers:
                 addr(self.h_req_slots), addr(self.h_flat_token_indices), addr(self.h_q_token_tiles),
                 addr(self._h_kv_splits_all), addr(self.h_cu_kv_splits), addr(self._h_row_index_all),
                 addr(self._h_worker_cu_all), addr(self._h_row_groups_all))
-        plan, uses = L.BatchMetadataStruct(), ctypes.c_uint32()
-        v = variant.struct() if variant is not None else None
-        self._last_prepare = (options, plan, uses, boundaries)  # what advance_decode() continues from
-        L.check(L.load().psi_hip_gqa_layer_prepare(
-            ctypes.byref(layer_struct), ctypes.byref(options), rs.ctypes.data, ti.ctypes.data, cu.ctypes.data, len(rs),
-            ctypes.byref(v) if v is not None else None, ctypes.byref(self._host_struct), ctypes.byref(plan),
-            ctypes.byref(uses)))
+        return self._host_struct
+
+    def _adopt(self, plan, uses: int) -> GQAReplayShape:
+        """Takes over what a preparation wrote into the host arrays (`plan`: the psi_hip_gqa_batch_metadata it
+        filled, `uses`: which dispatch tables are in use) and uploads it."""
         sh = plan.shape
         self._shape = GQAReplayShape(sh.num_tokens, sh.num_total_tokens, sh.num_q_token_tiles, sh.num_total_q_token_tiles,
                                      sh.num_kv_splits, sh.num_total_kv_splits, bool(sh.reduce_sdpa_partial_outputs))
         self._variant = GQASplitKVVariant.from_struct(plan.variant)
         self.h_kv_splits = self._h_kv_splits_all
-        use_index, use_workers, use_groups = bool(uses.value & 1), bool(uses.value & 2), bool(uses.value & 4)
+        use_index, use_workers, use_groups = bool(uses & 1), bool(uses & 2), bool(uses & 4)
         self.h_partial_row_index = self._h_row_index_all if use_index else None
         self.d_partial_row_index = self._d_row_index_all if use_index else None
         self.num_workers = plan.num_workers
@@ -1271,6 +1283,24 @@ class GQAInput:
     counts_uploaded: bool = False  # a replay cache reads the count words the metadata upload brought along
 
 
+@dataclass
+class GQAMixedPlan:
+    """What `GQA.prepare_mixed` planned: the batch's first `num_chunk_reqs` requests (`num_chunk_tokens` tokens) are
+    prefill chunks, the others decode requests; each part's arrays live in its own `GQAMetadataBuffers`."""
+    num_chunk_reqs: int
+    num_chunk_tokens: int
+    chunk_metadata: GQAMetadataBuffers
+    decode_metadata: GQAMetadataBuffers
+    has_chunk: bool
+    has_decode: bool
+
+    def struct(self):
+        empty = L.BatchMetadataStruct()
+        return L.MixedPlanStruct(self.num_chunk_reqs, self.num_chunk_tokens, 0, 0,
+                                 self.chunk_metadata.struct() if self.has_chunk else empty,
+                                 self.decode_metadata.struct() if self.has_decode else empty)
+
+
 class GQA:
     """`GQA` / `UngatedGQA` (attn/gqa/backend.rs:214-392, ungated_backend.rs:104-180): the attention part of a
     layer behind `record`.  `gated`: projection rows [q_0|g_0|...|k|v] and a sigmoid gate on the output."""
@@ -1333,6 +1363,53 @@ class GQA:
                                       capacity_mode=L.CAPACITY_FIXED_PARTITION, partition_tokens=partition_tokens,
                                       dispatch=dispatch, num_workers=num_workers, variant=variant,
                                       bucket_capacities=bucket_capacities, policy=policy)
+
+    def prepare_mixed(self, chunk_metadata: GQAMetadataBuffers, decode_metadata: GQAMetadataBuffers, req_slots,
+                      token_indices, cu_tokens, chunk_min_tokens: int = 8, chunk_partition: int = 4096,
+                      decode_partition: int = 512, num_workers: int = 0) -> "GQAMixedPlan":
+        """The host side of a step whose batch holds prefill chunks (more than `chunk_min_tokens` new tokens; they must
+        come first) and decode requests: one call (psi_hip_gqa_layer_prepare_mixed) plans the chunk part for the
+        row-group map and the decode part for the balanced decode map, each with fixed partitions, and uploads
+        both.  The reference plans such a batch for one variant (backend.rs:289-364)."""
+        rs = np.ascontiguousarray(req_slots, dtype=np.uint32)
+        ti = np.ascontiguousarray(token_indices, dtype=np.uint32)
+        cu = np.ascontiguousarray(cu_tokens, dtype=np.uint32)
+        assert len(rs) == len(ti) and len(cu) == len(rs) + 1
+        chunk_options = L.PlanOptionsStruct(L.CAPACITY_FIXED_PARTITION, chunk_partition, 0, L.DISPATCH_ROW_GROUPS, 0, 0,
+                                            None, 0, 0)
+        decode_options = L.PlanOptionsStruct(L.CAPACITY_FIXED_PARTITION, decode_partition, 0, L.DISPATCH_BALANCED,
+                                             num_workers, 0, None, 0, 0)
+        plan = L.MixedPlanStruct()
+        cfg = self.struct()
+        L.check(L.load().psi_hip_gqa_layer_prepare_mixed(
+            ctypes.byref(cfg), ctypes.byref(chunk_options), ctypes.byref(decode_options), chunk_min_tokens,
+            rs.ctypes.data, ti.ctypes.data, cu.ctypes.data, len(rs),
+            ctypes.byref(chunk_metadata._host_metadata(L.DISPATCH_ROW_GROUPS)),
+            ctypes.byref(decode_metadata._host_metadata(L.DISPATCH_BALANCED)), ctypes.byref(plan)))
+        if plan.chunk.shape.num_tokens:
+            chunk_metadata._adopt(plan.chunk, plan.chunk_uses)
+        if plan.decode.shape.num_tokens:
+            decode_metadata._adopt(plan.decode, plan.decode_uses)
+            decode_metadata._last_prepare = (decode_options, plan.decode, ctypes.c_uint32(plan.decode_uses), plan)
+        return GQAMixedPlan(plan.num_chunk_reqs, plan.num_chunk_tokens, chunk_metadata, decode_metadata,
+                            bool(plan.chunk.shape.num_tokens), bool(plan.decode.shape.num_tokens))
+
+    def mixed_scratch_bytes(self, plan: "GQAMixedPlan") -> int:
+        cfg, n = self.struct(), ctypes.c_uint64()
+        s = plan.struct()
+        L.check(L.load().psi_hip_gqa_layer_mixed_scratch_bytes(ctypes.byref(cfg), ctypes.byref(s), ctypes.byref(n)))
+        return n.value
+
+    def record_mixed(self, inp: GQAInput, plan: "GQAMixedPlan"):
+        """`GQA::record` for a mixed batch (psi_hip_gqa_layer_record_mixed): `inp` names the whole batch's rows and a
+        scratch of `mixed_scratch_bytes(plan)`; its `batch_metadata` is not used."""
+        cfg = self.struct()
+        inp.batch_metadata = plan.chunk_metadata if plan.has_chunk else plan.decode_metadata  # any prepared one
+        s, keep = self.input_struct(inp)
+        p = plan.struct()
+        L.check(self.device.lib.psi_hip_gqa_layer_record_mixed(self.device.ctx, ctypes.byref(cfg), ctypes.byref(s),
+                                                               ctypes.byref(p)))
+        return keep[1]
 
     def input_struct(self, inp: GQAInput):
         """(psi_hip_gqa_layer_input, keep-alive objects) for an input."""

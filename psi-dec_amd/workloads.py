@@ -378,14 +378,13 @@ class MixedStep:
     """A step that holds prefill chunks and decode tokens at once, over one arena and one page table.  The
     reference would run one SplitKV variant for the whole batch; here the requests with more than
     `chunk_min_tokens` new tokens go through the multi-query kernels with the row-group plan and the others
-    through the decode kernels (balanced worker plan, append inside the map launch): two `GQA.record` calls on
-    the same stream.  The chunk requests must come first in the batch, so that either part's tokens are one
-    contiguous run of the flat q / k / v / output rows."""
+    through the decode kernels (balanced worker plan, append inside the map launch): one planning call
+    (`GQA.prepare_mixed`) and one layer call (`GQA.record_mixed`) for the whole batch.  The chunk requests must
+    come first in the batch, so that either part's tokens are one contiguous run of the flat q / k / v / output
+    rows."""
 
     def __init__(self, device: G.Device, w: Workload, decode_partition: int = 512,
                  chunk_partition: Optional[int] = None, chunk_min_tokens: int = 8, f32_output: bool = False):
-        import dataclasses
-
         import torch
 
         q_lens = np.diff(w.cu_tokens).astype(np.int64)
@@ -394,35 +393,85 @@ class MixedStep:
         assert 0 < n_chunk < len(q_lens) and is_chunk[:n_chunk].all(), "chunk requests first, then decode requests"
         self.device, self.w, self.f32_output = device, w, f32_output
         self.pages, self.page_ids = device_pages(device, w), device.from_numpy(w.page_ids)
-        cut = int(w.cu_tokens[n_chunk])
-
-        def part(lo_req, hi_req, lo_tok, hi_tok):
-            return dataclasses.replace(
-                w, req_slots=w.req_slots[lo_req:hi_req], token_indices=w.token_indices[lo_req:hi_req],
-                cu_tokens=(w.cu_tokens[lo_req:hi_req + 1] - w.cu_tokens[lo_req]).astype(np.uint32),
-                q=w.q.reshape(w.num_tokens, -1)[lo_tok:hi_tok].reshape(-1),
-                flat_k=w.flat_k.reshape(w.num_tokens, -1)[lo_tok:hi_tok].reshape(-1),
-                flat_v=w.flat_v.reshape(w.num_tokens, -1)[lo_tok:hi_tok].reshape(-1))
-
-        chunk_w, decode_w = part(0, n_chunk, 0, cut), part(n_chunk, len(q_lens), cut, w.num_tokens)
+        self.q = device.from_numpy(w.q.reshape(-1))
+        self.flat_k = device.from_numpy(w.flat_k.reshape(-1))
+        self.flat_v = device.from_numpy(w.flat_v.reshape(-1))
+        n_chunk_tokens = int(w.cu_tokens[n_chunk])
+        chunk_ctx = w.context_lens[:n_chunk]
         if chunk_partition is None:
             # Two rows per query tile: the chunk's work items then number well above the compute units and are
             # small enough to fill them evenly (measured best on a 2048-token chunk over 4096 cached tokens).
-            chunk_partition = max(2048, 1 << int((int(chunk_w.context_lens.max()) + 1) // 2 - 1).bit_length())
-        group = w.num_q_heads // w.num_kv_heads
-        self.chunk = DeviceWorkload(device, chunk_w, partition_tokens=chunk_partition, f32_output=f32_output,
-                                    grouped=True, variant=G.GQASplitKVVariant.TiledQ(8, 16, min(group, 8)),
-                                    pages=self.pages, page_ids=self.page_ids)
-        self.decode = DeviceWorkload(device, decode_w, partition_tokens=decode_partition, f32_output=f32_output,
-                                     balanced=True, fused_append=True, pages=self.pages, page_ids=self.page_ids)
-        assert not self.decode.variant.is_tiled()
+            chunk_partition = max(2048, 1 << int((int(chunk_ctx.max()) + 1) // 2 - 1).bit_length())
+        self.chunk_partition, self.decode_partition, self.chunk_min_tokens = chunk_partition, decode_partition, chunk_min_tokens
+        chunk_rows = int(sum(-(-int(c) // chunk_partition) * -(-int(n) // 8) for c, n in zip(chunk_ctx, q_lens[:n_chunk])))
+        decode_rows = int(sum(-(-(int(t) + i + 1) // decode_partition)
+                              for t, n in zip(w.token_indices[n_chunk:], q_lens[n_chunk:]) for i in range(int(n))))
+        self.chunk_meta = G.GQAMetadataBuffers(device, n_chunk_tokens, max_kv_splits=chunk_rows)
+        self.decode_meta = G.GQAMetadataBuffers(device, w.num_tokens - n_chunk_tokens, max_kv_splits=decode_rows)
+        self.gqa = G.GQA(device, G.GQACore(0, w.num_q_heads * w.head_dim, w.head_dim, w.num_q_heads, w.num_kv_heads,
+                                           w.scale),
+                         G.GQAMetalConfig(w.page_bytes, 2, 1e-6, 10000.0, io_dtype=w.dtype), gated=False)
+        self.plan()
+        self.scratch = torch.empty(self.gqa.mixed_scratch_bytes(self.mixed_plan), dtype=torch.uint8,
+                                   device=device.torch_device)
+        out_dtype = torch.float32 if f32_output else w.dtype.torch()
+        self.output = torch.zeros(w.num_tokens * w.num_q_heads * w.head_dim, dtype=out_dtype, device=device.torch_device)
+
+        class _Scratch:  # the buffers of `GQAScratch` this path touches
+            qgkv = None
+            q_norm_rope = None
+            sdpa_partial = self.scratch
+            attention_output = self.output
+
+        self._input = G.GQAInput(w.layout, w.layer, self.chunk_meta, G.GQAKVCacheBindings(self.pages, self.page_ids),
+                                 _Scratch, replay_mode=G.GQAReplayMode.Bucketed, q=self.q, k=self.flat_k,
+                                 v=self.flat_v, output=self.output)
+
+    def plan(self):
+        """The host side of the step: both parts planned by one library call, two uploads."""
+        w = self.w
+        self.mixed_plan = self.gqa.prepare_mixed(self.chunk_meta, self.decode_meta, w.req_slots, w.token_indices,
+                                                 w.cu_tokens, chunk_min_tokens=self.chunk_min_tokens,
+                                                 chunk_partition=self.chunk_partition,
+                                                 decode_partition=self.decode_partition)
+        return self.mixed_plan
 
     def step(self):
-        self.chunk.step()
-        self.decode.step()
+        self.device.f32_output(self.f32_output)
+        try:
+            self.gqa.record_mixed(self._input, self.mixed_plan)
+        finally:
+            self.device.f32_output(False)
+
+    def algorithmic_bytes(self) -> int:
+        return self.w.algorithmic_bytes()
+
+    def chunk_flops(self) -> int:
+        """Matrix flops of the chunk part: 4 * Hq * D per visible (query, key) pair."""
+        w, n = self.w, self.mixed_plan.num_chunk_reqs
+        q_lens = np.diff(w.cu_tokens).astype(np.int64)
+        pairs = sum(int(w.token_indices[r]) * int(q_lens[r]) + int(q_lens[r]) * (int(q_lens[r]) + 1) // 2 for r in range(n))
+        return 4 * w.num_q_heads * w.head_dim * pairs
+
+    def decode_map_bytes(self) -> int:
+        """Algorithmic bytes of the decode part's map: its visible K and V once plus its Q rows."""
+        w, n = self.w, self.mixed_plan.num_chunk_reqs
+        es = w.dtype.item_size()
+        q_lens = np.diff(w.cu_tokens).astype(np.int64)
+        kv = int(w.context_lens[n:].astype(np.int64).sum()) * 2 * w.num_kv_heads * w.head_dim * es
+        return kv + int(q_lens[n:].sum()) * w.num_q_heads * w.head_dim * es
 
     def output_f32(self) -> np.ndarray:
-        return np.concatenate([self.chunk.output_f32(), self.decode.output_f32()])
+        import torch
+
+        self.device.sync()
+        return self.output.to(torch.float32).cpu().numpy()
+
+    def pages_host(self) -> np.ndarray:
+        import torch
+
+        self.device.sync()
+        return self.pages.view(torch.int16).cpu().numpy().view(np.uint16)
 
 
 def config_c5(seed: int = 5, chunk: int = 2048, prefix: int = 4096, batch: int = 128, lo: int = 512,

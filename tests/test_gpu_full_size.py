@@ -218,28 +218,28 @@ def test_c5_mixed_step(psi, oracle, device):
     wl = importlib_workloads(psi)
     w = wl.config_c5()
     step = wl.MixedStep(device, w, f32_output=True)
-    assert step.chunk.meta.num_row_groups > 0 and step.decode.balanced and step.decode.fused_append
+    plan = step.mixed_plan
+    assert (plan.num_chunk_reqs, plan.num_chunk_tokens) == (1, 2048)
+    assert step.chunk_meta.num_row_groups > 0 and step.chunk_meta.split_kv_variant().is_tiled()
+    assert step.decode_meta.num_workers > 0 and not step.decode_meta.split_kv_variant().is_tiled()
     step.step()
     got = step.output_f32().reshape(w.num_tokens, -1)
     assert np.isfinite(got).all()
+    assert device.take_device_error() == 0
     # decode side: whole requests
     order = 1 + np.argsort(w.context_lens[1:])
     picks = [int(order[0]), int(order[64]), int(order[-1])]
-    dec = step.decode
-    exp, rows = oracle_sample(oracle, dec, [p - 1 for p in picks])
-    assert_outputs_close(dec.output_f32().reshape(dec.w.num_tokens, -1)[rows].reshape(-1), exp.reshape(-1),
-                         "C5 mixed, decode side")
-    assert_appended_lines(dec)
-    assert_appended_lines(step.chunk)
+    exp, rows = oracle_sample(oracle, step, picks)
+    assert_outputs_close(got[rows].reshape(-1), exp.reshape(-1), "C5 mixed, decode side")
+    assert_appended_lines(step)  # both parts' new tokens
     # chunk side: single query tokens of the chunk, each as a one-token request at its own position
     import dataclasses
 
     tokens = np.array([0, 1, 511, 512, 1023, 2040, 2047])
-    cw = step.chunk.w
-    probe_w = dataclasses.replace(cw, req_slots=np.repeat(cw.req_slots, len(tokens)),
-                                  token_indices=(cw.token_indices[0] + tokens).astype(np.uint32),
+    probe_w = dataclasses.replace(w, req_slots=np.repeat(w.req_slots[:1], len(tokens)),
+                                  token_indices=(w.token_indices[0] + tokens).astype(np.uint32),
                                   cu_tokens=np.arange(len(tokens) + 1, dtype=np.uint32),
-                                  q=cw.q.reshape(cw.num_tokens, -1)[tokens].reshape(-1))
+                                  q=w.q.reshape(w.num_tokens, -1)[tokens].reshape(-1))
 
     class _Probe:  # what oracle_sample reads of a device workload
         w, pages, page_ids, device = probe_w, step.pages, step.page_ids, step.device

@@ -398,3 +398,68 @@ def test_replay_cache_records_again_when_a_context_flag_changes(psi, oracle, dev
     finally:
         device.f32_output(False)
         device.use_stream(main)
+
+
+@pytest.mark.parametrize("q_lens,ctx", [
+    ([200, 50, 1, 1, 3], [500, 300, 700, 33, 64]),   # two chunks, decode requests and a short verify request
+    ([1, 1, 2, 1], [600, 47, 1024, 9]),              # no chunk at all: the decode part alone
+    ([40, 130], [40, 900]),                          # chunks only
+])
+def test_mixed_batch_is_one_prepare_and_one_record(psi, oracle, device, q_lens, ctx):
+    """A batch of prefill chunks and decode requests behind one planning call and one layer call
+    (psi_hip_gqa_layer_prepare_mixed / _record_mixed): pages bit-exact and outputs within the bar of the CPU
+    oracle on the whole batch, whichever of the two parts the batch holds."""
+    wl = importlib_workloads(psi)
+    w = wl.make_workload(181, ctx, 24, 4, 256, psi.Dtype.Bfloat16, 16, q_lens=q_lens)
+    exp_pages, exp = oracle_step(oracle, w)
+    n_chunk = sum(1 for n in q_lens if n > 8)
+    if 0 < n_chunk < len(q_lens):
+        step = wl.MixedStep(device, w, decode_partition=512, chunk_partition=256, f32_output=True)
+    else:  # MixedStep insists on both parts; the entry points do not
+        step = _one_kind_mixed_step(psi, wl, device, w)
+    plan = step.mixed_plan
+    assert plan.num_chunk_reqs == n_chunk and plan.num_chunk_tokens == sum(n for n in q_lens if n > 8)
+    assert plan.has_chunk == (n_chunk > 0) and plan.has_decode == (n_chunk < len(q_lens))
+    step.step()
+    got = step.output_f32()
+    assert device.take_device_error() == 0
+    assert np.array_equal(step.pages_host().reshape(exp_pages.shape), exp_pages)
+    assert_outputs_close(got, exp, f"mixed batch {q_lens}")
+
+
+def _one_kind_mixed_step(psi, wl, device, w):
+    """`MixedStep` for a batch with only chunks or only decode requests (its constructor asks for both)."""
+    import torch
+
+    step = wl.MixedStep.__new__(wl.MixedStep)
+    step.device, step.w, step.f32_output = device, w, True
+    step.pages, step.page_ids = wl.device_pages(device, w), device.from_numpy(w.page_ids)
+    step.q, step.flat_k, step.flat_v = (device.from_numpy(a.reshape(-1)) for a in (w.q, w.flat_k, w.flat_v))
+    step.chunk_partition, step.decode_partition, step.chunk_min_tokens = 256, 512, 8
+    step.chunk_meta = psi.GQAMetadataBuffers(device, w.num_tokens, max_kv_splits=256)
+    step.decode_meta = psi.GQAMetadataBuffers(device, w.num_tokens, max_kv_splits=64)
+    step.gqa = _layer(psi, device, w, gated=False)
+    step.plan()
+    step.scratch = torch.empty(step.gqa.mixed_scratch_bytes(step.mixed_plan), dtype=torch.uint8,
+                               device=device.torch_device)
+    step.output = torch.zeros(w.num_tokens * w.num_q_heads * w.head_dim, dtype=torch.float32, device=device.torch_device)
+
+    class _Scratch:
+        qgkv = None
+        q_norm_rope = None
+        sdpa_partial = step.scratch
+        attention_output = step.output
+
+    step._input = psi.GQAInput(w.layout, w.layer, step.chunk_meta, psi.GQAKVCacheBindings(step.pages, step.page_ids),
+                               _Scratch, q=step.q, k=step.flat_k, v=step.flat_v, output=step.output)
+    return step
+
+
+def test_mixed_batch_wants_its_chunks_first(psi, device):
+    wl = importlib_workloads(psi)
+    w = wl.make_workload(182, [600, 300], 24, 4, 256, psi.Dtype.Bfloat16, 16, q_lens=[1, 100])
+    gqa = _layer(psi, device, w, gated=False)
+    chunk_meta = psi.GQAMetadataBuffers(device, 128, max_kv_splits=64)
+    decode_meta = psi.GQAMetadataBuffers(device, 128, max_kv_splits=64)
+    with pytest.raises(psi.PsiHipError, match="must come first"):
+        gqa.prepare_mixed(chunk_meta, decode_meta, w.req_slots, w.token_indices, w.cu_tokens)
