@@ -76,6 +76,7 @@ def parse_args():
     p.add_argument("--dtype", choices=["bf16", "f16", "f32"], default="bf16",
                    help="custom workload: element type (f32 runs the shape-generic kernels)")
     p.add_argument("--partition", type=int, default=512)
+    p.add_argument("--prefill-partition", type=int, default=4096, help="C5_prefill: tokens per KV partition")
     p.add_argument("--arenas", type=int, default=0, help="page arenas rotated between steps (0 = per workload)")
     p.add_argument("--identity-pages", action="store_true", help="unshuffled page pool (diagnostic)")
     p.add_argument("--plan-order", action="store_true", help="row-per-workgroup launch in plan order, not longest first")
@@ -242,7 +243,7 @@ def build_case(psi, wl, device, name, args):
         w = wl.make_workload(5, [4096 + 2048], 24, 4, 256, bf16, 16, q_lens=2048, host_pages=False)
         # 4096-token partitions: two rows per query tile, twice as many work items of half the size, which fill
         # the 256 compute units evenly (unsplit, 384 items make one and a half rounds: 375 against 323 us)
-        dw = wl.DeviceWorkload(device, w, partition_tokens=4096, grouped=True,
+        dw = wl.DeviceWorkload(device, w, partition_tokens=args.prefill_partition, grouped=True,
                                variant=psi.GQASplitKVVariant.TiledQ(8, 16, 6))
         case = Case(name, "prefill_chunk2048_on_prefix4096_24q4kv_d256_bf16_p16_part4096_seed5", [dw], "prefill",
                     "tiled_q_map", "split_kv_chunk_map", "kv append -> row-group (prefill-chunk) map -> LSE combine")

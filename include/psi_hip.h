@@ -114,9 +114,10 @@ int psi_hip_ctx_reset_timing(psi_hip_ctx* ctx);
 /* F32_OUTPUT makes the combine kernels store the attention output as f32 [tokens, Hq, D] instead of
  * the io dtype, so a harness can check the f32-accumulated result before output rounding. */
 #define PSI_HIP_FLAG_F32_OUTPUT 2u
-/* MUTE_LOADERS is for harnesses: while it is set, the loading waves of the multi-query and prefill-chunk maps never
- * say that a tile has landed, so that the other waves' waits (bounded at 65536 polls) run out, which sets
- * PSI_HIP_DEVICE_ERR_WAIT_GAVE_UP below while every kernel still runs to its end. */
+/* MUTE_LOADERS is for harnesses: while it is set, the loading waves of the multi-query map never say that a
+ * tile has landed, so that the other waves' waits (bounded at 65536 polls) run out, which sets
+ * PSI_HIP_DEVICE_ERR_WAIT_GAVE_UP below while every kernel still runs to its end.  (The prefill-chunk map
+ * has no such waits: its waves meet at workgroup barriers only.) */
 #define PSI_HIP_FLAG_MUTE_LOADERS 3u
 int psi_hip_ctx_set_flag(psi_hip_ctx* ctx, uint32_t flag, uint32_t value);
 
@@ -125,7 +126,7 @@ int psi_hip_ctx_set_flag(psi_hip_ctx* ctx, uint32_t flag, uint32_t value);
  * compute a row reports it in a word of pinned host memory that belongs to the context (written by the
  * GPU, read by the host after a synchronisation), and stores the affected partial rows as empty states
  * (maximum -inf, sum 0), so that no stale or half-computed row is merged.
- *   WAIT_GAVE_UP  a wave's bounded wait for another wave of its workgroup ran out;
+ *   WAIT_GAVE_UP  a wave's bounded wait for another wave of its workgroup ran out (multi-query map);
  *   V_RANGE       the prefill-chunk map met a V element of a bf16 cache that f16 cannot hold (finite
  *                 |v| > 65504, Inf or NaN): that map multiplies V as f16.  Run the batch through
  *                 psi_hip_split_kv_tiled_q_map instead, which keeps V in the storage type.
@@ -486,11 +487,11 @@ int psi_hip_split_kv_tiled_q_map_balanced(
     uint32_t num_active_q_token_tiles, uint32_t num_active_kv_splits, uint32_t max_active_q_tile_tokens);
 
 /* psi_hip_split_kv_tiled_q_map with one workgroup per (row group, KV head [, half of the Q heads]):
- * the group's K/V tiles are staged once in LDS for up to 128 query columns and both contractions run
+ * the group's K/V tiles are staged once in LDS for up to 256 query columns and both contractions run
  * on the matrix cores.  Same arguments, scratch layout and results (within rounding) as the plain map;
  * row_groups: device copy of the table of psi_hip_split_kv_tiled_q_group_rows for the same kv_splits.
- * Geometries outside the grouped kernel (other than bf16 / f16, head_dim 256, pages of 16*2^k tokens)
- * run the plain map. */
+ * Geometries outside the grouped kernel (other than bf16 / f16, head_dim 128 or 256, pages of 8*2^k
+ * tokens) run the plain map. */
 int psi_hip_split_kv_tiled_q_map_grouped(psi_hip_ctx* ctx, const psi_hip_gqa_config* cfg,
                                          const psi_hip_page_table_layout* layout, uint32_t q_token_tile_size,
                                          const void* q, const void* kv_pages, uint64_t kv_pages_bytes,

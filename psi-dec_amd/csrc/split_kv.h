@@ -138,9 +138,9 @@ inline int set_output_gate(ReduceArgs* a, const psi_hip_output_gate* gate, const
 // Prefill-chunk map: a workgroup serves up to kChunkCols query columns (tokens of a row group x
 // heads).  The heads of one KV head are dealt to chunk_head_subsets() workgroups, and a row group
 // holds up to chunk_group_tiles() Q-token tiles (0: the shape does not fit the kernel).
-constexpr int kChunkCols = 128;
-// Six heads per KV head go to three workgroups of two (two heads x 64 tokens fill the 128 columns; three heads x 40
-// tokens would leave eight of them empty).
+constexpr int kChunkCols = 256;
+// Six heads per KV head go to three workgroups of two (two heads x 128 tokens fill the 256 columns; three heads x 80
+// tokens would leave sixteen of them empty).
 inline uint32_t chunk_head_subsets(uint32_t group) { return group == 6 ? 3u : (group > 5 ? 2u : 1u); }
 inline uint32_t chunk_group_tiles(uint32_t group, uint32_t q_token_tile_size) {
     const uint32_t subsets = chunk_head_subsets(group);

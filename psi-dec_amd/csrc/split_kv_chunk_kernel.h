@@ -8,23 +8,31 @@
 //   one workgroup = one (row group, kv_head [, part of the query heads]).  A row group is a run of consecutive
 //   Q-token tiles of one request whose kv_split rows start at the same key (the rows of one KV partition).  With
 //   more than 5 query heads per KV head the heads are dealt to two or three workgroups.  The workgroup's query
-//   columns, column c = token_in_group * heads + head, are dealt out 16 per multiplying wave: a wave keeps the
-//   online-softmax state and the accumulators of its columns for the whole KV range, so wave states never merge.
+//   columns, column c = token_in_group * heads + head, are dealt out 32 per wave, as two blocks of 16: a wave keeps
+//   the online-softmax state and the accumulators of its columns for the whole KV range, so wave states never merge.
 //
-//   Twelve waves: eight that multiply (two per SIMD) and four that load (one per SIMD), around four LDS stages of
-//   32 keys.  A loading wave fetches its quarter of a tile into registers four tiles
-//   ahead (the tiles come from other compute units' L2 slices or from HBM, two microseconds away under load),
-//   stores it into the stage once every multiplying wave has said that it is through with the stage's previous
-//   tile, and announces it; a multiplying wave waits for the four announcements of its next tile, multiplies, and
-//   says so.  No barrier inside the range: the multiplying waves drift apart, and one wave's matrix work runs
-//   beside another's softmax and operand reads.  Every wait on another wave's word gives up after
-//   65536 polls: the wave then tells the host through MapArgs::status and waits no more, and the
-//   multiplying waves store empty states for the workgroup's columns; no wave stays behind.
+//   Eight waves, two per SIMD, each with half of the SIMD's registers.  Every operand of every product is read
+//   from LDS, and an operand read serves both column blocks of a wave, so a tile's K and V cross the LDS port once
+//   per 32 columns.  With 16 columns per wave (and then room for waves that only load) the same kernel spent its
+//   time on the LDS port - the transposing reads of V run at half the rate of 128-bit reads, 250 against 460
+//   bytes per nanosecond and compute unit - and reached a third of the matrix peak.  With one wave per SIMD nothing
+//   hides the latencies of a wave's own chain (operand reads, matrix results, exponentials); with two, each fills
+//   the other's gaps.
 //
-// Per 32-key tile and wave (16 columns)
+//   No wave only loads: every wave fetches four rows of K and four of V of every tile.  K goes straight to LDS
+//   with `global_load_lds_dwordx4`, which moves 16 bytes per lane from a per-lane global address to LDS address
+//   M0 + 16 * lane with no register in between, three tiles ahead, into a ring of four K tiles.  V goes through
+//   registers, two tiles ahead (two register sets, taken in turn), where bf16 becomes f16, into a ring of two V
+//   tiles.  One barrier per tile, B(t): before it a wave has stored its V rows of tile t and seen its K rows of
+//   tile t + 1 land (a wave's loads complete in the order of their issue); behind it everybody has, and every
+//   wave is through with tile t - 1.  No wait between waves other than the barrier, so none that could run out.
+//
+// Per 32-key tile and wave (2 x 16 columns)
 //   QK^T  S[key][column] on v_mfma_f32_16x16x32 of the storage type: A = K rows from LDS (key 16 * b + i in row i of
-//         key block b), B = the query columns, held in registers for the whole kernel.  A lane ends up with keys
-//         16 * b + 4 * (lane / 16) + r, r = 0..3, b = 0, 1, of its column.
+//         key block b), B = the query columns: the first block's held in registers for the whole kernel, the second
+//         block's read from LDS with the K operands (64 registers of queries next to 128 accumulators and the V
+//         rows under way are more than a wave has).  A lane ends up with keys 16 * b + 4 * (lane / 16) + r,
+//         r = 0..3, b = 0, 1, of its column.
 //   softmax  per column, in-lane over those 8 keys; masks only on tiles that touch the start of the range
 //         or a column's causal limit.  The reference maximum of a column moves only when a tile
 //         exceeds it by more than 2^8; a wave-wide vote guards the cross-lane maximum and the
@@ -37,50 +45,38 @@
 //         row-major V tile with the transposing LDS read of gfx950 (ds_read_b64_tr_b16: the 16 lanes of a quarter
 //         wave hand in 16 addresses of 4 elements each, a 16 x 4 block, and get it back transposed - lane 4a + c
 //         receives element c of the addresses a, a + 4, a + 8, a + 12), so no instruction of the kernel
-//         transposes V.  The V tile is kept as f16 in LDS: bf16 pages are converted once per tile, to nearest, on
-//         their way from the load registers into LDS (exact for 6.1e-5 <= |v| <= 65504; smaller magnitudes keep
+//         transposes V.  The V tile is kept as f16 in LDS: bf16 rows are converted once per tile, to nearest, by
+//         the wave that fetched them (exact for 6.1e-5 <= |v| <= 65504; smaller magnitudes keep
 //         an absolute spacing of 6e-8; larger ones become Inf, reach the accumulators as Inf or NaN, and are
 //         reported to the host through MapArgs::status).  The accumulators keep a column per lane, so rescaling
 //         needs no cross-lane traffic.
 //
-// LDS layout per stage
-//   K    [32 keys][D] elements, 16-byte chunk index XOR (key % 16): the 16 lanes of an operand read (16 rows, one
-//        chunk) then hit 16 different bank groups, and a row-wise store stays a permutation of its row.
-//   V    [32 keys][D] f16, rows padded to D * 2 + 32 bytes: the four keys of a quarter wave's transposing read
-//        (32 bytes each, 16 dims) then fall into different bank groups, and so do the eight keys of two quarters.
-//   and thirteen words: tiles stored, per loading wave; tiles read, per multiplying wave; and one that says that
-//   some wave's wait ran out (and four that nobody reads).
+// LDS layout
+//   K    four tiles of [32 keys][D] elements, 16-byte chunk index XOR (key % 16): the 16 lanes of an operand read
+//        (16 rows, one chunk) then hit 16 different bank groups.  (The loads write 1 KiB in lane order, so the
+//        layout can permute 16-byte chunks within a row, through the choice of each lane's global address, but
+//        cannot pad rows.)
+//   V    two tiles of [32 keys][D] f16, 32-byte chunk index XOR (key % 8): the four keys of a quarter wave's
+//        transposing read (32 bytes each, 16 dims) then fall into different bank groups, and so do the eight keys
+//        of two quarters.
+//   Q    the second column block's query operands, 4 or 8 KiB per wave.
 #pragma once
 #include <atomic>
+#include <type_traits>
 
 #include "split_kv_tiled_kernel.h"
 
 namespace psi {
 
-constexpr int kChunkKeys = 32;         // keys per KV tile
-constexpr int kChunkWaves = 8;          // multiplying waves
-constexpr int kChunkLoaders = 4;        // loading waves
-constexpr int kChunkStages = 4;         // KV tiles in LDS
-constexpr int kChunkWaveCols = 16;      // query columns of a multiplying wave
-static_assert(kChunkWaves * kChunkWaveCols == kChunkCols, "128 query columns per workgroup");
+constexpr int kChunkKeys = 32;      // keys per KV tile
+constexpr int kChunkColBlocks = 2;  // 16-column blocks of a wave
+constexpr int kChunkWaves = 8;
+constexpr int kChunkStages = 4;   // K tiles in LDS
+constexpr int kChunkVStages = 2;  // V tiles in LDS
+constexpr int kChunkWaveCols = 16 * kChunkColBlocks;
+static_assert(kChunkWaves * kChunkWaveCols == kChunkCols, "the workgroup's query columns");
 constexpr uint32_t kNoRow = 0xffffffffu;
 typedef __attribute__((ext_vector_type(4))) uint32_t u32x4_t;  // 128-bit word that stays in registers
-
-// Probabilities of 8 keys -> B operand of the 16x16x32 f16 contraction: one term, rounded to nearest.
-__device__ __forceinline__ uint4 prob_operand_f16(const float (&p)[8]) {
-    const f16x8_t h = {(_Float16)p[0], (_Float16)p[1], (_Float16)p[2], (_Float16)p[3],
-                       (_Float16)p[4], (_Float16)p[5], (_Float16)p[6], (_Float16)p[7]};
-    return __builtin_bit_cast(uint4, h);
-}
-
-// sum + the eight f16 values of `packed`, in f32.
-__device__ __forceinline__ float add_f16x8(uint4 packed, float sum) {
-    const f16x2_t ones = {(_Float16)1.0f, (_Float16)1.0f};
-    sum = __builtin_amdgcn_fdot2(__builtin_bit_cast(f16x2_t, packed.x), ones, sum, false);
-    sum = __builtin_amdgcn_fdot2(__builtin_bit_cast(f16x2_t, packed.y), ones, sum, false);
-    sum = __builtin_amdgcn_fdot2(__builtin_bit_cast(f16x2_t, packed.z), ones, sum, false);
-    return __builtin_amdgcn_fdot2(__builtin_bit_cast(f16x2_t, packed.w), ones, sum, false);
-}
 
 // max(a, b, c) in one instruction.  The logits are matrix-core results: a NaN among them (NaN in K or Q) ends up in
 // the probabilities either way, so the operands need not be canonicalised first, as fmaxf would have them.
@@ -119,42 +115,48 @@ __device__ __forceinline__ uint32_t wave_max_u32(uint32_t v) {
     return v;
 }
 
+// 16 bytes per lane from rows + lane_offset to LDS address lds_dst + 16 * lane.  `rows` and `lds_dst` are the same
+// in every lane (scalar registers).  Assembly, and so are the waits for these loads: the compiler does not know that
+// they write LDS, and where it does (the builtin) it waits for every outstanding one before any LDS read, which
+// would undo the prefetch.
+__device__ __forceinline__ void dma_16_bytes_per_lane(uint32_t lds_dst, const void* rows, uint32_t lane_offset) {
+    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2"
+                 :
+                 : "s"(lds_dst), "v"(lane_offset), "s"(rows)
+                 : "memory", "m0");
+}
+
 template <int D>
 struct ChunkLds {
-    static constexpr int kKBytes = kChunkKeys * D * 2;
-    static constexpr int kVStride = D * 2 + 32;  // bytes per key row of the V tile
-    static constexpr int kVtBytes = kChunkKeys * kVStride;
-    static constexpr int kStageBytes = kKBytes + kVtBytes;
-    static constexpr int kFlagsOffset = kChunkStages * kStageBytes;
-    // tiles stored per loading wave [4], tiles read per multiplying wave [8], a wait ran out [1]
-    static constexpr int bytes = kFlagsOffset + 64;
+    static constexpr int kKBytes = kChunkKeys * D * 2;  // a tile of K, and of V
+    static constexpr int kVOffset = kChunkStages * kKBytes;
+    static constexpr int kQOffset = kVOffset + kChunkVStages * kKBytes;
+    static constexpr int kQSteps = D / 32;  // k-steps of a wave's second column block whose query operands live here: all
+    static constexpr int bytes = kQOffset + kChunkWaves * kQSteps * 1024;
 };
 
-// kPage8: pages of eight tokens (a tile then spans four pages instead of one or two).
-template <typename Tag, int D, bool kPage8>
-__global__ __launch_bounds__(64 * (kChunkWaves + kChunkLoaders), 1) void split_kv_chunk_map(
+template <typename Tag, int D>
+__global__ __launch_bounds__(64 * kChunkWaves, 1) void split_kv_chunk_map(
     MapArgs a, const uint32_t* __restrict__ page_ids, const uint32_t* __restrict__ kv_splits,
     const uint32_t* __restrict__ req_slots, const uint16_t* __restrict__ q, const uint16_t* __restrict__ pages,
     const uint32_t* __restrict__ q_token_tiles, const uint32_t* __restrict__ flat_token_indices,
     const uint32_t* __restrict__ row_groups, uint32_t group_tiles, uint32_t num_groups, uint32_t head_subsets) {
     resolve_active(a);
     static_assert(D == 256 || D == 128, "head_dim 128 or 256");
+    constexpr int NB = kChunkColBlocks;
     constexpr int kKSteps = D / 32;
     constexpr int kDimBlocks = D / 16;
-    constexpr int kRowChunks = D / 8;                      // 16-byte chunks per key row
-    constexpr int kSubs = 64 * kChunkLoaders / kRowChunks;  // keys that the loading threads cover at a time (8 or 16)
-    constexpr int kLoads = kChunkKeys / kSubs;               // 128-bit loads per loading thread and operand (4 or 2)
+    constexpr int kRowBytes = D * 2;
+    constexpr int kRowChunks = D / 8;                    // 16-byte chunks per key row: 32 or 16
+    constexpr int kRowsPerLoad = 64 / kRowChunks;        // key rows that one load of a wave covers: 2 or 4
+    constexpr int kWaveRows = kChunkKeys / kChunkWaves;  // rows of K, and of V, that a wave fetches per tile
+    constexpr int kLoads = kWaveRows / kRowsPerLoad;     // loads per wave, tile and operand: 2 or 1
     constexpr int kKBytes = ChunkLds<D>::kKBytes;
-    constexpr int kVStride = ChunkLds<D>::kVStride;
-    constexpr int kStageBytes = ChunkLds<D>::kStageBytes;
+    constexpr int kVOffset = ChunkLds<D>::kVOffset;
+    constexpr int kQSteps = ChunkLds<D>::kQSteps;
+    static_assert(kQSteps == kKSteps, "the second block's queries live in LDS");
     constexpr float kSlack = 8.0f;
     extern __shared__ __attribute__((aligned(16))) unsigned char lds[];
-    // Progress words, addressed as LDS: through a generic pointer a volatile access becomes a flat one, which
-    // counts as a global load too, and waiting for its value would wait for every tile load in flight.
-    typedef volatile __attribute__((address_space(3))) uint32_t* LdsWords;
-    const LdsWords landed = (LdsWords)(lds + ChunkLds<D>::kFlagsOffset);  // tiles stored, per loading wave
-    const LdsWords done = landed + kChunkLoaders;                          // tiles read, per multiplying wave
-    const LdsWords failed = done + kChunkWaves;                            // some wave's wait ran out
 
     const uint32_t TS = a.rows_per_split_head;
     const uint32_t subset = blockIdx.x % head_subsets;
@@ -166,6 +168,7 @@ __global__ __launch_bounds__(64 * (kChunkWaves + kChunkLoaders), 1) void split_k
     const uint32_t lane = tid & 63;
     const uint32_t wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const uint32_t mt = lane & 15, mc = lane >> 4;
+    // (every exit before the tile loop is taken by the whole workgroup or by none of it)
     if (group >= num_groups || subset * heads_per_subset >= a.group) return;
     const uint32_t G = min(heads_per_subset, a.group - subset * heads_per_subset);
 
@@ -190,278 +193,298 @@ __global__ __launch_bounds__(64 * (kChunkWaves + kChunkLoaders), 1) void split_k
     const uint32_t key_base0 = kv_begin & ~(uint32_t)(kChunkKeys - 1);
     const uint32_t num_kv_tiles = (kv_end_max - key_base0 + kChunkKeys - 1) / kChunkKeys;
 
-    if (tid < kChunkLoaders + kChunkWaves + 1) landed[tid] = 0u;
-    __syncthreads();
-    // Both roles poll with the word of wave (lane % count) in each lane and a wave-wide vote.  A wait that runs out
-    // marks the workgroup's results as void (every multiplying wave looks at `failed` when it is through, tells the
-    // host and stores empty states); the wave itself goes on without waiting any more, so that nothing of this
-    // costs the tile loops a branch.
-    // The bound is a constant and the loop the only one, so that it stays the plain unrolled poll: a run-time bound
-    // in it, a second loop or a second path next to it each cost 1 to 5 % of the launch.
-    bool impatient = false;
-    auto wait_all_above = [&](LdsWords words, uint32_t count_mask, uint32_t value) __attribute__((always_inline)) {
-        bool there = impatient;
-        if (!impatient) {
-            for (uint32_t polls = 0; polls < kDefaultWaitPolls; ++polls) {
-                there = __all(words[lane & count_mask] > value);
-                if (there) break;
-                __builtin_amdgcn_s_sleep(1);
-            }
-        }
-        if (!there) {
-            // Only an LDS word here: a global store on this path would make every count of outstanding loads that
-            // the compiler keeps for the loading waves a guess, and its partial waits full ones.
-            impatient = true;  // `there` stays true from here on: the wave waits no more
-            if (lane == 0) *failed = 1u;
-        }
-        asm volatile("" ::: "memory");
+    // ---------------- the wave's columns ----------------
+    // The partial row of column block j of this lane's column: (row of the tile's split, head, token in the tile).
+    // Worked out where it is needed, at either end of the kernel, rather than kept in registers through the loop.
+    auto column_of = [&](int j, uint32_t* t, uint32_t* h) -> bool {
+        const uint32_t c = wave * kChunkWaveCols + 16 * j + mt;
+        *t = c < ncols ? c / G : 0u;
+        *h = c < ncols ? c % G : 0u;
+        return c < ncols;
     };
-
-    if (wave >= (uint32_t)kChunkWaves) {
-        // =========================== a loading wave ===========================
-        // A loading thread takes one 16-byte chunk of the keys sub, sub + kSubs, ... of every tile, so that a wave's
-        // load covers whole rows (two of 512 bytes, or four of 256).
-        const uint32_t lw = wave - kChunkWaves;
-        const uint32_t log2p = 31 - __builtin_clz(a.walk.tokens_per_page);
-        const uint32_t page_mask = a.walk.tokens_per_page - 1;
-        const uint32_t* table_row = page_ids + ((uint64_t)req_slot * a.walk.num_layers + a.layer) *
-                                                          a.walk.num_blocks * a.walk.ids_per_block;
-        const uint32_t last_page = (kv_end_max - 1) >> log2p;
-        const uint64_t page_bytes = a.walk.page_elems * 2;
-        const unsigned char* base = reinterpret_cast<const unsigned char*>(pages);
-        // Page ids come through the scalar cache: a vector load would queue behind the tile loads in flight, and
-        // waiting for it would wait for all of them.  A tile's ids are fetched one step before its loads are
-        // issued.  Tiles past the end of the range are clamped to the last one, so that loads stay unconditional.
-        typedef const __attribute__((address_space(4))) uint32_t* ConstantIds;
-        const ConstantIds ids_row = (ConstantIds)(uintptr_t)table_row;
-        constexpr int kIds = kPage8 ? 4 : 2;  // pages under a tile's 32 keys
-        struct TileIds {
-            uint32_t id[kIds];
-        };
-        auto tile_key = [&](uint32_t t) { return key_base0 + min(t, num_kv_tiles - 1) * kChunkKeys; };
-        auto fetch_ids = [&](uint32_t t) -> TileIds {
-            const uint32_t kb = tile_key(t);
-            TileIds ids;
+    bool used[NB];
+    uint32_t lim[NB];
+    unsigned char* q_lds = lds + ChunkLds<D>::kQOffset + wave * (kQSteps * 1024) + lane * 16;
+    uint4 qreg[kKSteps];  // the first block's; the second block's live in LDS
 #pragma unroll
-            for (int j = 0; j < kIds; ++j) ids.id[j] = ids_row[min((kb + (kChunkKeys / kIds) * j) >> log2p, last_page)];
-            return ids;
-        };
-        const uint32_t ltid = tid - 64 * kChunkWaves;
-        const uint32_t ld_chunk = ltid % kRowChunks;
-        const uint32_t ld_sub = ltid / kRowChunks;  // 0 .. kSubs - 1; load i takes key ld_sub + kSubs * i of the tile
-        // The keys of one load of a wave lie in one run of eight (ld_sub / 8 is the same for the whole wave): the
-        // run's rows are found with scalar arithmetic, and a lane adds a constant.
-        const uint32_t run_first = kSubs == 8 ? 0u : __builtin_amdgcn_readfirstlane(ld_sub & ~7u);
-        const uint32_t lane_off = (ld_sub & 7) * (D * 2) + ld_chunk * 16;
-        const uint32_t k_off = kv_head * a.walk.tokens_per_page * (D * 2) + lane_off;
-        const uint32_t v_off = (a.walk.hkv + kv_head) * a.walk.tokens_per_page * (D * 2) + lane_off;
-        struct Staging {
-            u32x4_t k[kLoads], v[kLoads];
-        };
-        auto issue_loads = [&](uint32_t t, const TileIds& ids) __attribute__((always_inline)) -> Staging {
-            const uint32_t kb = tile_key(t);
-            Staging st;
-            const unsigned char* rows_of_run[kLoads];
-#pragma unroll
-            for (int i = 0; i < kLoads; ++i) {
-                const uint32_t first = kSubs * i + run_first;  // of the tile's keys
-                uint32_t id;
-                if constexpr (kSubs == 8 || !kPage8) id = ids.id[(kSubs * i) / (kChunkKeys / kIds)];
-                else id = run_first == 0 ? ids.id[2 * i] : ids.id[2 * i + 1];
-                rows_of_run[i] = base + id * page_bytes + (uint64_t)((kb + first) & page_mask) * (D * 2);
-            }
-#pragma unroll
-            for (int i = 0; i < kLoads; ++i) st.k[i] = *reinterpret_cast<const u32x4_t*>(rows_of_run[i] + k_off);
-#pragma unroll
-            for (int i = 0; i < kLoads; ++i) st.v[i] = *reinterpret_cast<const u32x4_t*>(rows_of_run[i] + v_off);
-            return st;
-        };
-        // Where this wave says that a tile is stored.  A harness that wants to see waits run out (MapArgs::
-        // mute_loaders) has the word written where no wave looks.
-        const LdsWords announce = a.mute_loaders ? failed + 1 + lw : landed + lw;
-        uint32_t k_store[kLoads], v_store[kLoads];
-#pragma unroll
-        for (int i = 0; i < kLoads; ++i) {
-            const uint32_t key = ld_sub + kSubs * i;
-            k_store[i] = key * (D * 2) + ((ld_chunk ^ (key & 15)) * 16);
-            v_store[i] = kKBytes + key * kVStride + ld_chunk * 16;
-        }
-        auto store_tile = [&](uint32_t it, Staging& st) __attribute__((always_inline)) {
-            if (it >= (uint32_t)kChunkStages) wait_all_above(done, kChunkWaves - 1, it - kChunkStages);
-            unsigned char* stage = lds + (it % kChunkStages) * kStageBytes;
-            const uint32_t kb = key_base0 + it * kChunkKeys;
-            const bool edge = kb < kv_begin || kb + kChunkKeys > kv_end_max;  // first or last tile of the range
-#pragma unroll
-            for (int i = 0; i < kLoads; ++i) *reinterpret_cast<u32x4_t*>(stage + k_store[i]) = st.k[i];
-#pragma unroll
-            for (int i = 0; i < kLoads; ++i) {
-                u32x4_t w = to_f16x8<Tag>(st.v[i]);
-                const uint32_t token = kb + ld_sub + kSubs * i;
-                // V rows outside the range are zeroed: their probability is 0 but their bytes may be NaN / Inf
-                if (edge && (token < kv_begin || token >= kv_end_max)) w = u32x4_t{0u, 0u, 0u, 0u};
-                *reinterpret_cast<u32x4_t*>(stage + v_store[i]) = w;
-            }
-            if (lane == 0) *announce = it + 1;  // behind the stores in the LDS queue
-        };
-        // Four tiles of loads in flight per wave (one register set per stage): the tiles come from the other
-        // compute units' L2 slices or from HBM, two microseconds away under load, and a tile is used up in less
-        // than one.
-        Staging st_a = issue_loads(0, fetch_ids(0));
-        Staging st_b = issue_loads(1, fetch_ids(1));
-        Staging st_c = issue_loads(2, fetch_ids(2));
-        Staging st_d = issue_loads(3, fetch_ids(3));
-        TileIds ids = fetch_ids(4);
-        auto step = [&](uint32_t it, Staging& st) __attribute__((always_inline)) {
-            if (it < num_kv_tiles) store_tile(it, st);
-            st = issue_loads(it + kChunkStages, ids);
-            ids = fetch_ids(it + kChunkStages + 1);
-        };
-        for (uint32_t it = 0; it < num_kv_tiles; it += 4) {
-            step(it, st_a);
-            step(it + 1, st_b);
-            step(it + 2, st_c);
-            step(it + 3, st_d);
-        }
-        return;
-    }
-
-    // =========================== a multiplying wave ===========================
-    const uint32_t c = wave * kChunkWaveCols + mt;
-    const bool used = c < ncols;
-    uint32_t lim = 0;
-    uint64_t part_row = 0;
-    uint4 qreg[kKSteps];
-    {
-        const uint32_t t = used ? c / G : 0u, h = used ? c % G : 0u;
-        const uint32_t m = t / TS, r = t % TS;
-        const uint32_t row = rows[m];
-        if (used) {
-            lim = min(kv_splits[row * 3 + 2], flat_token_indices[flat_begin + t] + 1);
-            part_row = ((uint64_t)row * a.hq + head_first + h) * TS + r;
-        }
+    for (int j = 0; j < NB; ++j) {
+        uint32_t t, h;
+        used[j] = column_of(j, &t, &h);
+        lim[j] = 0;
+        if (used[j]) lim[j] = min(kv_splits[rows[t / TS] * 3 + 2], flat_token_indices[flat_begin + t] + 1);
         const uint16_t* q_row = q + ((uint64_t)(flat_begin + t) * a.hq + head_first + h) * D + mc * 8;
 #pragma unroll
-        for (int ks = 0; ks < kKSteps; ++ks)
-            qreg[ks] = used ? *reinterpret_cast<const uint4*>(q_row + ks * 32) : make_uint4(0, 0, 0, 0);
+        for (int ks = 0; ks < kKSteps; ++ks) {
+            const uint4 operand = used[j] ? *reinterpret_cast<const uint4*>(q_row + ks * 32) : make_uint4(0, 0, 0, 0);
+            if (j == 0) qreg[ks] = operand;
+            else *reinterpret_cast<uint4*>(q_lds + ks * 1024) = operand;
+        }
     }
-    const uint32_t wave_lo = __builtin_amdgcn_readfirstlane(wave_min_u32(used ? lim : 0xffffffffu));
-    const uint32_t wave_hi = __builtin_amdgcn_readfirstlane(wave_max_u32(lim));
-    // tiles that hold a visible key of this wave
-    const uint32_t my_tiles = wave_hi > key_base0 ? min(num_kv_tiles, (wave_hi - key_base0 + kChunkKeys - 1) / kChunkKeys) : 0u;
-
-    const uint32_t k_row0 = mt * (D * 2);
-    const uint32_t vt_base = (4 * mc + (mt >> 2)) * kVStride + (mt & 3) * 8;
-    float run_max = -INFINITY, lane_sum = 0.0f;
-    f32x4_t o[kDimBlocks];
+    uint32_t lo = 0xffffffffu, hi = 0;
 #pragma unroll
-    for (int db = 0; db < kDimBlocks; ++db) o[db] = f32x4_t{0.0f, 0.0f, 0.0f, 0.0f};
+    for (int j = 0; j < NB; ++j) {
+        lo = min(lo, used[j] ? lim[j] : 0xffffffffu);
+        hi = max(hi, lim[j]);
+    }
+    const uint32_t wave_lo = __builtin_amdgcn_readfirstlane(wave_min_u32(lo));
+    const uint32_t wave_hi = __builtin_amdgcn_readfirstlane(wave_max_u32(hi));
+    // tiles that hold a visible key of this wave, and of any wave of the workgroup
+    const uint32_t my_tiles =
+        wave_hi > key_base0 ? min(num_kv_tiles, (wave_hi - key_base0 + kChunkKeys - 1) / kChunkKeys) : 0u;
+    uint32_t* tile_counts = reinterpret_cast<uint32_t*>(lds);  // (where the first tile will land)
+    if (lane == 0) tile_counts[wave] = my_tiles;
+    __syncthreads();
+    const uint32_t group_kv_tiles =
+        __builtin_amdgcn_readfirstlane(wave_max_u32(lane < (uint32_t)kChunkWaves ? tile_counts[lane] : 0u));
+    __syncthreads();
+    // None of the loads above may be outstanding when the tile loads begin: the compiler's waits count the loads it
+    // knows of, and the tile loads are not among them.
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
 
-    constexpr int kAhead = kKSteps < 4 ? kKSteps : 4;  // k-steps between an operand's read and its product
-    for (uint32_t it = 0; it < my_tiles; ++it) {
-        wait_all_above(landed, kChunkLoaders - 1, it);
-        const unsigned char* kbuf = lds + (it % kChunkStages) * kStageBytes;
-        const unsigned char* vbuf = kbuf + kKBytes;
+    // ---------------- the wave's share of the tile loads ----------------
+    const uint32_t log2p = 31 - __builtin_clz(a.walk.tokens_per_page);
+    const uint32_t page_mask = a.walk.tokens_per_page - 1;
+    const uint32_t* table_row = page_ids + ((uint64_t)req_slot * a.walk.num_layers + a.layer) * a.walk.num_blocks *
+                                               a.walk.ids_per_block;
+    const uint64_t page_bytes = a.walk.page_elems * 2;
+    const unsigned char* base = reinterpret_cast<const unsigned char*>(pages);
+    // Page ids come through the scalar cache.  The wave's four rows of a tile lie in one page (pages hold at least
+    // 8 tokens).  Rows past the end of the range (the last tile's) are taken from the range's last page: the table
+    // need not hold a page for them, and nobody looks at what they hold.  Tiles past the last one are clamped to it,
+    // so that every iteration issues the same number of loads and the counts of outstanding ones stay constants.
+    const uint32_t last_page = (kv_end_max - 1) >> log2p;
+    typedef const __attribute__((address_space(4))) uint32_t* ConstantIds;
+    const ConstantIds ids_row = (ConstantIds)(uintptr_t)table_row;
+    auto first_key = [&](uint32_t t) { return key_base0 + min(t, group_kv_tiles - 1) * kChunkKeys + kWaveRows * wave; };
+    auto page_of = [&](uint32_t t) -> uint32_t { return ids_row[min(first_key(t) >> log2p, last_page)]; };
+    auto rows_of = [&](uint32_t t, uint32_t id) -> const unsigned char* {
+        return base + id * page_bytes + (uint64_t)(first_key(t) & page_mask) * kRowBytes;
+    };
+    const uint32_t k_plane = kv_head * a.walk.tokens_per_page * kRowBytes;
+    const uint32_t v_plane = (a.walk.hkv + kv_head) * a.walk.tokens_per_page * kRowBytes;
+    const uint32_t lds0 = (uint32_t)(size_t)(__attribute__((address_space(3))) unsigned char*)(lds);
+    const uint32_t row_in_load = lane / kRowChunks, slot = lane % kRowChunks;
+    // K goes from global memory straight to LDS; where in the wave's rows a lane's 16 bytes come from:
+    uint32_t k_lane[kLoads];
+    // V goes through registers, where bf16 becomes f16; where in the wave's rows of a stage a lane's 16 bytes go:
+    uint32_t v_lane[kLoads];
+#pragma unroll
+    for (int i = 0; i < kLoads; ++i) {
+        const uint32_t key = kWaveRows * wave + kRowsPerLoad * i + row_in_load;  // in the tile
+        k_lane[i] = (kRowsPerLoad * i + row_in_load) * kRowBytes + ((slot ^ (key & 15)) * 16);
+        v_lane[i] = (kRowsPerLoad * i + row_in_load) * kRowBytes + (((((slot >> 1) ^ (key & 7)) << 1) | (slot & 1)) * 16);
+    }
+    const uint32_t v_from = row_in_load * kRowBytes + slot * 16;  // (the rows of load i begin kRowsPerLoad * i rows on)
+    auto issue_k_loads = [&](uint32_t t, uint32_t id) __attribute__((always_inline)) {
+        const unsigned char* rows_at = rows_of(t, id) + k_plane;
+        const uint32_t dst = lds0 + (t % kChunkStages) * kKBytes + kWaveRows * wave * kRowBytes;
+#pragma unroll
+        for (int i = 0; i < kLoads; ++i) dma_16_bytes_per_lane(dst + i * 1024, rows_at, k_lane[i]);
+    };
+    struct VRows {
+        u32x4_t w[kLoads];
+    };
+    auto load_v_rows = [&](uint32_t t, uint32_t id, VRows& r) __attribute__((always_inline)) {
+        const unsigned char* rows_at = rows_of(t, id) + v_plane + v_from;
+#pragma unroll
+        for (int i = 0; i < kLoads; ++i)
+            r.w[i] = *reinterpret_cast<const u32x4_t*>(rows_at + i * (kRowsPerLoad * kRowBytes));
+    };
+    // The wave's V rows of tile t into their stage: as f16, and zero where a row lies outside the range - its
+    // probability is 0, but its bytes may be NaN or Inf.
+    auto store_v_rows = [&](uint32_t t, const VRows& r) __attribute__((always_inline)) {
+        const uint32_t kb = key_base0 + t * kChunkKeys;
+        const bool edge = kb < kv_begin || kb + kChunkKeys > kv_end_max;  // first or last tile of the range
+        unsigned char* mine = lds + kVOffset + (t % kChunkVStages) * kKBytes + kWaveRows * wave * kRowBytes;
+#pragma unroll
+        for (int i = 0; i < kLoads; ++i) {
+            u32x4_t w = to_f16x8<Tag>(r.w[i]);
+            const uint32_t token = kb + kWaveRows * wave + kRowsPerLoad * i + row_in_load;
+            if (edge && (token < kv_begin || token >= kv_end_max)) w = u32x4_t{0u, 0u, 0u, 0u};
+            *reinterpret_cast<u32x4_t*>(mine + v_lane[i]) = w;
+        }
+    };
+    // everything this wave has written to LDS is there, and every wave has come this far
+    auto barrier = []() __attribute__((always_inline)) { asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory"); };
+
+    const uint32_t k_row0 = mt * kRowBytes;
+    // transposing reads: key 4 * mc + mt / 4 (and 16 on), dims 16 * db + 4 * (mt % 4) ..; the 32-byte chunk db of a
+    // row sits at chunk db ^ (key % 8)
+    const uint32_t v_key = 4 * mc + (mt >> 2);
+    const uint32_t v_row0 = v_key * kRowBytes + (mt & 3) * 8;
+    const uint32_t v_swizzle = (v_key & 7) * 32;
+    float run_max[NB], lane_sum[NB];
+    f32x4_t o[NB][kDimBlocks];
+#pragma unroll
+    for (int j = 0; j < NB; ++j) {
+        run_max[j] = -INFINITY;
+        lane_sum[j] = 0.0f;
+#pragma unroll
+        for (int db = 0; db < kDimBlocks; ++db) o[j][db] = f32x4_t{0.0f, 0.0f, 0.0f, 0.0f};
+    }
+
+    // ---------------- the tile loop ----------------
+    // One barrier per tile, B(t).  Before it a wave has stored its V rows of tile t (in the middle of the tile
+    // before) and seen its K rows of tile t + 1 land; behind it everybody has, and every wave is through with tile
+    // t - 1: its K stage takes the loads of tile t + 3, and its V stage the rows of tile t + 1.  So behind B(t) a
+    // wave asks for its K rows of tile t + 3 and multiplies K * Q^T of tile t; then it stores its V rows of tile
+    // t + 1, which it asked for two tiles ago (two register sets, taken in turn), and asks for those of tile t + 3;
+    // then the softmax and the products with V.  The loads complete in the order of their issue: at the barrier
+    // the K rows of tile t + 1 are followed by the V rows of tile t + 1, the K rows of tile t + 2 and the V rows
+    // of tile t + 2.
+    constexpr int kAhead = 1;  // k-steps between an operand's read and its product
+    uint32_t next_id = 0;
+    auto tile = [&](uint32_t it, VRows& v_rows) __attribute__((always_inline)) {
+        asm volatile("s_waitcnt vmcnt(%0)" ::"n"(3 * kLoads) : "memory");
+        barrier();
+        const uint32_t id = next_id;   // of tile it + 3, asked for a tile ago: a page id takes as long as an LDS round trip,
+        next_id = page_of(it + 4);     // and waiting for it waits for every LDS read in flight as well
+        issue_k_loads(it + 3, id);
+        const bool mine = it < my_tiles;  // (a wave that sees none of the tile's keys still does its share of the loads)
+
+        const unsigned char* kbuf = lds + (it % kChunkStages) * kKBytes;
+        const unsigned char* vbuf = lds + kVOffset + (it % kChunkVStages) * kKBytes;
         const uint32_t kb = key_base0 + it * kChunkKeys;
         const bool masked = !(kb >= kv_begin && kb + kChunkKeys <= wave_lo);
-        f32x4_t s0 = f32x4_t{0.0f, 0.0f, 0.0f, 0.0f}, s1 = s0;
-        uint4 k0[kKSteps], k1[kKSteps];
+        f32x4_t s0[NB], s1[NB];
+#pragma unroll
+        for (int j = 0; j < NB; ++j) s0[j] = s1[j] = f32x4_t{0.0f, 0.0f, 0.0f, 0.0f};
+        if (mine) {
+        uint4 k0[kKSteps], k1[kKSteps], q1[kKSteps];
+        // the operands of k-step ks: two key blocks of K, and the second column block's queries
         auto read_k = [&](int ks) __attribute__((always_inline)) {
             const uint32_t off = k_row0 + (((4 * ks + mc) ^ mt) * 16);
             k0[ks] = *reinterpret_cast<const uint4*>(kbuf + off);
-            k1[ks] = *reinterpret_cast<const uint4*>(kbuf + off + 16 * (D * 2));
+            k1[ks] = *reinterpret_cast<const uint4*>(kbuf + off + 16 * kRowBytes);
+            q1[ks] = *reinterpret_cast<const uint4*>(q_lds + ks * 1024);
         };
         __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
         for (int ks = 0; ks < kAhead; ++ks) read_k(ks);
 #pragma unroll
         for (int ks = 0; ks < kKSteps; ++ks) {
-            s0 = mfma_16x16x32<Tag>(k0[ks], qreg[ks], s0);
-            s1 = mfma_16x16x32<Tag>(k1[ks], qreg[ks], s1);
+            s0[0] = mfma_16x16x32<Tag>(k0[ks], qreg[ks], s0[0]);
+            s1[0] = mfma_16x16x32<Tag>(k1[ks], qreg[ks], s1[0]);
+            s0[1] = mfma_16x16x32<Tag>(k0[ks], q1[ks], s0[1]);
+            s1[1] = mfma_16x16x32<Tag>(k1[ks], q1[ks], s1[1]);
             if (ks + kAhead < kKSteps) read_k(ks + kAhead);
         }
-        __builtin_amdgcn_sched_group_barrier(0x100, 2 * kAhead, 0);  // the first reads
+        __builtin_amdgcn_sched_group_barrier(0x100, 3 * kAhead, 0);  // the first reads
 #pragma unroll
         for (int ks = 0; ks < kKSteps - kAhead; ++ks) {
-            __builtin_amdgcn_sched_group_barrier(0x008, 2, 0);  // two products
-            __builtin_amdgcn_sched_group_barrier(0x100, 2, 0);  // the reads kAhead steps on
+            __builtin_amdgcn_sched_group_barrier(0x008, 4, 0);  // the products of a k-step
+            __builtin_amdgcn_sched_group_barrier(0x100, 3, 0);  // the reads kAhead steps on
         }
-        __builtin_amdgcn_sched_group_barrier(0x008, 2 * kAhead, 0);
+        __builtin_amdgcn_sched_group_barrier(0x008, 4 * kAhead, 0);
         __builtin_amdgcn_sched_barrier(0);
-        float v[8];
-#pragma unroll
-        for (int j = 0; j < 8; ++j) v[j] = j < 4 ? s0[j] : s1[j - 4];
-        if (masked) {
-#pragma unroll
-            for (int j = 0; j < 8; ++j) {
-                const uint32_t token = kb + 16 * (j >> 2) + 4 * mc + (j & 3);
-                if (token < kv_begin || token >= lim) v[j] = -INFINITY;
-            }
         }
-        float m = max3(max3(v[0], v[1], v[2]), max3(v[3], v[4], v[5]), fmaxf(v[6], v[7])) * a.scale_log2;
-        if (__any(m > run_max + kSlack)) {
-            m = fmaxf(m, __shfl_xor(m, 16, 64));
-            m = fmaxf(m, __shfl_xor(m, 32, 64));
-            if (m > run_max + kSlack) {
-                const float alpha = run_max > -INFINITY ? __builtin_amdgcn_exp2f(run_max - m) : 0.0f;
-                run_max = m;
-                lane_sum *= alpha;
+        if (it + 1 < group_kv_tiles) store_v_rows(it + 1, v_rows);
+        load_v_rows(it + 3, id, v_rows);
+        if (!mine) return;
+        uint4 pb[NB];
 #pragma unroll
-                for (int db = 0; db < kDimBlocks; ++db)
+        for (int j = 0; j < NB; ++j) {
+            float v[8];
 #pragma unroll
-                    for (int r = 0; r < 4; ++r) o[db][r] *= alpha;
+            for (int i = 0; i < 8; ++i) v[i] = i < 4 ? s0[j][i] : s1[j][i - 4];
+            if (masked) {
+#pragma unroll
+                for (int i = 0; i < 8; ++i) {
+                    const uint32_t token = kb + 16 * (i >> 2) + 4 * mc + (i & 3);
+                    if (token < kv_begin || token >= lim[j]) v[i] = -INFINITY;
+                }
             }
+            float m = max3(max3(v[0], v[1], v[2]), max3(v[3], v[4], v[5]), fmaxf(v[6], v[7])) * a.scale_log2;
+            if (__any(m > run_max[j] + kSlack)) {
+                m = fmaxf(m, __shfl_xor(m, 16, 64));
+                m = fmaxf(m, __shfl_xor(m, 32, 64));
+                if (m > run_max[j] + kSlack) {
+                    const float alpha = run_max[j] > -INFINITY ? __builtin_amdgcn_exp2f(run_max[j] - m) : 0.0f;
+                    run_max[j] = m;
+                    lane_sum[j] *= alpha;
+#pragma unroll
+                    for (int db = 0; db < kDimBlocks; ++db)
+#pragma unroll
+                        for (int r = 0; r < 4; ++r) o[j][db][r] *= alpha;
+                }
+            }
+            const float neg_ref = run_max[j] > -INFINITY ? -run_max[j] : 0.0f;
+            uint32_t words[4];
+#pragma unroll
+            for (int i = 0; i < 8; i += 2) {
+                // rounded to nearest, once, for the product and for the sum alike
+                const f16x2_t h = {(_Float16)__builtin_amdgcn_exp2f(__builtin_fmaf(v[i], a.scale_log2, neg_ref)),
+                                   (_Float16)__builtin_amdgcn_exp2f(__builtin_fmaf(v[i + 1], a.scale_log2, neg_ref))};
+                const f16x2_t ones = {(_Float16)1.0f, (_Float16)1.0f};
+                lane_sum[j] = __builtin_amdgcn_fdot2(h, ones, lane_sum[j], false);
+                words[i / 2] = __builtin_bit_cast(uint32_t, h);
+            }
+            pb[j] = make_uint4(words[0], words[1], words[2], words[3]);
         }
-        const float neg_ref = run_max > -INFINITY ? -run_max : 0.0f;
-        float p[8];
+        constexpr int kVGroup = 2;  // V operands read ahead of their products
 #pragma unroll
-        for (int j = 0; j < 8; ++j) p[j] = __builtin_amdgcn_exp2f(__builtin_fmaf(v[j], a.scale_log2, neg_ref));
-        const uint4 pb = prob_operand_f16(p);
-        lane_sum = add_f16x8(pb, lane_sum);
+        for (int g = 0; g < kDimBlocks; g += kVGroup) {
+            uint4 vt[kVGroup];
 #pragma unroll
-        for (int g = 0; g < kDimBlocks; g += 4) {
-            uint4 vt[4];
-#pragma unroll
-            for (int i = 0; i < 4; ++i) {
-                const unsigned char* src = vbuf + vt_base + (g + i) * 32;
-                const uint2 lo = lds_read_tr16_b64(src), hi = lds_read_tr16_b64(src + 16 * kVStride);
-                vt[i] = make_uint4(lo.x, lo.y, hi.x, hi.y);
+            for (int i = 0; i < kVGroup; ++i) {
+                const unsigned char* src = vbuf + v_row0 + (((g + i) * 32) ^ v_swizzle);
+                const uint2 lo2 = lds_read_tr16_b64(src), hi2 = lds_read_tr16_b64(src + 16 * kRowBytes);
+                vt[i] = make_uint4(lo2.x, lo2.y, hi2.x, hi2.y);
             }
 #pragma unroll
-            for (int i = 0; i < 4; ++i) o[g + i] = mfma_16x16x32<F16Tag>(vt[i], pb, o[g + i]);
+            for (int i = 0; i < kVGroup; ++i)
+#pragma unroll
+                for (int j = 0; j < NB; ++j) o[j][g + i] = mfma_16x16x32<F16Tag>(vt[i], pb[j], o[j][g + i]);
         }
-        if (lane == 0) done[wave] = it + 1;  // behind this tile's reads in the LDS queue
+    };
+    if (group_kv_tiles != 0) {
+        VRows first, even, odd;  // `odd` holds the rows of the odd tiles, and is taken in the even tiles
+        const uint32_t id0 = page_of(0), id1 = page_of(1), id2 = page_of(2);
+        next_id = page_of(3);
+        issue_k_loads(0, id0);
+        load_v_rows(0, id0, first);
+        issue_k_loads(1, id1);
+        load_v_rows(1, id1, odd);
+        issue_k_loads(2, id2);
+        load_v_rows(2, id2, even);
+        store_v_rows(0, first);
+        uint32_t it = 0;
+        for (; it + 1 < group_kv_tiles; it += 2) {
+            tile(it, odd);
+            tile(it + 1, even);
+        }
+        if (it < group_kv_tiles) tile(it, odd);
+        // The loads of tiles past the end go to LDS: they must be through before the workgroup gives it back.
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
     }
-    if (lane == 0) done[wave] = 0xffffffffu;
 
-    lane_sum += __shfl_xor(lane_sum, 16, 64);
-    lane_sum += __shfl_xor(lane_sum, 32, 64);
-    // A V element that f16 cannot hold has reached the accumulators as Inf or NaN (the conversion rounds to nearest,
-    // so that it overflows instead of saturating): the host is told, and the rows stay as they are, visibly wrong.
-    {
+#pragma unroll
+    for (int j = 0; j < NB; ++j) {
+        lane_sum[j] += __shfl_xor(lane_sum[j], 16, 64);
+        lane_sum[j] += __shfl_xor(lane_sum[j], 32, 64);
+        // A V element that f16 cannot hold has reached the accumulators as Inf or NaN (the conversion rounds to
+        // nearest, so that it overflows instead of saturating): the host is told, and the rows stay as they are,
+        // visibly wrong.
         float probe = 0.0f;
 #pragma unroll
         for (int db = 0; db < kDimBlocks; ++db)
 #pragma unroll
-            for (int r = 0; r < 4; ++r) probe = __builtin_fmaf(o[db][r], 0.0f, probe);
-        if (__any(lim != 0 && probe != probe) && lane == 0)
+            for (int r = 0; r < 4; ++r) probe = __builtin_fmaf(o[j][db][r], 0.0f, probe);
+        if (__any(lim[j] != 0 && probe != probe) && lane == 0)
             __hip_atomic_store(a.status + 1, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
-    }
-    if (*failed != 0u) {  // some wave's wait ran out: the host is told, and the columns get empty states
-        if (lane == 0) __hip_atomic_store(a.status, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
-        run_max = -INFINITY;
-        lane_sum = 0.0f;
+        if (lim[j] != 0) {
+            uint32_t t, h;
+            column_of(j, &t, &h);
+            const uint64_t part_row = ((uint64_t)rows[t / TS] * a.hq + head_first + h) * TS + t % TS;
+            if (mc == 0) {
+                a.part_max[part_row] = run_max[j];
+                a.part_sum[part_row] = lane_sum[j];
+            }
+            float* dst = a.part_acc + part_row * D + mc * 4;
 #pragma unroll
-        for (int db = 0; db < kDimBlocks; ++db) o[db] = f32x4_t{0.0f, 0.0f, 0.0f, 0.0f};
-    }
-    if (lim != 0) {
-        if (mc == 0) {
-            a.part_max[part_row] = run_max;
-            a.part_sum[part_row] = lane_sum;
+            for (int db = 0; db < kDimBlocks; ++db)
+                *reinterpret_cast<float4*>(dst + db * 16) = make_float4(o[j][db][0], o[j][db][1], o[j][db][2], o[j][db][3]);
         }
-        float* dst = a.part_acc + part_row * D + mc * 4;
-#pragma unroll
-        for (int db = 0; db < kDimBlocks; ++db)
-            *reinterpret_cast<float4*>(dst + db * 16) = make_float4(o[db][0], o[db][1], o[db][2], o[db][3]);
     }
 }
 
@@ -470,20 +493,19 @@ inline int launch_chunk_map_typed(psi_hip_ctx* ctx, const Geometry& g, const Map
                                   uint32_t group_tiles, uint32_t num_groups) {
     const uint32_t subsets = chunk_head_subsets(g.group);
     const dim3 grid(num_groups * g.hkv * subsets);
-    const bool page8 = g.tokens_per_page == 8;
-    auto* kernel = page8 ? &split_kv_chunk_map<Tag, D, true> : &split_kv_chunk_map<Tag, D, false>;
+    auto* kernel = &split_kv_chunk_map<Tag, D>;
     // The kernel's LDS is above the default limit of a launch; the limit is raised once per GPU and kernel (a
     // function's attributes belong to the device it is loaded on).
-    static std::atomic<uint64_t> raised_on[2] = {{0}, {0}};
+    static std::atomic<uint64_t> raised_on{0};
     const uint64_t device_bit = 1ull << (ctx->device & 63);
-    if ((raised_on[page8].load(std::memory_order_relaxed) & device_bit) == 0) {
+    if ((raised_on.load(std::memory_order_relaxed) & device_bit) == 0) {
         if (hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
                                 ChunkLds<D>::bytes) != hipSuccess)
             return PSI_HIP_ERR_UNSUPPORTED;
-        raised_on[page8].fetch_or(device_bit, std::memory_order_relaxed);
+        raised_on.fetch_or(device_bit, std::memory_order_relaxed);
     }
-    hipLaunchKernelGGL(kernel, grid, dim3(64 * (kChunkWaves + kChunkLoaders)), ChunkLds<D>::bytes, ctx->stream, a,
-                       a.walk.page_ids, a.kv_splits, a.req_slots, reinterpret_cast<const uint16_t*>(a.q),
+    hipLaunchKernelGGL(kernel, grid, dim3(64 * kChunkWaves), ChunkLds<D>::bytes, ctx->stream, a, a.walk.page_ids,
+                       a.kv_splits, a.req_slots, reinterpret_cast<const uint16_t*>(a.q),
                        reinterpret_cast<const uint16_t*>(a.kv_pages), a.q_token_tiles, a.flat_token_indices, row_groups,
                        group_tiles, num_groups, subsets);
     return PSI_HIP_OK;

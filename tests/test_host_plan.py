@@ -545,23 +545,23 @@ def check_groups(meta, shape, tile_size, max_tiles):
 
 def test_row_groups_of_a_prefill_chunk(psi):
     """A 70-token chunk on a 300-token prefix, 256-token partitions, next to two decode requests:
-    24 Q / 4 KV heads deal 2 heads to a workgroup, so a group holds 8 tiles of 8 tokens."""
+    24 Q / 4 KV heads deal 2 heads to a workgroup, so a group holds 16 tiles of 8 tokens."""
     meta = psi.GQAMetadataBuffers(None, 128, max_kv_splits=64)
     variant = psi.GQASplitKVVariant.TiledQ(8, 16, 6)
     shape = meta.update_fixed_partition([3, 1, 5], [300, 40, 999], [0, 70, 71, 72], variant, 256)
     assert meta.group_rows(tiled_config(psi, 24, 4)) == meta.num_row_groups > 0
-    table = check_groups(meta, shape, 8, 8)
+    table = check_groups(meta, shape, 8, 16)
     rows = meta.h_kv_splits.reshape(-1, 3)
-    # the chunk has 9 tiles; partition 0 is seen by all of them -> groups of 8 + 1
+    # the chunk has 9 tiles; partition 0 is seen by all of them -> one group of 9
     sizes = sorted(int((g != MAX).sum()) for g in table if rows[g[0]][1] == 0 and rows[g[0]][0] < 9)
-    assert sizes == [1, 8]
+    assert sizes == [9]
     # the groups survive a re-ordering of the rows (positions change, membership does not)
     meta.order_longest_first()
     meta.group_rows(tiled_config(psi, 24, 4))
-    check_groups(meta, shape, 8, 8)
+    check_groups(meta, shape, 8, 16)
 
 
-@pytest.mark.parametrize("hq,hkv,expected", [(16, 2, 4), (8, 2, 4), (4, 4, 16), (10, 2, 3), (14, 2, 4)])
+@pytest.mark.parametrize("hq,hkv,expected", [(16, 2, 8), (8, 2, 8), (4, 4, 32), (10, 2, 6), (14, 2, 8)])
 def test_row_group_size_follows_the_head_group(psi, hq, hkv, expected):
     meta = psi.GQAMetadataBuffers(None, 256, max_kv_splits=256)
     shape = meta.update_fixed_partition([0], [0], [0, 200], psi.GQASplitKVVariant.TiledQ(8, 16, min(hq // hkv, 8)), 128)
@@ -581,7 +581,7 @@ def test_row_groups_unsupported_geometry_and_greedy_plan(psi):
     assert meta.group_rows(tiled_config(psi, 8, 2, p=8)) > 0
     # the reference's greedy plan cuts every tile differently: groups degenerate but stay complete
     assert meta.group_rows(tiled_config(psi, 8, 2)) > 0
-    check_groups(meta, shape, 8, 4)
+    check_groups(meta, shape, 8, 8)
 
 
 def test_row_group_table_capacity_is_checked(psi):
@@ -597,11 +597,11 @@ def test_row_group_table_capacity_is_checked(psi):
     rc = lib.psi_hip_split_kv_tiled_q_group_rows(ctypes.byref(cfg), 8, p(rows), 2, p(tiles), 2, p(slots), p(table), 5,
                                                  ctypes.byref(n_tiles), ctypes.byref(n_groups))
     assert rc != 0 and b"row-group table too small" in lib.psi_hip_last_error()
-    table = np.zeros(16, np.uint32)
+    table = np.zeros(32, np.uint32)
     assert lib.psi_hip_split_kv_tiled_q_group_rows(ctypes.byref(cfg), 8, p(rows), 2, p(tiles), 2, p(slots), p(table),
-                                                   16, ctypes.byref(n_tiles), ctypes.byref(n_groups)) == 0
-    assert (n_tiles.value, n_groups.value) == (8, 2)  # two requests never share a group
-    assert table.tolist() == [0] + [MAX] * 7 + [1] + [MAX] * 7
+                                                   32, ctypes.byref(n_tiles), ctypes.byref(n_groups)) == 0
+    assert (n_tiles.value, n_groups.value) == (16, 2)  # two requests never share a group
+    assert table.tolist() == [0] + [MAX] * 15 + [1] + [MAX] * 15
 
 
 # ------------------------------------------------------------------ the whole plan in one call

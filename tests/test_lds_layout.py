@@ -1,9 +1,11 @@
-"""The LDS layout of the prefill-chunk map, checked on the host: the K tile in rows of head_dim * 2 bytes with the
-16-byte chunk index XORed with key % 16, the V tile in rows of head_dim * 2 + 32 bytes.  The operand reads must put
-the 16 lanes that a 128-bit LDS read serves together on 16 different bank groups, must find what the loading
-waves stored, and the stores must fill whole rows.  The address arithmetic below restates psi-dec_amd/csrc/split_kv_chunk_kernel.h (
-k_row0, vt_base, k_store, v_store); the lane groups are the ones measured on MI355X: lanes 0-3, 12-15 and 20-27 go together, then 4-11,
-16-19 and 28-31, and the same in the upper half of the wave."""
+"""The LDS layout of the prefill-chunk map, checked on the host.  A K tile is [32 keys][head_dim] elements with the
+16-byte chunk index XORed with key % 16; a V tile is [32 keys][head_dim] f16 with the 32-byte chunk index XORed with
+key % 8.  The operand reads must put the lanes that an LDS read serves together on different bank groups and must
+find what the fetching waves put there: K arrives by loads that write 1 KiB in lane order (the layout is made by each
+lane's choice of global address), V by 128-bit stores.  The address arithmetic below restates
+psi-dec_amd/csrc/split_kv_chunk_kernel.h (k_row0, v_row0, v_swizzle, k_lane, v_lane); the lane groups of a 128-bit
+access are the ones measured on MI355X: lanes 0-3, 12-15 and 20-27 go together, then 4-11, 16-19 and 28-31, and the
+same in the upper half of the wave."""
 import pytest
 
 READ_ROUNDS = [
@@ -12,10 +14,8 @@ READ_ROUNDS = [
 ]
 READ_ROUNDS += [[lane + 32 for lane in group] for group in READ_ROUNDS[:2]]
 KEYS = 32
-
-
-def pitch(d):
-    return d * 2 + 32
+WAVES = 8
+WAVE_ROWS = KEYS // WAVES
 
 
 def bank_group(byte_offset):
@@ -32,23 +32,32 @@ def k_read_offset(d, lane, ks, block):
 def v_read_offset(d, lane, db, block):
     """64-bit transposing read: the lane hands in key 16 * block + 4 * mc + mt / 4, dims 16 * db + 4 * (mt % 4) .. + 3."""
     mt, mc = lane & 15, lane >> 4
-    return (4 * mc + (mt >> 2)) * pitch(d) + (mt & 3) * 8 + db * 32 + block * 16 * pitch(d)
+    key = 4 * mc + (mt >> 2)
+    return key * d * 2 + (mt & 3) * 8 + ((db * 32) ^ ((key & 7) * 32)) + block * 16 * d * 2
 
 
-def loader_key_chunk(d, thread, i):
-    chunks = d // 8
-    return thread // chunks + (256 // chunks) * i, thread % chunks
+def fetch_geometry(d):
+    row_chunks = d // 8                 # 16-byte chunks per row
+    rows_per_load = 64 // row_chunks    # rows that one load of a wave covers
+    return row_chunks, rows_per_load, WAVE_ROWS // rows_per_load
 
 
-def k_store_offset(d, thread, i):
-    """128-bit store of loading thread `thread` (0 .. 255), load i, into the K tile."""
-    key, chunk = loader_key_chunk(d, thread, i)
-    return key * d * 2 + ((chunk ^ (key & 15)) * 16)
+def k_landing(d, wave, lane, i):
+    """Load i of a wave: (LDS offset in the tile where the lane's 16 bytes land, key, 16-byte chunk they come from)."""
+    row_chunks, rows_per_load, _ = fetch_geometry(d)
+    row_in_load, slot = lane // row_chunks, lane % row_chunks
+    key = WAVE_ROWS * wave + rows_per_load * i + row_in_load
+    lands = (WAVE_ROWS * wave + rows_per_load * i) * d * 2 + lane * 16
+    return lands, key, slot ^ (key & 15)
 
 
-def v_store_offset(d, thread, i):
-    key, chunk = loader_key_chunk(d, thread, i)
-    return key * pitch(d) + chunk * 16
+def v_store(d, wave, lane, i):
+    """Store i of a wave: (LDS offset in the tile, key, 16-byte chunk of the row that the lane holds)."""
+    row_chunks, rows_per_load, _ = fetch_geometry(d)
+    row_in_load, slot = lane // row_chunks, lane % row_chunks
+    key = WAVE_ROWS * wave + rows_per_load * i + row_in_load
+    where = key * d * 2 + ((((slot >> 1) ^ (key & 7)) << 1) | (slot & 1)) * 16
+    return where, key, slot
 
 
 def test_rounds_partition_the_wave():
@@ -56,12 +65,15 @@ def test_rounds_partition_the_wave():
 
 
 @pytest.mark.parametrize("d", [128, 256])
-def test_k_operand_reads_are_conflict_free_and_find_what_was_stored(d):
-    loads = KEYS * (d // 8) // 256
+def test_k_operand_reads_are_conflict_free_and_find_what_landed(d):
+    loads = fetch_geometry(d)[2]
     where = {}
-    for thread in range(256):
+    for wave in range(WAVES):
         for i in range(loads):
-            where[loader_key_chunk(d, thread, i)] = k_store_offset(d, thread, i)
+            for lane in range(64):
+                lands, key, chunk = k_landing(d, wave, lane, i)
+                assert lands // (d * 2) == key, "a lane's bytes land in the row of their key"
+                where[(key, chunk)] = lands
     assert len(where) == KEYS * d // 8 and len(set(where.values())) == len(where)
     for block in range(2):
         for ks in range(d // 32):
@@ -74,9 +86,18 @@ def test_k_operand_reads_are_conflict_free_and_find_what_was_stored(d):
 
 
 @pytest.mark.parametrize("d", [128, 256])
-def test_transposing_reads_spread_their_keys_over_the_banks(d):
+def test_transposing_reads_spread_their_keys_over_the_banks_and_find_what_was_stored(d):
     """The 16 lanes of a quarter wave read 4 keys x 32 bytes, two quarters 8 keys: every key's 32 bytes in a bank
     group pair of its own."""
+    loads = fetch_geometry(d)[2]
+    where = {}
+    for wave in range(WAVES):
+        for i in range(loads):
+            for lane in range(64):
+                at, key, chunk = v_store(d, wave, lane, i)
+                assert at // (d * 2) == key
+                where[(key, chunk)] = at
+    assert len(where) == KEYS * d // 8 and len(set(where.values())) == len(where)
     for block in range(2):
         for db in range(d // 16):
             for half in range(2):
@@ -85,29 +106,18 @@ def test_transposing_reads_spread_their_keys_over_the_banks(d):
                     off = v_read_offset(d, lane, db, block)
                     assert off % 8 == 0
                     mt, mc = lane & 15, lane >> 4
-                    assert off == (16 * block + 4 * mc + (mt >> 2)) * pitch(d) + (16 * db + 4 * (mt & 3)) * 2
+                    key = 16 * block + 4 * mc + (mt >> 2)
+                    first_dim = 16 * db + 4 * (mt & 3)  # 4 dims = 8 bytes inside chunk first_dim / 8
+                    assert off == where[(key, first_dim // 8)] + (first_dim % 8) * 2
                     pairs.add((off % 256) // 32)
                 assert len(pairs) == 8  # eight keys, eight different 32-byte bank ranges
 
 
 @pytest.mark.parametrize("d", [128, 256])
-def test_stores_fill_the_tiles_in_whole_rows(d):
-    loads = KEYS * (d // 8) // 256
-    covered = set()
-    for thread in range(256):
+def test_v_stores_are_conflict_free(d):
+    """A 128-bit store is served in the same rounds of 16 lanes."""
+    loads = fetch_geometry(d)[2]
+    for wave in range(WAVES):
         for i in range(loads):
-            key, byte = divmod(v_store_offset(d, thread, i), pitch(d))
-            assert key < KEYS and byte < d * 2 and byte % 16 == 0
-            covered.add((key, byte))
-            assert k_store_offset(d, thread, i) // (d * 2) == key  # the K store stays in its row
-    assert len(covered) == KEYS * d // 8
-
-
-def test_stores_of_head_dim_256_are_conflict_free():
-    """A 128-bit store is served in the same rounds of 16 lanes; with 512-byte rows every round stays inside one row,
-    where the XOR only permutes the chunks."""
-    for wave in range(4):
-        for i in range(4):
             for group in READ_ROUNDS:
-                assert len({bank_group(k_store_offset(256, 64 * wave + lane, i)) for lane in group}) == 16
-                assert len({bank_group(v_store_offset(256, 64 * wave + lane, i)) for lane in group}) == 16
+                assert len({bank_group(v_store(d, wave, lane, i)[0]) for lane in group}) == 16
