@@ -14,8 +14,10 @@ same sample on all of them).  `configs` carries the same figures for the other b
 headline batch with one workgroup per 512-token partition row, the headline's shape at batch 4 / 8 / 16, C3, C4 with
 one, three and seven drafts, C5's decode side, its prefill chunk, and the mixed step) and for the shapes the
 reference itself times (`REF_*`), each timed in this run with the same step and warm-up counts.  Every workload
-also carries a `cold` figure (the first steps after set-up), and every HBM roofline the read bandwidth of a bare
-page stream measured in the same run (`measured_stream_GBps`, `frac_of_measured_stream`).
+also carries a `cold` figure (the first steps after set-up), every HBM roofline the read bandwidth of a bare
+page stream measured in the same run (`measured_stream_GBps`, `frac_of_measured_stream`), and the matrix-core
+roofline of the prefill chunk the rate of a bare matrix-instruction loop and the LDS read rates of its two operand
+reads, measured in the same run (`measured_mfma_TFLOPs`, `frac_of_measured_mfma`, `measured_lds_read_GBps_per_cu`).
 
 Clocks.  `ms_per_step` / `us_per_layer_step`: host wall clock around K queued steps, device synchronised on both
 sides -- steps run back to back, as the layers of a decoder do.  `us_per_layer_step_p10_median_p90`: a HIP event
@@ -438,9 +440,15 @@ def time_case(psi, wl, device, case, args, with_spread=True):
            "frac_of_measured_stream": achieved / stream_gbps if stream_gbps else None, **timing}
     if case.flops:
         tflops = case.flops / (map_us / 1e6) / 1e12
+        rates = measured_matrix_rates(device)
         out["roofline"] = {"bound": "mfma", "kernel": case.roof_kernel, "achieved": tflops, "peak": MFMA_BF16_PEAK_TFLOPS,
                            "unit": "TFLOP/s", "frac": tflops / MFMA_BF16_PEAK_TFLOPS,
-                           "traffic": read_profile_traffic(case.key), "flops_per_launch": case.flops, **timing}
+                           "traffic": read_profile_traffic(case.key), "flops_per_launch": case.flops,
+                           "measured_mfma_TFLOPs": rates.get("mfma_tflops"),
+                           "frac_of_measured_mfma": tflops / rates["mfma_tflops"] if rates.get("mfma_tflops") else None,
+                           "measured_lds_read_GBps_per_cu": {"b128": rates.get("lds_b128"),
+                                                             "b64_transposing": rates.get("lds_b64_tr")},
+                           **timing}
         out["hbm_view"] = {k: hbm[k] for k in ("achieved", "peak", "unit", "frac", "algorithmic_bytes_per_launch")}
     else:
         out["roofline"] = hbm
@@ -538,6 +546,53 @@ def measured_stream_gbps(device):
         print(f"bench.py: stream probe unavailable ({e})", file=sys.stderr)
         _STREAM_PROBE["gbps"] = None
     return _STREAM_PROBE["gbps"]
+
+
+_MATRIX_PROBE = {}
+
+
+def measured_matrix_rates(device):
+    """What bounds the prefill-chunk map, measured in this run with the probes of psi-dec_amd/lib/libpsi_hip_probe.so:
+    the rate of back-to-back v_mfma_f32_16x16x32_bf16 from eight waves per compute unit (at the clock the chip keeps
+    under that load), and the LDS read rates per compute unit of the map's two operand reads (128-bit reads of a K
+    tile, transposing 64-bit reads of a V tile)."""
+    import ctypes
+
+    import torch
+
+    if _MATRIX_PROBE:
+        return _MATRIX_PROBE
+    try:
+        probe = ctypes.CDLL(os.path.join(ROOT, "psi-dec_amd", "lib", "libpsi_hip_probe.so"))
+        probe.psi_probe_mfma_rate.restype = ctypes.c_int
+        probe.psi_probe_mfma_rate.argtypes = [ctypes.c_void_p, ctypes.c_void_p, ctypes.c_uint32]
+        probe.psi_probe_lds_read_rate.restype = ctypes.c_int
+        probe.psi_probe_lds_read_rate.argtypes = [ctypes.c_void_p, ctypes.c_void_p, ctypes.c_int, ctypes.c_uint32]
+        sink = torch.zeros(512, dtype=torch.float32, device="cuda")
+        stream = ctypes.c_void_p(device.stream.cuda_stream)
+
+        def timed(launch, launches=10):
+            for _ in range(3):
+                if launch() != 0:
+                    raise RuntimeError("probe launch failed")
+            start, stop = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            start.record(device.stream)
+            for _ in range(launches):
+                launch()
+            stop.record(device.stream)
+            stop.synchronize()
+            return start.elapsed_time(stop) * 1e-3 / launches
+
+        iters = 2000  # about 250 us per launch, the length of the chunk map's own launches
+        seconds = timed(lambda: probe.psi_probe_mfma_rate(stream, sink.data_ptr(), iters))
+        _MATRIX_PROBE["mfma_tflops"] = 256 * 8 * 8 * iters * 16384 / seconds / 1e12
+        for name, pattern in (("lds_b128", 0), ("lds_b64_tr", 1)):
+            seconds = timed(lambda: probe.psi_probe_lds_read_rate(stream, sink.data_ptr(), pattern, 4000))
+            _MATRIX_PROBE[name] = 8 * 16384 * 4000 / seconds / 1e9
+    except (OSError, AttributeError, RuntimeError) as e:  # a measurement aid: a figure less, not a failure
+        print(f"bench.py: matrix probes unavailable ({e})", file=sys.stderr)
+        _MATRIX_PROBE["mfma_tflops"] = None
+    return _MATRIX_PROBE
 
 
 def calibrate_copy(device, args):

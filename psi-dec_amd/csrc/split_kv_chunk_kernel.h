@@ -13,11 +13,11 @@
 //
 //   Eight waves, two per SIMD, each with half of the SIMD's registers.  Every operand of every product is read
 //   from LDS, and an operand read serves both column blocks of a wave, so a tile's K and V cross the LDS port once
-//   per 32 columns.  With 16 columns per wave (and then room for waves that only load) the same kernel spent its
-//   time on the LDS port - the transposing reads of V run at half the rate of 128-bit reads, 250 against 460
-//   bytes per nanosecond and compute unit - and reached a third of the matrix peak.  With one wave per SIMD nothing
-//   hides the latencies of a wave's own chain (operand reads, matrix results, exponentials); with two, each fills
-//   the other's gaps.
+//   per 32 columns.  With 16 columns per wave (and then room for waves that only load) the same kernel's time
+//   followed its LDS traffic: taking the loading waves' stores away, or their loads, each bought back a tenth of
+//   the launch, and the products alone ran as long as the tile reads take at the LDS port's rate.  With one wave
+//   per SIMD nothing hides the latencies of a wave's own chain (operand reads, matrix results, exponentials);
+//   with two, each fills the other's gaps.
 //
 //   No wave only loads: every wave fetches four rows of K and four of V of every tile.  K goes straight to LDS
 //   with `global_load_lds_dwordx4`, which moves 16 bytes per lane from a per-lane global address to LDS address
