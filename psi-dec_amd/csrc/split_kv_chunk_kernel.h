@@ -346,10 +346,12 @@ __global__ __launch_bounds__(64 * kChunkWaves, 1) void split_kv_chunk_map(
         const unsigned char* vbuf = lds + kVOffset + (it % kChunkVStages) * kKBytes;
         const uint32_t kb = key_base0 + it * kChunkKeys;
         const bool masked = !(kb >= kv_begin && kb + kChunkKeys <= wave_lo);
+        float logits[NB][8];
+        if (mine) {
+        // (zeroed here, where the first products can take the zeros as a constant operand, not from registers)
         f32x4_t s0[NB], s1[NB];
 #pragma unroll
         for (int j = 0; j < NB; ++j) s0[j] = s1[j] = f32x4_t{0.0f, 0.0f, 0.0f, 0.0f};
-        if (mine) {
         uint4 k0[kKSteps], k1[kKSteps], q1[kKSteps];
         // the operands of k-step ks: two key blocks of K, and the second column block's queries
         auto read_k = [&](int ks) __attribute__((always_inline)) {
@@ -377,6 +379,10 @@ __global__ __launch_bounds__(64 * kChunkWaves, 1) void split_kv_chunk_map(
         }
         __builtin_amdgcn_sched_group_barrier(0x008, 4 * kAhead, 0);
         __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+        for (int j = 0; j < NB; ++j)
+#pragma unroll
+            for (int i = 0; i < 8; ++i) logits[j][i] = i < 4 ? s0[j][i] : s1[j][i - 4];
         }
         if (it + 1 < group_kv_tiles) store_v_rows(it + 1, v_rows);
         load_v_rows(it + 3, id, v_rows);
@@ -384,9 +390,7 @@ __global__ __launch_bounds__(64 * kChunkWaves, 1) void split_kv_chunk_map(
         uint4 pb[NB];
 #pragma unroll
         for (int j = 0; j < NB; ++j) {
-            float v[8];
-#pragma unroll
-            for (int i = 0; i < 8; ++i) v[i] = i < 4 ? s0[j][i] : s1[j][i - 4];
+            float (&v)[8] = logits[j];
             if (masked) {
 #pragma unroll
                 for (int i = 0; i < 8; ++i) {
@@ -394,7 +398,7 @@ __global__ __launch_bounds__(64 * kChunkWaves, 1) void split_kv_chunk_map(
                     if (token < kv_begin || token >= lim[j]) v[i] = -INFINITY;
                 }
             }
-            float m = max3(max3(v[0], v[1], v[2]), max3(v[3], v[4], v[5]), fmaxf(v[6], v[7])) * a.scale_log2;
+            float m = max3(max3(v[0], v[1], v[2]), max3(v[3], v[4], v[5]), max3(v[6], v[7], v[7])) * a.scale_log2;
             if (__any(m > run_max[j] + kSlack)) {
                 m = fmaxf(m, __shfl_xor(m, 16, 64));
                 m = fmaxf(m, __shfl_xor(m, 32, 64));
