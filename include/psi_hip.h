@@ -351,6 +351,14 @@ int psi_hip_qk_norm_rope_kv_page_write(
 
 /* ------------------------------------------------------------------ split-KV decode (SingleQ) */
 
+/* Which kernels a geometry gets (all map and combine entry points below, SingleQ and TiledQ):
+ *   bf16 / f16 K/V, head_dim 128 or 256, tokens_per_page a power of two  -> the gfx950 kernels (HBM-bound
+ *       decode map, matrix-core multi-query map; prefill-chunk map for pages of at least 8 tokens);
+ *   anything else the reference's config admits (f32 K/V, other head dims, other page sizes)  -> the
+ *       shape-generic kernels: the same results, correct for every shape, not tuned (a batch of 8
+ *       sequences in f32 runs at about 1 % of the HBM peak);
+ *   PSI_HIP_FLAG_FORCE_GENERIC sends every geometry to the generic kernels (the cross-check variant). */
+
 /* Scratch for the partial states of `num_total_kv_splits` splits: replaces `GQASplitKVSingleQScratch::new`
  * (gqa_split_kv_single_q.rs:236-246).  The layout is private to the library. */
 int psi_hip_split_kv_single_q_scratch_bytes(const psi_hip_gqa_config* cfg, uint32_t num_total_kv_splits,
