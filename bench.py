@@ -15,7 +15,9 @@ headline batch with one workgroup per 512-token partition row, the headline's sh
 one, three and seven drafts, C5's decode side, its prefill chunk, and the mixed step) and for the shapes the
 reference itself times (`REF_*`), each timed in this run with the same step and warm-up counts.  Every workload
 also carries a `cold` figure (the first steps after set-up), every HBM roofline the read bandwidth of a bare
-page stream measured in the same run (`measured_stream_GBps`, `frac_of_measured_stream`), and the matrix-core
+page stream measured in the same run, in launches of 1 GiB and in launches of the map's own size
+(`measured_stream_GBps`, `frac_of_measured_stream`, `measured_stream_same_size_GBps`,
+`frac_of_measured_stream_same_size`), and the matrix-core
 roofline of the prefill chunk the rate of a bare matrix-instruction loop and the LDS read rates of its two operand
 reads, measured in the same run (`measured_mfma_TFLOPs`, `frac_of_measured_mfma`, `measured_lds_read_GBps_per_cu`).
 
@@ -433,11 +435,16 @@ def time_case(psi, wl, device, case, args, with_spread=True):
               "timing": "HIP events on the launch stream; the smaller of the back-to-back and per-launch figures"}
     achieved = map_bytes / (map_us / 1e6) / 1e9
     stream_gbps = measured_stream_gbps(device)
+    # ... and in a launch that reads as many bytes as this map does (a short launch's start and end weigh more)
+    same_size = (map_bytes // (16 << 20)) * (16 << 20)
+    stream_same_gbps = measured_stream_gbps(device, same_size) if 0 < same_size <= 9 << 30 else None
     hbm = {"bound": "hbm", "kernel": case.roof_kernel, "achieved": achieved,
            "peak": HBM_PEAK_GBPS, "unit": "GB/s", "frac": achieved / HBM_PEAK_GBPS,
            "traffic": read_profile_traffic(case.key), "algorithmic_bytes_per_launch": map_bytes,
            "measured_stream_GBps": stream_gbps,
-           "frac_of_measured_stream": achieved / stream_gbps if stream_gbps else None, **timing}
+           "frac_of_measured_stream": achieved / stream_gbps if stream_gbps else None,
+           "measured_stream_same_size_GBps": stream_same_gbps,
+           "frac_of_measured_stream_same_size": achieved / stream_same_gbps if stream_same_gbps else None, **timing}
     if case.flops:
         tflops = case.flops / (map_us / 1e6) / 1e12
         rates = measured_matrix_rates(device)
@@ -510,42 +517,46 @@ def cpu_baseline(psi, wl, w, dw, budget_s):
 _STREAM_PROBE = {}
 
 
-def measured_stream_gbps(device):
+def measured_stream_gbps(device, nbytes=1 << 30):
     """Read bandwidth of a bare stream in the attention's access pattern, measured in this run: the page-stream
-    probe of psi-dec_amd/lib/libpsi_hip_probe.so over 1 GiB of scattered 64 KiB pages, 1 KiB per load through LDS,
-    eight loads in flight per wave.  What the HBM-bound maps could reach at best on this box."""
+    probe of psi-dec_amd/lib/libpsi_hip_probe.so over `nbytes` (1 GiB unless a launch of a workload's own size is asked
+    for; a multiple of 16 MiB) of scattered 64 KiB pages, 1 KiB per load through LDS, eight loads in flight per wave.
+    What the HBM-bound maps could reach at best on this box, in a launch of that size."""
     import ctypes
 
     import torch
 
-    if "gbps" in _STREAM_PROBE:
-        return _STREAM_PROBE["gbps"]
+    key = "gbps" if nbytes == 1 << 30 else f"gbps_{nbytes}"
+    if key in _STREAM_PROBE:
+        return _STREAM_PROBE[key]
     try:
         probe = ctypes.CDLL(os.path.join(ROOT, "psi-dec_amd", "lib", "libpsi_hip_probe.so"))
         probe.psi_probe_page_stream.restype = ctypes.c_int
         probe.psi_probe_page_stream.argtypes = [ctypes.c_void_p, ctypes.c_void_p, ctypes.c_uint64, ctypes.c_int]
-        nbytes = 1 << 30
-        src = torch.empty(nbytes, dtype=torch.uint8, device="cuda").random_(0, 255)
+        # successive launches read successive slices of at least 1 GiB in all, so that none finds its bytes in the
+        # 256 MiB last-level cache (the workloads rotate their arenas for the same reason)
+        copies = max(1, -(-(1 << 30) // nbytes))
+        src = torch.empty(nbytes * copies, dtype=torch.uint8, device="cuda").random_(0, 255)
         stream = ctypes.c_void_p(device.stream.cuda_stream)
         best = 0.0
         for _ in range(2):
-            for _ in range(5):
-                if probe.psi_probe_page_stream(stream, src.data_ptr(), nbytes, 8) != 0:
+            for i in range(5):
+                if probe.psi_probe_page_stream(stream, src.data_ptr() + (i % copies) * nbytes, nbytes, 8) != 0:
                     raise RuntimeError("psi_probe_page_stream failed")
             start, stop = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
             start.record(device.stream)
-            for _ in range(20):
-                probe.psi_probe_page_stream(stream, src.data_ptr(), nbytes, 8)
+            for i in range(20):
+                probe.psi_probe_page_stream(stream, src.data_ptr() + (i % copies) * nbytes, nbytes, 8)
             stop.record(device.stream)
             stop.synchronize()
             best = max(best, nbytes / (start.elapsed_time(stop) * 1e-3 / 20) / 1e9)
         del src
         torch.cuda.empty_cache()
-        _STREAM_PROBE["gbps"] = best
+        _STREAM_PROBE[key] = best
     except (OSError, RuntimeError) as e:  # the probe library is a measurement aid: a figure less, not a failure
         print(f"bench.py: stream probe unavailable ({e})", file=sys.stderr)
-        _STREAM_PROBE["gbps"] = None
-    return _STREAM_PROBE["gbps"]
+        _STREAM_PROBE[key] = None
+    return _STREAM_PROBE[key]
 
 
 _MATRIX_PROBE = {}
