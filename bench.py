@@ -42,7 +42,7 @@ sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBPS = 8000.0
 MFMA_BF16_PEAK_TFLOPS = 2500.0
-CONFIG_NAMES = ["C1", "C2_rows512", "C2_b4", "C2_b8", "C2_b16", "C3", "C4_q2", "C4_q4", "C4_q8", "C5_decode", "C5_prefill",
+CONFIG_NAMES = ["C1", "C2_rows512", "C2_b4", "C2_b8", "C2_b16", "C3", "C4_q2", "C4_q4", "C4_q8", "C5_decode", "C5_prefill", "PREFILL_d128",
                 "C5_mixed", "GENERIC_f32_b8"]
 # The shapes the reference itself times (the only figures it publishes for these kernels, on an Apple M3 Max):
 #   REF_tiled      "SplitKV TiledQ only", 40 Q / 8 KV heads, head_dim 128, 8-token pages, one request with 8 new tokens
@@ -252,6 +252,16 @@ def build_case(psi, wl, device, name, args):
         case = Case(name, "prefill_chunk2048_on_prefix4096_24q4kv_d256_bf16_p16_part4096_seed5", [dw], "prefill",
                     "tiled_q_map", "split_kv_chunk_map", "kv append -> row-group (prefill-chunk) map -> LSE combine")
         case.flops = 4 * 24 * 256 * sum(4096 + i + 1 for i in range(2048))
+        return case
+    if name == "PREFILL_d128":
+        # the same chunk on the geometry of the reference's published figures (Qwen3-14B: 40 Q / 8 KV heads of 128,
+        # 8-token pages; gqa_split_kv_tiled_q.rs:66-76 profile (128, 8))
+        w = wl.make_workload(5, [4096 + 2048], 40, 8, 128, bf16, 8, q_lens=2048, host_pages=False)
+        dw = wl.DeviceWorkload(device, w, partition_tokens=args.prefill_partition, grouped=True,
+                               variant=psi.GQASplitKVVariant.TiledQ(8, 16, 5))
+        case = Case(name, "prefill_chunk2048_on_prefix4096_40q8kv_d128_bf16_p8_part4096_seed5", [dw], "prefill",
+                    "tiled_q_map", "split_kv_chunk_map", "kv append -> row-group (prefill-chunk) map -> LSE combine")
+        case.flops = 4 * 40 * 128 * sum(4096 + i + 1 for i in range(2048))
         return case
     if name == "C5_mixed":
         step = wl.MixedStep(device, wl.config_c5())

@@ -189,6 +189,33 @@ def test_c5_prefill_chunk_full_size(psi, oracle, device):
     assert_outputs_close(outs["grouped 2048"][picks].reshape(-1), exp, "C5 chunk sampled")
 
 
+def test_prefill_chunk_full_size_on_the_reference_geometry(psi, oracle, device):
+    """The same chunk on the geometry of the reference's published figures and TiledQ profile (128, 8)
+    (gqa_split_kv_tiled_q.rs:66-76): 40 Q / 8 KV heads of 128, 8-token pages.  Row-group map against the plain
+    multi-query map on the whole chunk, and sampled query tokens against the scalar oracle."""
+    wl = importlib_workloads(psi)
+    w = wl.make_workload(5, [4096 + 2048], 40, 8, 128, psi.Dtype.Bfloat16, 8, q_lens=2048, host_pages=False)
+    variant = psi.GQASplitKVVariant.TiledQ(8, 16, 5)
+    outs = {}
+    for name, partition, grouped in (("grouped 4096", 4096, True), ("plain 2048", 2048, False)):
+        dw = wl.DeviceWorkload(device, w, partition_tokens=partition, f32_output=True, grouped=grouped, variant=variant)
+        assert (dw.meta.num_row_groups > 0) == grouped
+        dw.step()
+        outs[name] = dw.output_f32().reshape(2048, -1)
+        if grouped:
+            pages = dw.pages_host()
+        del dw
+    assert np.isfinite(outs["grouped 4096"]).all()
+    assert np.abs(outs["grouped 4096"] - outs["plain 2048"]).max() < 1e-4
+    picks = np.array([0, 1, 47, 48, 1023, 2040, 2047])
+    dt = oracle_dtype(oracle, w)
+    exp = oracle.paged_gqa(w.num_q_heads, w.num_kv_heads, w.head_dim, w.scale, w.page_bytes, dt, layout_tuple(w),
+                           w.layer, np.repeat(w.req_slots, len(picks)), (w.token_indices[0] + picks).astype(np.uint32),
+                           np.arange(len(picks) + 1, dtype=np.uint32), w.q.reshape(2048, -1)[picks].reshape(-1), pages,
+                           w.page_ids, num_threads=16)
+    assert_outputs_close(outs["grouped 4096"][picks].reshape(-1), exp, "head_dim 128 chunk sampled")
+
+
 @pytest.mark.parametrize("how", DECODE_MODES)
 def test_c5_decode_batch_full_size(psi, oracle, device, how):
     """C5's decode side: 128 sequences with contexts 512..32768 (about 8.7 GB of K/V).  512- and 4096-token
