@@ -131,7 +131,9 @@ struct ChunkLds {
     static constexpr int kKBytes = kChunkKeys * D * 2;  // a tile of K, and of V
     static constexpr int kVOffset = kChunkStages * kKBytes;
     static constexpr int kQOffset = kVOffset + kChunkVStages * kKBytes;
-    static constexpr int kQSteps = D / 32;  // k-steps of a wave's second column block whose query operands live here: all
+    // k-steps of a wave's second column block whose query operands live here: all of them at head_dim 256 (128
+    // accumulators + 64 registers of queries + the V rows under way are more than a wave has), none at 128
+    static constexpr int kQSteps = D == 256 ? D / 32 : 0;
     static constexpr int bytes = kQOffset + kChunkWaves * kQSteps * 1024;
 };
 
@@ -154,7 +156,8 @@ __global__ __launch_bounds__(64 * kChunkWaves, 1) void split_kv_chunk_map(
     constexpr int kKBytes = ChunkLds<D>::kKBytes;
     constexpr int kVOffset = ChunkLds<D>::kVOffset;
     constexpr int kQSteps = ChunkLds<D>::kQSteps;
-    static_assert(kQSteps == kKSteps, "the second block's queries live in LDS");
+    constexpr bool kQInLds = kQSteps != 0;
+    static_assert(kQSteps == kKSteps || kQSteps == 0, "the second block's queries live in LDS, or in registers");
     constexpr float kSlack = 8.0f;
     extern __shared__ __attribute__((aligned(16))) unsigned char lds[];
 
@@ -205,7 +208,8 @@ __global__ __launch_bounds__(64 * kChunkWaves, 1) void split_kv_chunk_map(
     bool used[NB];
     uint32_t lim[NB];
     unsigned char* q_lds = lds + ChunkLds<D>::kQOffset + wave * (kQSteps * 1024) + lane * 16;
-    uint4 qreg[kKSteps];  // the first block's; the second block's live in LDS
+    uint4 qreg[kKSteps];                     // the first block's
+    uint4 qreg1[kQInLds ? 1 : kKSteps];      // the second block's, unless they live in LDS
 #pragma unroll
     for (int j = 0; j < NB; ++j) {
         uint32_t t, h;
@@ -217,7 +221,8 @@ __global__ __launch_bounds__(64 * kChunkWaves, 1) void split_kv_chunk_map(
         for (int ks = 0; ks < kKSteps; ++ks) {
             const uint4 operand = used[j] ? *reinterpret_cast<const uint4*>(q_row + ks * 32) : make_uint4(0, 0, 0, 0);
             if (j == 0) qreg[ks] = operand;
-            else *reinterpret_cast<uint4*>(q_lds + ks * 1024) = operand;
+            else if constexpr (kQInLds) *reinterpret_cast<uint4*>(q_lds + ks * 1024) = operand;
+            else qreg1[ks] = operand;
         }
     }
     uint32_t lo = 0xffffffffu, hi = 0;
@@ -332,7 +337,8 @@ __global__ __launch_bounds__(64 * kChunkWaves, 1) void split_kv_chunk_map(
     // then the softmax and the products with V.  The loads complete in the order of their issue: at the barrier
     // the K rows of tile t + 1 are followed by the V rows of tile t + 1, the K rows of tile t + 2 and the V rows
     // of tile t + 2.
-    constexpr int kAhead = 1;  // k-steps between an operand's read and its product
+    // k-steps between an operand's read and its product (head_dim 128 has the registers for two)
+    constexpr int kAhead = D == 256 ? 1 : 2;
     uint32_t next_id = 0;
     auto tile = [&](uint32_t it, VRows& v_rows) __attribute__((always_inline)) {
         asm volatile("s_waitcnt vmcnt(%0)" ::"n"(3 * kLoads) : "memory");
@@ -358,7 +364,8 @@ __global__ __launch_bounds__(64 * kChunkWaves, 1) void split_kv_chunk_map(
             const uint32_t off = k_row0 + (((4 * ks + mc) ^ mt) * 16);
             k0[ks] = *reinterpret_cast<const uint4*>(kbuf + off);
             k1[ks] = *reinterpret_cast<const uint4*>(kbuf + off + 16 * kRowBytes);
-            q1[ks] = *reinterpret_cast<const uint4*>(q_lds + ks * 1024);
+            if constexpr (kQInLds) q1[ks] = *reinterpret_cast<const uint4*>(q_lds + ks * 1024);
+            else q1[ks] = qreg1[ks];
         };
         __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
@@ -371,11 +378,12 @@ __global__ __launch_bounds__(64 * kChunkWaves, 1) void split_kv_chunk_map(
             s1[1] = mfma_16x16x32<Tag>(k1[ks], q1[ks], s1[1]);
             if (ks + kAhead < kKSteps) read_k(ks + kAhead);
         }
-        __builtin_amdgcn_sched_group_barrier(0x100, 3 * kAhead, 0);  // the first reads
+        constexpr int kReads = kQInLds ? 3 : 2;  // LDS reads of a k-step
+        __builtin_amdgcn_sched_group_barrier(0x100, kReads * kAhead, 0);  // the first reads
 #pragma unroll
         for (int ks = 0; ks < kKSteps - kAhead; ++ks) {
             __builtin_amdgcn_sched_group_barrier(0x008, 4, 0);  // the products of a k-step
-            __builtin_amdgcn_sched_group_barrier(0x100, 3, 0);  // the reads kAhead steps on
+            __builtin_amdgcn_sched_group_barrier(0x100, kReads, 0);  // the reads kAhead steps on
         }
         __builtin_amdgcn_sched_group_barrier(0x008, 4 * kAhead, 0);
         __builtin_amdgcn_sched_barrier(0);
