@@ -30,8 +30,8 @@
 // Per 32-key tile and wave (2 x 16 columns)
 //   QK^T  S[key][column] on v_mfma_f32_16x16x32 of the storage type: A = K rows from LDS (key 16 * b + i in row i of
 //         key block b), B = the query columns: the first block's held in registers for the whole kernel, the second
-//         block's read from LDS with the K operands (64 registers of queries next to 128 accumulators and the V
-//         rows under way are more than a wave has).  A lane ends up with keys 16 * b + 4 * (lane / 16) + r,
+//         block's too at head_dim 128, and read from LDS with the K operands at head_dim 256 (64 registers of
+//         queries next to 128 accumulators and the V rows under way are more than a wave has).  A lane ends up with keys 16 * b + 4 * (lane / 16) + r,
 //         r = 0..3, b = 0, 1, of its column.
 //   softmax  per column, in-lane over those 8 keys; masks only on tiles that touch the start of the range
 //         or a column's causal limit.  The reference maximum of a column moves only when a tile
@@ -59,7 +59,7 @@
 //   V    two tiles of [32 keys][D] f16, 32-byte chunk index XOR (key % 8): the four keys of a quarter wave's
 //        transposing read (32 bytes each, 16 dims) then fall into different bank groups, and so do the eight keys
 //        of two quarters.
-//   Q    the second column block's query operands, 4 or 8 KiB per wave.
+//   Q    at head_dim 256, the second column block's query operands, 8 KiB per wave.
 #pragma once
 #include <atomic>
 #include <type_traits>
