@@ -329,6 +329,33 @@ def test_grouped_geometries(psi, oracle, device, dtype_name, hq, hkv, d, p, q_le
     assert dw.meta.num_row_groups > 0
 
 
+@pytest.mark.parametrize("seed", range(16))
+def test_grouped_random_batches(psi, oracle, device, seed):
+    """Seeded random batches through the row-group map against the oracle: head groups 1..8, both head dims, pages
+    of 8..64 tokens, both 16-bit types, partitions that do and do not divide the contexts, chunks from one token to
+    a few hundred next to decode-sized requests, contexts that end inside a tile, on a tile boundary and inside
+    the first tile."""
+    rng = np.random.default_rng(7000 + seed)
+    wl = importlib_workloads(psi)
+    group = int(rng.choice([1, 2, 4, 5, 6, 7, 8]))
+    hkv = int(rng.choice([1, 2, 4]))
+    d = int(rng.choice([128, 256]))
+    p = int(rng.choice([8, 16, 32, 64]))
+    dtype = psi.Dtype.Bfloat16 if rng.random() < 0.7 else psi.Dtype.Float16
+    n = int(rng.integers(1, 5))
+    q_lens = [int(rng.choice([1, 2, 7, 8, 9, 33, 64, 100, 257])) for _ in range(n)]
+    prefixes = [int(rng.choice([0, 1, 15, 31, 32, 33, 200, 511, 777])) for _ in range(n)]
+    ctx = [a + b for a, b in zip(prefixes, q_lens)]
+    partition = int(rng.choice([64, 128, 256, 2048]))
+    w = wl.make_workload(7100 + seed, ctx, group * hkv, hkv, d, dtype, p, q_lens=q_lens,
+                         num_page_ids_per_block=int(rng.choice([1, 2])))
+    variant = psi.GQASplitKVVariant.TiledQ(8, 16, group)
+    _, dw = run_and_check(psi, oracle, device, w,
+                          f"grouped random {seed}: G={group} Hkv={hkv} D={d} P={p} q={q_lens} on {prefixes} part={partition}",
+                          max_tokens=1024, variant=variant, partition_tokens=partition, grouped=True)
+    assert dw.meta.num_row_groups > 0
+
+
 def test_grouped_and_plain_maps_agree(psi, oracle, device):
     """Same plan through both maps: the outputs differ only in rounding, the grouped table falls
     back to the plain map where the geometry has no grouped kernel (head_dim 64)."""
