@@ -70,6 +70,11 @@ struct psi_hip_ctx {
     // with plain stores: nothing on the GPU reads or clears them.
     volatile uint32_t* status_host = nullptr;
     uint32_t* status_device = nullptr;
+    // Two zeroed words of device memory through which the workgroups of a prefill-chunk map launch share out its work
+    // items; the launch leaves them zero again.  One launch at a time uses them: the context's launches run on its
+    // stream, one after the other.
+    uint32_t* work_claim = nullptr;
+    int num_cus = 0;  // compute units of the device
     bool mute_loaders = false;  // harness switch: the maps' loading waves announce nothing, so that waits run out
     std::map<std::string, psi::KernelTimer> timers;
     std::vector<hipEvent_t> event_pool;

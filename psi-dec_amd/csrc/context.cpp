@@ -112,7 +112,15 @@ int psi_hip_ctx_create(int device, void* stream, psi_hip_ctx** out_ctx) {
         return psi::fail(PSI_HIP_ERR_RUNTIME, "the device status words cannot be mapped into device %d", device);
     }
     memset(status_host, 0, 64);
+    void* work_claim = nullptr;
+    if (hipMalloc(&work_claim, 64) != hipSuccess || hipMemset(work_claim, 0, 64) != hipSuccess) {
+        (void)hipHostFree(status_host);
+        if (work_claim != nullptr) (void)hipFree(work_claim);
+        return psi::fail(PSI_HIP_ERR_RUNTIME, "no device memory for the context's work counters on device %d", device);
+    }
     auto* ctx = new psi_hip_ctx();
+    ctx->work_claim = static_cast<uint32_t*>(work_claim);
+    ctx->num_cus = prop.multiProcessorCount;
     ctx->status_host = static_cast<volatile uint32_t*>(status_host);
     ctx->status_device = static_cast<uint32_t*>(status_device);
     ctx->device = device;
@@ -130,6 +138,7 @@ int psi_hip_ctx_destroy(psi_hip_ctx* ctx) {
         }
     for (auto ev : ctx->event_pool) (void)hipEventDestroy(ev);
     if (ctx->status_host != nullptr) (void)hipHostFree(const_cast<uint32_t*>(ctx->status_host));
+    if (ctx->work_claim != nullptr) (void)hipFree(ctx->work_claim);
     delete ctx;
     return PSI_HIP_OK;
 }

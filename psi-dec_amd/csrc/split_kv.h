@@ -64,12 +64,15 @@ struct MapArgs {
     // have landed, so that the other waves' waits run out.
     uint32_t* status = nullptr;
     uint32_t mute_loaders = 0;
+    // Prefill-chunk map: the context's two work-sharing words (psi_hip_ctx::work_claim).
+    uint32_t* work_claim = nullptr;
 };
 
-// Fills the two fields above from the context.
+// Fills the three fields above from the context.
 inline void set_device_status(MapArgs* a, const psi_hip_ctx* ctx) {
     a->status = ctx->status_device;
     a->mute_loaders = ctx->mute_loaders ? 1u : 0u;
+    a->work_claim = ctx->work_claim;
 }
 
 // First statement of every map kernel.

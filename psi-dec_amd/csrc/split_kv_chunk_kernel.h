@@ -61,6 +61,7 @@
 //        of two quarters.
 //   Q    at head_dim 256, the second column block's query operands, 8 KiB per wave.
 #pragma once
+#include <algorithm>
 #include <atomic>
 #include <type_traits>
 
@@ -137,13 +138,15 @@ struct ChunkLds {
     static constexpr int bytes = kQOffset + kChunkWaves * kQSteps * 1024;
 };
 
+// One work item: (row group, kv_head, part of the query heads) = item / (head_subsets * hkv), item / head_subsets %
+// hkv, item % head_subsets.  `next_item` (thread 0's) and `claimed`: see the kernel below.
 template <typename Tag, int D>
-__global__ __launch_bounds__(64 * kChunkWaves, 1) void split_kv_chunk_map(
-    MapArgs a, const uint32_t* __restrict__ page_ids, const uint32_t* __restrict__ kv_splits,
+__device__ __forceinline__ void chunk_map_item(
+    const MapArgs& a, const uint32_t* __restrict__ page_ids, const uint32_t* __restrict__ kv_splits,
     const uint32_t* __restrict__ req_slots, const uint16_t* __restrict__ q, const uint16_t* __restrict__ pages,
     const uint32_t* __restrict__ q_token_tiles, const uint32_t* __restrict__ flat_token_indices,
-    const uint32_t* __restrict__ row_groups, uint32_t group_tiles, uint32_t num_groups, uint32_t head_subsets) {
-    resolve_active(a);
+    const uint32_t* __restrict__ row_groups, uint32_t group_tiles, uint32_t num_groups, uint32_t head_subsets,
+    uint32_t item, uint32_t& next_item, bool& claimed) {
     static_assert(D == 256 || D == 128, "head_dim 128 or 256");
     constexpr int NB = kChunkColBlocks;
     constexpr int kKSteps = D / 32;
@@ -162,9 +165,9 @@ __global__ __launch_bounds__(64 * kChunkWaves, 1) void split_kv_chunk_map(
     extern __shared__ __attribute__((aligned(16))) unsigned char lds[];
 
     const uint32_t TS = a.rows_per_split_head;
-    const uint32_t subset = blockIdx.x % head_subsets;
-    const uint32_t kv_head = (blockIdx.x / head_subsets) % a.walk.hkv;
-    const uint32_t group = blockIdx.x / (head_subsets * a.walk.hkv);
+    const uint32_t subset = item % head_subsets;
+    const uint32_t kv_head = (item / head_subsets) % a.walk.hkv;
+    const uint32_t group = item / (head_subsets * a.walk.hkv);
     const uint32_t heads_per_subset = (a.group + head_subsets - 1) / head_subsets;
     const uint32_t head_first = kv_head * a.group + subset * heads_per_subset;
     const uint32_t tid = threadIdx.x;
@@ -277,7 +280,8 @@ __global__ __launch_bounds__(64 * kChunkWaves, 1) void split_kv_chunk_map(
     for (int i = 0; i < kLoads; ++i) {
         const uint32_t key = kWaveRows * wave + kRowsPerLoad * i + row_in_load;  // in the tile
         k_lane[i] = (kRowsPerLoad * i + row_in_load) * kRowBytes + ((slot ^ (key & 15)) * 16);
-        v_lane[i] = (kRowsPerLoad * i + row_in_load) * kRowBytes + (((((slot >> 1) ^ (key & 7)) << 1) | (slot & 1)) * 16);
+        v_lane[i] = kVOffset + (kWaveRows * wave + kRowsPerLoad * i + row_in_load) * kRowBytes +
+                    (((((slot >> 1) ^ (key & 7)) << 1) | (slot & 1)) * 16);
     }
     const uint32_t v_from = row_in_load * kRowBytes + slot * 16;  // (the rows of load i begin kRowsPerLoad * i rows on)
     auto issue_k_loads = [&](uint32_t t, uint32_t id) __attribute__((always_inline)) {
@@ -297,10 +301,11 @@ __global__ __launch_bounds__(64 * kChunkWaves, 1) void split_kv_chunk_map(
     };
     // The wave's V rows of tile t into their stage: as f16, and zero where a row lies outside the range - its
     // probability is 0, but its bytes may be NaN or Inf.
-    auto store_v_rows = [&](uint32_t t, const VRows& r) __attribute__((always_inline)) {
+    // (the stage, t % kChunkVStages, is a constant where this is called: it goes into the store's immediate offset)
+    auto store_v_rows = [&](uint32_t t, auto stage, const VRows& r) __attribute__((always_inline)) {
         const uint32_t kb = key_base0 + t * kChunkKeys;
         const bool edge = kb < kv_begin || kb + kChunkKeys > kv_end_max;  // first or last tile of the range
-        unsigned char* mine = lds + kVOffset + (t % kChunkVStages) * kKBytes + kWaveRows * wave * kRowBytes;
+        unsigned char* mine = lds + decltype(stage)::value * kKBytes;
 #pragma unroll
         for (int i = 0; i < kLoads; ++i) {
             u32x4_t w = to_f16x8<Tag>(r.w[i]);
@@ -312,12 +317,14 @@ __global__ __launch_bounds__(64 * kChunkWaves, 1) void split_kv_chunk_map(
     // everything this wave has written to LDS is there, and every wave has come this far
     auto barrier = []() __attribute__((always_inline)) { asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory"); };
 
-    const uint32_t k_row0 = mt * kRowBytes;
+    // Where a lane reads its K operand of k-step ks: chunk (4 * ks + mc) ^ mt of row mt.  4 * ks and mc share no bit,
+    // so that is the lane's chunk of k-step 0 with ks * 64 bytes XORed in: one register, not one per k-step.
+    const uint32_t k_lane0 = mt * kRowBytes + ((mc ^ mt) * 16);
     // transposing reads: key 4 * mc + mt / 4 (and 16 on), dims 16 * db + 4 * (mt % 4) ..; the 32-byte chunk db of a
     // row sits at chunk db ^ (key % 8)
     const uint32_t v_key = 4 * mc + (mt >> 2);
-    const uint32_t v_row0 = v_key * kRowBytes + (mt & 3) * 8;
-    const uint32_t v_swizzle = (v_key & 7) * 32;
+    // (likewise one register: the lane's place in chunk 0 ^ (key % 8), with (db % 8) * 32 XORed in and db / 8 * 256 added)
+    const uint32_t v_lane0 = kVOffset + v_key * kRowBytes + (mt & 3) * 8 + (v_key & 7) * 32;
     float run_max[NB], lane_sum[NB];
     f32x4_t o[NB][kDimBlocks];
 #pragma unroll
@@ -340,7 +347,8 @@ __global__ __launch_bounds__(64 * kChunkWaves, 1) void split_kv_chunk_map(
     // k-steps between an operand's read and its product (head_dim 128 has the registers for two)
     constexpr int kAhead = D == 256 ? 1 : 2;
     uint32_t next_id = 0;
-    auto tile = [&](uint32_t it, VRows& v_rows) __attribute__((always_inline)) {
+    auto tile = [&](uint32_t it, auto v_stage, VRows& v_rows) __attribute__((always_inline)) {
+        constexpr int kVStage = decltype(v_stage)::value;  // it % kChunkVStages
         asm volatile("s_waitcnt vmcnt(%0)" ::"n"(3 * kLoads) : "memory");
         barrier();
         const uint32_t id = next_id;   // of tile it + 3, asked for a tile ago: a page id takes as long as an LDS round trip,
@@ -348,8 +356,7 @@ __global__ __launch_bounds__(64 * kChunkWaves, 1) void split_kv_chunk_map(
         issue_k_loads(it + 3, id);
         const bool mine = it < my_tiles;  // (a wave that sees none of the tile's keys still does its share of the loads)
 
-        const unsigned char* kbuf = lds + (it % kChunkStages) * kKBytes;
-        const unsigned char* vbuf = lds + kVOffset + (it % kChunkVStages) * kKBytes;
+        const uint32_t k_at = (it % kChunkStages) * kKBytes + k_lane0;
         const uint32_t kb = key_base0 + it * kChunkKeys;
         const bool masked = !(kb >= kv_begin && kb + kChunkKeys <= wave_lo);
         float logits[NB][8];
@@ -361,9 +368,9 @@ __global__ __launch_bounds__(64 * kChunkWaves, 1) void split_kv_chunk_map(
         uint4 k0[kKSteps], k1[kKSteps], q1[kKSteps];
         // the operands of k-step ks: two key blocks of K, and the second column block's queries
         auto read_k = [&](int ks) __attribute__((always_inline)) {
-            const uint32_t off = k_row0 + (((4 * ks + mc) ^ mt) * 16);
-            k0[ks] = *reinterpret_cast<const uint4*>(kbuf + off);
-            k1[ks] = *reinterpret_cast<const uint4*>(kbuf + off + 16 * kRowBytes);
+            const unsigned char* src = lds + (k_at ^ (ks * 64));
+            k0[ks] = *reinterpret_cast<const uint4*>(src);
+            k1[ks] = *reinterpret_cast<const uint4*>(src + 16 * kRowBytes);
             if constexpr (kQInLds) q1[ks] = *reinterpret_cast<const uint4*>(q_lds + ks * 1024);
             else q1[ks] = qreg1[ks];
         };
@@ -372,18 +379,18 @@ __global__ __launch_bounds__(64 * kChunkWaves, 1) void split_kv_chunk_map(
         for (int ks = 0; ks < kAhead; ++ks) read_k(ks);
 #pragma unroll
         for (int ks = 0; ks < kKSteps; ++ks) {
+            if (ks + kAhead < kKSteps) read_k(ks + kAhead);
             s0[0] = mfma_16x16x32<Tag>(k0[ks], qreg[ks], s0[0]);
             s1[0] = mfma_16x16x32<Tag>(k1[ks], qreg[ks], s1[0]);
             s0[1] = mfma_16x16x32<Tag>(k0[ks], q1[ks], s0[1]);
             s1[1] = mfma_16x16x32<Tag>(k1[ks], q1[ks], s1[1]);
-            if (ks + kAhead < kKSteps) read_k(ks + kAhead);
         }
         constexpr int kReads = kQInLds ? 3 : 2;  // LDS reads of a k-step
         __builtin_amdgcn_sched_group_barrier(0x100, kReads * kAhead, 0);  // the first reads
 #pragma unroll
         for (int ks = 0; ks < kKSteps - kAhead; ++ks) {
-            __builtin_amdgcn_sched_group_barrier(0x008, 4, 0);  // the products of a k-step
             __builtin_amdgcn_sched_group_barrier(0x100, kReads, 0);  // the reads kAhead steps on
+            __builtin_amdgcn_sched_group_barrier(0x008, 4, 0);  // the products of a k-step
         }
         __builtin_amdgcn_sched_group_barrier(0x008, 4 * kAhead, 0);
         __builtin_amdgcn_sched_barrier(0);
@@ -392,7 +399,7 @@ __global__ __launch_bounds__(64 * kChunkWaves, 1) void split_kv_chunk_map(
 #pragma unroll
             for (int i = 0; i < 8; ++i) logits[j][i] = i < 4 ? s0[j][i] : s1[j][i - 4];
         }
-        if (it + 1 < group_kv_tiles) store_v_rows(it + 1, v_rows);
+        if (it + 1 < group_kv_tiles) store_v_rows(it + 1, std::integral_constant<int, 1 - kVStage>{}, v_rows);
         load_v_rows(it + 3, id, v_rows);
         if (!mine) return;
         uint4 pb[NB];
@@ -439,7 +446,7 @@ __global__ __launch_bounds__(64 * kChunkWaves, 1) void split_kv_chunk_map(
             uint4 vt[kVGroup];
 #pragma unroll
             for (int i = 0; i < kVGroup; ++i) {
-                const unsigned char* src = vbuf + v_row0 + (((g + i) * 32) ^ v_swizzle);
+                const unsigned char* src = lds + (v_lane0 ^ (((g + i) & 7) * 32)) + (kVStage * kKBytes + ((g + i) & 8) * 32);
                 const uint2 lo2 = lds_read_tr16_b64(src), hi2 = lds_read_tr16_b64(src + 16 * kRowBytes);
                 vt[i] = make_uint4(lo2.x, lo2.y, hi2.x, hi2.y);
             }
@@ -459,17 +466,33 @@ __global__ __launch_bounds__(64 * kChunkWaves, 1) void split_kv_chunk_map(
         load_v_rows(1, id1, odd);
         issue_k_loads(2, id2);
         load_v_rows(2, id2, even);
-        store_v_rows(0, first);
+        store_v_rows(0, std::integral_constant<int, 0>{}, first);
         uint32_t it = 0;
         for (; it + 1 < group_kv_tiles; it += 2) {
-            tile(it, odd);
-            tile(it + 1, even);
+            tile(it, std::integral_constant<int, 0>{}, odd);
+            tile(it + 1, std::integral_constant<int, 1>{}, even);
         }
-        if (it < group_kv_tiles) tile(it, odd);
+        if (it < group_kv_tiles) tile(it, std::integral_constant<int, 0>{}, odd);
         // The loads of tiles past the end go to LDS: they must be through before the workgroup gives it back.
         asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
     }
 
+    // The workgroup's next item is asked for here, so that the answer travels while the results are stored.
+    if (tid == 0) next_item = gridDim.x + atomicAdd(a.work_claim, 1u);
+    claimed = true;
+
+    // Where the columns' partial rows go.  Both blocks' rows are known before either block's stores are issued: the
+    // row numbers come from memory, and a wait for a load waits for every store issued before it as well.  (A row
+    // number fits 32 bits: the partial accumulators, D floats a row, fit the GPU's memory.)
+    uint32_t part_row[NB];
+#pragma unroll
+    for (int j = 0; j < NB; ++j) {
+        uint32_t t, h;
+        column_of(j, &t, &h);
+        part_row[j] = (rows[t / TS] * a.hq + head_first + h) * TS + t % TS;
+    }
+#pragma unroll
+    for (int j = 0; j < NB; ++j) asm volatile("" : "+v"(part_row[j]));
 #pragma unroll
     for (int j = 0; j < NB; ++j) {
         lane_sum[j] += __shfl_xor(lane_sum[j], 16, 64);
@@ -485,14 +508,11 @@ __global__ __launch_bounds__(64 * kChunkWaves, 1) void split_kv_chunk_map(
         if (__any(lim[j] != 0 && probe != probe) && lane == 0)
             __hip_atomic_store(a.status + 1, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
         if (lim[j] != 0) {
-            uint32_t t, h;
-            column_of(j, &t, &h);
-            const uint64_t part_row = ((uint64_t)rows[t / TS] * a.hq + head_first + h) * TS + t % TS;
             if (mc == 0) {
-                a.part_max[part_row] = run_max[j];
-                a.part_sum[part_row] = lane_sum[j];
+                a.part_max[part_row[j]] = run_max[j];
+                a.part_sum[part_row[j]] = lane_sum[j];
             }
-            float* dst = a.part_acc + part_row * D + mc * 4;
+            float* dst = a.part_acc + (uint64_t)part_row[j] * D + mc * 4;
 #pragma unroll
             for (int db = 0; db < kDimBlocks; ++db)
                 *reinterpret_cast<float4*>(dst + db * 16) = make_float4(o[j][db][0], o[j][db][1], o[j][db][2], o[j][db][3]);
@@ -500,26 +520,73 @@ __global__ __launch_bounds__(64 * kChunkWaves, 1) void split_kv_chunk_map(
     }
 }
 
+// The grid is as many workgroups as the GPU holds at once, and a workgroup takes items until there are none left:
+// the first is its own number, the others come from a counter, in the order of the list (longest first).  The
+// hardware hands the workgroups of a larger grid to the compute units in a fixed rotation, and a workgroup waits for
+// the unit whose turn it is while others stand idle: with items of 4 to 128 tiles a launch then ended a tenth later
+// than with items taken as units become free.
+//   work_claim[0] counts the items handed out beyond the first of each workgroup, work_claim[1] the workgroups that
+// are through; the last one out sets both back to zero for the next launch (launches of a context run one after
+// the other, on its stream).
+template <typename Tag, int D>
+__global__ __launch_bounds__(64 * kChunkWaves, 1) void split_kv_chunk_map(
+    MapArgs a, const uint32_t* __restrict__ page_ids, const uint32_t* __restrict__ kv_splits,
+    const uint32_t* __restrict__ req_slots, const uint16_t* __restrict__ q, const uint16_t* __restrict__ pages,
+    const uint32_t* __restrict__ q_token_tiles, const uint32_t* __restrict__ flat_token_indices,
+    const uint32_t* __restrict__ row_groups, uint32_t group_tiles, uint32_t num_groups, uint32_t head_subsets,
+    uint32_t num_items) {
+    resolve_active(a);
+    extern __shared__ __attribute__((aligned(16))) unsigned char lds[];
+    volatile uint32_t* mailbox = reinterpret_cast<volatile uint32_t*>(lds + 1024);  // (clear of the item's first LDS words)
+    uint32_t item = blockIdx.x;
+    while (item < num_items) {
+        uint32_t next_item = 0;
+        bool claimed = false;
+        chunk_map_item<Tag, D>(a, page_ids, kv_splits, req_slots, q, pages, q_token_tiles, flat_token_indices, row_groups,
+                               group_tiles, num_groups, head_subsets, item, next_item, claimed);
+        if (!claimed && threadIdx.x == 0) next_item = gridDim.x + atomicAdd(a.work_claim, 1u);
+        __syncthreads();  // every wave is through with the item's LDS
+        if (threadIdx.x == 0) *mailbox = next_item;
+        __syncthreads();
+        item = __builtin_amdgcn_readfirstlane(*mailbox);
+    }
+    if (threadIdx.x == 0 && atomicAdd(a.work_claim + 1, 1u) == gridDim.x - 1) {
+        __hip_atomic_store(a.work_claim, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        __hip_atomic_store(a.work_claim + 1, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    }
+}
+
 template <typename Tag, int D>
 inline int launch_chunk_map_typed(psi_hip_ctx* ctx, const Geometry& g, const MapArgs& a, const uint32_t* row_groups,
                                   uint32_t group_tiles, uint32_t num_groups) {
     const uint32_t subsets = chunk_head_subsets(g.group);
-    const dim3 grid(num_groups * g.hkv * subsets);
+    const uint32_t num_items = num_groups * g.hkv * subsets;
+    if (num_items == 0) return PSI_HIP_OK;
     auto* kernel = &split_kv_chunk_map<Tag, D>;
     // The kernel's LDS is above the default limit of a launch; the limit is raised once per GPU and kernel (a
-    // function's attributes belong to the device it is loaded on).
+    // function's attributes belong to the device it is loaded on).  How many workgroups the GPU holds at once is
+    // asked then, too.
     static std::atomic<uint64_t> raised_on{0};
+    static std::atomic<int> resident_per_cu{0};
     const uint64_t device_bit = 1ull << (ctx->device & 63);
     if ((raised_on.load(std::memory_order_relaxed) & device_bit) == 0) {
         if (hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
                                 ChunkLds<D>::bytes) != hipSuccess)
             return PSI_HIP_ERR_UNSUPPORTED;
+        int per_cu = 0;
+        if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, kernel, 64 * kChunkWaves, ChunkLds<D>::bytes) !=
+                hipSuccess ||
+            per_cu < 1)
+            return PSI_HIP_ERR_UNSUPPORTED;
+        resident_per_cu.store(per_cu, std::memory_order_relaxed);
         raised_on.fetch_or(device_bit, std::memory_order_relaxed);
     }
+    const uint32_t resident = (uint32_t)resident_per_cu.load(std::memory_order_relaxed) * (uint32_t)ctx->num_cus;
+    const dim3 grid(std::min(num_items, resident));
     hipLaunchKernelGGL(kernel, grid, dim3(64 * kChunkWaves), ChunkLds<D>::bytes, ctx->stream, a, a.walk.page_ids,
                        a.kv_splits, a.req_slots, reinterpret_cast<const uint16_t*>(a.q),
                        reinterpret_cast<const uint16_t*>(a.kv_pages), a.q_token_tiles, a.flat_token_indices, row_groups,
-                       group_tiles, num_groups, subsets);
+                       group_tiles, num_groups, subsets, num_items);
     return PSI_HIP_OK;
 }
 
