@@ -161,6 +161,9 @@ __device__ __forceinline__ void chunk_map_item(
     constexpr int kQSteps = ChunkLds<D>::kQSteps;
     constexpr bool kQInLds = kQSteps != 0;
     static_assert(kQSteps == kKSteps || kQSteps == 0, "the second block's queries live in LDS, or in registers");
+    // k-steps of the second block whose queries are in registers.  (At head_dim 256 two of the eight fit instead of
+    // the second set of operand registers below, and bought less than that set does; three spill inside the loop.)
+    constexpr int kQ1Regs = kQInLds ? 0 : kKSteps;
     constexpr float kSlack = 8.0f;
     extern __shared__ __attribute__((aligned(16))) unsigned char lds[];
 
@@ -212,7 +215,7 @@ __device__ __forceinline__ void chunk_map_item(
     uint32_t lim[NB];
     unsigned char* q_lds = lds + ChunkLds<D>::kQOffset + wave * (kQSteps * 1024) + lane * 16;
     uint4 qreg[kKSteps];                     // the first block's
-    uint4 qreg1[kQInLds ? 1 : kKSteps];      // the second block's, unless they live in LDS
+    uint4 qreg1[kQ1Regs > 0 ? kQ1Regs : 1];  // the second block's, as far as they live in registers
 #pragma unroll
     for (int j = 0; j < NB; ++j) {
         uint32_t t, h;
@@ -224,8 +227,8 @@ __device__ __forceinline__ void chunk_map_item(
         for (int ks = 0; ks < kKSteps; ++ks) {
             const uint4 operand = used[j] ? *reinterpret_cast<const uint4*>(q_row + ks * 32) : make_uint4(0, 0, 0, 0);
             if (j == 0) qreg[ks] = operand;
-            else if constexpr (kQInLds) *reinterpret_cast<uint4*>(q_lds + ks * 1024) = operand;
-            else qreg1[ks] = operand;
+            else if (ks < kQ1Regs) qreg1[ks] = operand;
+            else *reinterpret_cast<uint4*>(q_lds + ks * 1024) = operand;
         }
     }
     uint32_t lo = 0xffffffffu, hi = 0;
@@ -346,6 +349,9 @@ __device__ __forceinline__ void chunk_map_item(
     // of tile t + 2.
     // k-steps between an operand's read and its product (head_dim 128 has the registers for two)
     constexpr int kAhead = D == 256 ? 1 : 2;
+    // whether those reads are issued ahead of the products of the step before them (a second set of operand
+    // registers) or behind them (the same registers again, and the products' 64 cycles to cover the read)
+    constexpr bool kReadsFirst = true;
     uint32_t next_id = 0;
     auto tile = [&](uint32_t it, auto v_stage, VRows& v_rows) __attribute__((always_inline)) {
         constexpr int kVStage = decltype(v_stage)::value;  // it % kChunkVStages
@@ -371,8 +377,8 @@ __device__ __forceinline__ void chunk_map_item(
             const unsigned char* src = lds + (k_at ^ (ks * 64));
             k0[ks] = *reinterpret_cast<const uint4*>(src);
             k1[ks] = *reinterpret_cast<const uint4*>(src + 16 * kRowBytes);
-            if constexpr (kQInLds) q1[ks] = *reinterpret_cast<const uint4*>(q_lds + ks * 1024);
-            else q1[ks] = qreg1[ks];
+            if (ks < kQ1Regs) q1[ks] = qreg1[ks];
+            else q1[ks] = *reinterpret_cast<const uint4*>(q_lds + ks * 1024);
         };
         __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
@@ -385,12 +391,18 @@ __device__ __forceinline__ void chunk_map_item(
             s0[1] = mfma_16x16x32<Tag>(k0[ks], q1[ks], s0[1]);
             s1[1] = mfma_16x16x32<Tag>(k1[ks], q1[ks], s1[1]);
         }
-        constexpr int kReads = kQInLds ? 3 : 2;  // LDS reads of a k-step
-        __builtin_amdgcn_sched_group_barrier(0x100, kReads * kAhead, 0);  // the first reads
+        // LDS reads of k-step ks: the two K operands, and the second block's queries unless they are in registers
+        auto reads_of = [](int ks) __attribute__((always_inline)) {
+            if (ks < kQ1Regs) __builtin_amdgcn_sched_group_barrier(0x100, 2, 0);
+            else __builtin_amdgcn_sched_group_barrier(0x100, 3, 0);
+        };
+#pragma unroll
+        for (int ks = 0; ks < kAhead; ++ks) reads_of(ks);  // the first reads
 #pragma unroll
         for (int ks = 0; ks < kKSteps - kAhead; ++ks) {
-            __builtin_amdgcn_sched_group_barrier(0x100, kReads, 0);  // the reads kAhead steps on
+            if constexpr (kReadsFirst) reads_of(ks + kAhead);  // the reads kAhead steps on
             __builtin_amdgcn_sched_group_barrier(0x008, 4, 0);  // the products of a k-step
+            if constexpr (!kReadsFirst) reads_of(ks + kAhead);
         }
         __builtin_amdgcn_sched_group_barrier(0x008, 4 * kAhead, 0);
         __builtin_amdgcn_sched_barrier(0);
@@ -497,16 +509,6 @@ __device__ __forceinline__ void chunk_map_item(
     for (int j = 0; j < NB; ++j) {
         lane_sum[j] += __shfl_xor(lane_sum[j], 16, 64);
         lane_sum[j] += __shfl_xor(lane_sum[j], 32, 64);
-        // A V element that f16 cannot hold has reached the accumulators as Inf or NaN (the conversion rounds to
-        // nearest, so that it overflows instead of saturating): the host is told, and the rows stay as they are,
-        // visibly wrong.
-        float probe = 0.0f;
-#pragma unroll
-        for (int db = 0; db < kDimBlocks; ++db)
-#pragma unroll
-            for (int r = 0; r < 4; ++r) probe = __builtin_fmaf(o[j][db][r], 0.0f, probe);
-        if (__any(lim[j] != 0 && probe != probe) && lane == 0)
-            __hip_atomic_store(a.status + 1, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
         if (lim[j] != 0) {
             if (mc == 0) {
                 a.part_max[part_row[j]] = run_max[j];
@@ -518,6 +520,26 @@ __device__ __forceinline__ void chunk_map_item(
                 *reinterpret_cast<float4*>(dst + db * 16) = make_float4(o[j][db][0], o[j][db][1], o[j][db][2], o[j][db][3]);
         }
     }
+    // A V element that f16 cannot hold has reached the accumulators as Inf or NaN (the conversion rounds to nearest,
+    // so that it overflows instead of saturating): the host is told, and the rows stay as they are, visibly wrong.
+    // (Looked for behind the stores, which do not wait for it, and along eight chains rather than one.)
+    float probe[NB][4];
+#pragma unroll
+    for (int j = 0; j < NB; ++j)
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+            probe[j][r] = 0.0f;
+#pragma unroll
+            for (int db = 0; db < kDimBlocks; ++db) probe[j][r] = __builtin_fmaf(o[j][db][r], 0.0f, probe[j][r]);
+        }
+    bool out_of_range = false;
+#pragma unroll
+    for (int j = 0; j < NB; ++j) {
+        const float all = (probe[j][0] + probe[j][1]) + (probe[j][2] + probe[j][3]);
+        out_of_range |= lim[j] != 0 && all != all;
+    }
+    if (__any(out_of_range) && lane == 0)
+        __hip_atomic_store(a.status + 1, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
 }
 
 // The grid is as many workgroups as the GPU holds at once, and a workgroup takes items until there are none left:
