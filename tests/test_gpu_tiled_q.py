@@ -356,6 +356,28 @@ def test_grouped_random_batches(psi, oracle, device, seed):
     assert dw.meta.num_row_groups > 0
 
 
+def test_grouped_more_items_than_workgroups(psi, oracle, device):
+    """The row-group map runs one workgroup per compute unit, and a workgroup that is through with its item takes the
+    next from a counter that the launch leaves at zero.  Here the launch has several times as many items as the GPU
+    has compute units, of one to four KV tiles each; the outputs match the oracle, and a second and a third
+    step on the same context, the third after a small launch in between, repeat the first bit for bit."""
+    wl = importlib_workloads(psi)
+    w = wl.make_workload(95, [1100, 40], 24, 4, 256, psi.Dtype.Bfloat16, 16, q_lens=[900, 40])
+    _, dw = run_and_check(psi, oracle, device, w, "grouped chunk 900 on 200, 128-token partitions", max_tokens=1024,
+                          variant=psi.GQASplitKVVariant.TiledQ(8, 16, 6), partition_tokens=128, grouped=True,
+                          check_rounded=False)
+    items = dw.meta.num_row_groups * 4 * 3  # KV heads x head subsets
+    assert items > 512, items
+    first = dw.output_f32().copy()
+    dw.step()
+    assert np.array_equal(dw.output_f32(), first)
+    small = wl.make_workload(96, [70], 24, 4, 256, psi.Dtype.Bfloat16, 16, q_lens=[9])
+    run_and_check(psi, oracle, device, small, "grouped chunk 9 on 61", max_tokens=64,
+                  variant=psi.GQASplitKVVariant.TiledQ(8, 16, 6), partition_tokens=256, grouped=True, check_rounded=False)
+    dw.step()
+    assert np.array_equal(dw.output_f32(), first)
+
+
 def test_grouped_and_plain_maps_agree(psi, oracle, device):
     """Same plan through both maps: the outputs differ only in rounding, the grouped table falls
     back to the plain map where the geometry has no grouped kernel (head_dim 64)."""
