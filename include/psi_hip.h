@@ -95,7 +95,11 @@ const char* psi_hip_version(void);
 
 /* Replaces `Device::system_default()` + `Stream::new` (crates/inference-backend-metal/src/metal/mod.rs:12-40).
  * `stream` is a hipStream_t (NULL = the default stream); every launch of this context goes to
- * it.  A context is confined to one thread, like the reference's executor. */
+ * it.  A context is confined to one thread, like the reference's executor.  The context owns 64 bytes of pinned
+ * host memory (the device error words) and 64 bytes of device memory (the counters through which the workgroups of
+ * a prefill-chunk map share out its work: zero between launches, so the launches of one context must follow one
+ * another on its stream, as they do, and two contexts never share them); both are allocated here and freed by
+ * psi_hip_ctx_destroy, no launch allocates. */
 int psi_hip_ctx_create(int device, void* stream, psi_hip_ctx** out_ctx);
 int psi_hip_ctx_destroy(psi_hip_ctx* ctx);
 int psi_hip_ctx_set_stream(psi_hip_ctx* ctx, void* stream);
@@ -494,9 +498,10 @@ int psi_hip_split_kv_tiled_q_map_balanced(
     uint32_t num_total_q_token_tiles, uint32_t num_total_kv_splits, uint32_t num_active_tokens,
     uint32_t num_active_q_token_tiles, uint32_t num_active_kv_splits, uint32_t max_active_q_tile_tokens);
 
-/* psi_hip_split_kv_tiled_q_map with one workgroup per (row group, KV head [, half of the Q heads]):
+/* psi_hip_split_kv_tiled_q_map with one work item per (row group, KV head [, half or a third of the Q heads]):
  * the group's K/V tiles are staged once in LDS for up to 256 query columns and both contractions run
- * on the matrix cores.  Same arguments, scratch layout and results (within rounding) as the plain map;
+ * on the matrix cores.  The launch is one workgroup per compute unit; a workgroup takes items, in the table's
+ * order, until none is left.  Same arguments, scratch layout and results (within rounding) as the plain map;
  * row_groups: device copy of the table of psi_hip_split_kv_tiled_q_group_rows for the same kv_splits.
  * Geometries outside the grouped kernel (other than bf16 / f16, head_dim 128 or 256, pages of 8*2^k
  * tokens) run the plain map. */
