@@ -9,9 +9,9 @@ int launch_decode_map_bf16_d128(psi_hip_ctx* ctx, const Geometry& g, const MapAr
 int launch_decode_map_f16_d256(psi_hip_ctx* ctx, const Geometry& g, const MapArgs& a);
 int launch_decode_map_f16_d128(psi_hip_ctx* ctx, const Geometry& g, const MapArgs& a);
 
-// Log-sum-exp combine: one wave per (token, q_head), lanes over head_dim.  The row maxima are
-// fetched lane-parallel first; the accumulator rows are then read four at a time so that a wave
-// keeps several 1 KiB reads in flight instead of one.
+// Log-sum-exp combine: one wave per (token, q_head), lanes over head_dim.  The accumulator rows are
+// read four at a time so that a wave keeps several 1 KiB reads in flight instead of one; the overall
+// maximum comes from the first four rows' own values and a lane-parallel pass over the rest.
 template <typename Tag, int D, bool kIndexed>
 __global__ __launch_bounds__(256) void split_kv_reduce_fast(ReduceArgs a) {
     resolve_active(a);
@@ -22,34 +22,45 @@ __global__ __launch_bounds__(256) void split_kv_reduce_fast(ReduceArgs a) {
     if (row_out >= (uint64_t)a.num_active_tokens * a.hq) return;
     const uint32_t token = (uint32_t)(row_out / a.hq), q_head = (uint32_t)(row_out % a.hq);
     const uint32_t begin = a.cu_kv_splits[token], end = a.cu_kv_splits[token + 1];
-    float global_max = -INFINITY;
     const uint32_t* row_index = a.row_index;
-    for (uint32_t p = begin + lane; p < end; p += 64)
-        global_max = fmaxf(global_max, a.part_max[(uint64_t)(kIndexed ? row_index[p] : p) * a.hq + q_head]);
-#pragma unroll
-    for (int off = 32; off > 0; off >>= 1) global_max = fmaxf(global_max, __shfl_xor(global_max, off, 64));
-    float weight_sum = 0.0f, value[kPerLane];
-#pragma unroll
-    for (int e = 0; e < kPerLane; ++e) value[e] = 0.0f;
-    for (uint32_t p0 = begin; p0 < end; p0 += kUnroll) {
-        float w[kUnroll], sums[kUnroll], part[kUnroll][kPerLane];
+    auto row_of = [&](uint32_t p) -> uint64_t { return (uint64_t)(kIndexed ? row_index[p] : p) * a.hq + q_head; };
+    // The first four rows are asked for before anything waits: their maxima (the same in every lane) enter the
+    // overall maximum from registers, and the lane-parallel pass over the maxima covers the rows behind them only,
+    // so that a short list - the usual case - costs one round trip to memory instead of two.
+    float m[kUnroll], sums[kUnroll], part[kUnroll][kPerLane];
+    auto fetch = [&](uint32_t p0) __attribute__((always_inline)) {
 #pragma unroll
         for (int u = 0; u < kUnroll; ++u) {
             const bool live = p0 + u < end;
-            const uint32_t p = live ? p0 + u : begin;
-            const uint64_t row = (uint64_t)(kIndexed ? row_index[p] : p) * a.hq + q_head;
-            const float m = a.part_max[row];
+            const uint64_t row = row_of(live ? p0 + u : begin);
+            m[u] = a.part_max[row];
+            if (!live) m[u] = -INFINITY;
             sums[u] = a.part_sum[row];
-            w[u] = live && m > -INFINITY ? exp2f(m - global_max) : 0.0f;
             const float* src = a.part_acc + row * D + lane * kPerLane;
 #pragma unroll
             for (int e = 0; e < kPerLane; ++e) part[u][e] = src[e];
         }
+    };
+    if (begin < end) fetch(begin);
+    float global_max = -INFINITY;
+    for (uint32_t p = begin + kUnroll + lane; p < end; p += 64) global_max = fmaxf(global_max, a.part_max[row_of(p)]);
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) global_max = fmaxf(global_max, __shfl_xor(global_max, off, 64));
+    if (begin < end) {
+#pragma unroll
+        for (int u = 0; u < kUnroll; ++u) global_max = fmaxf(global_max, m[u]);
+    }
+    float weight_sum = 0.0f, value[kPerLane];
+#pragma unroll
+    for (int e = 0; e < kPerLane; ++e) value[e] = 0.0f;
+    for (uint32_t p0 = begin; p0 < end; p0 += kUnroll) {
+        if (p0 != begin) fetch(p0);
 #pragma unroll
         for (int u = 0; u < kUnroll; ++u) {
-            weight_sum = fmaf(w[u], sums[u], weight_sum);
+            const float w = m[u] > -INFINITY ? exp2f(m[u] - global_max) : 0.0f;
+            weight_sum = fmaf(w, sums[u], weight_sum);
 #pragma unroll
-            for (int e = 0; e < kPerLane; ++e) value[e] = fmaf(w[u], part[u][e], value[e]);
+            for (int e = 0; e < kPerLane; ++e) value[e] = fmaf(w, part[u][e], value[e]);
         }
     }
     const float inv = weight_sum > 0.0f ? 1.0f / weight_sum : 0.0f;
@@ -152,35 +163,45 @@ __global__ __launch_bounds__(256) void split_kv_reduce_tiled_fast(ReduceArgs a) 
     if (token >= flat_end) return;
     const uint32_t begin = a.cu_kv_splits[tile], end = a.cu_kv_splits[tile + 1];
     constexpr int kUnroll = 4;
-    float global_max = -INFINITY;
     const uint32_t* row_index = a.row_index;
-    for (uint32_t p = begin + lane; p < end; p += 64)
-        global_max = fmaxf(global_max,
-                           a.part_max[((uint64_t)(kIndexed ? row_index[p] : p) * a.hq + q_head) * rows + tile_row]);
-#pragma unroll
-    for (int off = 32; off > 0; off >>= 1) global_max = fmaxf(global_max, __shfl_xor(global_max, off, 64));
-    float weight_sum = 0.0f, value[kPerLane];
-#pragma unroll
-    for (int e = 0; e < kPerLane; ++e) value[e] = 0.0f;
-    for (uint32_t p0 = begin; p0 < end; p0 += kUnroll) {
-        float w[kUnroll], sums[kUnroll], part[kUnroll][kPerLane];
+    auto row_of = [&](uint32_t p) -> uint64_t {
+        return ((uint64_t)(kIndexed ? row_index[p] : p) * a.hq + q_head) * rows + tile_row;
+    };
+    // (the first four rows ahead of the pass over the maxima, as in split_kv_reduce_fast)
+    float m[kUnroll], sums[kUnroll], part[kUnroll][kPerLane];
+    auto fetch = [&](uint32_t p0) __attribute__((always_inline)) {
 #pragma unroll
         for (int u = 0; u < kUnroll; ++u) {
             const bool live = p0 + u < end;
-            const uint32_t p = live ? p0 + u : begin;
-            const uint64_t row = ((uint64_t)(kIndexed ? row_index[p] : p) * a.hq + q_head) * rows + tile_row;
-            const float m = a.part_max[row];
+            const uint64_t row = row_of(live ? p0 + u : begin);
+            m[u] = a.part_max[row];
+            if (!live) m[u] = -INFINITY;
             sums[u] = a.part_sum[row];
-            w[u] = live && m > -INFINITY ? exp2f(m - global_max) : 0.0f;
             const float* src = a.part_acc + row * D + lane * kPerLane;
 #pragma unroll
             for (int e = 0; e < kPerLane; ++e) part[u][e] = src[e];
         }
+    };
+    if (begin < end) fetch(begin);
+    float global_max = -INFINITY;
+    for (uint32_t p = begin + kUnroll + lane; p < end; p += 64) global_max = fmaxf(global_max, a.part_max[row_of(p)]);
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) global_max = fmaxf(global_max, __shfl_xor(global_max, off, 64));
+    if (begin < end) {
+#pragma unroll
+        for (int u = 0; u < kUnroll; ++u) global_max = fmaxf(global_max, m[u]);
+    }
+    float weight_sum = 0.0f, value[kPerLane];
+#pragma unroll
+    for (int e = 0; e < kPerLane; ++e) value[e] = 0.0f;
+    for (uint32_t p0 = begin; p0 < end; p0 += kUnroll) {
+        if (p0 != begin) fetch(p0);
 #pragma unroll
         for (int u = 0; u < kUnroll; ++u) {
-            weight_sum = fmaf(w[u], sums[u], weight_sum);
+            const float w = m[u] > -INFINITY ? exp2f(m[u] - global_max) : 0.0f;
+            weight_sum = fmaf(w, sums[u], weight_sum);
 #pragma unroll
-            for (int e = 0; e < kPerLane; ++e) value[e] = fmaf(w[u], part[u][e], value[e]);
+            for (int e = 0; e < kPerLane; ++e) value[e] = fmaf(w, part[u][e], value[e]);
         }
     }
     const float inv = weight_sum > 0.0f ? 1.0f / weight_sum : 0.0f;
