@@ -19,7 +19,8 @@
 //   per SIMD nothing hides the latencies of a wave's own chain (operand reads, matrix results, exponentials);
 //   with two, each fills the other's gaps.
 //
-//   No wave only loads: every wave fetches four rows of K and four of V of every tile.  K goes straight to LDS
+//   A KV tile is 16 KiB of K and 16 KiB of V: 32 keys at head_dim 256, 64 at head_dim 128.  No wave only loads:
+//   every wave fetches an eighth of the rows of K and of V of every tile.  K goes straight to LDS
 //   with `global_load_lds_dwordx4`, which moves 16 bytes per lane from a per-lane global address to LDS address
 //   M0 + 16 * lane with no register in between, three tiles ahead, into a ring of four K tiles.  V goes through
 //   registers, two tiles ahead (two register sets, taken in turn), where bf16 becomes f16, into a ring of two V
@@ -27,7 +28,7 @@
 //   tile t + 1 land (a wave's loads complete in the order of their issue); behind it everybody has, and every
 //   wave is through with tile t - 1.  No wait between waves other than the barrier, so none that could run out.
 //
-// Per 32-key tile and wave (2 x 16 columns)
+// Per tile and wave (2 x 16 columns), for each 32 keys of the tile
 //   QK^T  S[key][column] on v_mfma_f32_16x16x32 of the storage type: A = K rows from LDS (key 16 * b + i in row i of
 //         key block b), B = the query columns: the first block's held in registers for the whole kernel, the second
 //         block's too at head_dim 128, and read from LDS with the K operands at head_dim 256 (64 registers of
@@ -52,11 +53,11 @@
 //         needs no cross-lane traffic.
 //
 // LDS layout
-//   K    four tiles of [32 keys][D] elements, 16-byte chunk index XOR (key % 16): the 16 lanes of an operand read
+//   K    four tiles of [32 or 64 keys][D] elements, 16-byte chunk index XOR (key % 16): the 16 lanes of an operand read
 //        (16 rows, one chunk) then hit 16 different bank groups.  (The loads write 1 KiB in lane order, so the
 //        layout can permute 16-byte chunks within a row, through the choice of each lane's global address, but
 //        cannot pad rows.)
-//   V    two tiles of [32 keys][D] f16, 32-byte chunk index XOR (key % 8): the four keys of a quarter wave's
+//   V    two tiles of [32 or 64 keys][D] f16, 32-byte chunk index XOR (key % 8): the four keys of a quarter wave's
 //        transposing read (32 bytes each, 16 dims) then fall into different bank groups, and so do the eight keys
 //        of two quarters.
 //   Q    at head_dim 256, the second column block's query operands, 8 KiB per wave.
@@ -69,7 +70,11 @@
 
 namespace psi {
 
-constexpr int kChunkKeys = 32;      // keys per KV tile
+// Keys per KV tile: 32 at head_dim 256, 64 at head_dim 128 (the same 16 KiB of K and of V, and as many matrix
+// instructions between two barriers; with 32 keys at head_dim 128 a tile's fixed costs - barrier, first operand reads,
+// the way from the last product of K * Q^T to the first of V^T * P^T - weighed twice as much).
+template <int D>
+constexpr int kChunkKeysOf = D == 128 ? 64 : 32;
 constexpr int kChunkColBlocks = 2;  // 16-column blocks of a wave
 constexpr int kChunkWaves = 8;
 constexpr int kChunkStages = 4;   // K tiles in LDS
@@ -129,7 +134,7 @@ __device__ __forceinline__ void dma_16_bytes_per_lane(uint32_t lds_dst, const vo
 
 template <int D>
 struct ChunkLds {
-    static constexpr int kKBytes = kChunkKeys * D * 2;  // a tile of K, and of V
+    static constexpr int kKBytes = kChunkKeysOf<D> * D * 2;  // a tile of K, and of V
     static constexpr int kVOffset = kChunkStages * kKBytes;
     static constexpr int kQOffset = kVOffset + kChunkVStages * kKBytes;
     // k-steps of a wave's second column block whose query operands live here: all of them at head_dim 256 (128
@@ -154,7 +159,10 @@ __device__ __forceinline__ void chunk_map_item(
     constexpr int kRowBytes = D * 2;
     constexpr int kRowChunks = D / 8;                    // 16-byte chunks per key row: 32 or 16
     constexpr int kRowsPerLoad = 64 / kRowChunks;        // key rows that one load of a wave covers: 2 or 4
-    constexpr int kWaveRows = kChunkKeys / kChunkWaves;  // rows of K, and of V, that a wave fetches per tile
+    constexpr int kKeys = kChunkKeysOf<D>;
+    constexpr int kSub = kKeys / 32;                     // 32-key halves of a tile (what one V^T * P^T product spans)
+    constexpr int kKeyBlocks = kKeys / 16;               // 16-key blocks of a tile (what one K * Q^T product spans)
+    constexpr int kWaveRows = kKeys / kChunkWaves;       // rows of K, and of V, that a wave fetches per tile: 4 or 8
     constexpr int kLoads = kWaveRows / kRowsPerLoad;     // loads per wave, tile and operand: 2 or 1
     constexpr int kKBytes = ChunkLds<D>::kKBytes;
     constexpr int kVOffset = ChunkLds<D>::kVOffset;
@@ -199,8 +207,8 @@ __device__ __forceinline__ void chunk_map_item(
     const uint32_t ncols = (flat_end - flat_begin) * G;
     if (ncols > (uint32_t)kChunkCols || flat_end - flat_begin > num_tiles * TS) return;
     const uint32_t req_slot = req_slots[flat_begin];
-    const uint32_t key_base0 = kv_begin & ~(uint32_t)(kChunkKeys - 1);
-    const uint32_t num_kv_tiles = (kv_end_max - key_base0 + kChunkKeys - 1) / kChunkKeys;
+    const uint32_t key_base0 = kv_begin & ~(uint32_t)(kKeys - 1);
+    const uint32_t num_kv_tiles = (kv_end_max - key_base0 + kKeys - 1) / kKeys;
 
     // ---------------- the wave's columns ----------------
     // The partial row of column block j of this lane's column: (row of the tile's split, head, token in the tile).
@@ -241,7 +249,7 @@ __device__ __forceinline__ void chunk_map_item(
     const uint32_t wave_hi = __builtin_amdgcn_readfirstlane(wave_max_u32(hi));
     // tiles that hold a visible key of this wave, and of any wave of the workgroup
     const uint32_t my_tiles =
-        wave_hi > key_base0 ? min(num_kv_tiles, (wave_hi - key_base0 + kChunkKeys - 1) / kChunkKeys) : 0u;
+        wave_hi > key_base0 ? min(num_kv_tiles, (wave_hi - key_base0 + kKeys - 1) / kKeys) : 0u;
     uint32_t* tile_counts = reinterpret_cast<uint32_t*>(lds);  // (where the first tile will land)
     if (lane == 0) tile_counts[wave] = my_tiles;
     __syncthreads();
@@ -259,14 +267,14 @@ __device__ __forceinline__ void chunk_map_item(
                                                a.walk.ids_per_block;
     const uint64_t page_bytes = a.walk.page_elems * 2;
     const unsigned char* base = reinterpret_cast<const unsigned char*>(pages);
-    // Page ids come through the scalar cache.  The wave's four rows of a tile lie in one page (pages hold at least
-    // 8 tokens).  Rows past the end of the range (the last tile's) are taken from the range's last page: the table
+    // Page ids come through the scalar cache.  The wave's four or eight rows of a tile lie in one page (pages hold
+    // at least 8 tokens).  Rows past the end of the range (the last tile's) are taken from the range's last page: the table
     // need not hold a page for them, and nobody looks at what they hold.  Tiles past the last one are clamped to it,
     // so that every iteration issues the same number of loads and the counts of outstanding ones stay constants.
     const uint32_t last_page = (kv_end_max - 1) >> log2p;
     typedef const __attribute__((address_space(4))) uint32_t* ConstantIds;
     const ConstantIds ids_row = (ConstantIds)(uintptr_t)table_row;
-    auto first_key = [&](uint32_t t) { return key_base0 + min(t, group_kv_tiles - 1) * kChunkKeys + kWaveRows * wave; };
+    auto first_key = [&](uint32_t t) { return key_base0 + min(t, group_kv_tiles - 1) * kKeys + kWaveRows * wave; };
     auto page_of = [&](uint32_t t) -> uint32_t { return ids_row[min(first_key(t) >> log2p, last_page)]; };
     auto rows_of = [&](uint32_t t, uint32_t id) -> const unsigned char* {
         return base + id * page_bytes + (uint64_t)(first_key(t) & page_mask) * kRowBytes;
@@ -306,8 +314,8 @@ __device__ __forceinline__ void chunk_map_item(
     // probability is 0, but its bytes may be NaN or Inf.
     // (the stage, t % kChunkVStages, is a constant where this is called: it goes into the store's immediate offset)
     auto store_v_rows = [&](uint32_t t, auto stage, const VRows& r) __attribute__((always_inline)) {
-        const uint32_t kb = key_base0 + t * kChunkKeys;
-        const bool edge = kb < kv_begin || kb + kChunkKeys > kv_end_max;  // first or last tile of the range
+        const uint32_t kb = key_base0 + t * kKeys;
+        const bool edge = kb < kv_begin || kb + kKeys > kv_end_max;  // first or last tile of the range
         unsigned char* mine = lds + decltype(stage)::value * kKBytes;
 #pragma unroll
         for (int i = 0; i < kLoads; ++i) {
@@ -347,8 +355,8 @@ __device__ __forceinline__ void chunk_map_item(
     // then the softmax and the products with V.  The loads complete in the order of their issue: at the barrier
     // the K rows of tile t + 1 are followed by the V rows of tile t + 1, the K rows of tile t + 2 and the V rows
     // of tile t + 2.
-    // k-steps between an operand's read and its product (head_dim 128 has the registers for two)
-    constexpr int kAhead = D == 256 ? 1 : 2;
+    // k-steps between an operand's read and its product
+    constexpr int kAhead = 1;
     // whether those reads are issued ahead of the products of the step before them (a second set of operand
     // registers) or behind them (the same registers again, and the products' 64 cycles to cover the read)
     constexpr bool kReadsFirst = true;
@@ -363,20 +371,22 @@ __device__ __forceinline__ void chunk_map_item(
         const bool mine = it < my_tiles;  // (a wave that sees none of the tile's keys still does its share of the loads)
 
         const uint32_t k_at = (it % kChunkStages) * kKBytes + k_lane0;
-        const uint32_t kb = key_base0 + it * kChunkKeys;
-        const bool masked = !(kb >= kv_begin && kb + kChunkKeys <= wave_lo);
-        float logits[NB][8];
+        const uint32_t kb = key_base0 + it * kKeys;
+        const bool masked = !(kb >= kv_begin && kb + kKeys <= wave_lo);
+        float logits[NB][4 * kKeyBlocks];
         if (mine) {
         // (zeroed here, where the first products can take the zeros as a constant operand, not from registers)
-        f32x4_t s0[NB], s1[NB];
+        f32x4_t sc[kKeyBlocks][NB];
 #pragma unroll
-        for (int j = 0; j < NB; ++j) s0[j] = s1[j] = f32x4_t{0.0f, 0.0f, 0.0f, 0.0f};
-        uint4 k0[kKSteps], k1[kKSteps], q1[kKSteps];
-        // the operands of k-step ks: two key blocks of K, and the second column block's queries
+        for (int b = 0; b < kKeyBlocks; ++b)
+#pragma unroll
+            for (int j = 0; j < NB; ++j) sc[b][j] = f32x4_t{0.0f, 0.0f, 0.0f, 0.0f};
+        uint4 kk[kKeyBlocks][kKSteps], q1[kKSteps];
+        // the operands of k-step ks: the key blocks of K, and the second column block's queries
         auto read_k = [&](int ks) __attribute__((always_inline)) {
             const unsigned char* src = lds + (k_at ^ (ks * 64));
-            k0[ks] = *reinterpret_cast<const uint4*>(src);
-            k1[ks] = *reinterpret_cast<const uint4*>(src + 16 * kRowBytes);
+#pragma unroll
+            for (int b = 0; b < kKeyBlocks; ++b) kk[b][ks] = *reinterpret_cast<const uint4*>(src + 16 * b * kRowBytes);
             if (ks < kQ1Regs) q1[ks] = qreg1[ks];
             else q1[ks] = *reinterpret_cast<const uint4*>(q_lds + ks * 1024);
         };
@@ -386,46 +396,58 @@ __device__ __forceinline__ void chunk_map_item(
 #pragma unroll
         for (int ks = 0; ks < kKSteps; ++ks) {
             if (ks + kAhead < kKSteps) read_k(ks + kAhead);
-            s0[0] = mfma_16x16x32<Tag>(k0[ks], qreg[ks], s0[0]);
-            s1[0] = mfma_16x16x32<Tag>(k1[ks], qreg[ks], s1[0]);
-            s0[1] = mfma_16x16x32<Tag>(k0[ks], q1[ks], s0[1]);
-            s1[1] = mfma_16x16x32<Tag>(k1[ks], q1[ks], s1[1]);
+#pragma unroll
+            for (int j = 0; j < NB; ++j)
+#pragma unroll
+                for (int b = 0; b < kKeyBlocks; ++b)
+                    sc[b][j] = mfma_16x16x32<Tag>(kk[b][ks], j == 0 ? qreg[ks] : q1[ks], sc[b][j]);
         }
-        // LDS reads of k-step ks: the two K operands, and the second block's queries unless they are in registers
+        // LDS reads of k-step ks: the K operands, and the second block's queries unless they are in registers
+        static_assert(kKeyBlocks == 2 || (kKeyBlocks == 4 && kQ1Regs == kKSteps), "the literal counts below");
         auto reads_of = [](int ks) __attribute__((always_inline)) {
-            if (ks < kQ1Regs) __builtin_amdgcn_sched_group_barrier(0x100, 2, 0);
+            if (kKeyBlocks == 4) __builtin_amdgcn_sched_group_barrier(0x100, 4, 0);
+            else if (ks < kQ1Regs) __builtin_amdgcn_sched_group_barrier(0x100, 2, 0);
             else __builtin_amdgcn_sched_group_barrier(0x100, 3, 0);
+        };
+        auto products_of_a_step = []() __attribute__((always_inline)) {
+            if (kKeyBlocks == 4) __builtin_amdgcn_sched_group_barrier(0x008, 8, 0);
+            else __builtin_amdgcn_sched_group_barrier(0x008, 4, 0);
         };
 #pragma unroll
         for (int ks = 0; ks < kAhead; ++ks) reads_of(ks);  // the first reads
 #pragma unroll
         for (int ks = 0; ks < kKSteps - kAhead; ++ks) {
             if constexpr (kReadsFirst) reads_of(ks + kAhead);  // the reads kAhead steps on
-            __builtin_amdgcn_sched_group_barrier(0x008, 4, 0);  // the products of a k-step
+            products_of_a_step();
             if constexpr (!kReadsFirst) reads_of(ks + kAhead);
         }
-        __builtin_amdgcn_sched_group_barrier(0x008, 4 * kAhead, 0);
+#pragma unroll
+        for (int ks = 0; ks < kAhead; ++ks) products_of_a_step();
         __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
         for (int j = 0; j < NB; ++j)
 #pragma unroll
-            for (int i = 0; i < 8; ++i) logits[j][i] = i < 4 ? s0[j][i] : s1[j][i - 4];
+            for (int i = 0; i < 4 * kKeyBlocks; ++i) logits[j][i] = sc[i >> 2][j][i & 3];
         }
         if (it + 1 < group_kv_tiles) store_v_rows(it + 1, std::integral_constant<int, 1 - kVStage>{}, v_rows);
         load_v_rows(it + 3, id, v_rows);
         if (!mine) return;
-        uint4 pb[NB];
+        uint4 pb[NB][kSub];
 #pragma unroll
         for (int j = 0; j < NB; ++j) {
-            float (&v)[8] = logits[j];
+            constexpr int kMine = 4 * kKeyBlocks;  // the lane's keys of its column: 4 * mc + r of every key block
+            float (&v)[kMine] = logits[j];
             if (masked) {
 #pragma unroll
-                for (int i = 0; i < 8; ++i) {
+                for (int i = 0; i < kMine; ++i) {
                     const uint32_t token = kb + 16 * (i >> 2) + 4 * mc + (i & 3);
                     if (token < kv_begin || token >= lim[j]) v[i] = -INFINITY;
                 }
             }
-            float m = max3(max3(v[0], v[1], v[2]), max3(v[3], v[4], v[5]), max3(v[6], v[7], v[7])) * a.scale_log2;
+            float m = max3(max3(v[0], v[1], v[2]), max3(v[3], v[4], v[5]), max3(v[6], v[7], v[7]));
+            if constexpr (kMine == 16)
+                m = max3(m, max3(max3(v[8], v[9], v[10]), max3(v[11], v[12], v[13]), v[14]), v[15]);
+            m *= a.scale_log2;
             if (__any(m > run_max[j] + kSlack)) {
                 m = fmaxf(m, __shfl_xor(m, 16, 64));
                 m = fmaxf(m, __shfl_xor(m, 32, 64));
@@ -440,9 +462,9 @@ __device__ __forceinline__ void chunk_map_item(
                 }
             }
             const float neg_ref = run_max[j] > -INFINITY ? -run_max[j] : 0.0f;
-            uint32_t words[4];
+            uint32_t words[kMine / 2];
 #pragma unroll
-            for (int i = 0; i < 8; i += 2) {
+            for (int i = 0; i < kMine; i += 2) {
                 // rounded to nearest, once, for the product and for the sum alike
                 const f16x2_t h = {(_Float16)__builtin_amdgcn_exp2f(__builtin_fmaf(v[i], a.scale_log2, neg_ref)),
                                    (_Float16)__builtin_amdgcn_exp2f(__builtin_fmaf(v[i + 1], a.scale_log2, neg_ref))};
@@ -450,22 +472,28 @@ __device__ __forceinline__ void chunk_map_item(
                 lane_sum[j] = __builtin_amdgcn_fdot2(h, ones, lane_sum[j], false);
                 words[i / 2] = __builtin_bit_cast(uint32_t, h);
             }
-            pb[j] = make_uint4(words[0], words[1], words[2], words[3]);
+#pragma unroll
+            for (int sub = 0; sub < kSub; ++sub)
+                pb[j][sub] = make_uint4(words[4 * sub], words[4 * sub + 1], words[4 * sub + 2], words[4 * sub + 3]);
         }
         constexpr int kVGroup = 2;  // V operands read ahead of their products
 #pragma unroll
-        for (int g = 0; g < kDimBlocks; g += kVGroup) {
-            uint4 vt[kVGroup];
+        for (int sub = 0; sub < kSub; ++sub) {
 #pragma unroll
-            for (int i = 0; i < kVGroup; ++i) {
-                const unsigned char* src = lds + (v_lane0 ^ (((g + i) & 7) * 32)) + (kVStage * kKBytes + ((g + i) & 8) * 32);
-                const uint2 lo2 = lds_read_tr16_b64(src), hi2 = lds_read_tr16_b64(src + 16 * kRowBytes);
-                vt[i] = make_uint4(lo2.x, lo2.y, hi2.x, hi2.y);
+            for (int g = 0; g < kDimBlocks; g += kVGroup) {
+                uint4 vt[kVGroup];
+#pragma unroll
+                for (int i = 0; i < kVGroup; ++i) {
+                    const unsigned char* src = lds + (v_lane0 ^ (((g + i) & 7) * 32)) +
+                                               (kVStage * kKBytes + 32 * sub * kRowBytes + ((g + i) & 8) * 32);
+                    const uint2 lo2 = lds_read_tr16_b64(src), hi2 = lds_read_tr16_b64(src + 16 * kRowBytes);
+                    vt[i] = make_uint4(lo2.x, lo2.y, hi2.x, hi2.y);
+                }
+#pragma unroll
+                for (int i = 0; i < kVGroup; ++i)
+#pragma unroll
+                    for (int j = 0; j < NB; ++j) o[j][g + i] = mfma_16x16x32<F16Tag>(vt[i], pb[j][sub], o[j][g + i]);
             }
-#pragma unroll
-            for (int i = 0; i < kVGroup; ++i)
-#pragma unroll
-                for (int j = 0; j < NB; ++j) o[j][g + i] = mfma_16x16x32<F16Tag>(vt[i], pb[j], o[j][g + i]);
         }
     };
     if (group_kv_tiles != 0) {

@@ -1,6 +1,6 @@
-"""The LDS layout of the prefill-chunk map, checked on the host.  A K tile is [32 keys][head_dim] elements with the
-16-byte chunk index XORed with key % 16; a V tile is [32 keys][head_dim] f16 with the 32-byte chunk index XORed with
-key % 8.  The operand reads must put the lanes that an LDS read serves together on different bank groups and must
+"""The LDS layout of the prefill-chunk map, checked on the host.  A tile holds 32 keys at head_dim 256 and 64 at
+head_dim 128 (16 KiB either way).  A K tile is [keys][head_dim] elements with the 16-byte chunk index XORed with
+key % 16; a V tile is [keys][head_dim] f16 with the 32-byte chunk index XORed with key % 8.  The operand reads must put the lanes that an LDS read serves together on different bank groups and must
 find what the fetching waves put there: K arrives by loads that write 1 KiB in lane order (the layout is made by each
 lane's choice of global address), V by 128-bit stores.  The address arithmetic below restates
 psi-dec_amd/csrc/split_kv_chunk_kernel.h (k_row0, v_row0, v_swizzle, k_lane, v_lane); the lane groups of a 128-bit
@@ -13,9 +13,15 @@ READ_ROUNDS = [
     [4, 5, 6, 7, 8, 9, 10, 11, 16, 17, 18, 19, 28, 29, 30, 31],
 ]
 READ_ROUNDS += [[lane + 32 for lane in group] for group in READ_ROUNDS[:2]]
-KEYS = 32
 WAVES = 8
-WAVE_ROWS = KEYS // WAVES
+
+
+def keys_of(d):
+    return 64 if d == 128 else 32
+
+
+def wave_rows(d):
+    return keys_of(d) // WAVES
 
 
 def bank_group(byte_offset):
@@ -39,15 +45,15 @@ def v_read_offset(d, lane, db, block):
 def fetch_geometry(d):
     row_chunks = d // 8                 # 16-byte chunks per row
     rows_per_load = 64 // row_chunks    # rows that one load of a wave covers
-    return row_chunks, rows_per_load, WAVE_ROWS // rows_per_load
+    return row_chunks, rows_per_load, wave_rows(d) // rows_per_load
 
 
 def k_landing(d, wave, lane, i):
     """Load i of a wave: (LDS offset in the tile where the lane's 16 bytes land, key, 16-byte chunk they come from)."""
     row_chunks, rows_per_load, _ = fetch_geometry(d)
     row_in_load, slot = lane // row_chunks, lane % row_chunks
-    key = WAVE_ROWS * wave + rows_per_load * i + row_in_load
-    lands = (WAVE_ROWS * wave + rows_per_load * i) * d * 2 + lane * 16
+    key = wave_rows(d) * wave + rows_per_load * i + row_in_load
+    lands = (wave_rows(d) * wave + rows_per_load * i) * d * 2 + lane * 16
     return lands, key, slot ^ (key & 15)
 
 
@@ -55,7 +61,7 @@ def v_store(d, wave, lane, i):
     """Store i of a wave: (LDS offset in the tile, key, 16-byte chunk of the row that the lane holds)."""
     row_chunks, rows_per_load, _ = fetch_geometry(d)
     row_in_load, slot = lane // row_chunks, lane % row_chunks
-    key = WAVE_ROWS * wave + rows_per_load * i + row_in_load
+    key = wave_rows(d) * wave + rows_per_load * i + row_in_load
     where = key * d * 2 + ((((slot >> 1) ^ (key & 7)) << 1) | (slot & 1)) * 16
     return where, key, slot
 
@@ -74,8 +80,8 @@ def test_k_operand_reads_are_conflict_free_and_find_what_landed(d):
                 lands, key, chunk = k_landing(d, wave, lane, i)
                 assert lands // (d * 2) == key, "a lane's bytes land in the row of their key"
                 where[(key, chunk)] = lands
-    assert len(where) == KEYS * d // 8 and len(set(where.values())) == len(where)
-    for block in range(2):
+    assert len(where) == keys_of(d) * d // 8 and len(set(where.values())) == len(where)
+    for block in range(keys_of(d) // 16):
         for ks in range(d // 32):
             for group in READ_ROUNDS:
                 assert len({bank_group(k_read_offset(d, lane, ks, block)) for lane in group}) == 16
@@ -97,8 +103,8 @@ def test_transposing_reads_spread_their_keys_over_the_banks_and_find_what_was_st
                 at, key, chunk = v_store(d, wave, lane, i)
                 assert at // (d * 2) == key
                 where[(key, chunk)] = at
-    assert len(where) == KEYS * d // 8 and len(set(where.values())) == len(where)
-    for block in range(2):
+    assert len(where) == keys_of(d) * d // 8 and len(set(where.values())) == len(where)
+    for block in range(keys_of(d) // 16):
         for db in range(d // 16):
             for half in range(2):
                 pairs = set()
