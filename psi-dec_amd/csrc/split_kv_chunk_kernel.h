@@ -5,9 +5,10 @@
 // decomposition: here the matrix cores and the LDS are the bound, not HBM.
 //
 // Work decomposition
-//   one workgroup = one (row group, kv_head [, part of the query heads]).  A row group is a run of consecutive
-//   Q-token tiles of one request whose kv_split rows start at the same key (the rows of one KV partition).  With
-//   more than 5 query heads per KV head the heads are dealt to two or three workgroups.  The workgroup's query
+//   one work item = one (row group, kv_head [, part of the query heads]); the launch is one workgroup per compute
+//   unit, and a workgroup takes items until none is left (see the kernel at the end of this file).  A row group is
+//   a run of consecutive Q-token tiles of one request whose kv_split rows start at the same key (the rows of one KV
+//   partition).  With more than 5 query heads per KV head the heads are dealt to two or three items.  An item's query
 //   columns, column c = token_in_group * heads + head, are dealt out 32 per wave, as two blocks of 16: a wave keeps
 //   the online-softmax state and the accumulators of its columns for the whole KV range, so wave states never merge.
 //
