@@ -43,7 +43,7 @@ sys.path.insert(0, ROOT)
 HBM_PEAK_GBPS = 8000.0
 MFMA_BF16_PEAK_TFLOPS = 2500.0
 CONFIG_NAMES = ["C1", "C2_rows512", "C2_b4", "C2_b8", "C2_b16", "C3", "C4_q2", "C4_q4", "C4_q8", "C5_decode", "C5_prefill", "PREFILL_d128",
-                "C5_mixed", "GENERIC_f32_b8"]
+                "PREFILL_p16k", "PREFILL_c512", "C5_mixed", "GENERIC_f32_b8"]
 # The shapes the reference itself times (the only figures it publishes for these kernels, on an Apple M3 Max):
 #   REF_tiled      "SplitKV TiledQ only", 40 Q / 8 KV heads, head_dim 128, 8-token pages, one request with 8 new tokens
 #                  on 128 cached ones: 0.319 ms median, map + reduce (docs/qwen3_dspark_design_draft.md:1453-1458, the
@@ -80,7 +80,8 @@ def parse_args():
     p.add_argument("--dtype", choices=["bf16", "f16", "f32"], default="bf16",
                    help="custom workload: element type (f32 runs the shape-generic kernels)")
     p.add_argument("--partition", type=int, default=512)
-    p.add_argument("--prefill-partition", type=int, default=4096, help="C5_prefill: tokens per KV partition")
+    p.add_argument("--prefill-partition", type=int, default=4096,
+                   help="C5_prefill, PREFILL_d128: tokens per KV partition (0: what the library's partition planner picks)")
     p.add_argument("--arenas", type=int, default=0, help="page arenas rotated between steps (0 = per workload)")
     p.add_argument("--identity-pages", action="store_true", help="unshuffled page pool (diagnostic)")
     p.add_argument("--plan-order", action="store_true", help="row-per-workgroup launch in plan order, not longest first")
@@ -190,8 +191,9 @@ def build_case(psi, wl, device, name, args):
         if args.grouped:
             w = wl.make_workload(args.seed, ctx, args.q_heads, args.kv_heads, d, elem, p, q_lens=args.q_len,
                                  host_pages=False)
-            dw = wl.DeviceWorkload(device, w, partition_tokens=args.partition, grouped=True,
+            dw = wl.DeviceWorkload(device, w, partition_tokens=args.partition or "auto", grouped=True,
                                    variant=psi.GQASplitKVVariant.TiledQ(8, 16, group))
+            key = key.replace(f"_part{args.partition}_", f"_part{dw.partition_tokens}_")
             return Case(name, key + "_grouped", [dw], "verify", "tiled_q_map", "split_kv_chunk_map",
                         "kv append -> row-group (prefill-chunk) map -> LSE combine")
         return verify_case(key, ctx, args.q_len, args.partition, args.arenas or 1, args.seed, hq=args.q_heads,
@@ -247,9 +249,9 @@ def build_case(psi, wl, device, name, args):
         w = wl.make_workload(5, [4096 + 2048], 24, 4, 256, bf16, 16, q_lens=2048, host_pages=False)
         # 4096-token partitions: two rows per query tile, twice as many work items of half the size, which fill
         # the 256 compute units evenly (unsplit, 384 items make one and a half rounds: 375 against 323 us)
-        dw = wl.DeviceWorkload(device, w, partition_tokens=args.prefill_partition, grouped=True,
+        dw = wl.DeviceWorkload(device, w, partition_tokens=args.prefill_partition or "auto", grouped=True,
                                variant=psi.GQASplitKVVariant.TiledQ(8, 16, 6))
-        case = Case(name, "prefill_chunk2048_on_prefix4096_24q4kv_d256_bf16_p16_part4096_seed5", [dw], "prefill",
+        case = Case(name, f"prefill_chunk2048_on_prefix4096_24q4kv_d256_bf16_p16_part{dw.partition_tokens}_seed5", [dw], "prefill",
                     "tiled_q_map", "split_kv_chunk_map", "kv append -> row-group (prefill-chunk) map -> LSE combine")
         case.flops = 4 * 24 * 256 * sum(4096 + i + 1 for i in range(2048))
         return case
@@ -257,11 +259,23 @@ def build_case(psi, wl, device, name, args):
         # the same chunk on the geometry of the reference's published figures (Qwen3-14B: 40 Q / 8 KV heads of 128,
         # 8-token pages; gqa_split_kv_tiled_q.rs:66-76 profile (128, 8))
         w = wl.make_workload(5, [4096 + 2048], 40, 8, 128, bf16, 8, q_lens=2048, host_pages=False)
-        dw = wl.DeviceWorkload(device, w, partition_tokens=args.prefill_partition, grouped=True,
+        dw = wl.DeviceWorkload(device, w, partition_tokens=args.prefill_partition or "auto", grouped=True,
                                variant=psi.GQASplitKVVariant.TiledQ(8, 16, 5))
-        case = Case(name, "prefill_chunk2048_on_prefix4096_40q8kv_d128_bf16_p8_part4096_seed5", [dw], "prefill",
+        case = Case(name, f"prefill_chunk2048_on_prefix4096_40q8kv_d128_bf16_p8_part{dw.partition_tokens}_seed5", [dw], "prefill",
                     "tiled_q_map", "split_kv_chunk_map", "kv append -> row-group (prefill-chunk) map -> LSE combine")
         case.flops = 4 * 40 * 128 * sum(4096 + i + 1 for i in range(2048))
+        return case
+    if name in ("PREFILL_p16k", "PREFILL_c512"):
+        # other shapes of the same model, with the partition that psi_hip_split_kv_chunk_partition_tokens picks:
+        # a chunk of 2048 tokens on a 16384-token prefix, and one of 512 tokens on a 4096-token prefix
+        prefix, chunk = (16384, 2048) if name == "PREFILL_p16k" else (4096, 512)
+        w = wl.make_workload(5, [prefix + chunk], 24, 4, 256, bf16, 16, q_lens=chunk, host_pages=False)
+        dw = wl.DeviceWorkload(device, w, partition_tokens="auto", grouped=True,
+                               variant=psi.GQASplitKVVariant.TiledQ(8, 16, 6))
+        case = Case(name, f"prefill_chunk{chunk}_on_prefix{prefix}_24q4kv_d256_bf16_p16_part{dw.partition_tokens}_planned_seed5",
+                    [dw], "prefill", "tiled_q_map", "split_kv_chunk_map",
+                    "kv append -> row-group (prefill-chunk) map -> LSE combine")
+        case.flops = 4 * 24 * 256 * sum(prefix + i + 1 for i in range(chunk))
         return case
     if name == "C5_mixed":
         step = wl.MixedStep(device, wl.config_c5())

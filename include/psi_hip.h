@@ -485,6 +485,22 @@ int psi_hip_split_kv_tiled_q_group_rows(const psi_hip_gqa_config* cfg, uint32_t 
                                         uint64_t row_groups_capacity, uint32_t* out_group_tiles,
                                         uint32_t* out_num_groups);
 
+/* Partition length for a batch of prefill chunks (no counterpart in the reference, which has no fixed partitions).
+ * Host helper: the `partition_tokens` of a FIXED_PARTITION plan, a multiple of 256 tokens, with which the work items of
+ * psi_hip_split_kv_tiled_q_map_grouped -- (token group, partition, KV head, head subset) -- and the combine behind it
+ * end soonest on `num_compute_units` compute units (0 = 256), by a model of that launch: an item costs its KV tiles
+ * plus a fixed share, a unit that is through takes the heaviest item left, and every item's partial rows are written
+ * and read once.  token_indices[r] is the position of request r's first new token and cu_tokens[r + 1] - cu_tokens[r]
+ * the number of its new tokens, as for psi_hip_gqa_metadata_update.  On the shape this library is measured on (2048
+ * tokens on a 4096-token prefix, 24 Q / 4 KV heads of 256) it answers 4096; for 512 tokens on the same prefix 1024,
+ * where 4096 leaves 96 items for 256 units and takes three times as long.  The answer depends on the batch's lengths
+ * only: cache it per shape class.  *out_partition_tokens = 0 when the geometry has no grouped kernel or the batch
+ * is empty. */
+int psi_hip_split_kv_chunk_partition_tokens(const psi_hip_gqa_config* cfg, uint32_t q_token_tile_size,
+                                            const uint32_t* token_indices, const uint32_t* cu_tokens,
+                                            uint32_t num_reqs, uint32_t num_compute_units,
+                                            uint32_t* out_partition_tokens);
+
 /* The multi-query map launched over a balanced plan (psi_hip_split_kv_balance_plan on the TiledQ tables: its
  * `num_tokens` is then the number of Q-token tiles and cu_in the per-tile cu_kv_splits): workgroup w of each KV head
  * serves kv_splits rows [worker_cu[w], worker_cu[w + 1]).  Same results as psi_hip_split_kv_tiled_q_map up to the

@@ -345,6 +345,8 @@ PROTOTYPES = {
     ),
     "psi_hip_split_kv_tiled_q_group_rows": (
         c_int, [_CFG, c_uint32, _U32P, c_uint32, _U32P, c_uint32, _U32P, _U32P, c_uint64, _U32P, _U32P]),
+    "psi_hip_split_kv_chunk_partition_tokens": (
+        c_int, [_CFG, c_uint32, _U32P, _U32P, c_uint32, c_uint32, _U32P]),
     "psi_hip_split_kv_tiled_q_reduce": (
         c_int,
         [c_void_p, _CFG, c_uint32, c_void_p, c_uint64, c_void_p, c_void_p, c_void_p, c_uint32, c_uint32, c_uint32,

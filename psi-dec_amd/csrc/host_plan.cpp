@@ -6,6 +6,7 @@
 //   crates/inference-executor-metal/src/attn/gqa/mod.rs:64-316             (batch selector)
 //   crates/inference-executor-metal/src/attn/gqa/batch_metadata.rs:192-523 (metadata + split plans)
 #include <algorithm>
+#include <functional>
 #include <queue>
 
 #include "split_kv.h"
@@ -665,6 +666,80 @@ extern "C" int psi_hip_split_kv_order_longest_first(uint32_t* kv_splits, uint32_
         partial_row_index[order[pos]] = pos;
     }
     std::copy(sorted.begin(), sorted.end(), kv_splits);
+    return PSI_HIP_OK;
+}
+
+// Partition length for prefill chunks: a model of the row-group map's launch.  An item = (token group of a request,
+// partition, KV head, head subset) costs its KV tiles plus a fixed share (its start, its partial rows); the units
+// take items heaviest first as they become free; every item's partial rows are written once and read once by the
+// combine.  The figures are this library's own measurements on MI355X: an item's fixed cost is that of nine tiles,
+// and the partial rows of an item of 256 columns at head_dim 256 cost the launch 0.06 tiles.
+extern "C" int psi_hip_split_kv_chunk_partition_tokens(const psi_hip_gqa_config* cfg, uint32_t q_token_tile_size,
+                                                       const uint32_t* token_indices, const uint32_t* cu_tokens,
+                                                       uint32_t num_reqs, uint32_t num_compute_units,
+                                                       uint32_t* out_partition_tokens) {
+    Geometry g;
+    int rc = make_geometry(cfg, &g);
+    if (rc != PSI_HIP_OK) return rc;
+    PSI_REQUIRE(out_partition_tokens != nullptr, "out_partition_tokens must not be null");
+    PSI_REQUIRE(num_reqs == 0 || (token_indices && cu_tokens), "request arrays must not be null");
+    *out_partition_tokens = 0;
+    if (num_reqs == 0 || !chunk_map_supported(g, q_token_tile_size)) return PSI_HIP_OK;
+    const uint32_t units = num_compute_units ? num_compute_units : 256u;
+    const uint32_t tile_keys = chunk_tile_keys(g.d);
+    const uint32_t group_tokens = chunk_group_tiles(g.group, q_token_tile_size) * q_token_tile_size;
+    const uint32_t copies = g.hkv * chunk_head_subsets(g.group);  // items of equal cost per (group, partition)
+    constexpr double kItemTiles = 9.0;
+    const double partial_tiles = 0.06 * g.d / 256.0;
+    uint64_t longest = 0;
+    for (uint32_t r = 0; r < num_reqs; ++r)
+        longest = std::max<uint64_t>(longest, (uint64_t)token_indices[r] + (cu_tokens[r + 1] - cu_tokens[r]));
+    if (longest == 0) return PSI_HIP_OK;
+    const uint32_t unsplit = (uint32_t)std::min<uint64_t>((longest + 255) / 256 * 256, 1u << 20);
+    std::vector<uint32_t> candidates;
+    for (uint32_t p = 256; p < unsplit && p <= 32768; p += p < 2048 ? 256 : (p < 8192 ? 1024 : 2048)) candidates.push_back(p);
+    candidates.push_back(unsplit);
+    double best = 0.0;
+    std::vector<double> costs;
+    std::vector<double> free_at;
+    for (uint32_t partition : candidates) {
+        costs.clear();
+        for (uint32_t r = 0; r < num_reqs; ++r) {
+            const uint32_t prefix = token_indices[r], chunk = cu_tokens[r + 1] - cu_tokens[r];
+            for (uint32_t a = 0; a < chunk; a += group_tokens) {
+                const uint64_t kv_end = (uint64_t)prefix + std::min(a + group_tokens, chunk);  // causal limit of the group's last token
+                for (uint64_t lo = 0; lo < kv_end; lo += partition) {
+                    const uint64_t keys = std::min<uint64_t>(lo + partition, kv_end) - lo;
+                    costs.push_back((double)((keys + tile_keys - 1) / tile_keys) + kItemTiles);
+                }
+            }
+        }
+        std::sort(costs.begin(), costs.end(), std::greater<double>());
+        const double items = (double)costs.size() * copies;
+        double total = 0.0;
+        for (double c : costs) total += c * copies;
+        double end;
+        if (items > 8.0 * units) {
+            // so many items that the units end within the lightest item of each other
+            end = std::max(total / units + 0.5 * costs.back(), costs.front());
+        } else {
+            free_at.assign(units, 0.0);  // a min-heap of the times at which the units become free
+            std::make_heap(free_at.begin(), free_at.end(), std::greater<double>());
+            end = 0.0;
+            for (double c : costs)
+                for (uint32_t k = 0; k < copies; ++k) {
+                    std::pop_heap(free_at.begin(), free_at.end(), std::greater<double>());
+                    free_at.back() += c;
+                    end = std::max(end, free_at.back());
+                    std::push_heap(free_at.begin(), free_at.end(), std::greater<double>());
+                }
+        }
+        const double cost = end + partial_tiles * items;
+        if (*out_partition_tokens == 0 || cost <= best) {  // (ties go to the longer partition: fewer partial rows)
+            best = cost;
+            *out_partition_tokens = partition;
+        }
+    }
     return PSI_HIP_OK;
 }
 

@@ -144,6 +144,8 @@ inline int set_output_gate(ReduceArgs* a, const psi_hip_output_gate* gate, const
 constexpr int kChunkCols = 256;
 // Six heads per KV head go to three workgroups of two (two heads x 128 tokens fill the 256 columns; three heads x 80
 // tokens would leave sixteen of them empty).
+// Keys of one KV tile of the prefill-chunk map (16 KiB of K and of V at either head_dim).
+constexpr uint32_t chunk_tile_keys(uint32_t d) { return d == 128 ? 64u : 32u; }
 inline uint32_t chunk_head_subsets(uint32_t group) { return group == 6 ? 3u : (group > 5 ? 2u : 1u); }
 inline uint32_t chunk_group_tiles(uint32_t group, uint32_t q_token_tile_size) {
     const uint32_t subsets = chunk_head_subsets(group);

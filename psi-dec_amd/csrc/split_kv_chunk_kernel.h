@@ -75,7 +75,7 @@ namespace psi {
 // instructions between two barriers; with 32 keys at head_dim 128 a tile's fixed costs - barrier, first operand reads,
 // the way from the last product of K * Q^T to the first of V^T * P^T - weighed twice as much).
 template <int D>
-constexpr int kChunkKeysOf = D == 128 ? 64 : 32;
+constexpr int kChunkKeysOf = (int)chunk_tile_keys(D);
 constexpr int kChunkColBlocks = 2;  // 16-column blocks of a wave
 constexpr int kChunkWaves = 8;
 constexpr int kChunkStages = 4;   // K tiles in LDS

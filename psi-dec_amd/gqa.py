@@ -503,6 +503,20 @@ def balanced_workers(config: "GQASplitKVConfig") -> int:
     return out.value
 
 
+def chunk_partition_tokens(config, q_token_tile_size: int, token_indices: Sequence[int], cu_tokens: Sequence[int],
+                           num_compute_units: int = 0) -> int:
+    """Partition length (tokens) for a FIXED_PARTITION plan of a batch of prefill chunks that the row-group map and its
+    combine finish soonest with, by the library's model of that launch (psi_hip_split_kv_chunk_partition_tokens);
+    `config` is any of the kernels' configs (it gives the heads, head_dim and page size), token_indices[r] the position
+    of request r's first new token, cu_tokens the prefix sums of the new tokens.  0: the geometry has no row-group
+    kernel.  Depends on the lengths only; cache it per shape class."""
+    out, cfg = ctypes.c_uint32(), config.struct()
+    L.check(L.load().psi_hip_split_kv_chunk_partition_tokens(
+        ctypes.byref(cfg), q_token_tile_size, L.u32_array(token_indices), L.u32_array(cu_tokens), len(token_indices),
+        num_compute_units, ctypes.byref(out)))
+    return out.value
+
+
 def select_split_kv_variant(split_kv: GQASplitKV, max_tokens: int, replay_policy: Optional[GQAReplayBucketPolicy],
                             token_indices: Sequence[int], cu_tokens: Sequence[int]) -> GQASplitKVVariant:
     """`select_split_kv_variant` (attn/gqa/mod.rs:64-94); the (256, 8) work model applies by itself."""

@@ -203,6 +203,13 @@ class DeviceWorkload:
             variant = split_kv.select(w.num_tokens, int(sum(-(-int(n) // 8) for n in q_lens)))
         self.variant = variant
         rows = variant.q_token_tile_size if variant.is_tiled() else 1
+        if partition_tokens == "auto":
+            # prefill chunks through the row-group map: the partition that the library's model of the launch picks
+            assert grouped and variant.is_tiled(), "the partition planner serves the row-group map"
+            partition_tokens = G.chunk_partition_tokens(split_kv.config, variant.q_token_tile_size,
+                                                        [int(t) for t in w.token_indices],
+                                                        [int(c) for c in w.cu_tokens]) or None
+        self.partition_tokens = partition_tokens
         if partition_tokens is not None:
             if variant.is_tiled():
                 tile = variant.q_token_tile_size

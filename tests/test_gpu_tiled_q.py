@@ -356,6 +356,19 @@ def test_grouped_random_batches(psi, oracle, device, seed):
     assert dw.meta.num_row_groups > 0
 
 
+@pytest.mark.parametrize("prefix,chunk", [(0, 700), (1500, 300), (37, 64)])
+def test_grouped_with_the_planned_partition(psi, oracle, device, prefix, chunk):
+    """The partition length that the library's planner picks for the batch (psi_hip_split_kv_chunk_partition_tokens)
+    instead of a given one: a multiple of 256 tokens, and the same outputs against the oracle as with any other."""
+    wl = importlib_workloads(psi)
+    w = wl.make_workload(99, [prefix + chunk, 40], 24, 4, 256, psi.Dtype.Bfloat16, 16, q_lens=[chunk, 5])
+    _, dw = run_and_check(psi, oracle, device, w, f"grouped chunk {chunk} on {prefix}, planned partition",
+                          max_tokens=1024, variant=psi.GQASplitKVVariant.TiledQ(8, 16, 6), partition_tokens="auto",
+                          grouped=True, check_rounded=False)
+    assert dw.partition_tokens % 256 == 0 and 256 <= dw.partition_tokens <= (prefix + chunk + 255) // 256 * 256
+    assert dw.meta.num_row_groups > 0
+
+
 def test_grouped_more_items_than_workgroups(psi, oracle, device):
     """The row-group map runs one workgroup per compute unit, and a workgroup that is through with its item takes the
     next from a counter that the launch leaves at zero.  Here the launch has several times as many items as the GPU
