@@ -622,7 +622,7 @@ typedef struct psi_hip_gqa_layer_input {
 
 typedef struct psi_hip_gqa_plan_options {
     uint32_t capacity_mode;           /* PSI_HIP_CAPACITY_* */
-    uint32_t partition_tokens;        /* FIXED_PARTITION */
+    uint32_t partition_tokens;        /* FIXED_PARTITION (prefill chunks: see psi_hip_split_kv_chunk_partition_tokens) */
     uint32_t caller_num_total_tokens; /* CALLER_TOKENS */
     uint32_t dispatch;                /* PSI_HIP_DISPATCH_* */
     uint32_t num_workers;             /* BALANCED: workers per KV head, 0 = psi_hip_split_kv_balanced_workers */
