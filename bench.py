@@ -80,8 +80,9 @@ def parse_args():
     p.add_argument("--dtype", choices=["bf16", "f16", "f32"], default="bf16",
                    help="custom workload: element type (f32 runs the shape-generic kernels)")
     p.add_argument("--partition", type=int, default=512)
-    p.add_argument("--prefill-partition", type=int, default=4096,
-                   help="C5_prefill, PREFILL_d128: tokens per KV partition (0: what the library's partition planner picks)")
+    p.add_argument("--prefill-partition", type=int, default=0,
+                   help="C5_prefill, PREFILL_d128: tokens per KV partition (0, the default: what the library's partition "
+                        "planner picks - 4096 and 3072)")
     p.add_argument("--arenas", type=int, default=0, help="page arenas rotated between steps (0 = per workload)")
     p.add_argument("--identity-pages", action="store_true", help="unshuffled page pool (diagnostic)")
     p.add_argument("--plan-order", action="store_true", help="row-per-workgroup launch in plan order, not longest first")
@@ -247,8 +248,8 @@ def build_case(psi, wl, device, name, args):
                            args.arenas or 1, 5)
     if name == "C5_prefill":
         w = wl.make_workload(5, [4096 + 2048], 24, 4, 256, bf16, 16, q_lens=2048, host_pages=False)
-        # 4096-token partitions: two rows per query tile, twice as many work items of half the size, which fill
-        # the 256 compute units evenly (unsplit, 384 items make one and a half rounds: 375 against 323 us)
+        # the planner's 4096-token partitions: two rows per query tile, 192 work items of 128 KV tiles and 192 of
+        # 4 to 64 that fill the end of the launch
         dw = wl.DeviceWorkload(device, w, partition_tokens=args.prefill_partition or "auto", grouped=True,
                                variant=psi.GQASplitKVVariant.TiledQ(8, 16, 6))
         case = Case(name, f"prefill_chunk2048_on_prefix4096_24q4kv_d256_bf16_p16_part{dw.partition_tokens}_seed5", [dw], "prefill",

@@ -473,9 +473,9 @@ int psi_hip_split_kv_tiled_q_map(psi_hip_ctx* ctx, const psi_hip_gqa_config* cfg
 /* Row groups for prefill chunks (no counterpart in the reference, whose TiledQ map launches one
  * threadgroup per (row, Q-head tile), gqa_split_kv_tiled_q.rs:402-409).  Host helper: gathers the
  * kv_split rows of consecutive Q-token tiles of one request that start at the same key (the rows of one
- * KV partition of a fixed-partition plan) into groups of up to *out_group_tiles rows, heaviest group
- * first.  row_groups: host u32[row_groups_capacity], written as [*out_num_groups][*out_group_tiles] row
- * indices padded with PSI_HIP_SENTINEL; capacity of num_kv_splits * 32 words always suffices.  req_slots
+ * KV partition of a fixed-partition plan) into groups of up to *out_group_tiles rows, the group with the
+ * longest KV range first (its work items walk that range whatever the number of its tokens).  row_groups:
+ * host u32[row_groups_capacity], written as [*out_num_groups][*out_group_tiles] row indices padded with PSI_HIP_SENTINEL; capacity of num_kv_splits * 32 words always suffices.  req_slots
  * is the per-token slot array of psi_hip_gqa_metadata_update.  Every non-padding row lands in exactly
  * one group.  *out_group_tiles = 0 when the geometry has no grouped kernel (use the plain map then). */
 int psi_hip_split_kv_tiled_q_group_rows(const psi_hip_gqa_config* cfg, uint32_t q_token_tile_size,

@@ -784,7 +784,8 @@ extern "C" int psi_hip_split_kv_tiled_q_group_rows(const psi_hip_gqa_config* cfg
     });
     struct Group {
         uint32_t first, count;  // range of `rows`
-        uint64_t work;          // query tokens x keys, the dispatch-order key
+        uint32_t keys;          // its longest KV range: what an item of the group costs, and the dispatch-order key
+        uint64_t work;          // query tokens x keys: the order among groups of equal range
     };
     std::vector<Group> groups;
     auto tile_tokens = [&](uint32_t tile) { return q_token_tiles[(size_t)tile * 2 + 1] - q_token_tiles[(size_t)tile * 2]; };
@@ -797,15 +798,20 @@ extern "C" int psi_hip_split_kv_tiled_q_group_rows(const psi_hip_gqa_config* cfg
                    prev.tile + 1 == rows[i].tile && tile_tokens(prev.tile) == q_token_tile_size &&
                    q_token_tiles[(size_t)prev.tile * 2 + 1] == q_token_tiles[(size_t)rows[i].tile * 2];
         }
-        if (!join) groups.push_back(Group{i, 0, 0});
+        if (!join) groups.push_back(Group{i, 0, 0, 0});
         groups.back().count += 1;
+        groups.back().keys = std::max(groups.back().keys, rows[i].kv_end - rows[i].kv_begin);
         groups.back().work += (uint64_t)tile_tokens(rows[i].tile) * (rows[i].kv_end - rows[i].kv_begin);
     }
     PSI_REQUIRE((uint64_t)groups.size() * max_tiles <= row_groups_capacity,
                 "row-group table too small: %llu groups of %u rows, capacity %llu words",
                 (unsigned long long)groups.size(), max_tiles, (unsigned long long)row_groups_capacity);
-    // heaviest groups first, so that the light ones fill the end of the launch
-    std::stable_sort(groups.begin(), groups.end(), [](const Group& x, const Group& y) { return x.work > y.work; });
+    // Longest groups first, so that the short ones fill the end of the launch.  A work item walks the group's KV
+    // range whatever the number of its query tokens (a request's last group may hold a few), so the range is the
+    // key, not the tokens x keys product, by which such a group was claimed last and ended the launch.
+    std::stable_sort(groups.begin(), groups.end(), [](const Group& x, const Group& y) {
+        return x.keys != y.keys ? x.keys > y.keys : x.work > y.work;
+    });
     for (size_t gi = 0; gi < groups.size(); ++gi) {
         uint32_t* out = row_groups + gi * max_tiles;
         for (uint32_t m = 0; m < max_tiles; ++m)

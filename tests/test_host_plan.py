@@ -522,14 +522,14 @@ def check_groups(meta, shape, tile_size, max_tiles):
     table = meta.h_row_groups.reshape(meta.num_row_groups, meta.group_tiles)
     assert meta.group_tiles == max_tiles
     seen = []
-    work = []
+    order = []
     for g in table:
         members = [int(r) for r in g if r != MAX]
         assert members and [int(r) for r in g[:len(members)]] == members, "padding only at the end"
         seen += members
         first = rows[members[0]]
         slot = meta.h_req_slots[tiles[first[0]][0]]
-        w = 0
+        w, longest = 0, 0
         for i, r in enumerate(members):
             tile, begin, end = (int(x) for x in rows[r])
             assert begin == first[1] and tile == first[0] + i
@@ -537,9 +537,12 @@ def check_groups(meta, shape, tile_size, max_tiles):
             if i + 1 < len(members):
                 assert tiles[tile][1] - tiles[tile][0] == tile_size and tiles[tile][1] == tiles[tile + 1][0]
             w += int(tiles[tile][1] - tiles[tile][0]) * (end - begin)
-        work.append(w)
+            longest = max(longest, end - begin)
+        order.append((longest, w))
     assert sorted(seen) == list(range(shape.num_sdpa_map_task_templates)), "rows lost or duplicated"
-    assert work == sorted(work, reverse=True), "heaviest group first"
+    # a work item walks its group's KV range whatever the number of its tokens: the longest range goes first, and
+    # among equal ranges the group with more tokens x keys
+    assert order == sorted(order, reverse=True), "longest group first"
     return table
 
 
