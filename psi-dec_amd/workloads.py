@@ -406,9 +406,13 @@ class MixedStep:
         n_chunk_tokens = int(w.cu_tokens[n_chunk])
         chunk_ctx = w.context_lens[:n_chunk]
         if chunk_partition is None:
-            # Two rows per query tile: the chunk's work items then number well above the compute units and are
-            # small enough to fill them evenly (measured best on a 2048-token chunk over 4096 cached tokens).
-            chunk_partition = max(2048, 1 << int((int(chunk_ctx.max()) + 1) // 2 - 1).bit_length())
+            # what the library's model of the row-group launch picks for these chunks (4096 tokens for a 2048-token
+            # chunk over 4096 cached tokens: 192 work items of 128 KV tiles and 192 of 4 to 64)
+            config = G.GQASplitKVConfig(w.dtype, w.page_bytes, w.num_q_heads, w.num_kv_heads, w.head_dim)
+            chunk_partition = G.chunk_partition_tokens(config, 8, [int(t) for t in w.token_indices[:n_chunk]],
+                                                       [int(c) for c in w.cu_tokens[:n_chunk + 1]])
+            if chunk_partition == 0:  # no row-group kernel for this geometry: the multi-query map's partitions
+                chunk_partition = 512
         self.chunk_partition, self.decode_partition, self.chunk_min_tokens = chunk_partition, decode_partition, chunk_min_tokens
         chunk_rows = int(sum(-(-int(c) // chunk_partition) * -(-int(n) // 8) for c, n in zip(chunk_ctx, q_lens[:n_chunk])))
         decode_rows = int(sum(-(-(int(t) + i + 1) // decode_partition)
