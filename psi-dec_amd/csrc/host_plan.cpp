@@ -703,6 +703,7 @@ extern "C" int psi_hip_split_kv_chunk_partition_tokens(const psi_hip_gqa_config*
     std::vector<double> costs;
     std::vector<double> free_at;
     for (uint32_t partition : candidates) {
+        if ((uint64_t)partition * 64 < longest) continue;  // (more than 64 partitions of a request are never the answer)
         costs.clear();
         for (uint32_t r = 0; r < num_reqs; ++r) {
             const uint32_t prefix = token_indices[r], chunk = cu_tokens[r + 1] - cu_tokens[r];

@@ -57,6 +57,8 @@ def planned(reqs, hq, hkv, d, ts, units=256):
     longest = max(prefix + chunk for prefix, chunk in reqs)
     best, answer = None, 0
     for p in candidates(longest):
+        if p * 64 < longest:
+            continue
         cost = model(reqs, hq, hkv, d, ts, p, units)
         if best is None or cost <= best:
             best, answer = cost, p
@@ -90,7 +92,7 @@ def test_library_and_restatement_agree_on_random_batches(psi):
         group = rng.choice([1, 2, 4, 5, 6, 7, 8])
         d = rng.choice([128, 256])
         cfg = config(psi, hkv * group, hkv, d, rng.choice([8, 16, 32]))
-        reqs = [(rng.choice([0, 1, 17, 500, 4096, 9000, 20000]), rng.choice([1, 8, 100, 512, 2048, 5000]))
+        reqs = [(rng.choice([0, 1, 17, 500, 4096, 9000, 20000, 300000]), rng.choice([1, 8, 100, 512, 2048, 5000]))
                 for _ in range(rng.randint(1, 4))]
         units = rng.choice([0, 64, 256, 304])
         got = ask(psi, cfg, 8, reqs, units)
