@@ -102,6 +102,9 @@ const char* psi_hip_version(void);
  * psi_hip_ctx_destroy, no launch allocates. */
 int psi_hip_ctx_create(int device, void* stream, psi_hip_ctx** out_ctx);
 int psi_hip_ctx_destroy(psi_hip_ctx* ctx);
+/* Later launches go to `stream`.  They are ordered behind what the context has launched on its previous stream (an
+ * event recorded there, awaited here: no host synchronisation), so the one-after-the-other rule above survives the
+ * switch.  Not while either stream is being captured into a graph: then the order is the capturing caller's. */
 int psi_hip_ctx_set_stream(psi_hip_ctx* ctx, void* stream);
 /* `ReplaySubmission::wait` (stream synchronisation). */
 int psi_hip_sync(psi_hip_ctx* ctx);

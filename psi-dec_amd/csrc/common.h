@@ -75,6 +75,7 @@ struct psi_hip_ctx {
     // stream, one after the other.
     uint32_t* work_claim = nullptr;
     int num_cus = 0;  // compute units of the device
+    hipEvent_t order_event = nullptr;  // psi_hip_ctx_set_stream: the old stream's work before the new stream's
     bool mute_loaders = false;  // harness switch: the maps' loading waves announce nothing, so that waits run out
     std::map<std::string, psi::KernelTimer> timers;
     std::vector<hipEvent_t> event_pool;

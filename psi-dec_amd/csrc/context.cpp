@@ -139,13 +139,32 @@ int psi_hip_ctx_destroy(psi_hip_ctx* ctx) {
     for (auto ev : ctx->event_pool) (void)hipEventDestroy(ev);
     if (ctx->status_host != nullptr) (void)hipHostFree(const_cast<uint32_t*>(ctx->status_host));
     if (ctx->work_claim != nullptr) (void)hipFree(ctx->work_claim);
+    if (ctx->order_event != nullptr) (void)hipEventDestroy(ctx->order_event);
     delete ctx;
     return PSI_HIP_OK;
 }
 
 int psi_hip_ctx_set_stream(psi_hip_ctx* ctx, void* stream) {
     PSI_REQUIRE(ctx != nullptr, "ctx must not be null");
-    ctx->stream = (hipStream_t)stream;
+    const hipStream_t next = (hipStream_t)stream;
+    if (next == ctx->stream) return PSI_HIP_OK;
+    // What the context has launched on the old stream stays ahead of what it launches on the new one: its launches
+    // share the context's work counters and the arena the caller hands them, and rely on running one after the other.
+    // (A stream that is being captured takes no dependency on work outside its capture, and the other way round:
+    // there the order is the capturing caller's.)
+    hipStreamCaptureStatus from = hipStreamCaptureStatusNone, to = hipStreamCaptureStatusNone;
+    const bool plain = hipStreamIsCapturing(ctx->stream, &from) == hipSuccess &&
+                       hipStreamIsCapturing(next, &to) == hipSuccess && from == hipStreamCaptureStatusNone &&
+                       to == hipStreamCaptureStatusNone;
+    if (plain) {
+        if (ctx->order_event == nullptr)
+            PSI_HIP_CHECK(hipEventCreateWithFlags(&ctx->order_event, hipEventDisableTiming));
+        PSI_HIP_CHECK(hipEventRecord(ctx->order_event, ctx->stream));
+        PSI_HIP_CHECK(hipStreamWaitEvent(next, ctx->order_event, 0));
+    } else {
+        (void)hipGetLastError();
+    }
+    ctx->stream = next;
     return PSI_HIP_OK;
 }
 

@@ -303,3 +303,40 @@ def test_wide_combine_leaves_inactive_tokens_alone(psi, oracle, device):
                            w.layer, w.req_slots[:1], w.token_indices[:1], np.arange(2, dtype=np.uint32),
                            w.q.reshape(2, -1)[:1].reshape(-1), dw.pages_host(), w.page_ids, num_threads=8)
     assert_outputs_close(got[0], exp, "wide combine under device-side counts")
+
+
+def test_a_stream_switch_keeps_the_contexts_launches_in_order(psi, oracle, device):
+    """`psi_hip_ctx_set_stream`: what the context launches on the new stream runs behind what it launched on the old
+    one, with no synchronisation by the caller.  The old stream is held busy while a step is queued on it; the step
+    queued on the new stream right after must see that step's pages (it appends to the same slots and reads the
+    history) and leave the output of its own inputs."""
+    import dataclasses
+
+    import torch
+
+    wl = importlib_workloads(psi)
+    w = wl.make_workload(77, [900, 40, 2100], 24, 4, 256, psi.Dtype.Bfloat16, 16, q_lens=2)
+    dw = wl.DeviceWorkload(device, w, partition_tokens=512, f32_output=True)
+    rng = np.random.default_rng(5)
+    fresh = {name: wl.to_storage(rng.standard_normal(t.numel(), dtype=np.float32), w.dtype)
+             for name, t in (("q", dw.q), ("flat_k", dw.flat_k), ("flat_v", dw.flat_v))}
+    staged = {name: device.from_numpy(a) for name, a in fresh.items()}
+    second = dataclasses.replace(w, **fresh)
+    side, main = torch.cuda.Stream(), device.stream
+    torch.cuda.synchronize()
+    try:
+        torch.cuda._sleep(50_000_000)  # the old stream is busy for tens of milliseconds
+        dw.step()                       # first inputs, queued behind the sleep
+        for name, t in (("q", dw.q), ("flat_k", dw.flat_k), ("flat_v", dw.flat_v)):
+            t.copy_(staged[name])       # second inputs, behind the first step on the old stream
+        device.use_stream(side)
+        dw.step()                       # on the new stream: must run behind all of the above
+        side.synchronize()
+    finally:
+        device.use_stream(main)
+    torch.cuda.synchronize()
+    n = w.num_tokens * w.num_q_heads * w.head_dim
+    exp_pages, exp = oracle_step(oracle, second)
+    assert_outputs_close(dw.output[:n].cpu().numpy(), exp, "the step on the new stream")
+    got_pages = dw.pages.view(torch.int16).cpu().numpy().view(np.uint16)
+    assert np.array_equal(got_pages.reshape(exp_pages.shape), exp_pages)
