@@ -692,8 +692,10 @@ extern "C" int psi_hip_split_kv_chunk_partition_tokens(const psi_hip_gqa_config*
     constexpr double kItemTiles = 9.0;
     const double partial_tiles = 0.06 * g.d / 256.0;
     uint64_t longest = 0;
-    for (uint32_t r = 0; r < num_reqs; ++r)
+    for (uint32_t r = 0; r < num_reqs; ++r) {
+        PSI_REQUIRE(cu_tokens[r + 1] >= cu_tokens[r], "cu_tokens must not decrease (request %u)", r);
         longest = std::max<uint64_t>(longest, (uint64_t)token_indices[r] + (cu_tokens[r + 1] - cu_tokens[r]));
+    }
     if (longest == 0) return PSI_HIP_OK;
     const uint32_t unsplit = (uint32_t)std::min<uint64_t>((longest + 255) / 256 * 256, 1u << 20);
     std::vector<uint32_t> candidates;
@@ -703,7 +705,8 @@ extern "C" int psi_hip_split_kv_chunk_partition_tokens(const psi_hip_gqa_config*
     std::vector<double> costs;
     std::vector<double> free_at;
     for (uint32_t partition : candidates) {
-        if ((uint64_t)partition * 64 < longest) continue;  // (more than 64 partitions of a request are never the answer)
+        // (more than 64 partitions of a request are never the answer)
+        if ((uint64_t)partition * 64 < longest && partition != unsplit) continue;
         costs.clear();
         for (uint32_t r = 0; r < num_reqs; ++r) {
             const uint32_t prefix = token_indices[r], chunk = cu_tokens[r + 1] - cu_tokens[r];

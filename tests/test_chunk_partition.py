@@ -57,7 +57,7 @@ def planned(reqs, hq, hkv, d, ts, units=256):
     longest = max(prefix + chunk for prefix, chunk in reqs)
     best, answer = None, 0
     for p in candidates(longest):
-        if p * 64 < longest:
+        if p * 64 < longest and p != candidates(longest)[-1]:
             continue
         cost = model(reqs, hq, hkv, d, ts, p, units)
         if best is None or cost <= best:
@@ -109,3 +109,14 @@ def test_geometries_without_a_row_group_kernel_and_empty_batches(psi):
 def test_fewer_units_want_fewer_longer_items(psi):
     cfg = config(psi, 24, 4, 256, 16)
     assert ask(psi, cfg, 8, [(4096, 512)], 32) >= ask(psi, cfg, 8, [(4096, 512)], 256)
+
+
+def test_a_decreasing_prefix_sum_is_refused(psi):
+    with pytest.raises(Exception, match="cu_tokens must not decrease"):
+        psi.chunk_partition_tokens(config(psi, 24, 4, 256, 16), 8, [4096, 100], [0, 2048, 1000])
+
+
+def test_contexts_beyond_64_of_the_longest_candidate_stay_unsplit_at_worst(psi):
+    """The planner never answers 0 for a geometry it serves: the unsplit candidate always stands."""
+    got = ask(psi, config(psi, 24, 4, 256, 16), 8, [(3_000_000, 64)])
+    assert got % 256 == 0 and got >= 32768
