@@ -42,7 +42,7 @@ sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBPS = 8000.0
 MFMA_BF16_PEAK_TFLOPS = 2500.0
-CONFIG_NAMES = ["C1", "C2_rows512", "C2_b4", "C2_b8", "C2_b16", "C3", "C4_q2", "C4_q4", "C4_q8", "C5_decode", "C5_prefill", "PREFILL_d128",
+CONFIG_NAMES = ["C1", "C2_rows512", "C2_b4", "C2_b8", "C2_b16", "C3", "C4_q2", "C4_q4", "C4_q8", "C4_q8_g8", "C5_decode", "C5_prefill", "PREFILL_d128",
                 "PREFILL_p16k", "PREFILL_c512", "C5_mixed", "GENERIC_f32_b8"]
 # The shapes the reference itself times (the only figures it publishes for these kernels, on an Apple M3 Max):
 #   REF_tiled      "SplitKV TiledQ only", 40 Q / 8 KV heads, head_dim 128, 8-token pages, one request with 8 new tokens
@@ -242,6 +242,18 @@ def build_case(psi, wl, device, name, args):
         ctx = wl.config_c2_context_lens(4, 64, 2048, 16384) + q_len
         return verify_case(f"verify_q{q_len}_b64_ctx2048-16384_24q4kv_d256_bf16_p16_part512_seed4", ctx, q_len, 512,
                            args.arenas or 1, 4)
+    if name == "C4_q8_g8":
+        # the same batch with 8 heads per KV head (32 Q / 4 KV): 64 query columns per tile, more than the multi-query
+        # map's pipeline holds, so the step goes through the row-group map - short chunks whose tokens times all the
+        # heads fit one workgroup, walked once per KV head, with the partition the planner picks
+        ctx = wl.config_c2_context_lens(4, 64, 2048, 16384) + 8
+        w = wl.make_workload(4, ctx, 32, 4, 256, bf16, 16, q_lens=8, host_pages=False,
+                             shuffle_pages=not args.identity_pages)
+        dw = wl.DeviceWorkload(device, w, partition_tokens="auto", grouped=True,
+                               variant=psi.GQASplitKVVariant.TiledQ(8, 16, 8))
+        return Case(name, f"verify_q8_b64_ctx2048-16384_32q4kv_d256_bf16_p16_part{dw.partition_tokens}_planned_seed4_grouped",
+                    [dw], "verify", "tiled_q_map", "split_kv_chunk_map",
+                    "kv append -> row-group map (all heads of a KV head per work item) -> LSE combine")
     if name == "C5_decode":
         ctx = wl.config_c2_context_lens(5, 128, 512, 32768) + 1
         return decode_case("decode_b128_ctx512-32768_24q4kv_d256_bf16_p16_part512_seed5", ctx, 24, 4, bf16, 512,

@@ -687,8 +687,19 @@ extern "C" int psi_hip_split_kv_chunk_partition_tokens(const psi_hip_gqa_config*
     if (num_reqs == 0 || !chunk_map_supported(g, q_token_tile_size)) return PSI_HIP_OK;
     const uint32_t units = num_compute_units ? num_compute_units : 256u;
     const uint32_t tile_keys = chunk_tile_keys(g.d);
-    const uint32_t group_tokens = chunk_group_tiles(g.group, q_token_tile_size) * q_token_tile_size;
-    const uint32_t copies = g.hkv * chunk_head_subsets(g.group);  // items of equal cost per (group, partition)
+    uint32_t longest_chunk = 0;
+    for (uint32_t r = 0; r < num_reqs; ++r)
+        if (cu_tokens[r + 1] >= cu_tokens[r]) longest_chunk = std::max(longest_chunk, cu_tokens[r + 1] - cu_tokens[r]);
+    // (as psi_hip_split_kv_tiled_q_group_rows and the launch have it: no head subsets when every chunk fits one
+    // workgroup with all the heads)
+    const uint32_t chunk_tiles = (longest_chunk + q_token_tile_size - 1) / q_token_tile_size;
+    const uint32_t width = std::max(std::min(chunk_tiles, chunk_group_tiles(g.group, q_token_tile_size)), 1u);
+    const uint32_t subsets = chunk_launch_subsets(g.group, width, q_token_tile_size);
+    const uint32_t group_tokens =
+        (subsets == 1 ? std::max(std::min(chunk_all_heads_tiles(g.group, q_token_tile_size),
+                                          chunk_group_tiles(g.group, q_token_tile_size)), 1u)
+                      : chunk_group_tiles(g.group, q_token_tile_size)) * q_token_tile_size;
+    const uint32_t copies = g.hkv * subsets;  // items of equal cost per (group, partition)
     constexpr double kItemTiles = 9.0;
     const double partial_tiles = 0.06 * g.d / 256.0;
     uint64_t longest = 0;
@@ -807,21 +818,30 @@ extern "C" int psi_hip_split_kv_tiled_q_group_rows(const psi_hip_gqa_config* cfg
         groups.back().keys = std::max(groups.back().keys, rows[i].kv_end - rows[i].kv_begin);
         groups.back().work += (uint64_t)tile_tokens(rows[i].tile) * (rows[i].kv_end - rows[i].kv_begin);
     }
-    PSI_REQUIRE((uint64_t)groups.size() * max_tiles <= row_groups_capacity,
-                "row-group table too small: %llu groups of %u rows, capacity %llu words",
-                (unsigned long long)groups.size(), max_tiles, (unsigned long long)row_groups_capacity);
     // Longest groups first, so that the short ones fill the end of the launch.  A work item walks the group's KV
     // range whatever the number of its query tokens (a request's last group may hold a few), so the range is the
     // key, not the tokens x keys product, by which such a group was claimed last and ended the launch.
     std::stable_sort(groups.begin(), groups.end(), [](const Group& x, const Group& y) {
         return x.keys != y.keys ? x.keys > y.keys : x.work > y.work;
     });
+    // No group wider than what fits one workgroup with all the heads of a KV head (short chunks, verify steps): the
+    // table is written that narrow, which tells the launch to deal no heads to separate work items.
+    uint32_t stride = max_tiles;
+    const uint32_t all_heads_tiles = chunk_all_heads_tiles(g.group, q_token_tile_size);
+    if (all_heads_tiles >= 1 && all_heads_tiles < max_tiles) {
+        uint32_t widest = 0;
+        for (const Group& grp : groups) widest = std::max(widest, grp.count);
+        if (widest <= all_heads_tiles) stride = all_heads_tiles;
+    }
+    PSI_REQUIRE((uint64_t)groups.size() * stride <= row_groups_capacity,
+                "row-group table too small: %llu groups of %u rows, capacity %llu words",
+                (unsigned long long)groups.size(), stride, (unsigned long long)row_groups_capacity);
     for (size_t gi = 0; gi < groups.size(); ++gi) {
-        uint32_t* out = row_groups + gi * max_tiles;
-        for (uint32_t m = 0; m < max_tiles; ++m)
+        uint32_t* out = row_groups + gi * stride;
+        for (uint32_t m = 0; m < stride; ++m)
             out[m] = m < groups[gi].count ? rows[groups[gi].first + m].row : PSI_HIP_SENTINEL;
     }
-    *out_group_tiles = max_tiles;
+    *out_group_tiles = stride;
     *out_num_groups = (uint32_t)groups.size();
     return PSI_HIP_OK;
 }

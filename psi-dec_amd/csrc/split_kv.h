@@ -153,6 +153,17 @@ inline uint32_t chunk_group_tiles(uint32_t group, uint32_t q_token_tile_size) {
     const uint32_t tiles = (uint32_t)kChunkCols / (heads * q_token_tile_size);
     return tiles > 32 ? 32u : tiles;
 }
+// Q-token tiles of a row group whose tokens times all the heads of a KV head fit the columns of one workgroup.
+inline uint32_t chunk_all_heads_tiles(uint32_t group, uint32_t q_token_tile_size) {
+    return (uint32_t)kChunkCols / (group * q_token_tile_size);
+}
+// Head subsets of a launch over a row-group table `group_tiles` wide.  A table that narrow that a group's tokens
+// times all the heads fit one workgroup (short chunks, verify steps) is walked without subsets: a work item then
+// reads its KV range once for all the heads.  (The width of the table says it: psi_hip_split_kv_tiled_q_group_rows
+// writes the narrow form when no group is wider.)
+inline uint32_t chunk_launch_subsets(uint32_t group, uint32_t group_tiles, uint32_t q_token_tile_size) {
+    return group_tiles <= chunk_all_heads_tiles(group, q_token_tile_size) ? 1u : chunk_head_subsets(group);
+}
 // True when the prefill-chunk map covers the geometry: 2-byte elements, head_dim 128 or 256, pages of 8 * 2^k tokens
 // (the reference's TiledQ profiles (128, 8), (256, 8), (256, 16) among them,
 // crates/inference-backend-metal/src/components/gqa_split_kv_tiled_q.rs:66-76).

@@ -610,7 +610,7 @@ __global__ __launch_bounds__(64 * kChunkWaves, 1) void split_kv_chunk_map(
 template <typename Tag, int D>
 inline int launch_chunk_map_typed(psi_hip_ctx* ctx, const Geometry& g, const MapArgs& a, const uint32_t* row_groups,
                                   uint32_t group_tiles, uint32_t num_groups) {
-    const uint32_t subsets = chunk_head_subsets(g.group);
+    const uint32_t subsets = chunk_launch_subsets(g.group, group_tiles, a.rows_per_split_head);
     const uint32_t num_items = num_groups * g.hkv * subsets;
     if (num_items == 0) return PSI_HIP_OK;
     auto* kernel = &split_kv_chunk_map<Tag, D>;

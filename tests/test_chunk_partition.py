@@ -20,7 +20,13 @@ def model(reqs, hq, hkv, d, ts, partition, units=256):
     group = hq // hkv
     subsets = 3 if group == 6 else (2 if group > 5 else 1)
     heads = (group + subsets - 1) // subsets
-    group_tokens = min(256 // (heads * ts), 32) * ts
+    group_tiles = min(256 // (heads * ts), 32)
+    # chunks that short that their tokens times all the heads of a KV head fit one workgroup: no head subsets
+    all_heads_tiles = 256 // (group * ts)
+    widest = max(min(max((chunk + ts - 1) // ts for _, chunk in reqs), group_tiles), 1)
+    if widest <= all_heads_tiles:
+        subsets, group_tiles = 1, max(min(all_heads_tiles, group_tiles), 1)
+    group_tokens = group_tiles * ts
     tile_keys = 64 if d == 128 else 32
     costs = []
     for prefix, chunk in reqs:

@@ -160,6 +160,34 @@ def test_c4_verify_full_batch(psi, oracle, device, how, q_len):
     assert np.abs(outs[0] - outs[1]).max() < 2e-5
 
 
+@pytest.mark.parametrize("hq", [32, 28])
+def test_c4_verify_with_eight_tokens_and_64_columns_through_row_groups(psi, oracle, device, hq):
+    """C4's batch with 8 (and 7) heads per KV head and eight new tokens per sequence: 64 (56) query columns per tile.
+    The row-group map with the planned partition (tables written narrow: a work item serves all the heads of its KV
+    head), the same with 512-token partitions and the plain multi-query map agree to f32 rounding; the shortest,
+    median and longest sequence match the scalar oracle, every appended line is in its page slot."""
+    wl = importlib_workloads(psi)
+    ctx = wl.config_c2_context_lens(4, 64, 2048, 16384) + 8
+    w = wl.make_workload(4, ctx, hq, 4, 256, psi.Dtype.Bfloat16, 16, q_lens=8, host_pages=False)
+    variant = psi.GQASplitKVVariant.TiledQ(8, 16, hq // 4)
+    outs = {}
+    for name, partition, grouped in (("planned", "auto", True), ("grouped 512", 512, True), ("plain 512", 512, False)):
+        dw = wl.DeviceWorkload(device, w, partition_tokens=partition, f32_output=True, grouped=grouped, variant=variant)
+        assert (dw.meta.num_row_groups > 0) == grouped
+        if grouped:
+            assert dw.meta.group_tiles == 4  # 4 tiles x 8 tokens x 8 heads = 256 columns: no head subsets
+        dw.step()
+        outs[name] = dw.output_f32()
+        if name == "planned":
+            assert dw.partition_tokens >= 2048
+            order = np.argsort(w.context_lens)
+            _sampled_check(oracle, dw, [int(order[0]), int(order[32]), int(order[-1])], f"C4 q_len 8, {hq} heads, sampled")
+        del dw
+    assert np.isfinite(outs["planned"]).all()
+    assert np.abs(outs["planned"] - outs["grouped 512"]).max() < 1e-4
+    assert np.abs(outs["planned"] - outs["plain 512"]).max() < 1e-4
+
+
 def test_c5_prefill_chunk_full_size(psi, oracle, device):
     """C5's chunk: 2048 new tokens on a 4096-token prefix, 24 Q / 4 KV heads.  The row-group map and
     the plain multi-query map agree to rounding on the whole chunk, partition lengths do not matter,

@@ -329,6 +329,27 @@ def test_grouped_geometries(psi, oracle, device, dtype_name, hq, hkv, d, p, q_le
     assert dw.meta.num_row_groups > 0
 
 
+@pytest.mark.parametrize("hq,hkv,d,p,q_lens,width", [
+    (32, 4, 256, 16, [8, 8, 5, 8, 1], 4),   # verify steps at 8 heads per KV head: 64 columns, all heads in one item
+    (28, 4, 256, 16, [8, 1, 8], 4),         # 7 heads: 56 columns
+    (24, 4, 128, 8, [8, 8, 40], 5),         # 6 heads: a chunk of five tiles still fits (240 columns)
+    (16, 2, 128, 16, [32, 8], 4),           # 8 heads x 32 tokens: all 256 columns of one item
+    (16, 2, 256, 32, [33, 8], 8),           # one token more: back to two head subsets, tables 8 tiles wide
+])
+def test_grouped_short_chunks_walk_their_range_once_for_all_heads(psi, oracle, device, hq, hkv, d, p, q_lens, width):
+    """With more than five heads per KV head a row group's heads are dealt to two or three work items - unless no
+    group of the batch is wider than what fits one workgroup with all the heads: then the table is written that
+    narrow and a work item serves every head of its KV head, reading the KV range once."""
+    wl = importlib_workloads(psi)
+    prefixes = [700, 64, 1500, 0, 333][:len(q_lens)]
+    ctx = [a + b for a, b in zip(prefixes, q_lens)]
+    w = wl.make_workload(411, ctx, hq, hkv, d, psi.Dtype.Bfloat16, p, q_lens=q_lens)
+    variant = psi.GQASplitKVVariant.TiledQ(8, 16, hq // hkv)
+    _, dw = run_and_check(psi, oracle, device, w, f"grouped short chunks {hq}/{hkv}/{d} q={q_lens}", max_tokens=256,
+                          variant=variant, partition_tokens=512, grouped=True)
+    assert dw.meta.num_row_groups > 0 and dw.meta.group_tiles == width
+
+
 @pytest.mark.parametrize("seed", range(16))
 def test_grouped_random_batches(psi, oracle, device, seed):
     """Seeded random batches through the row-group map against the oracle: head groups 1..8, both head dims, pages

@@ -603,8 +603,19 @@ def test_row_group_table_capacity_is_checked(psi):
     table = np.zeros(32, np.uint32)
     assert lib.psi_hip_split_kv_tiled_q_group_rows(ctypes.byref(cfg), 8, p(rows), 2, p(tiles), 2, p(slots), p(table),
                                                    32, ctypes.byref(n_tiles), ctypes.byref(n_groups)) == 0
-    assert (n_tiles.value, n_groups.value) == (16, 2)  # two requests never share a group
-    assert table.tolist() == [0] + [MAX] * 15 + [1] + [MAX] * 15
+    # two requests never share a group; and no group is wider than the 5 tiles whose tokens fit one workgroup with
+    # all six heads of a KV head, so the table is written that narrow (the launch then deals no heads to separate
+    # work items)
+    assert (n_tiles.value, n_groups.value) == (5, 2)
+    assert table[:10].tolist() == [0] + [MAX] * 4 + [1] + [MAX] * 4
+    # a group of six tiles is wider than that: the full width, 16 tiles of two heads each
+    rows = np.array([[t, 0, 64] for t in range(6)], np.uint32).reshape(-1)
+    tiles = np.array([[8 * t, 8 * t + 8] for t in range(6)], np.uint32).reshape(-1)
+    slots = np.zeros(48, np.uint32)
+    assert lib.psi_hip_split_kv_tiled_q_group_rows(ctypes.byref(cfg), 8, p(rows), 6, p(tiles), 6, p(slots), p(table),
+                                                   32, ctypes.byref(n_tiles), ctypes.byref(n_groups)) == 0
+    assert (n_tiles.value, n_groups.value) == (16, 1)
+    assert table[:16].tolist() == list(range(6)) + [MAX] * 10
 
 
 # ------------------------------------------------------------------ the whole plan in one call
