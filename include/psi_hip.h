@@ -480,7 +480,17 @@ int psi_hip_split_kv_tiled_q_map(psi_hip_ctx* ctx, const psi_hip_gqa_config* cfg
  * longest KV range first (its work items walk that range whatever the number of its tokens).  row_groups:
  * host u32[row_groups_capacity], written as [*out_num_groups][*out_group_tiles] row indices padded with PSI_HIP_SENTINEL; capacity of num_kv_splits * 32 words always suffices.  req_slots
  * is the per-token slot array of psi_hip_gqa_metadata_update.  Every non-padding row lands in exactly
- * one group.  *out_group_tiles = 0 when the geometry has no grouped kernel (use the plain map then). */
+ * one group.  *out_group_tiles = 0 when the geometry has no grouped kernel (use the plain map then).
+ * With more than five Q heads per KV head a group's heads are dealt to two or three work items, so that an item's
+ * tokens x heads fit the 256 query columns of a workgroup -- unless no group of the batch is wider than
+ * 256 / (heads per KV head * q_token_tile_size) tiles (short chunks, verify steps): then *out_group_tiles is that
+ * number, and the launch, which goes by the table's width, lets one work item serve all the heads of its KV head and
+ * read its KV range once.
+ * When to use row groups: for requests of more than one Q-token tile (the plain map walks a request's KV range once per
+ * tile), and for single tiles of more than 48 query columns (8 tokens x 7 or 8 heads per KV head), where the plain map
+ * falls back to a kernel that reads K/V twice: 64 sequences of 2048..16384 tokens with 8 new tokens each at 32 Q /
+ * 4 KV heads of 256 take 487 us here against 786 us, with 16 new tokens 529 us against 1534 us.  Single tiles of up to
+ * 48 columns are faster through the plain map with a balanced plan (447 us against 483 us at 24 Q heads). */
 int psi_hip_split_kv_tiled_q_group_rows(const psi_hip_gqa_config* cfg, uint32_t q_token_tile_size,
                                         const uint32_t* kv_splits, uint32_t num_kv_splits,
                                         const uint32_t* q_token_tiles, uint32_t num_q_token_tiles,
@@ -496,8 +506,8 @@ int psi_hip_split_kv_tiled_q_group_rows(const psi_hip_gqa_config* cfg, uint32_t 
  * and read once.  token_indices[r] is the position of request r's first new token and cu_tokens[r + 1] - cu_tokens[r]
  * the number of its new tokens, as for psi_hip_gqa_metadata_update.  On the shape this library is measured on (2048
  * tokens on a 4096-token prefix, 24 Q / 4 KV heads of 256) it answers 4096; for 512 tokens on the same prefix 1024,
- * where 4096 leaves 96 items for 256 units and takes three times as long.  The answer depends on the batch's lengths
- * only: cache it per shape class.  *out_partition_tokens = 0 when the geometry has no grouped kernel or the batch
+ * where 4096 leaves 96 items for 256 units and takes three times as long; for 64 verify requests of 8 tokens on
+ * 2048..16384 cached ones 10240.  The answer depends on the batch's lengths only: cache it per shape class.  *out_partition_tokens = 0 when the geometry has no grouped kernel or the batch
  * is empty. */
 int psi_hip_split_kv_chunk_partition_tokens(const psi_hip_gqa_config* cfg, uint32_t q_token_tile_size,
                                             const uint32_t* token_indices, const uint32_t* cu_tokens,
@@ -517,7 +527,8 @@ int psi_hip_split_kv_tiled_q_map_balanced(
     uint32_t num_total_q_token_tiles, uint32_t num_total_kv_splits, uint32_t num_active_tokens,
     uint32_t num_active_q_token_tiles, uint32_t num_active_kv_splits, uint32_t max_active_q_tile_tokens);
 
-/* psi_hip_split_kv_tiled_q_map with one work item per (row group, KV head [, half or a third of the Q heads]):
+/* psi_hip_split_kv_tiled_q_map with one work item per (row group, KV head [, half or a third of the Q heads, by the
+ * width of the table: see psi_hip_split_kv_tiled_q_group_rows]):
  * the group's K/V tiles are staged once in LDS for up to 256 query columns and both contractions run
  * on the matrix cores.  The launch is one workgroup per compute unit; a workgroup takes items, in the table's
  * order, until none is left.  Same arguments, scratch layout and results (within rounding) as the plain map;
