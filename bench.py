@@ -160,7 +160,9 @@ def build_case(psi, wl, device, name, args):
                                  shuffle_pages=not args.identity_pages)
             w.seed = seed + 1000 * i
             out.append(wl.DeviceWorkload(device, w, partition_tokens=partition, variant=variant, **verify_how))
-        return Case(name, key, out, "verify", "tiled_q_map", "split_kv_tiled_map",
+        # (tiles of more than 48 query columns go to the row-group kernel, a row per group)
+        wide = min(hq // hkv, 8) * min(int(np.max(q_len)), 8) > 48
+        return Case(name, key, out, "verify", "tiled_q_map", "split_kv_chunk_map" if wide else "split_kv_tiled_paired_map",
                     "kv append -> multi-query split-KV map -> LSE combine")
 
     def map_and_reduce_only(case):

@@ -487,10 +487,11 @@ int psi_hip_split_kv_tiled_q_map(psi_hip_ctx* ctx, const psi_hip_gqa_config* cfg
  * number, and the launch, which goes by the table's width, lets one work item serve all the heads of its KV head and
  * read its KV range once.
  * When to use row groups: for requests of more than one Q-token tile (the plain map walks a request's KV range once per
- * tile), and for single tiles of more than 48 query columns (8 tokens x 7 or 8 heads per KV head), where the plain map
- * falls back to a kernel that reads K/V twice: 64 sequences of 2048..16384 tokens with 8 new tokens each at 32 Q /
- * 4 KV heads of 256 take 487 us here against 786 us, with 16 new tokens 529 us against 1534 us.  Single tiles of up to
- * 48 columns are faster through the plain map with a balanced plan (447 us against 483 us at 24 Q heads). */
+ * tile), and for single tiles of more than 48 query columns (8 tokens x 7 or 8 heads per KV head): the plain and the
+ * balanced map hand those to the same kernel, every row a group of its own, but cut for another kernel's shares --
+ * 64 sequences of 2048..16384 tokens with 8 new tokens each at 32 Q / 4 KV heads of 256 take 487 us as row groups over
+ * the planned partition against 661 us over a balanced plan; with 16 new tokens 529 us against 1534 us.  Single tiles
+ * of up to 48 columns are faster through the plain map with a balanced plan (447 us against 483 us at 24 Q heads). */
 int psi_hip_split_kv_tiled_q_group_rows(const psi_hip_gqa_config* cfg, uint32_t q_token_tile_size,
                                         const uint32_t* kv_splits, uint32_t num_kv_splits,
                                         const uint32_t* q_token_tiles, uint32_t num_q_token_tiles,

@@ -190,12 +190,14 @@ __device__ __forceinline__ void chunk_map_item(
     if (group >= num_groups || subset * heads_per_subset >= a.group) return;
     const uint32_t G = min(heads_per_subset, a.group - subset * heads_per_subset);
 
+    // (no table: every kv_split row is a group of its own, group_tiles is 1)
     const uint32_t* rows = row_groups + (uint64_t)group * group_tiles;
-    const uint32_t my_row = lane < group_tiles ? rows[lane] : kNoRow;
+    auto row_of = [&](uint32_t i) -> uint32_t { return row_groups != nullptr ? rows[i] : group; };
+    const uint32_t my_row = lane < group_tiles ? row_of(lane) : kNoRow;
     const bool my_row_ok = my_row != kNoRow && my_row < a.num_active_kv_splits;
     const uint32_t num_tiles = __builtin_amdgcn_readfirstlane(__popcll(__ballot(my_row_ok)));
     if (num_tiles == 0) return;
-    const uint32_t row0 = __builtin_amdgcn_readfirstlane(rows[0]);
+    const uint32_t row0 = __builtin_amdgcn_readfirstlane(row_of(0));
     if (row0 >= a.num_active_kv_splits) return;
     const uint32_t q_tile0 = kv_splits[row0 * 3];
     if (q_tile0 >= a.num_active_q_token_tiles || q_tile0 + num_tiles > a.num_active_q_token_tiles) return;
@@ -230,7 +232,7 @@ __device__ __forceinline__ void chunk_map_item(
         uint32_t t, h;
         used[j] = column_of(j, &t, &h);
         lim[j] = 0;
-        if (used[j]) lim[j] = min(kv_splits[rows[t / TS] * 3 + 2], flat_token_indices[flat_begin + t] + 1);
+        if (used[j]) lim[j] = min(kv_splits[row_of(t / TS) * 3 + 2], flat_token_indices[flat_begin + t] + 1);
         const uint16_t* q_row = q + ((uint64_t)(flat_begin + t) * a.hq + head_first + h) * D + mc * 8;
 #pragma unroll
         for (int ks = 0; ks < kKSteps; ++ks) {
@@ -530,7 +532,7 @@ __device__ __forceinline__ void chunk_map_item(
     for (int j = 0; j < NB; ++j) {
         uint32_t t, h;
         column_of(j, &t, &h);
-        part_row[j] = (rows[t / TS] * a.hq + head_first + h) * TS + t % TS;
+        part_row[j] = (row_of(t / TS) * a.hq + head_first + h) * TS + t % TS;
     }
 #pragma unroll
     for (int j = 0; j < NB; ++j) asm volatile("" : "+v"(part_row[j]));

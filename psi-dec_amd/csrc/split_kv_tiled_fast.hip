@@ -43,6 +43,9 @@ int launch_tiled_map_fast(psi_hip_ctx* ctx, const Geometry& g, const MapArgs& a)
     if (max_tile_tokens > a.rows_per_split_head) max_tile_tokens = a.rows_per_split_head;
     if (max_tile_tokens * g.group > 64) return PSI_HIP_ERR_UNSUPPORTED;
     if ((uint64_t)a.num_total_kv_splits * g.hkv > 0x7fffffffull) return PSI_HIP_ERR_UNSUPPORTED;
+    // More columns than the paired pipeline holds (8 tokens x 7 or 8 heads per KV head): the row-group kernel with
+    // every row a group of its own, which takes 256 columns and reads the row's K/V once.
+    if (max_tile_tokens * g.group > 48) return launch_chunk_map(ctx, g, a, nullptr, 1, a.num_total_kv_splits);
     if (g.dtype == PSI_HIP_BF16)
         return g.d == 256 ? launch_tiled_map_bf16_d256(ctx, g, a, max_tile_tokens)
                           : launch_tiled_map_bf16_d128(ctx, g, a, max_tile_tokens);

@@ -10,8 +10,8 @@
 //   (stream p takes the 16-token tiles p, p + 4, ...), each with its own online-softmax state per column; the
 //   states merge through LDS at the end of the row.
 //   Up to 48 columns (three blocks): split_kv_tiled_paired_map, two waves per stream, KV tiles through LDS by
-//   global_load_lds.  49 to 64 columns: split_kv_tiled_map with two groups of four waves (CG = 2), one per 32
-//   columns, each wave with its tile in registers; the second group finds most tiles in cache.
+//   global_load_lds.  49 to 64 columns (8 tokens x 7 or 8 heads per KV head) are more than its stages and registers
+//   hold: those launches go to the row-group kernel (split_kv_chunk_kernel.h) with every row a group of its own.
 //
 // Per 16-token KV tile
 //   QK^T  S[token][column] on v_mfma_f32_16x16x32: A = the K tile (lane = token lane%16, 8 contiguous dims), B =
@@ -89,397 +89,11 @@ __device__ __forceinline__ uint2 lds_read_tr16_b64(const void* p) {
     return __builtin_bit_cast(uint2, v);
 }
 
-constexpr float kMaxSlack = 8.0f;   // see the softmax of split_kv_tiled_map
+// The reference maximum of a column moves only when a tile exceeds it by more than kMaxSlack (log2 domain), a few
+// times per range: probabilities stay below 2^kMaxSlack, and the rescaling of the accumulators is rare.
+constexpr float kMaxSlack = 8.0f;
 constexpr int kTiledTileWaves = 4;  // waves that share the KV tiles of a split among them
 
-// Two workgroups per SIMD for every shape.  Three would hold the one-column-block variant to 168 registers, which
-// it overflows into a private segment since it walks a range of rows (at a great loss, and the balanced launch
-// keeps one workgroup per compute unit anyway); one would let the wider variants move their accumulators into
-// AGPRs, which measured slower (verify q_len 4: 521 vs 455 us).  At two workgroups per SIMD only the two-group
-// variants at head_dim 256 keep a private segment (40-44 bytes, outside the tile loop).
-template <int NB, int CG>
-struct TiledOccupancy {
-    static constexpr int value = 2;
-};
-
-// NB: column blocks per wave (1 or 2); CG: column groups (1 or 2), each a set of four waves.
-template <typename Tag, int D, int NB, int CG, bool kHalfPage>
-__global__ __launch_bounds__(64 * kTiledTileWaves * CG, (TiledOccupancy<NB, CG>::value)) void split_kv_tiled_map(
-    MapArgs a, const uint32_t* __restrict__ page_ids, const uint32_t* __restrict__ kv_splits,
-    const uint32_t* __restrict__ req_slots, const uint16_t* __restrict__ q, const uint16_t* __restrict__ pages,
-    const uint32_t* __restrict__ q_token_tiles, const uint32_t* __restrict__ flat_token_indices,
-    const uint32_t* __restrict__ worker_cu) {
-    resolve_active(a);
-    constexpr int kTileWaves = kTiledTileWaves;
-    constexpr int kWaves = kTileWaves * CG;
-    constexpr int kVLanesPerToken = D / 8;                  // 32 (D=256) or 16 (D=128)
-    constexpr int kVTokensPerLoad = 64 / kVLanesPerToken;   // 2 or 4
-    constexpr int kVLoads = kTileTokens / kVTokensPerLoad;  // 8 or 4
-    constexpr int kKSteps = D / 32;                         // MFMA k-steps of QK^T
-    constexpr int kDimBlocks = D / 16;                      // 16-dim output blocks of PV
-    constexpr int kVStride = D + 16;                        // elements per token row of the V buffer: the four rows of a
-                                                            // quarter wave's transposing read fall into different banks
-    constexpr int kCols = CG * NB * 16;
-    constexpr int kMergeStride = D + 4;                     // floats per column row of the merge buffer
-
-    // LDS: the main loop's V buffers and Q operands share their bytes with the epilogue's merge buffer.
-    constexpr int kVBytes = kWaves * kTileTokens * kVStride * 2;
-    constexpr int kQBytes = CG * NB * kKSteps * 64 * 16;
-    constexpr int kMergeBytes = kCols * kMergeStride * 4;
-    constexpr int kUnionBytes = (kVBytes + kQBytes) > kMergeBytes ? (kVBytes + kQBytes) : kMergeBytes;
-    __shared__ __attribute__((aligned(16))) unsigned char lds_union[kUnionBytes];
-    __shared__ float wave_max_lds[kTileWaves][kCols];
-    __shared__ float col_max_lds[kCols];
-    __shared__ float col_sum_lds[kCols];
-    uint16_t* v_lds = reinterpret_cast<uint16_t*>(lds_union);
-    uint4* qb_lds = reinterpret_cast<uint4*>(lds_union + kVBytes);  // [CG * NB][kKSteps][64]
-    float* merge = reinterpret_cast<float*>(lds_union);
-
-    const uint32_t G = a.group;
-    const uint32_t kv_head = blockIdx.x % a.walk.hkv;
-    const uint32_t wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
-    const uint32_t tile_wave = wave % kTileWaves;       // which KV tiles this wave takes
-    const uint32_t col_base = (wave / kTileWaves) * NB;  // first column block of this wave
-
-    // Rows of kv_splits this workgroup serves: one row (blockIdx / Hkv) in the plain launch, or the worker's row
-    // range when a balanced plan hands each workgroup an equal share of tiles.  Every skip below is uniform over
-    // the workgroup.
-    uint32_t row_begin = blockIdx.x / a.walk.hkv, row_end = row_begin + 1;
-    if (worker_cu != nullptr) {
-        row_begin = worker_cu[blockIdx.x / a.walk.hkv];
-        row_end = worker_cu[blockIdx.x / a.walk.hkv + 1];
-    }
-    bool lds_in_use = false;
-    for (uint32_t split = row_begin; split < row_end; ++split) {
-    if (split >= a.num_active_kv_splits) break;
-    const uint32_t q_tile = kv_splits[split * 3];
-    if (q_tile >= a.num_active_q_token_tiles) continue;  // sentinel padding
-    const uint32_t kv_begin = kv_splits[split * 3 + 1];
-    const uint32_t kv_end = kv_splits[split * 3 + 2];
-    const uint32_t flat_begin = q_token_tiles[q_tile * 2], flat_end = q_token_tiles[q_tile * 2 + 1];
-    if (flat_begin >= a.num_active_tokens || flat_end > a.num_active_tokens || flat_end <= flat_begin) continue;
-    const uint32_t tile_tokens = flat_end - flat_begin;
-    const uint32_t ncols = tile_tokens * G;
-    if (ncols > (uint32_t)kCols) {
-        // A tile wider than the launch was sized for (the caller's largest-tile bound was too small, e.g. a
-        // capture made for two-token tiles replayed on a four-token batch).  The row cannot be computed here;
-        // it is entered as an empty state, so that the combine merges nothing stale, and the tile's output is
-        // then wrong in a visible way (zeros for a tile with no other row) rather than silently mixed.
-        const uint32_t rows = a.rows_per_split_head;
-        for (uint32_t idx = threadIdx.x; idx < ncols * (D / 4); idx += 64 * kWaves) {
-            const uint32_t c = idx / (D / 4), d4 = idx % (D / 4);
-            const uint64_t row = ((uint64_t)split * a.hq + (uint64_t)kv_head * G + c % G) * rows + c / G;
-            *reinterpret_cast<float4*>(&a.part_acc[row * D + d4 * 4]) = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
-            if (d4 == 0) {
-                a.part_max[row] = -INFINITY;
-                a.part_sum[row] = 0.0f;
-            }
-        }
-        continue;
-    }
-    if (lds_in_use) __syncthreads();  // the previous row's merge buffer has been read out
-    lds_in_use = true;
-    // Lane coordinates, re-derived per row from a value the optimiser cannot see through: nothing computed from
-    // them is loop-invariant, so no per-lane address survives from one row into the next row's register budget.
-    uint32_t tid = threadIdx.x;
-    asm volatile("" : "+v"(tid));
-    const uint32_t lane = tid & 63;
-    const uint32_t mt = lane & 15, mc = lane >> 4;
-    const uint32_t vsub = lane / kVLanesPerToken, vdl = lane % kVLanesPerToken;
-    const uint32_t nb_total = (ncols + 15) / 16;
-    // column blocks this wave works on: col_base + [0, nb_active)
-    const uint32_t nb_active = nb_total > col_base ? min(nb_total - col_base, (uint32_t)NB) : 0u;
-    const uint32_t req_slot = req_slots[flat_begin];
-
-    // Column of this lane in its block nb: c = 16*(col_base + nb) + mt; its query token, head and
-    // visible key range.
-    uint32_t lim[NB];  // keys [kv_begin, lim) are visible to the column (0: column unused)
-#pragma unroll
-    for (int nb = 0; nb < NB; ++nb) {
-        const uint32_t c = (col_base + nb) * 16 + mt;
-        lim[nb] = 0;
-        if (c < ncols) lim[nb] = min(kv_end, flat_token_indices[flat_begin + c / G] + 1);
-    }
-
-    // Query columns as MFMA B operands [nb][k-step][lane]; unused columns are zero.
-    for (uint32_t nb = wave; nb < nb_total; nb += kWaves) {
-        const uint32_t c = nb * 16 + mt;
-        const bool used = c < ncols;
-        const uint32_t cc = used ? c : 0;
-        const uint16_t* q_row =
-            q + ((uint64_t)(flat_begin + cc / G) * a.hq + (uint64_t)kv_head * G + cc % G) * D + mc * 8;
-#pragma unroll
-        for (int i = 0; i < kKSteps; ++i) {
-            const uint4 v = *reinterpret_cast<const uint4*>(q_row + i * 32);
-            qb_lds[(nb * kKSteps + i) * 64 + lane] = used ? v : make_uint4(0, 0, 0, 0);
-        }
-    }
-    __syncthreads();
-
-    const uint32_t log2p = 31 - __builtin_clz(a.walk.tokens_per_page);
-    const uint32_t page_mask = a.walk.tokens_per_page - 1;
-    const uint32_t* table_row = page_ids + ((uint64_t)req_slot * a.walk.num_layers + a.layer) *
-                                                      a.walk.num_blocks * a.walk.ids_per_block;
-    const uint64_t v_region = (uint64_t)a.walk.hkv * a.walk.tokens_per_page * D;
-    const uint32_t tile_begin = kv_begin / kTileTokens;
-    const uint32_t tile_end = (kv_end + kTileTokens - 1) / kTileTokens;
-
-    float run_max[NB], lane_sum[NB];
-    f32x4_t o[NB][kDimBlocks];
-#pragma unroll
-    for (int nb = 0; nb < NB; ++nb) {
-        run_max[nb] = -INFINITY;
-        lane_sum[nb] = 0.0f;
-#pragma unroll
-        for (int db = 0; db < kDimBlocks; ++db) o[nb][db] = f32x4_t{0.0f, 0.0f, 0.0f, 0.0f};
-    }
-
-    const uint32_t last_page = (kv_end - 1) >> log2p;
-    auto load_page_id = [&](uint32_t tile) -> TilePages {
-        TilePages p{0u, 0u};
-        if (tile < tile_end) {
-            const uint32_t first = (tile * kTileTokens) >> log2p;
-            p.a = table_row[first];
-            if (kHalfPage) p.b = table_row[min(first + 1, last_page)];
-        }
-        return p;
-    };
-    auto head_base = [&](uint32_t page_id) -> const uint16_t* {
-        return pages + (uint64_t)page_id * a.walk.page_elems + (uint64_t)kv_head * a.walk.tokens_per_page * D;
-    };
-    uint4 kreg[kKSteps];
-    uint4 vreg[kVLoads];
-    auto issue_k = [&](uint32_t tile, TilePages p) {
-        const uint16_t* k_lane;
-        if (kHalfPage)
-            k_lane = head_base(mt < 8 ? p.a : p.b) + (mt & 7) * D + mc * 8;
-        else
-            k_lane = head_base(p.a) + (((tile * kTileTokens) & page_mask) + mt) * D + mc * 8;
-#pragma unroll
-        for (int i = 0; i < kKSteps; ++i) kreg[i] = *reinterpret_cast<const uint4*>(k_lane + i * 32);
-    };
-    auto issue_v = [&](uint32_t tile, TilePages p) {
-#pragma unroll
-        for (int j = 0; j < kVLoads; ++j) {
-            const uint16_t* v_lane;
-            if (kHalfPage)
-                v_lane = head_base(j * kVTokensPerLoad < 8 ? p.a : p.b) + v_region +
-                         ((j * kVTokensPerLoad + vsub) & 7) * D + vdl * 8;
-            else
-                v_lane = head_base(p.a) + v_region +
-                         (((tile * kTileTokens) & page_mask) + j * kVTokensPerLoad + vsub) * D + vdl * 8;
-            vreg[j] = stream_load_b128(v_lane);  // V rows are whole lines read once; K keeps ordinary loads (two loads share each line)
-        }
-    };
-
-    uint16_t* my_v = v_lds + wave * kTileTokens * kVStride;
-    // B operand of PV for dim block db (tokens 4 * mc .. + 3 of dim 16 * db + mt) through the transposing LDS read:
-    // the lane hands in the address of token 4 * mc + mt / 4, dims 16 * db + 4 * (mt % 4) .. + 3, and the 16 lanes of
-    // a quarter wave get their 16 x 4 block back transposed.
-    const uint16_t* my_v_read = my_v + (mc * 4 + (mt >> 2)) * kVStride + (mt & 3) * 4;
-
-    auto process_tile = [&](uint32_t tile, bool partial, auto has_next_tag, uint32_t next, TilePages next_pid)
-                            __attribute__((always_inline)) {
-        constexpr bool has_next = decltype(has_next_tag)::value;
-        // ---- logits S[token][column] on the matrix cores
-        f32x4_t s[NB];
-#pragma unroll
-        for (int nb = 0; nb < NB; ++nb) {
-            s[nb] = f32x4_t{0.0f, 0.0f, 0.0f, 0.0f};
-            if ((uint32_t)nb < nb_active) {
-#pragma unroll
-                for (int i = 0; i < kKSteps; ++i)
-                    s[nb] = mfma_16x16x32<Tag>(kreg[i], qb_lds[((col_base + nb) * kKSteps + i) * 64 + lane], s[nb]);
-            }
-        }
-        __builtin_amdgcn_sched_barrier(0);
-        if (has_next) issue_k(next, next_pid);
-        __builtin_amdgcn_sched_barrier(0);
-
-        ProbOperand<Tag> pa[NB];
-        float alpha[NB];
-        bool moved = false;
-        auto softmax = [&]() __attribute__((always_inline)) {
-            // ---- online softmax per column over this lane's tokens 4*mc + r
-#pragma unroll
-            for (int nb = 0; nb < NB; ++nb) {
-                alpha[nb] = 1.0f;
-                if ((uint32_t)nb < nb_active) {
-                    float v[4];
-                    bool valid[4];
-                    float m = -INFINITY;
-#pragma unroll
-                    for (int r = 0; r < 4; ++r) {
-                        const uint32_t token = tile * kTileTokens + mc * 4 + r;
-                        valid[r] = token >= kv_begin && token < lim[nb];
-                        v[r] = valid[r] ? s[nb][r] * a.scale_log2 : -INFINITY;
-                        m = fmaxf(m, v[r]);
-                    }
-                    m = fmaxf(m, __shfl_xor(m, 16, 64));
-                    m = fmaxf(m, __shfl_xor(m, 32, 64));
-                    // The reference maximum of a column moves only when a tile exceeds it by more than kMaxSlack
-                    // (log2 domain), a few times per range: probabilities stay below 2^kMaxSlack, and the rescaling
-                    // of the accumulators, which every move of any of the wave's columns triggers, becomes rare.
-                    const float next_max = m > run_max[nb] + kMaxSlack ? m : run_max[nb];
-                    // a column with no visible key so far keeps max = -inf, sum = 0, O = 0
-                    alpha[nb] = run_max[nb] > -INFINITY ? __builtin_amdgcn_exp2f(run_max[nb] - next_max) : 0.0f;
-                    moved = moved || next_max != run_max[nb];
-                    run_max[nb] = next_max;
-                    float p[4], tile_sum = 0.0f;
-#pragma unroll
-                    for (int r = 0; r < 4; ++r) {
-                        p[r] = valid[r] ? __builtin_amdgcn_exp2f(v[r] - next_max) : 0.0f;
-                        tile_sum += p[r];
-                    }
-                    lane_sum[nb] = lane_sum[nb] * alpha[nb] + tile_sum;
-                    pa[nb].set(p);
-                }
-            }
-        };
-        auto stage_v = [&]() __attribute__((always_inline)) {
-            // ---- V tile: registers -> this wave's LDS buffer (rows outside the split zeroed: their
-            // probability is 0 but their bytes may be NaN/Inf), then refill the registers for the next tile
-            wave_lds_fence();  // the previous tile's reads of the buffer are complete
-#pragma unroll
-            for (int j = 0; j < kVLoads; ++j) {
-                const uint32_t tok_in_tile = j * kVTokensPerLoad + vsub;
-                uint4 val = vreg[j];
-                if (partial) {
-                    const uint32_t vtoken = tile * kTileTokens + tok_in_tile;
-                    if (vtoken < kv_begin || vtoken >= kv_end) val = make_uint4(0, 0, 0, 0);
-                }
-                *reinterpret_cast<uint4*>(my_v + tok_in_tile * kVStride + vdl * 8) = val;
-            }
-            __builtin_amdgcn_sched_barrier(0);
-            if (has_next) issue_v(next, next_pid);
-            __builtin_amdgcn_sched_barrier(0);
-        };
-        // One column group: V goes to LDS, and the next tile's V loads go out, before the softmax - a tile's period is
-        // the memory latency plus the time from the tile's start to the issue of the next tile's last load (verify
-        // with 3 / 4 query tokens: 437 / 442 -> 420 / 431 us).  Two column groups, two waves per SIMD, measure faster
-        // the other way round (8 tokens: 721 against 747 us).
-        if constexpr (CG == 1) {
-            stage_v();
-            softmax();
-        } else {
-            softmax();
-            stage_v();
-        }
-        const bool rescale = __any(moved);
-        wave_lds_fence();  // the V tile is in LDS
-
-        // ---- O[column][dim] = alpha * O + P^T V
-        if (rescale) {
-#pragma unroll
-            for (int nb = 0; nb < NB; ++nb) {
-                if ((uint32_t)nb < nb_active) {
-                    float al[4];
-#pragma unroll
-                    for (int r = 0; r < 4; ++r) al[r] = __shfl(alpha[nb], mc * 4 + r, 64);
-#pragma unroll
-                    for (int db = 0; db < kDimBlocks; ++db)
-#pragma unroll
-                        for (int r = 0; r < 4; ++r) o[nb][db][r] *= al[r];
-                }
-            }
-        }
-#pragma unroll
-        for (int db = 0; db < kDimBlocks; ++db) {
-            const uint2 b = lds_read_tr16_b64(my_v_read + db * 16);
-#pragma unroll
-            for (int nb = 0; nb < NB; ++nb) {
-                if ((uint32_t)nb < nb_active) {
-#pragma unroll
-                    for (int t = 0; t < ProbOperand<Tag>::kTerms; ++t)
-                        o[nb][db] = mfma_16x16x16<Tag>(pa[nb].term[t], b, o[nb][db]);
-                }
-            }
-        }
-        __builtin_amdgcn_sched_barrier(0);
-    };
-
-    uint32_t tile = tile_begin + tile_wave;
-    if (tile < tile_end && nb_active != 0) {
-        {
-            const TilePages pid = load_page_id(tile);
-            issue_k(tile, pid);
-            issue_v(tile, pid);
-        }
-        TilePages pid_next = load_page_id(tile + kTileWaves);
-        auto is_partial = [&](uint32_t t) { return t * kTileTokens < kv_begin || (t + 1) * kTileTokens > kv_end; };
-        while (tile + kTileWaves < tile_end) {
-            const uint32_t next = tile + kTileWaves;
-            const TilePages pid_after = load_page_id(next + kTileWaves);
-            process_tile(tile, is_partial(tile), std::true_type(), next, pid_next);
-            pid_next = pid_after;
-            tile = next;
-        }
-        process_tile(tile, is_partial(tile), std::false_type(), 0u, TilePages{0u, 0u});
-    }
-
-    // ---- merge the four wave states of each column group.  Column statistics live in the S layout
-    // (lane <-> column mt), the accumulators in the MFMA output layout (lane <-> columns 4*mc + r, dim mt).
-#pragma unroll
-    for (int nb = 0; nb < NB; ++nb) {
-        lane_sum[nb] += __shfl_xor(lane_sum[nb], 16, 64);
-        lane_sum[nb] += __shfl_xor(lane_sum[nb], 32, 64);
-        if (mc == 0) wave_max_lds[tile_wave][(col_base + nb) * 16 + mt] = run_max[nb];
-    }
-    __syncthreads();  // every wave has left the main loop: the V / Q bytes may now be reused
-#pragma unroll
-    for (int nb = 0; nb < NB; ++nb) {
-        const uint32_t c = (col_base + nb) * 16 + mt;
-        float gm = wave_max_lds[0][c];
-#pragma unroll
-        for (int w = 1; w < kTileWaves; ++w) gm = fmaxf(gm, wave_max_lds[w][c]);
-        const float f = run_max[nb] > -INFINITY ? __builtin_amdgcn_exp2f(run_max[nb] - gm) : 0.0f;
-        lane_sum[nb] *= f;
-        if (tile_wave == 0 && mc == 0) col_max_lds[c] = gm;
-        float fr[4];
-#pragma unroll
-        for (int r = 0; r < 4; ++r) fr[r] = __shfl(f, mc * 4 + r, 64);
-#pragma unroll
-        for (int db = 0; db < kDimBlocks; ++db)
-#pragma unroll
-            for (int r = 0; r < 4; ++r) o[nb][db][r] *= fr[r];
-    }
-    for (uint32_t w = 0; w < (uint32_t)kTileWaves; ++w) {
-        if (tile_wave == w) {
-#pragma unroll
-            for (int nb = 0; nb < NB; ++nb) {
-                if ((uint32_t)nb < nb_active) {
-                    if (mc == 0) {
-                        const uint32_t c = (col_base + nb) * 16 + mt;
-                        col_sum_lds[c] = (w == 0 ? 0.0f : col_sum_lds[c]) + lane_sum[nb];
-                    }
-#pragma unroll
-                    for (int db = 0; db < kDimBlocks; ++db)
-#pragma unroll
-                        for (int r = 0; r < 4; ++r) {
-                            float* dst = merge + ((col_base + nb) * 16 + mc * 4 + r) * kMergeStride + db * 16 + mt;
-                            *dst = (w == 0 ? 0.0f : *dst) + o[nb][db][r];
-                        }
-                }
-            }
-        }
-        __syncthreads();
-    }
-
-    // ---- emit: partial row of (split, q_head, token_in_tile); 1 KiB of contiguous f32 per wave store
-    const uint32_t rows = a.rows_per_split_head;
-    for (uint32_t idx = tid; idx < ncols * (D / 4); idx += 64 * kWaves) {
-        const uint32_t c = idx / (D / 4), d4 = idx % (D / 4);
-        const uint64_t row = ((uint64_t)split * a.hq + (uint64_t)kv_head * G + c % G) * rows + c / G;
-        const float4 val = *reinterpret_cast<const float4*>(merge + c * kMergeStride + d4 * 4);
-        *reinterpret_cast<float4*>(&a.part_acc[row * D + d4 * 4]) = val;
-    }
-    if (tid < ncols) {
-        const uint64_t row = ((uint64_t)split * a.hq + (uint64_t)kv_head * G + tid % G) * rows + tid / G;
-        a.part_max[row] = col_max_lds[tid];
-        a.part_sum[row] = col_sum_lds[tid];
-    }
-    }  // rows of this workgroup
-}
 
 // ---------------------------------------------------------------------------------------------------------------
 // KV tiles through LDS without registers (tiles of up to 48 query columns; see split_kv_tiled_paired_map below).
@@ -706,7 +320,10 @@ __global__ __launch_bounds__(64 * tiled_paired_waves(NB), 1) void split_kv_tiled
     if (!cur.valid) continue;  // sentinel padding or a tile outside the active ones
     const uint32_t kv_begin = cur.kv_begin, kv_end = cur.kv_end, flat_begin = cur.flat_begin, ncols = cur.ncols;
     if (ncols > (uint32_t)kCols) {
-        // A tile wider than the launch was sized for: entered as an empty state (see split_kv_tiled_map).
+        // A tile wider than the launch was sized for (the caller's largest-tile bound was too small, e.g. a
+        // capture made for two-token tiles replayed on a four-token batch).  The row cannot be computed here;
+        // it is entered as an empty state, so that the combine merges nothing stale, and the tile's output is
+        // then wrong in a visible way (zeros for a tile with no other row) rather than silently mixed.
         const uint32_t rows = a.rows_per_split_head;
         for (uint32_t idx = threadIdx.x; idx < ncols * (D / 4); idx += 64 * kWaves) {
             const uint32_t c = idx / (D / 4), d4 = idx % (D / 4);
@@ -721,8 +338,10 @@ __global__ __launch_bounds__(64 * tiled_paired_waves(NB), 1) void split_kv_tiled
     }
     if (lds_in_use) __syncthreads();  // the previous row's merge buffer has been read out
     lds_in_use = true;
+    // Lane coordinates, re-derived per row from a value the optimiser cannot see through: nothing computed from
+    // them is loop-invariant, so no per-lane address survives from one row into the next row's register budget.
     uint32_t tid = threadIdx.x;
-    asm volatile("" : "+v"(tid));  // lane coordinates re-derived per row (see split_kv_tiled_map)
+    asm volatile("" : "+v"(tid));
     const uint32_t lane = tid & 63;
     const uint32_t mt = lane & 15, mc = lane >> 4;
 
@@ -898,7 +517,7 @@ __global__ __launch_bounds__(64 * tiled_paired_waves(NB), 1) void split_kv_tiled
             }
 
             if constexpr (kBlocks > 0) {
-                // ---- online softmax per column over this lane's tokens 4*mc + r (see split_kv_tiled_map); nearly
+                // ---- online softmax per column over this lane's tokens 4*mc + r; nearly
                 // every tile lies inside the range of every column and needs no mask
                 ProbOperand<Tag> pa[kB];
                 float alpha[kB];
@@ -1060,17 +679,6 @@ inline int launch_tiled_map_typed(psi_hip_ctx* ctx, const Geometry& g, const Map
     const dim3 grid((a.worker_cu ? a.num_workers : a.num_total_kv_splits) * g.hkv);
     const uint16_t* q = reinterpret_cast<const uint16_t*>(a.q);
     const uint16_t* pages = reinterpret_cast<const uint16_t*>(a.kv_pages);
-#define PSI_TILED_LAUNCH(NB, CG)                                                                                       \
-    do {                                                                                                               \
-        if (g.tokens_per_page == 8)                                                                                    \
-            hipLaunchKernelGGL((split_kv_tiled_map<Tag, D, NB, CG, true>), grid, dim3(64 * kTiledTileWaves * CG), 0,    \
-                               ctx->stream, a, a.walk.page_ids, a.kv_splits, a.req_slots, q, pages, a.q_token_tiles,   \
-                               a.flat_token_indices, a.worker_cu);                                                     \
-        else                                                                                                           \
-            hipLaunchKernelGGL((split_kv_tiled_map<Tag, D, NB, CG, false>), grid, dim3(64 * kTiledTileWaves * CG), 0,   \
-                               ctx->stream, a, a.walk.page_ids, a.kv_splits, a.req_slots, q, pages, a.q_token_tiles,   \
-                               a.flat_token_indices, a.worker_cu);                                                     \
-    } while (0)
 #define PSI_TILED_PAIRED_LAUNCH(NB)                                                                                    \
     do {                                                                                                               \
         if (g.tokens_per_page == 8)                                                                                    \
@@ -1085,9 +693,7 @@ inline int launch_tiled_map_typed(psi_hip_ctx* ctx, const Geometry& g, const Map
     if (nb == 1) PSI_TILED_PAIRED_LAUNCH(1);
     else if (nb == 2) PSI_TILED_PAIRED_LAUNCH(2);
     else if (nb == 3) PSI_TILED_PAIRED_LAUNCH(3);
-    else if (nb <= 4) PSI_TILED_LAUNCH(2, 2);
-    else return PSI_HIP_ERR_UNSUPPORTED;
-#undef PSI_TILED_LAUNCH
+    else return PSI_HIP_ERR_UNSUPPORTED;  // (wider tiles: see launch_tiled_map_fast)
 #undef PSI_TILED_PAIRED_LAUNCH
     return PSI_HIP_OK;
 }

@@ -44,7 +44,7 @@ def test_prefill_chunk_on_prefix(psi, oracle, device, partition):
     ("Float32", 4, 2, 64, 4, 3),
     ("Bfloat16", 24, 4, 256, 8, 8),  # the reference's (256, 8) profile, full tiles
     ("Float16", 8, 1, 128, 8, 3),
-    ("Float16", 16, 2, 256, 16, 8),   # 8 heads per KV head, full tiles: 64 columns, the two-group kernel
+    ("Float16", 16, 2, 256, 16, 8),   # 8 heads per KV head, full tiles: 64 columns: the row-group kernel, a row per group
     ("Bfloat16", 16, 2, 256, 16, 7),  # 56 columns
 ])
 def test_tiled_geometries(psi, oracle, device, dtype_name, hq, hkv, d, p, q_len):
@@ -436,7 +436,7 @@ def test_grouped_and_plain_maps_agree(psi, oracle, device):
     ("Bfloat16", 24, 4, 256, 16, 2),                        # one-draft verify: one column block
     ("Bfloat16", 24, 4, 256, 16, 4),                        # three drafts: two column blocks
     ("Bfloat16", 24, 4, 256, 16, [8, 3, 1, 8, 5, 2, 7]),    # full tiles: three column blocks, the loading wave takes one
-    ("Bfloat16", 16, 2, 256, 16, [8, 2, 8, 1, 8, 3, 8]),    # 64 columns: the two-group kernel
+    ("Bfloat16", 16, 2, 256, 16, [8, 2, 8, 1, 8, 3, 8]),    # 64 columns: the row-group kernel, a row per group
     ("Float16", 16, 2, 256, 8, 3),                          # 8-token pages
     ("Bfloat16", 32, 8, 128, 16, [20, 1, 9, 2, 1, 1, 12]),  # several Q-token tiles per request
     ("Float32", 6, 2, 64, 8, 2),                            # generic kernels: one workgroup per row
@@ -456,5 +456,7 @@ def test_balanced_plan_for_multi_query_rows(psi, oracle, device, dtype_name, hq,
     assert dw.balanced and dw.shape.num_sdpa_map_task_templates <= dw.meta.num_workers + dw.shape.num_q_token_tiles
     plain = wl.DeviceWorkload(device, w, partition_tokens=512, variant=variant, f32_output=True, max_tokens=64)
     plain.step()
-    # f16 probabilities are one 11-bit term: their rounding depends on where the rows are cut
-    assert np.abs(plain.output_f32() - dw.output_f32()).max() < (2e-4 if dtype_name == "Float16" else 2e-5)
+    # f16 probabilities are one 11-bit term: their rounding depends on where the rows are cut (the row-group kernel
+    # rounds them to f16 for bf16 K/V, too)
+    one_term = dtype_name == "Float16" or hq // hkv * 8 > 48
+    assert np.abs(plain.output_f32() - dw.output_f32()).max() < (2e-4 if one_term else 2e-5)
