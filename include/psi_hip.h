@@ -634,10 +634,17 @@ typedef struct psi_hip_gqa_layer_input {
 #define PSI_HIP_DISPATCH_LONGEST_FIRST 1u /* psi_hip_split_kv_order_longest_first */
 #define PSI_HIP_DISPATCH_BALANCED 2u      /* psi_hip_split_kv_balance_plan */
 #define PSI_HIP_DISPATCH_ROW_GROUPS 3u    /* psi_hip_split_kv_tiled_q_group_rows (TiledQ; SingleQ batches get BALANCED) */
+#define PSI_HIP_DISPATCH_AUTO 4u          /* per batch: ROW_GROUPS over the partition length of
+                                             psi_hip_split_kv_chunk_partition_tokens when the batch is TiledQ with
+                                             FIXED_PARTITION capacities, the host arrays hold a row-group table, and a
+                                             request brings more than one Q-token tile or a tile more than 48 query
+                                             columns (new tokens x Q heads per KV head); BALANCED over
+                                             partition_tokens otherwise */
 
 typedef struct psi_hip_gqa_plan_options {
     uint32_t capacity_mode;           /* PSI_HIP_CAPACITY_* */
-    uint32_t partition_tokens;        /* FIXED_PARTITION (prefill chunks: see psi_hip_split_kv_chunk_partition_tokens) */
+    uint32_t partition_tokens;        /* FIXED_PARTITION; with ROW_GROUPS 0 = what
+                                         psi_hip_split_kv_chunk_partition_tokens answers for the batch */
     uint32_t caller_num_total_tokens; /* CALLER_TOKENS */
     uint32_t dispatch;                /* PSI_HIP_DISPATCH_* */
     uint32_t num_workers;             /* BALANCED: workers per KV head, 0 = psi_hip_split_kv_balanced_workers */

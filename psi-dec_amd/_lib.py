@@ -26,7 +26,7 @@ FLAG_MUTE_LOADERS = 3
 DEVICE_ERR_WAIT_GAVE_UP = 1
 DEVICE_ERR_V_RANGE = 2
 REPLAY_EXACT, REPLAY_BUCKETED = 0, 1
-DISPATCH_PLAN_ORDER, DISPATCH_LONGEST_FIRST, DISPATCH_BALANCED, DISPATCH_ROW_GROUPS = 0, 1, 2, 3
+DISPATCH_PLAN_ORDER, DISPATCH_LONGEST_FIRST, DISPATCH_BALANCED, DISPATCH_ROW_GROUPS, DISPATCH_AUTO = 0, 1, 2, 3, 4
 STATIC_SCRATCH_BYTES = 16 << 20
 
 

@@ -306,7 +306,7 @@ extern "C" int psi_hip_gqa_layer_prepare(const psi_hip_gqa_layer_config* cfg, co
     PSI_REQUIRE(host->req_slots_by_token && host->flat_token_indices && host->q_token_tiles && host->kv_splits &&
                     host->cu_kv_splits,
                 "GQA prepare: the metadata arrays must not be null");
-    PSI_REQUIRE(options->dispatch <= PSI_HIP_DISPATCH_ROW_GROUPS, "unknown dispatch plan %u", options->dispatch);
+    PSI_REQUIRE(options->dispatch <= PSI_HIP_DISPATCH_AUTO, "unknown dispatch plan %u", options->dispatch);
     psi_hip_split_kv_variant chosen;
     int rc;
     if (variant != nullptr) {
@@ -318,7 +318,38 @@ extern "C" int psi_hip_gqa_layer_prepare(const psi_hip_gqa_layer_config* cfg, co
     }
     const bool tiled = chosen.kind == PSI_HIP_VARIANT_TILED_Q;
     uint32_t dispatch = options->dispatch;
+    uint32_t partition_tokens = options->partition_tokens;
+    if (dispatch == PSI_HIP_DISPATCH_AUTO) {
+        // Row groups where they are the faster launch: a request brings more than one Q-token tile (the plain map
+        // walks its KV range once per tile), or a tile more query columns than the multi-query pipeline holds.
+        dispatch = PSI_HIP_DISPATCH_BALANCED;
+        if (tiled && host->row_groups != nullptr && options->capacity_mode == PSI_HIP_CAPACITY_FIXED_PARTITION &&
+            cfg->attention.num_kv_heads != 0) {
+            uint32_t most = 0;
+            for (uint32_t r = 0; r < num_reqs; ++r)
+                if (cu_tokens[r + 1] > cu_tokens[r]) most = std::max(most, cu_tokens[r + 1] - cu_tokens[r]);
+            const uint32_t heads = cfg->attention.num_q_heads / cfg->attention.num_kv_heads;
+            uint32_t planned = 0;
+            if (most > chosen.q_token_tile_size || most * heads > 48) {
+                rc = psi_hip_split_kv_chunk_partition_tokens(&cfg->attention, chosen.q_token_tile_size, token_indices,
+                                                             cu_tokens, num_reqs, 0, &planned);
+                if (rc != PSI_HIP_OK) return rc;
+            }
+            if (planned != 0) {  // (0: no row-group kernel for the geometry)
+                dispatch = PSI_HIP_DISPATCH_ROW_GROUPS;
+                partition_tokens = planned;
+            }
+        }
+    }
     if (dispatch == PSI_HIP_DISPATCH_ROW_GROUPS && !tiled) dispatch = PSI_HIP_DISPATCH_BALANCED;
+    if (dispatch == PSI_HIP_DISPATCH_ROW_GROUPS && partition_tokens == 0 &&
+        options->capacity_mode == PSI_HIP_CAPACITY_FIXED_PARTITION) {
+        rc = psi_hip_split_kv_chunk_partition_tokens(&cfg->attention, chosen.q_token_tile_size, token_indices, cu_tokens,
+                                                     num_reqs, 0, &partition_tokens);
+        if (rc != PSI_HIP_OK) return rc;
+        PSI_REQUIRE(partition_tokens != 0,
+                    "GQA prepare: no row-group kernel for this geometry, so no partition length to plan; pass one");
+    }
     uint32_t workers = 0;
     if (dispatch == PSI_HIP_DISPATCH_BALANCED || dispatch == PSI_HIP_DISPATCH_ROW_GROUPS) {
         workers = options->num_workers;
@@ -347,7 +378,7 @@ extern "C" int psi_hip_gqa_layer_prepare(const psi_hip_gqa_layer_config* cfg, co
     psi_hip_gqa_replay_shape shape;
     rc = psi_hip_gqa_metadata_update(host->max_tokens, req_slots, token_indices, cu_tokens, num_reqs, &chosen,
                                      options->capacity_mode, options->caller_num_total_tokens,
-                                     options->topology_boundaries, options->num_boundaries, options->partition_tokens,
+                                     options->topology_boundaries, options->num_boundaries, partition_tokens,
                                      plan_capacity, host->req_slots_by_token, host->flat_token_indices,
                                      host->q_token_tiles, plan_rows, plan_cu, &shape);
     if (rc != PSI_HIP_OK) return rc;

@@ -808,7 +808,7 @@ class GQAMetadataBuffers:
         """The host arrays as psi_hip_gqa_layer_prepare takes them (`psi_hip_gqa_host_metadata`); waits until the last
         upload has left the staging block."""
         self._staging_free()
-        if dispatch == L.DISPATCH_ROW_GROUPS and self._row_groups_words() == 0:
+        if dispatch in (L.DISPATCH_ROW_GROUPS, L.DISPATCH_AUTO) and self._row_groups_words() == 0:
             self._alloc_row_groups((self._max_kv_splits + self._max_workers) * 32)
         if self._host_struct is None or self._host_struct.row_groups_capacity != self._row_groups_words():
             def addr(a):
@@ -1366,13 +1366,16 @@ class GQA:
                                 balanced: bool = True, grouped: bool = False,
                                 variant: Optional[GQASplitKVVariant] = None, num_workers: int = 0,
                                 bucket_capacities: bool = False,
-                                policy: Optional[GQAReplayBucketPolicy] = None) -> GQAReplayShape:
+                                policy: Optional[GQAReplayBucketPolicy] = None, auto: bool = False) -> GQAReplayShape:
         """Not in the reference: partitions of fixed length instead of the greedy budget, then (by default) the
         balanced worker plan that gives every compute unit an equal share of the batch's tiles; `grouped`
-        selects the row-group plan of the prefill-chunk map instead.  One host call and one upload.
-        `bucket_capacities`: the recorded capacities (the re-cut row count included) are rounded up to
-        `ReplayBucketPolicy` buckets, so that a `GQAReplayCache` keeps one program per bucket."""
-        dispatch = (L.DISPATCH_ROW_GROUPS if grouped else L.DISPATCH_BALANCED if balanced else L.DISPATCH_PLAN_ORDER)
+        selects the row-group plan of the prefill-chunk map instead (`partition_tokens` 0: the planner's), and `auto`
+        lets the library pick between the two per batch (PSI_HIP_DISPATCH_AUTO: row groups over the planner's
+        partition when a request brings more than one Q-token tile or a tile more than 48 query columns).  One host
+        call and one upload.  `bucket_capacities`: the recorded capacities (the re-cut row count included) are rounded
+        up to `ReplayBucketPolicy` buckets, so that a `GQAReplayCache` keeps one program per bucket."""
+        dispatch = (L.DISPATCH_AUTO if auto else L.DISPATCH_ROW_GROUPS if grouped else
+                    L.DISPATCH_BALANCED if balanced else L.DISPATCH_PLAN_ORDER)
         return batch_metadata.prepare(self.struct(), req_slots, token_indices, cu_tokens,
                                       capacity_mode=L.CAPACITY_FIXED_PARTITION, partition_tokens=partition_tokens,
                                       dispatch=dispatch, num_workers=num_workers, variant=variant,

@@ -183,9 +183,11 @@ class DeviceWorkload:
                  max_tokens: Optional[int] = None, variant: Optional[G.GQASplitKVVariant] = None,
                  f32_output: bool = False, balanced: bool = False, longest_first: bool = False,
                  grouped: bool = False, fused_append: bool = False, num_workers: Optional[int] = None,
-                 pages=None, page_ids=None):
+                 pages=None, page_ids=None, auto: bool = False):
         """`pages` / `page_ids`: an arena and a page table already on the device (shared with another workload
-        of the same step) instead of this workload's own."""
+        of the same step) instead of this workload's own.  `auto`: the library picks the dispatch for the batch
+        (PSI_HIP_DISPATCH_AUTO): row groups over the planner's partition, or the balanced plan over
+        `partition_tokens`."""
         import torch
 
         self.device, self.w = device, w
@@ -210,10 +212,15 @@ class DeviceWorkload:
                                                         [int(t) for t in w.token_indices],
                                                         [int(c) for c in w.cu_tokens]) or None
         self.partition_tokens = partition_tokens
+        self._auto = bool(auto)
+        if auto:
+            assert partition_tokens is not None and not grouped, "auto dispatch plans over fixed partitions"
+            balanced = True
         if partition_tokens is not None:
             if variant.is_tiled():
                 tile = variant.q_token_tile_size
-                splits_cap = int(sum(-(-int(c) // partition_tokens) * -(-int(n) // tile)
+                shortest = min(partition_tokens, 256) if auto else partition_tokens  # (the planner's are 256 * k)
+                splits_cap = int(sum(-(-int(c) // shortest) * -(-int(n) // tile)
                                      for c, n in zip(w.context_lens, q_lens)))
             else:
                 splits_cap = int(sum(-(-(int(t) + i + 1) // partition_tokens)
@@ -262,13 +269,17 @@ class DeviceWorkload:
         groups) in one library call, and one upload into the metadata buffers' fixed device arrays."""
         w = self.w
         L = G.L
-        dispatch = (L.DISPATCH_ROW_GROUPS if self.grouped else L.DISPATCH_BALANCED if self.balanced else
+        dispatch = (L.DISPATCH_AUTO if self._auto else L.DISPATCH_ROW_GROUPS if self.grouped else
+                    L.DISPATCH_BALANCED if self.balanced else
                     L.DISPATCH_LONGEST_FIRST if self._longest_first else L.DISPATCH_PLAN_ORDER)
         fixed = self._partition_tokens is not None
         self.shape = self.meta.prepare(self._layer_struct, w.req_slots, w.token_indices, w.cu_tokens,
                                        capacity_mode=L.CAPACITY_FIXED_PARTITION if fixed else L.CAPACITY_EXACT,
                                        partition_tokens=self._partition_tokens or 0, dispatch=dispatch,
                                        num_workers=self._num_workers or 0, variant=self.variant)
+        if self._auto:  # what the library picked
+            self.grouped = self.meta.num_row_groups > 0
+            self.balanced = not self.grouped
         return self.shape
 
     def append(self):

@@ -44,13 +44,14 @@ def assert_outputs_close(actual, expected, what=""):
 
 
 def run_and_check(psi, oracle, device, w, what, partition_tokens=None, max_tokens=None, variant=None,
-                  check_rounded=True, balanced=False, longest_first=False, grouped=False, fused_append=False):
+                  check_rounded=True, balanced=False, longest_first=False, grouped=False, fused_append=False,
+                  **more):
     """GPU layer-step vs oracle: pages bit-exact, f32 outputs within tolerance, io-dtype outputs
     equal to the f32 outputs rounded once."""
     wl = importlib_workloads(psi)
     dw = wl.DeviceWorkload(device, w, partition_tokens=partition_tokens, max_tokens=max_tokens, variant=variant,
                            f32_output=True, balanced=balanced, longest_first=longest_first, grouped=grouped,
-                           fused_append=fused_append)
+                           fused_append=fused_append, **more)
     dw.step()
     got = dw.output_f32()
     exp_pages, exp = oracle_step(oracle, w)
@@ -63,7 +64,7 @@ def run_and_check(psi, oracle, device, w, what, partition_tokens=None, max_token
     if check_rounded and int(w.dtype) != 0:
         dw2 = wl.DeviceWorkload(device, w, partition_tokens=partition_tokens, max_tokens=max_tokens,
                                 variant=variant, f32_output=False, balanced=balanced, longest_first=longest_first,
-                                grouped=grouped, fused_append=fused_append)
+                                grouped=grouped, fused_append=fused_append, **more)
         dw2.step()
         rounded = dw2.output_f32()
         ref = oracle.to_f32(oracle.from_f32(got, oracle_dtype(oracle, w)), oracle_dtype(oracle, w))

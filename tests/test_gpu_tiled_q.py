@@ -350,6 +350,26 @@ def test_grouped_short_chunks_walk_their_range_once_for_all_heads(psi, oracle, d
     assert dw.meta.num_row_groups > 0 and dw.meta.group_tiles == width
 
 
+@pytest.mark.parametrize("hq,q_lens,expect_groups", [
+    (24, [8, 3, 8, 1], False),      # single tiles of up to 48 columns: the multi-query pipeline over a balanced plan
+    (24, [8, 16, 8, 1], True),      # a request with two Q-token tiles
+    (32, [8, 8, 2, 8], True),       # 64 columns per tile
+    (24, [1, 1, 1, 1], False),      # decode
+    (24, [200, 1, 2, 8], True),     # a prefill chunk among decode-sized requests
+])
+def test_the_library_picks_the_dispatch(psi, oracle, device, hq, q_lens, expect_groups):
+    """PSI_HIP_DISPATCH_AUTO through the one-call preparation: whichever launch it picks, the step matches the
+    oracle."""
+    wl = importlib_workloads(psi)
+    prefixes = [3000, 700, 1025, 64]
+    ctx = [a + b for a, b in zip(prefixes, q_lens)]
+    w = wl.make_workload(433, ctx, hq, 4, 256, psi.Dtype.Bfloat16, 16, q_lens=q_lens)
+    _, dw = run_and_check(psi, oracle, device, w, f"auto dispatch {hq} heads q={q_lens}", partition_tokens=512,
+                          max_tokens=512, auto=True)
+    assert dw.grouped == expect_groups and dw.balanced != expect_groups
+    assert (dw.meta.num_row_groups > 0) == expect_groups and (dw.meta.num_workers > 0) != expect_groups
+
+
 @pytest.mark.parametrize("seed", range(16))
 def test_grouped_random_batches(psi, oracle, device, seed):
     """Seeded random batches through the row-group map against the oracle: head groups 1..8, both head dims, pages

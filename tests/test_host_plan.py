@@ -681,6 +681,56 @@ def test_single_call_prepare_equals_the_step_by_step_plan(psi, seed):
             assert b.max_active_q_tile_tokens == min(int(q_lens.max()), variant.q_token_tile_size)
 
 
+@pytest.mark.parametrize("hq,q_lens,expect_groups", [
+    (24, [1, 1, 1], False),        # decode: SingleQ, balanced
+    (24, [4, 2, 4], False),        # one tile of up to 24 columns per request: the multi-query pipeline, balanced
+    (24, [8, 8, 8], False),        # 48 columns: still the pipeline
+    (24, [8, 9, 8], True),         # one request with a second Q-token tile: row groups
+    (32, [8, 8, 3], True),         # 64 columns per tile: row groups
+    (28, [7, 2, 1], True),         # 49 columns
+    (28, [6, 6, 6], False),        # 42
+    (24, [300, 1, 2], True),       # a prefill chunk among decode-sized requests
+])
+def test_prepare_picks_the_dispatch_by_the_batch(psi, hq, q_lens, expect_groups):
+    """PSI_HIP_DISPATCH_AUTO: row groups over the planner's partition when a request brings more than one Q-token
+    tile or a tile more than 48 query columns, the balanced plan over the caller's partition otherwise - and either
+    way exactly what the explicit dispatch writes."""
+    import importlib
+
+    L = importlib.import_module("psi-dec_amd._lib")
+    core = psi.GQACore(0, hq * 256, 256, hq, 4, 0.0625)
+    gqa = psi.GQA(None, core, psi.GQAMetalConfig(65536, 64, 1e-6, 1e6))
+    q_lens = np.array(q_lens)
+    starts = np.array([5000, 300, 12000], np.uint32)
+    slots = np.array([2, 0, 1], np.uint32)
+    cu = np.concatenate([[0], np.cumsum(q_lens)]).astype(np.uint32)
+    variant = psi.select_split_kv_variant(gqa.split_kv, 512, None, starts.tolist(), cu.tolist())
+    assert variant.is_tiled() == (int(q_lens.max()) > 1)
+
+    def arrays(md):
+        s = md.replay_shape()
+        return dict(shape=s, splits=md.h_kv_splits[:3 * s.num_total_sdpa_map_task_templates].tolist(),
+                    workers=None if md.h_worker_cu is None else md.h_worker_cu.tolist(),
+                    groups=None if md.h_row_groups is None or not md.num_row_groups else
+                    (md.group_tiles, md.h_row_groups[:md.group_tiles * md.num_row_groups].tolist()))
+
+    auto = psi.GQAMetadataBuffers(None, 512, max_kv_splits=2048, max_workers=8)
+    gqa.prepare_fixed_partition(auto, slots, starts, cu, 512, auto=True, num_workers=8)
+    assert (auto.num_row_groups > 0) == expect_groups
+    explicit = psi.GQAMetadataBuffers(None, 512, max_kv_splits=2048, max_workers=8)
+    if expect_groups:
+        planned = psi.chunk_partition_tokens(gqa.split_kv.config, variant.q_token_tile_size, starts.tolist(), cu.tolist())
+        assert planned > 0
+        gqa.prepare_fixed_partition(explicit, slots, starts, cu, planned, grouped=True)
+        assert arrays(auto) == arrays(explicit)
+        # a partition length of 0 asks for the planner's, too
+        gqa.prepare_fixed_partition(explicit, slots, starts, cu, 0, grouped=True)
+        assert arrays(auto) == arrays(explicit)
+    else:
+        gqa.prepare_fixed_partition(explicit, slots, starts, cu, 512, balanced=True, num_workers=8)
+        assert auto.num_workers == 8 and arrays(auto) == arrays(explicit)
+
+
 @pytest.mark.parametrize("dispatch_name", ["plan", "balanced", "groups"])
 def test_prepare_buckets_the_dispatch_plans_capacities(psi, dispatch_name):
     """With `bucket_capacities` the one-call preparation rounds the recorded capacities - tokens, Q-token tiles,
