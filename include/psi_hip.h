@@ -461,7 +461,11 @@ int psi_hip_split_kv_tiled_q_scratch_bytes(const psi_hip_gqa_config* cfg, uint32
  * tile holds, e.g. 2 for a verify step with one draft; it sizes the kernel's query-column blocks.
  * 0 = unknown, any tile may hold q_token_tile_size tokens.  It is a contract, not a hint: it must bound every
  * batch the launch serves, including every batch later replayed on a graph captured from this call.  A row whose
- * tile holds more tokens is entered as an empty partial state (its keys are not attended). */
+ * tile holds more tokens is entered as an empty partial state (its keys are not attended).
+ * Kernels, for bf16 / f16 with head_dim 128 or 256 and pages of 8 * 2^k tokens: up to 48 query columns per tile
+ * (max_active_q_tile_tokens x Q heads per KV head) the multi-query pipeline; 49 to 64 the row-group kernel with every
+ * row a group of its own (its probabilities are rounded to f16 for bf16 K/V, too, and it needs the context's work
+ * counters: see psi_hip_ctx_create).  Everything else: the shape-generic kernel. */
 int psi_hip_split_kv_tiled_q_map(psi_hip_ctx* ctx, const psi_hip_gqa_config* cfg,
                                  const psi_hip_page_table_layout* layout, uint32_t q_token_tile_size,
                                  const void* q, const void* kv_pages, uint64_t kv_pages_bytes,
