@@ -136,7 +136,9 @@ int psi_hip_ctx_set_flag(psi_hip_ctx* ctx, uint32_t flag, uint32_t value);
  *   WAIT_GAVE_UP  a wave's bounded wait for another wave of its workgroup ran out (multi-query map);
  *   V_RANGE       the prefill-chunk map met a V element of a bf16 cache that f16 cannot hold (finite
  *                 |v| > 65504, Inf or NaN): that map multiplies V as f16.  Run the batch through
- *                 psi_hip_split_kv_tiled_q_map instead, which keeps V in the storage type.
+ *                 psi_hip_split_kv_tiled_q_map instead, which keeps V in the storage type -- except for tiles of
+ *                 more than 48 query columns, which that entry point hands to the same kernel: for those, set
+ *                 PSI_HIP_FLAG_FORCE_GENERIC for the step (the shape-generic kernels multiply in f32).
  * psi_hip_sync returns PSI_HIP_ERR_RUNTIME while a bit is set; psi_hip_ctx_take_device_error
  * synchronises the context's stream, returns the bits and clears them. */
 #define PSI_HIP_DEVICE_ERR_WAIT_GAVE_UP 1u
@@ -464,8 +466,9 @@ int psi_hip_split_kv_tiled_q_scratch_bytes(const psi_hip_gqa_config* cfg, uint32
  * tile holds more tokens is entered as an empty partial state (its keys are not attended).
  * Kernels, for bf16 / f16 with head_dim 128 or 256 and pages of 8 * 2^k tokens: up to 48 query columns per tile
  * (max_active_q_tile_tokens x Q heads per KV head) the multi-query pipeline; 49 to 64 the row-group kernel with every
- * row a group of its own (its probabilities are rounded to f16 for bf16 K/V, too, and it needs the context's work
- * counters: see psi_hip_ctx_create).  Everything else: the shape-generic kernel. */
+ * row a group of its own (for bf16 K/V, too, it rounds the probabilities to f16 and multiplies V as f16, reporting
+ * V values beyond f16's range as PSI_HIP_DEVICE_ERR_V_RANGE; it uses the context's work counters: see
+ * psi_hip_ctx_create).  Everything else: the shape-generic kernel. */
 int psi_hip_split_kv_tiled_q_map(psi_hip_ctx* ctx, const psi_hip_gqa_config* cfg,
                                  const psi_hip_page_table_layout* layout, uint32_t q_token_tile_size,
                                  const void* q, const void* kv_pages, uint64_t kv_pages_bytes,

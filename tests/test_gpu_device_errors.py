@@ -116,6 +116,36 @@ def test_chunk_map_reports_v_beyond_f16(psi, oracle, device):
     assert (err <= 2e-3 * np.maximum(1.0, np.abs(exp))).all()
 
 
+def test_wide_tiles_report_v_beyond_f16_and_the_generic_kernels_take_it(psi, oracle, device):
+    """Tiles of more than 48 query columns (8 tokens x 8 heads per KV head) go to the row-group kernel through every
+    entry point, so a V element beyond f16 is reported there too; the shape-generic kernels, which multiply in f32,
+    give the oracle's result on the same batch."""
+    L = _lib(psi)
+    wl = importlib_workloads(psi)
+    w = wl.make_workload(95, [700, 40, 1300], 16, 2, 256, psi.Dtype.Bfloat16, 16, q_lens=8, host_pages=True)
+    _set_v(w, psi, wl, 0, 37, 1, 5, 1.0e5)
+    _set_v(w, psi, wl, 2, 901, 0, 200, -3.0e7)
+    _, exp = oracle_step(oracle, w)
+    for how in (dict(balanced=True), dict()):
+        dw = wl.DeviceWorkload(device, w, partition_tokens=256, max_tokens=64, f32_output=True, **how)
+        dw.step()
+        with pytest.raises(psi.PsiHipError, match="f16 range"):
+            device.sync()
+        assert device.take_device_error() == L.DEVICE_ERR_V_RANGE
+    device.force_generic(True)
+    try:
+        slow = wl.DeviceWorkload(device, w, partition_tokens=256, max_tokens=64, f32_output=True)
+        slow.step()
+        got = slow.output_f32()
+        assert device.take_device_error() == 0
+    finally:
+        device.force_generic(False)
+    exp = np.asarray(exp, dtype=np.float64).ravel()
+    err = np.abs(got.ravel() - exp)
+    assert np.sqrt((err ** 2).sum() / (exp ** 2).sum()) <= 1e-3
+    assert (err <= 2e-3 * np.maximum(1.0, np.abs(exp))).all()
+
+
 def test_chunk_map_keeps_small_v(psi, oracle, device):
     """V magnitudes around 1e-6 lie below f16's normal range (6.1e-5): as f16 they keep an absolute spacing of
     6e-8, so each output element, a convex combination of them, is within 3e-8 of the oracle's - far inside the
