@@ -146,7 +146,7 @@ struct ChunkLds {
 
 // One work item: (row group, kv_head, part of the query heads) = item / (head_subsets * hkv), item / head_subsets %
 // hkv, item % head_subsets.  `next_item` (thread 0's) and `claimed`: see the kernel below.
-template <typename Tag, int D>
+template <typename Tag, int D, bool kTable>
 __device__ __forceinline__ void chunk_map_item(
     const MapArgs& a, const uint32_t* __restrict__ page_ids, const uint32_t* __restrict__ kv_splits,
     const uint32_t* __restrict__ req_slots, const uint16_t* __restrict__ q, const uint16_t* __restrict__ pages,
@@ -190,9 +190,9 @@ __device__ __forceinline__ void chunk_map_item(
     if (group >= num_groups || subset * heads_per_subset >= a.group) return;
     const uint32_t G = min(heads_per_subset, a.group - subset * heads_per_subset);
 
-    // (no table: every kv_split row is a group of its own, group_tiles is 1)
+    // (kTable false: no table, every kv_split row is a group of its own, group_tiles is 1)
     const uint32_t* rows = row_groups + (uint64_t)group * group_tiles;
-    auto row_of = [&](uint32_t i) -> uint32_t { return row_groups != nullptr ? rows[i] : group; };
+    auto row_of = [&](uint32_t i) -> uint32_t { return kTable ? rows[i] : group; };
     const uint32_t my_row = lane < group_tiles ? row_of(lane) : kNoRow;
     const bool my_row_ok = my_row != kNoRow && my_row < a.num_active_kv_splits;
     const uint32_t num_tiles = __builtin_amdgcn_readfirstlane(__popcll(__ballot(my_row_ok)));
@@ -581,7 +581,7 @@ __device__ __forceinline__ void chunk_map_item(
 //   work_claim[0] counts the items handed out beyond the first of each workgroup, work_claim[1] the workgroups that
 // are through; the last one out sets both back to zero for the next launch (launches of a context run one after
 // the other, on its stream).
-template <typename Tag, int D>
+template <typename Tag, int D, bool kTable>
 __global__ __launch_bounds__(64 * kChunkWaves, 1) void split_kv_chunk_map(
     MapArgs a, const uint32_t* __restrict__ page_ids, const uint32_t* __restrict__ kv_splits,
     const uint32_t* __restrict__ req_slots, const uint16_t* __restrict__ q, const uint16_t* __restrict__ pages,
@@ -595,7 +595,7 @@ __global__ __launch_bounds__(64 * kChunkWaves, 1) void split_kv_chunk_map(
     while (item < num_items) {
         uint32_t next_item = 0;
         bool claimed = false;
-        chunk_map_item<Tag, D>(a, page_ids, kv_splits, req_slots, q, pages, q_token_tiles, flat_token_indices, row_groups,
+        chunk_map_item<Tag, D, kTable>(a, page_ids, kv_splits, req_slots, q, pages, q_token_tiles, flat_token_indices, row_groups,
                                group_tiles, num_groups, head_subsets, item, next_item, claimed);
         if (!claimed && threadIdx.x == 0) next_item = gridDim.x + atomicAdd(a.work_claim, 1u);
         __syncthreads();  // every wave is through with the item's LDS
@@ -609,13 +609,13 @@ __global__ __launch_bounds__(64 * kChunkWaves, 1) void split_kv_chunk_map(
     }
 }
 
-template <typename Tag, int D>
-inline int launch_chunk_map_typed(psi_hip_ctx* ctx, const Geometry& g, const MapArgs& a, const uint32_t* row_groups,
-                                  uint32_t group_tiles, uint32_t num_groups) {
+template <typename Tag, int D, bool kTable>
+inline int launch_chunk_map_form(psi_hip_ctx* ctx, const Geometry& g, const MapArgs& a, const uint32_t* row_groups,
+                                 uint32_t group_tiles, uint32_t num_groups) {
     const uint32_t subsets = chunk_launch_subsets(g.group, group_tiles, a.rows_per_split_head);
     const uint32_t num_items = num_groups * g.hkv * subsets;
     if (num_items == 0) return PSI_HIP_OK;
-    auto* kernel = &split_kv_chunk_map<Tag, D>;
+    auto* kernel = &split_kv_chunk_map<Tag, D, kTable>;
     // The kernel's LDS is above the default limit of a launch; the limit is raised once per GPU and kernel (a
     // function's attributes belong to the device it is loaded on).  How many workgroups the GPU holds at once is
     // asked then, too.
@@ -641,6 +641,18 @@ inline int launch_chunk_map_typed(psi_hip_ctx* ctx, const Geometry& g, const Map
                        reinterpret_cast<const uint16_t*>(a.kv_pages), a.q_token_tiles, a.flat_token_indices, row_groups,
                        group_tiles, num_groups, subsets, num_items);
     return PSI_HIP_OK;
+}
+
+// With a table, or without one: every kv_split row a group of its own (group_tiles 1), which is how the plain and the
+// balanced multi-query entry points launch this kernel for tiles of more than 48 query columns.
+template <typename Tag, int D>
+inline int launch_chunk_map_typed(psi_hip_ctx* ctx, const Geometry& g, const MapArgs& a, const uint32_t* row_groups,
+                                  uint32_t group_tiles, uint32_t num_groups) {
+    if (row_groups == nullptr) {
+        if (group_tiles != 1) return PSI_HIP_ERR_UNSUPPORTED;
+        return launch_chunk_map_form<Tag, D, false>(ctx, g, a, nullptr, 1, num_groups);
+    }
+    return launch_chunk_map_form<Tag, D, true>(ctx, g, a, row_groups, group_tiles, num_groups);
 }
 
 }  // namespace psi
